@@ -1,0 +1,77 @@
+"""Builds libcgptx.so (HIP kernels + C-ABI, gfx950) in-tree with hipcc.
+
+`python -m cgpt_amd.build` compiles every translation unit under
+cgpt_amd/csrc into cgpt_amd/lib/libcgptx.so. hipcc cross-compiles for gfx950
+without a GPU, so this runs in a CPU-only container.
+"""
+from __future__ import annotations
+
+import concurrent.futures
+import os
+import pathlib
+import shutil
+import subprocess
+import sys
+
+ROOT = pathlib.Path(__file__).resolve().parent.parent
+CSRC = ROOT / "cgpt_amd" / "csrc"
+LIB_DIR = ROOT / "cgpt_amd" / "lib"
+OBJ_DIR = ROOT / "build" / "obj"
+LIB_PATH = LIB_DIR / "libcgptx.so"
+
+HIPCC = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+
+DEVICE_FLAGS = [
+    "--offload-arch=gfx950",
+    "-O3",
+    "-std=c++20",
+    "-fPIC",
+    "-fno-gpu-rdc",
+    "-Wall",
+    "-Wno-unused-function",
+    # Keep the compiler from forming packed-fp32 VALU ops.
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    f"-I{ROOT / 'include'}",
+    f"-I{CSRC}",
+]
+
+
+def sources() -> list[pathlib.Path]:
+    return sorted(CSRC.glob("*.hip")) + sorted(CSRC.glob("*.cpp"))
+
+
+def _compile(src: pathlib.Path, force: bool) -> pathlib.Path:
+    obj = OBJ_DIR / (src.name + ".o")
+    deps = [src] + list(CSRC.glob("*.hpp")) + list((ROOT / "include").glob("*.h"))
+    if not force and obj.exists() and all(obj.stat().st_mtime >= d.stat().st_mtime for d in deps):
+        return obj
+    cmd = [HIPCC, *DEVICE_FLAGS, "-c", str(src), "-o", str(obj)]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    noise = "is not a recognized feature for this target"
+    err = "\n".join(line for line in proc.stderr.splitlines() if noise not in line)
+    if proc.returncode != 0:
+        raise RuntimeError(f"hipcc failed for {src.name}:\n{err}")
+    if err.strip():
+        print(err, file=sys.stderr)
+    return obj
+
+
+def build(force: bool = True, jobs: int | None = None) -> pathlib.Path:
+    """Compiles all sources (always, when force) and links the shared library."""
+    OBJ_DIR.mkdir(parents=True, exist_ok=True)
+    LIB_DIR.mkdir(parents=True, exist_ok=True)
+    srcs = sources()
+    jobs = jobs or min(8, len(srcs), os.cpu_count() or 1)
+    with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as pool:
+        objs = list(pool.map(lambda s: _compile(s, force), srcs))
+    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-rdc", "-o", str(LIB_PATH),
+           *map(str, objs)]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"link failed:\n{proc.stderr}")
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    path = build(force="--incremental" not in sys.argv)
+    print(path)

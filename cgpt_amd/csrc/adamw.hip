@@ -1,0 +1,478 @@
+// Fused multi-tensor AdamW for gfx950.
+//
+// Semantics: src/optim/adamw.cu:74-187 (gradient statistics, device-side step
+// preparation, batched update) and 269-435 (host entry points). The reference
+// launches two kernels per tensor (181 launches for the 104m model); here the
+// whole parameter list is covered by three launches:
+//   1. stats:   every block owns one 4096-element chunk of one tensor, reads the
+//               gradient with 128-bit loads and writes one partial Σ(g/scale)²;
+//               a non-finite value sets an integer flag.
+//   2. prepare: one block sums the partials in a fixed order (in double), decides
+//               skip / step++ / bias corrections / clip factor on the device.
+//   3. update:  same chunking; reads g, m, v, master, writes m, v, master, param.
+// The block → (tensor, offset) map is a binary search in a small prefix table
+// that lives in the workspace. HBM traffic per parameter: g twice, m/v/master
+// read+write, param write = 30 B with 16-bit params.
+//
+// The squared norm is order-independent here (fixed partial order), where the
+// reference adds block sums with float atomics.
+#include "common.hpp"
+
+#include <cmath>
+#include <limits>
+#include <vector>
+
+namespace cgptx {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kChunk = 4096;  // elements per block
+
+struct DeviceEntry {
+    void* parameter;
+    const void* gradient;
+    float* master;
+    float* first;
+    float* second;
+    unsigned long long count;
+    int dtype;
+    int pad;
+};
+
+struct Hyper {
+    float learning_rate, beta1, beta2, epsilon, weight_decay, loss_scale, max_grad_norm;
+};
+
+// Device-side scalars of one workspace.
+struct DeviceState {
+    unsigned int non_finite;
+    unsigned int observed_non_finite;
+    unsigned long long step;
+    float scalars[4];  // bias_correction1, bias_correction2, clip, unused
+    float squared_norm;
+    float pad;
+};
+
+__device__ __forceinline__ int find_entry(const unsigned int* __restrict__ chunk_begin, int entries,
+                                          unsigned int chunk) {
+    int lo = 0, hi = entries;  // chunk_begin[lo] <= chunk < chunk_begin[hi]
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (chunk_begin[mid] <= chunk) lo = mid; else hi = mid;
+    }
+    return lo;
+}
+
+__device__ __forceinline__ float block_sum(float v, float* stage) {
+    v = wave_sum(v);
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    if (lane == 0) stage[wave] = v;
+    __syncthreads();
+    float total = 0.0f;
+#pragma unroll
+    for (int w = 0; w < kThreads / kWave; ++w) total += stage[w];
+    return total;
+}
+
+template <typename T>
+__device__ __forceinline__ void stats_chunk(const T* __restrict__ g, unsigned long long begin, unsigned long long end,
+                                            float inv_scale_unused, float loss_scale, float& sum, bool& bad) {
+    constexpr int VEC = kVec128<T>;
+    const bool aligned = (reinterpret_cast<std::uintptr_t>(g + begin) & 15u) == 0;
+    const unsigned long long count = end - begin;
+    const unsigned long long vectors = aligned ? count / VEC : 0;
+    for (unsigned long long v = threadIdx.x; v < vectors; v += kThreads) {
+        const vec_t<float, VEC> x = vec_to_f32<T, VEC>(load_vec<T, VEC>(g + begin + v * VEC));
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            const float grad = x[e] / loss_scale;
+            if (isfinite(grad)) sum = fmaf(grad, grad, sum); else bad = true;
+        }
+    }
+    for (unsigned long long i = begin + vectors * VEC + threadIdx.x; i < end; i += kThreads) {
+        const float grad = to_f32(g[i]) / loss_scale;
+        if (isfinite(grad)) sum = fmaf(grad, grad, sum); else bad = true;
+    }
+}
+
+__global__ __launch_bounds__(kThreads) void adamw_stats_kernel(const DeviceEntry* __restrict__ entries,
+                                                              const unsigned int* __restrict__ chunk_begin,
+                                                              int entry_count, float loss_scale,
+                                                              float* __restrict__ partial, DeviceState* state) {
+    __shared__ float stage[kThreads / kWave];
+    __shared__ int any_bad;
+    if (threadIdx.x == 0) any_bad = 0;
+    __syncthreads();
+    const int e = find_entry(chunk_begin, entry_count, blockIdx.x);
+    const DeviceEntry entry = entries[e];
+    const unsigned long long begin = static_cast<unsigned long long>(blockIdx.x - chunk_begin[e]) * kChunk;
+    const unsigned long long end = begin + kChunk < entry.count ? begin + kChunk : entry.count;
+    float sum = 0.0f;
+    bool bad = false;
+    switch (entry.dtype) {
+        case CGPTX_F16: stats_chunk(static_cast<const f16_t*>(entry.gradient), begin, end, 0.f, loss_scale, sum, bad); break;
+        case CGPTX_BF16: stats_chunk(static_cast<const bf16_t*>(entry.gradient), begin, end, 0.f, loss_scale, sum, bad); break;
+        default: stats_chunk(static_cast<const float*>(entry.gradient), begin, end, 0.f, loss_scale, sum, bad); break;
+    }
+    if (bad) any_bad = 1;  // benign race: every writer stores 1
+    const float total = block_sum(sum, stage);
+    if (threadIdx.x == 0) {
+        partial[blockIdx.x] = total;
+        if (any_bad) atomicExch(&state->non_finite, 1u);
+    }
+}
+
+// One block. Fixed-order sum of the partials, then the decision logic of
+// adamw_prepare_step_kernel (src/optim/adamw.cu:166-187).
+__global__ __launch_bounds__(kThreads) void adamw_prepare_kernel(const float* __restrict__ partial,
+                                                                unsigned int partial_count, DeviceState* state,
+                                                                float beta1, float beta2, float max_grad_norm,
+                                                                int advance_step) {
+    __shared__ double stage[kThreads];
+    double sum = 0.0;
+    for (unsigned int i = threadIdx.x; i < partial_count; i += kThreads) sum += static_cast<double>(partial[i]);
+    stage[threadIdx.x] = sum;
+    __syncthreads();
+    for (int stride = kThreads / 2; stride > 0; stride >>= 1) {
+        if (threadIdx.x < stride) stage[threadIdx.x] += stage[threadIdx.x + stride];
+        __syncthreads();
+    }
+    if (threadIdx.x != 0) return;
+    const float squared = static_cast<float>(stage[0]);
+    state->squared_norm = squared;
+    if (state->non_finite != 0u || !isfinite(squared)) {
+        state->non_finite = 1u;
+        state->observed_non_finite = 1u;
+        return;
+    }
+    if (advance_step) {
+        const unsigned long long next_step = state->step + 1ull;
+        state->step = next_step;
+        state->scalars[0] = 1.0f - powf(beta1, static_cast<float>(next_step));
+        state->scalars[1] = 1.0f - powf(beta2, static_cast<float>(next_step));
+    }
+    if (isinf(max_grad_norm)) {
+        state->scalars[2] = 1.0f;
+    } else {
+        const float norm = sqrtf(squared);
+        state->scalars[2] = norm > max_grad_norm ? max_grad_norm / norm : 1.0f;
+    }
+}
+
+__global__ void adamw_reset_kernel(DeviceState* state) {
+    state->non_finite = 0u;
+    state->squared_norm = 0.0f;
+}
+
+__device__ __forceinline__ void adamw_element(float grad_raw, float& m, float& v, float& master, const Hyper& h,
+                                              float bc1, float bc2, float clip) {
+    const float grad = grad_raw / h.loss_scale * clip;
+    m = h.beta1 * m + (1.0f - h.beta1) * grad;
+    v = h.beta2 * v + (1.0f - h.beta2) * grad * grad;
+    const float normalized = m / bc1 / (sqrtf(v / bc2) + h.epsilon);
+    master = master * (1.0f - h.learning_rate * h.weight_decay) - h.learning_rate * normalized;
+}
+
+template <typename T>
+__device__ __forceinline__ void update_chunk(const DeviceEntry& entry, unsigned long long begin,
+                                             unsigned long long end, const Hyper& h, float bc1, float bc2,
+                                             float clip) {
+    constexpr int VEC = kVec128<T>;
+    T* p = static_cast<T*>(entry.parameter);
+    const T* g = static_cast<const T*>(entry.gradient);
+    const bool aligned = ((reinterpret_cast<std::uintptr_t>(p + begin) | reinterpret_cast<std::uintptr_t>(g + begin) |
+                           reinterpret_cast<std::uintptr_t>(entry.master + begin) |
+                           reinterpret_cast<std::uintptr_t>(entry.first + begin) |
+                           reinterpret_cast<std::uintptr_t>(entry.second + begin)) & 15u) == 0;
+    const unsigned long long count = end - begin;
+    const unsigned long long vectors = aligned ? count / VEC : 0;
+    for (unsigned long long vi = threadIdx.x; vi < vectors; vi += kThreads) {
+        const unsigned long long at = begin + vi * VEC;
+        const vec_t<float, VEC> gr = vec_to_f32<T, VEC>(load_vec<T, VEC>(g + at));
+        vec_t<float, VEC> mm, vv, ww;
+#pragma unroll
+        for (int q = 0; q < VEC / 4; ++q) {
+            const vec_t<float, 4> a = load_vec<float, 4>(entry.first + at + 4 * q);
+            const vec_t<float, 4> b = load_vec<float, 4>(entry.second + at + 4 * q);
+            const vec_t<float, 4> c = load_vec<float, 4>(entry.master + at + 4 * q);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                mm[4 * q + e] = a[e];
+                vv[4 * q + e] = b[e];
+                ww[4 * q + e] = c[e];
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            float m = mm[e], v = vv[e], w = ww[e];
+            adamw_element(gr[e], m, v, w, h, bc1, bc2, clip);
+            mm[e] = m;
+            vv[e] = v;
+            ww[e] = w;
+        }
+#pragma unroll
+        for (int q = 0; q < VEC / 4; ++q) {
+            vec_t<float, 4> a, b, c;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                a[e] = mm[4 * q + e];
+                b[e] = vv[4 * q + e];
+                c[e] = ww[4 * q + e];
+            }
+            store_vec<float, 4>(entry.first + at + 4 * q, a);
+            store_vec<float, 4>(entry.second + at + 4 * q, b);
+            store_vec<float, 4>(entry.master + at + 4 * q, c);
+        }
+        store_vec<T, VEC>(p + at, vec_from_f32<T, VEC>(ww));
+    }
+    for (unsigned long long i = begin + vectors * VEC + threadIdx.x; i < end; i += kThreads) {
+        float m = entry.first[i], v = entry.second[i], w = entry.master[i];
+        adamw_element(to_f32(g[i]), m, v, w, h, bc1, bc2, clip);
+        entry.first[i] = m;
+        entry.second[i] = v;
+        entry.master[i] = w;
+        p[i] = from_f32<T>(w);
+    }
+}
+
+__global__ __launch_bounds__(kThreads) void adamw_update_kernel(const DeviceEntry* __restrict__ entries,
+                                                               const unsigned int* __restrict__ chunk_begin,
+                                                               int entry_count, Hyper h,
+                                                               const DeviceState* __restrict__ state) {
+    if (state->non_finite != 0u) return;
+    const float bc1 = state->scalars[0], bc2 = state->scalars[1], clip = state->scalars[2];
+    const int e = find_entry(chunk_begin, entry_count, blockIdx.x);
+    const DeviceEntry entry = entries[e];
+    const unsigned long long begin = static_cast<unsigned long long>(blockIdx.x - chunk_begin[e]) * kChunk;
+    const unsigned long long end = begin + kChunk < entry.count ? begin + kChunk : entry.count;
+    switch (entry.dtype) {
+        case CGPTX_F16: update_chunk<f16_t>(entry, begin, end, h, bc1, bc2, clip); break;
+        case CGPTX_BF16: update_chunk<bf16_t>(entry, begin, end, h, bc1, bc2, clip); break;
+        default: update_chunk<float>(entry, begin, end, h, bc1, bc2, clip); break;
+    }
+}
+
+__global__ void adamw_set_scalars_kernel(DeviceState* state, float bc1, float bc2) {
+    state->scalars[0] = bc1;
+    state->scalars[1] = bc2;
+}
+
+int validate_options(const cgptx_adamw_options* o, const char* name) {
+    if (o == nullptr) return fail(CGPTX_INVALID_ARGUMENT, std::string(name) + ": null options");
+    if (!std::isfinite(o->learning_rate) || o->learning_rate < 0.0f || !std::isfinite(o->beta1) || o->beta1 < 0.0f ||
+        o->beta1 >= 1.0f || !std::isfinite(o->beta2) || o->beta2 < 0.0f || o->beta2 >= 1.0f ||
+        !std::isfinite(o->epsilon) || o->epsilon <= 0.0f || !std::isfinite(o->weight_decay) ||
+        o->weight_decay < 0.0f || !std::isfinite(o->loss_scale) || o->loss_scale <= 0.0f ||
+        o->max_grad_norm <= 0.0f || std::isnan(o->max_grad_norm))
+        return fail(CGPTX_INVALID_ARGUMENT, std::string(name) + ": invalid optimizer options");
+    return CGPTX_OK;
+}
+
+int validate_entry(const cgptx_adamw_entry& e, const char* name) {
+    if (e.parameter == nullptr || e.gradient == nullptr || e.master_parameter == nullptr ||
+        e.first_moment == nullptr || e.second_moment == nullptr)
+        return fail(CGPTX_INVALID_ARGUMENT, std::string(name) + ": null entry");
+    if (!valid_dtype(e.dtype)) return fail(CGPTX_INVALID_ARGUMENT, std::string(name) + ": unsupported dtype");
+    if (e.count == 0) return fail(CGPTX_INVALID_ARGUMENT, std::string(name) + ": empty tensor");
+    return CGPTX_OK;
+}
+
+Hyper to_hyper(const cgptx_adamw_options& o) {
+    return {o.learning_rate, o.beta1, o.beta2, o.epsilon, o.weight_decay, o.loss_scale, o.max_grad_norm};
+}
+
+}  // namespace
+}  // namespace cgptx
+
+struct cgptx_adamw_workspace {
+    cgptx::DeviceState* state = nullptr;       // device
+    cgptx::DeviceEntry* entries = nullptr;     // device
+    unsigned int* chunk_begin = nullptr;       // device, entry_count + 1
+    float* partial = nullptr;                  // device, total_chunks
+    std::vector<cgptx_adamw_entry> bound;      // host copy of the bound entry list
+    unsigned int total_chunks = 0;
+    bool initialized = false;
+};
+
+namespace cgptx {
+namespace {
+
+int bind_entries(cgptx_adamw_workspace* ws, const cgptx_adamw_entry* entries, std::size_t entry_count,
+                 hipStream_t stream) {
+    std::vector<DeviceEntry> host(entry_count);
+    std::vector<unsigned int> begin(entry_count + 1);
+    unsigned long long chunks = 0;
+    for (std::size_t i = 0; i < entry_count; ++i) {
+        const auto& e = entries[i];
+        host[i] = {e.parameter, e.gradient, e.master_parameter, e.first_moment, e.second_moment,
+                   static_cast<unsigned long long>(e.count), e.dtype, 0};
+        begin[i] = static_cast<unsigned int>(chunks);
+        chunks += (e.count + kChunk - 1) / kChunk;
+        if (chunks > 0x7fffffffull) return fail(CGPTX_OVERFLOW, "adamw: too many elements for one launch");
+    }
+    begin[entry_count] = static_cast<unsigned int>(chunks);
+    if (ws->entries != nullptr) CGPTX_HIP(hipFree(ws->entries));
+    if (ws->chunk_begin != nullptr) CGPTX_HIP(hipFree(ws->chunk_begin));
+    if (ws->partial != nullptr) CGPTX_HIP(hipFree(ws->partial));
+    CGPTX_HIP(hipMalloc(reinterpret_cast<void**>(&ws->entries), entry_count * sizeof(DeviceEntry)));
+    CGPTX_HIP(hipMalloc(reinterpret_cast<void**>(&ws->chunk_begin), (entry_count + 1) * sizeof(unsigned int)));
+    CGPTX_HIP(hipMalloc(reinterpret_cast<void**>(&ws->partial), chunks * sizeof(float)));
+    // Pageable sources: these copies complete before hipMemcpyAsync returns control
+    // to a later kernel on the same stream, and the vectors die at scope exit, so
+    // use the synchronous form.
+    CGPTX_HIP(hipStreamSynchronize(stream));
+    CGPTX_HIP(hipMemcpy(ws->entries, host.data(), entry_count * sizeof(DeviceEntry), hipMemcpyHostToDevice));
+    CGPTX_HIP(hipMemcpy(ws->chunk_begin, begin.data(), (entry_count + 1) * sizeof(unsigned int),
+                        hipMemcpyHostToDevice));
+    ws->total_chunks = static_cast<unsigned int>(chunks);
+    ws->bound.assign(entries, entries + entry_count);
+    return CGPTX_OK;
+}
+
+bool same_entries(const std::vector<cgptx_adamw_entry>& bound, const cgptx_adamw_entry* entries, std::size_t n) {
+    if (bound.size() != n) return false;
+    for (std::size_t i = 0; i < n; ++i) {
+        const auto &a = bound[i], &b = entries[i];
+        if (a.parameter != b.parameter || a.gradient != b.gradient || a.master_parameter != b.master_parameter ||
+            a.first_moment != b.first_moment || a.second_moment != b.second_moment || a.count != b.count ||
+            a.dtype != b.dtype)
+            return false;
+    }
+    return true;
+}
+
+}  // namespace
+}  // namespace cgptx
+
+extern "C" int cgptx_adamw_workspace_create(cgptx_adamw_workspace** workspace) {
+    using namespace cgptx;
+    if (workspace == nullptr) return fail(CGPTX_INVALID_ARGUMENT, "adamw_workspace_create: null output");
+    auto* ws = new cgptx_adamw_workspace();
+    if (int s = check_hip(hipMalloc(reinterpret_cast<void**>(&ws->state), sizeof(DeviceState)), "hipMalloc")) {
+        delete ws;
+        return s;
+    }
+    if (int s = check_hip(hipMemset(ws->state, 0, sizeof(DeviceState)), "hipMemset")) {
+        (void)hipFree(ws->state);
+        delete ws;
+        return s;
+    }
+    *workspace = ws;
+    return CGPTX_OK;
+}
+
+extern "C" int cgptx_adamw_workspace_destroy(cgptx_adamw_workspace* ws) {
+    using namespace cgptx;
+    if (ws == nullptr) return CGPTX_OK;
+    (void)hipDeviceSynchronize();
+    if (ws->state) (void)hipFree(ws->state);
+    if (ws->entries) (void)hipFree(ws->entries);
+    if (ws->chunk_begin) (void)hipFree(ws->chunk_begin);
+    if (ws->partial) (void)hipFree(ws->partial);
+    delete ws;
+    return CGPTX_OK;
+}
+
+extern "C" int cgptx_adamw_step_many_async(cgptx_adamw_workspace* ws, const cgptx_adamw_entry* entries,
+                                           size_t entry_count, const cgptx_adamw_options* options,
+                                           uint64_t initial_step, cgptx_stream stream_) {
+    using namespace cgptx;
+    const char* name = "adamw_step_many_async";
+    if (int s = validate_options(options, name)) return s;
+    if (ws == nullptr) return fail(CGPTX_INVALID_ARGUMENT, std::string(name) + ": null workspace");
+    if (entries == nullptr || entry_count == 0)
+        return fail(CGPTX_INVALID_ARGUMENT, std::string(name) + ": empty parameter list");
+    for (std::size_t i = 0; i < entry_count; ++i)
+        if (int s = validate_entry(entries[i], name)) return s;
+    auto stream = static_cast<hipStream_t>(stream_);
+    if (!ws->initialized) {
+        if (int s = bind_entries(ws, entries, entry_count, stream)) return s;
+        DeviceState init{};
+        init.step = initial_step;
+        CGPTX_HIP(hipMemcpy(ws->state, &init, sizeof(init), hipMemcpyHostToDevice));
+        ws->initialized = true;
+    } else if (!same_entries(ws->bound, entries, entry_count)) {
+        return fail(CGPTX_INVALID_ARGUMENT, std::string(name) + ": workspace entries changed");
+    }
+    const Hyper h = to_hyper(*options);
+    const int n = static_cast<int>(entry_count);
+    hipLaunchKernelGGL(adamw_reset_kernel, dim3(1), dim3(1), 0, stream, ws->state);
+    CGPTX_LAUNCH_CHECK();
+    hipLaunchKernelGGL(adamw_stats_kernel, dim3(ws->total_chunks), dim3(kThreads), 0, stream, ws->entries,
+                       ws->chunk_begin, n, h.loss_scale, ws->partial, ws->state);
+    CGPTX_LAUNCH_CHECK();
+    hipLaunchKernelGGL(adamw_prepare_kernel, dim3(1), dim3(kThreads), 0, stream, ws->partial, ws->total_chunks,
+                       ws->state, h.beta1, h.beta2, h.max_grad_norm, 1);
+    CGPTX_LAUNCH_CHECK();
+    hipLaunchKernelGGL(adamw_update_kernel, dim3(ws->total_chunks), dim3(kThreads), 0, stream, ws->entries,
+                       ws->chunk_begin, n, h, ws->state);
+    CGPTX_LAUNCH_CHECK();
+    return CGPTX_OK;
+}
+
+extern "C" int cgptx_adamw_check(cgptx_adamw_workspace* ws, int* all_finite, uint64_t* step, cgptx_stream stream_) {
+    using namespace cgptx;
+    if (ws == nullptr || all_finite == nullptr || step == nullptr)
+        return fail(CGPTX_INVALID_ARGUMENT, "adamw_check: null argument");
+    auto stream = static_cast<hipStream_t>(stream_);
+    CGPTX_HIP(hipStreamSynchronize(stream));
+    DeviceState host{};
+    CGPTX_HIP(hipMemcpy(&host, ws->state, sizeof(host), hipMemcpyDeviceToHost));
+    *all_finite = host.observed_non_finite == 0u ? 1 : 0;
+    *step = host.step;
+    const unsigned int zero = 0;
+    CGPTX_HIP(hipMemcpy(&ws->state->observed_non_finite, &zero, sizeof(zero), hipMemcpyHostToDevice));
+    return CGPTX_OK;
+}
+
+extern "C" int cgptx_adamw_step(void* parameter, const void* gradient, float* master_parameter, float* first_moment,
+                                float* second_moment, size_t count, int dtype, const cgptx_adamw_options* options,
+                                uint64_t next_step, int* updated, cgptx_stream stream_) {
+    using namespace cgptx;
+    const char* name = "adamw_step";
+    if (int s = validate_options(options, name)) return s;
+    if (updated == nullptr) return fail(CGPTX_INVALID_ARGUMENT, std::string(name) + ": null output flag");
+    const cgptx_adamw_entry entry{parameter, gradient, master_parameter, first_moment, second_moment, count, dtype};
+    if (int s = validate_entry(entry, name)) return s;
+    if (next_step == 0) return fail(CGPTX_OVERFLOW, std::string(name) + ": step counter overflow");
+    auto stream = static_cast<hipStream_t>(stream_);
+    const unsigned long long chunks = (count + kChunk - 1) / kChunk;
+    if (chunks > 0x7fffffffull) return fail(CGPTX_OVERFLOW, std::string(name) + ": tensor too large");
+    // Scratch layout: DeviceState | DeviceEntry | chunk_begin[2] | partial[chunks]
+    const std::size_t off_entry = 256, off_begin = 512, off_partial = 768;
+    void* mem = nullptr;
+    if (int s = scratch(stream, off_partial + chunks * sizeof(float), &mem)) return s;
+    auto* base = static_cast<char*>(mem);
+    auto* state = reinterpret_cast<DeviceState*>(base);
+    auto* d_entry = reinterpret_cast<DeviceEntry*>(base + off_entry);
+    auto* d_begin = reinterpret_cast<unsigned int*>(base + off_begin);
+    auto* partial = reinterpret_cast<float*>(base + off_partial);
+    const DeviceEntry h_entry{parameter, gradient, master_parameter, first_moment, second_moment,
+                              static_cast<unsigned long long>(count), dtype, 0};
+    const unsigned int h_begin[2] = {0u, static_cast<unsigned int>(chunks)};
+    DeviceState init{};
+    CGPTX_HIP(hipStreamSynchronize(stream));
+    CGPTX_HIP(hipMemcpy(state, &init, sizeof(init), hipMemcpyHostToDevice));
+    CGPTX_HIP(hipMemcpy(d_entry, &h_entry, sizeof(h_entry), hipMemcpyHostToDevice));
+    CGPTX_HIP(hipMemcpy(d_begin, h_begin, sizeof(h_begin), hipMemcpyHostToDevice));
+    const Hyper h = to_hyper(*options);
+    hipLaunchKernelGGL(adamw_stats_kernel, dim3(static_cast<unsigned int>(chunks)), dim3(kThreads), 0, stream,
+                       d_entry, d_begin, 1, h.loss_scale, partial, state);
+    CGPTX_LAUNCH_CHECK();
+    hipLaunchKernelGGL(adamw_prepare_kernel, dim3(1), dim3(kThreads), 0, stream, partial,
+                       static_cast<unsigned int>(chunks), state, h.beta1, h.beta2, h.max_grad_norm, 0);
+    CGPTX_LAUNCH_CHECK();
+    // Bias corrections in double on the host, as adamw_step does (src/optim/adamw.cu:413-415).
+    const float bc1 = static_cast<float>(1.0 - std::pow(static_cast<double>(h.beta1), static_cast<double>(next_step)));
+    const float bc2 = static_cast<float>(1.0 - std::pow(static_cast<double>(h.beta2), static_cast<double>(next_step)));
+    hipLaunchKernelGGL(adamw_set_scalars_kernel, dim3(1), dim3(1), 0, stream, state, bc1, bc2);
+    CGPTX_LAUNCH_CHECK();
+    hipLaunchKernelGGL(adamw_update_kernel, dim3(static_cast<unsigned int>(chunks)), dim3(kThreads), 0, stream,
+                       d_entry, d_begin, 1, h, state);
+    CGPTX_LAUNCH_CHECK();
+    CGPTX_HIP(hipStreamSynchronize(stream));
+    DeviceState result{};
+    CGPTX_HIP(hipMemcpy(&result, state, sizeof(result), hipMemcpyDeviceToHost));
+    *updated = result.non_finite == 0u ? 1 : 0;
+    return CGPTX_OK;
+}

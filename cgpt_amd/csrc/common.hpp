@@ -1,0 +1,110 @@
+// Shared device/host helpers for the gfx950 kernels: storage types, 128-bit
+// vector access, wavefront (64-lane) reductions, status plumbing and the
+// per-stream scratch arena.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstddef>
+#include <cstdint>
+#include <cstdio>
+#include <string>
+
+#include "cgptx.h"
+
+namespace cgptx {
+
+using bf16_t = __bf16;
+using f16_t = _Float16;
+
+constexpr int kWave = 64;
+
+template <typename T, int N>
+struct VecOf {
+    typedef T type __attribute__((ext_vector_type(N)));
+};
+template <typename T, int N>
+using vec_t = typename VecOf<T, N>::type;
+
+// Elements of T in one 128-bit access.
+template <typename T>
+constexpr int kVec128 = 16 / sizeof(T);
+
+template <typename T>
+__device__ __forceinline__ float to_f32(T v) { return static_cast<float>(v); }
+template <typename T>
+__device__ __forceinline__ T from_f32(float v) { return static_cast<T>(v); }
+
+// Round a float through storage type T (what a store followed by a load does).
+template <typename T>
+__device__ __forceinline__ float round_to(float v) { return static_cast<float>(static_cast<T>(v)); }
+
+template <typename T, int N>
+__device__ __forceinline__ vec_t<float, N> vec_to_f32(vec_t<T, N> v) {
+    return __builtin_convertvector(v, vec_t<float, N>);
+}
+template <typename T, int N>
+__device__ __forceinline__ vec_t<T, N> vec_from_f32(vec_t<float, N> v) {
+    return __builtin_convertvector(v, vec_t<T, N>);
+}
+
+template <typename T, int N>
+__device__ __forceinline__ vec_t<T, N> load_vec(const T* p) {
+    return *reinterpret_cast<const vec_t<T, N>*>(p);
+}
+template <typename T, int N>
+__device__ __forceinline__ void store_vec(T* p, vec_t<T, N> v) {
+    *reinterpret_cast<vec_t<T, N>*>(p) = v;
+}
+
+// Butterfly reductions across `width` adjacent lanes (width a power of two <= 64).
+template <int width = kWave>
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int offset = width / 2; offset > 0; offset >>= 1) v += __shfl_xor(v, offset, kWave);
+    return v;
+}
+template <int width = kWave>
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int offset = width / 2; offset > 0; offset >>= 1) v = fmaxf(v, __shfl_xor(v, offset, kWave));
+    return v;
+}
+
+inline bool is_aligned16(const void* p) { return (reinterpret_cast<std::uintptr_t>(p) & 15u) == 0; }
+
+// ---- status ---------------------------------------------------------------
+int fail(int code, const std::string& message);   // records the message, returns code
+int check_hip(hipError_t error, const char* what); // CGPTX_OK or CGPTX_RUNTIME
+void clear_error();
+
+#define CGPTX_HIP(expr)                                              \
+    do {                                                             \
+        if (int status_ = ::cgptx::check_hip((expr), #expr)) return status_; \
+    } while (0)
+
+#define CGPTX_LAUNCH_CHECK() CGPTX_HIP(hipGetLastError())
+
+inline bool valid_dtype(int dtype) { return dtype == CGPTX_F16 || dtype == CGPTX_BF16 || dtype == CGPTX_F32; }
+inline std::size_t dtype_size(int dtype) { return dtype == CGPTX_F32 ? 4 : 2; }
+
+// Calls fn.template operator()<T>() with T chosen from a dtype code.
+template <typename Fn>
+int dispatch_dtype(int dtype, Fn&& fn) {
+    switch (dtype) {
+        case CGPTX_F16: return fn.template operator()<f16_t>();
+        case CGPTX_BF16: return fn.template operator()<bf16_t>();
+        case CGPTX_F32: return fn.template operator()<float>();
+        default: return fail(CGPTX_INVALID_ARGUMENT, "unsupported dtype");
+    }
+}
+
+// ---- scratch arena ----------------------------------------------------------
+// Returns `bytes` of device scratch bound to (current device, stream), 256-byte
+// aligned. Grows by reallocation on eager calls; refuses to grow during capture.
+int scratch(hipStream_t stream, std::size_t bytes, void** out);
+
+// Number of compute units of the current device (cached).
+int compute_units();
+
+}  // namespace cgptx

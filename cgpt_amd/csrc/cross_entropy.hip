@@ -1,0 +1,185 @@
+// Dense softmax cross-entropy (loss + logits gradient) for gfx950.
+//
+// Semantics: include/ops/cross_entropy.h:25-42; arithmetic of
+// src/ops/cpu/backward/cross_entropy_backward_cpu.cpp:122-148:
+//   loss = mean_r [ y_r < V ] (log Σ_j e^{z_rj} − z_{r,y_r}),
+//   grad_rj = (softmax(z_r)_j − [j = y_r]) · scale / rows   (stored in the logits dtype).
+//
+// One block per row. Pass 1 streams the row once with 128-bit loads keeping an
+// online (max, Σexp) pair per thread; pass 2 re-reads the row (64 KB at V=32000
+// in 16-bit, still resident in L2) and writes the gradient. HBM traffic is one
+// read and one write of the logits. Per-row losses go to scratch and one block
+// adds them in a fixed order, where the reference uses a float atomicAdd
+// (src/ops/cross_entropy.cu:134-245).
+#include "common.hpp"
+
+#include <cmath>
+#include <limits>
+
+namespace cgptx {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kWaves = kThreads / kWave;
+
+struct MaxSum {
+    float m, s;
+};
+
+__device__ __forceinline__ MaxSum combine(MaxSum a, MaxSum b) {
+    const float m = fmaxf(a.m, b.m);
+    if (m == -INFINITY) return {m, 0.0f};
+    return {m, a.s * __expf(a.m - m) + b.s * __expf(b.m - m)};
+}
+
+__device__ __forceinline__ MaxSum block_combine(MaxSum v, MaxSum* stage) {
+#pragma unroll
+    for (int offset = kWave / 2; offset > 0; offset >>= 1) {
+        MaxSum other{__shfl_xor(v.m, offset, kWave), __shfl_xor(v.s, offset, kWave)};
+        v = combine(v, other);
+    }
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    if (lane == 0) stage[wave] = v;
+    __syncthreads();
+    MaxSum total = stage[0];
+#pragma unroll
+    for (int w = 1; w < kWaves; ++w) total = combine(total, stage[w]);
+    return total;
+}
+
+template <typename T, bool WithGradient>
+__global__ __launch_bounds__(kThreads) void cross_entropy_row_kernel(float* __restrict__ row_loss,
+                                                                    T* __restrict__ gradient,
+                                                                    const T* __restrict__ logits,
+                                                                    const std::uint32_t* __restrict__ targets,
+                                                                    unsigned int vocab, float factor,
+                                                                    bool vector_ok) {
+    constexpr int VEC = kVec128<T>;
+    __shared__ MaxSum stage[kWaves];
+    const std::size_t base = static_cast<std::size_t>(blockIdx.x) * vocab;
+    const T* row = logits + base;
+    const unsigned int vectors = vector_ok ? vocab / VEC : 0;
+
+    MaxSum acc{-INFINITY, 0.0f};
+    for (unsigned int v = threadIdx.x; v < vectors; v += kThreads) {
+        const vec_t<float, VEC> x = vec_to_f32<T, VEC>(load_vec<T, VEC>(row + v * VEC));
+        float vmax = x[0];
+#pragma unroll
+        for (int e = 1; e < VEC; ++e) vmax = fmaxf(vmax, x[e]);
+        if (vmax > acc.m) {
+            acc.s *= __expf(acc.m - vmax);
+            acc.m = vmax;
+        }
+        if (acc.m != -INFINITY) {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) acc.s += __expf(x[e] - acc.m);
+        }
+    }
+    for (unsigned int i = vectors * VEC + threadIdx.x; i < vocab; i += kThreads) {
+        const float x = to_f32(row[i]);
+        if (x > acc.m) {
+            acc.s *= __expf(acc.m - x);
+            acc.m = x;
+        }
+        if (acc.m != -INFINITY) acc.s += __expf(x - acc.m);
+    }
+    const MaxSum total = block_combine(acc, stage);
+    const std::uint32_t target = targets[blockIdx.x];
+    if (threadIdx.x == 0) {
+        float loss = 0.0f;
+        if (target < vocab) loss = __logf(total.s) + total.m - to_f32(row[target]);
+        row_loss[blockIdx.x] = loss;
+    }
+    if constexpr (WithGradient) {
+        const float inv = 1.0f / total.s;
+        T* out = gradient + base;
+        for (unsigned int v = threadIdx.x; v < vectors; v += kThreads) {
+            const vec_t<float, VEC> x = vec_to_f32<T, VEC>(load_vec<T, VEC>(row + v * VEC));
+            vec_t<float, VEC> g;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                float value = __expf(x[e] - total.m) * inv;
+                if (v * VEC + e == target) value -= 1.0f;
+                g[e] = value * factor;
+            }
+            store_vec<T, VEC>(out + v * VEC, vec_from_f32<T, VEC>(g));
+        }
+        for (unsigned int i = vectors * VEC + threadIdx.x; i < vocab; i += kThreads) {
+            float value = __expf(to_f32(row[i]) - total.m) * inv;
+            if (i == target) value -= 1.0f;
+            out[i] = from_f32<T>(value * factor);
+        }
+    }
+}
+
+}  // namespace
+
+// Shared with the cut-cross-entropy path: loss[0] = (Σ row_loss) / rows, fixed order.
+__global__ __launch_bounds__(256) void mean_reduce_kernel(float* __restrict__ loss,
+                                                         const float* __restrict__ row_loss, unsigned int rows,
+                                                         float inv_rows) {
+    __shared__ double stage[256];
+    double sum = 0.0;
+    for (unsigned int i = threadIdx.x; i < rows; i += 256) sum += static_cast<double>(row_loss[i]);
+    stage[threadIdx.x] = sum;
+    __syncthreads();
+    for (int stride = 128; stride > 0; stride >>= 1) {
+        if (threadIdx.x < static_cast<unsigned int>(stride)) stage[threadIdx.x] += stage[threadIdx.x + stride];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) loss[0] = static_cast<float>(stage[0]) * inv_rows;
+}
+
+namespace {
+
+int run(float* loss, void* gradient, const void* logits, const std::uint32_t* targets, std::size_t rows,
+        std::size_t vocab, float gradient_scale, int dtype, hipStream_t stream, bool with_gradient,
+        const char* name) {
+    if (!valid_dtype(dtype)) return fail(CGPTX_INVALID_ARGUMENT, std::string(name) + ": unsupported dtype");
+    if (loss == nullptr || logits == nullptr || targets == nullptr || rows == 0 || vocab == 0 ||
+        (with_gradient && gradient == nullptr))
+        return fail(CGPTX_INVALID_ARGUMENT, std::string(name) + ": invalid tensors or targets");
+    if (with_gradient && (!std::isfinite(gradient_scale) || gradient_scale <= 0.0f))
+        return fail(CGPTX_INVALID_ARGUMENT, std::string(name) + ": gradient scale must be finite and positive");
+    constexpr std::size_t i32max = std::numeric_limits<int>::max();
+    if (rows > i32max || vocab > i32max) return fail(CGPTX_OVERFLOW, std::string(name) + ": dimension exceeds int range");
+    void* mem = nullptr;
+    if (int s = scratch(stream, rows * sizeof(float), &mem)) return s;
+    auto* row_loss = static_cast<float*>(mem);
+    const float factor = gradient_scale / static_cast<float>(rows);
+    const auto r = static_cast<unsigned int>(rows), v = static_cast<unsigned int>(vocab);
+    int status = dispatch_dtype(dtype, [&]<typename T>() -> int {
+        const bool vector_ok = vocab % kVec128<T> == 0 && is_aligned16(logits) &&
+                               (!with_gradient || is_aligned16(gradient));
+        if (with_gradient) {
+            hipLaunchKernelGGL((cross_entropy_row_kernel<T, true>), dim3(r), dim3(kThreads), 0, stream, row_loss,
+                               static_cast<T*>(gradient), static_cast<const T*>(logits), targets, v, factor, vector_ok);
+        } else {
+            hipLaunchKernelGGL((cross_entropy_row_kernel<T, false>), dim3(r), dim3(kThreads), 0, stream, row_loss,
+                               static_cast<T*>(nullptr), static_cast<const T*>(logits), targets, v, factor, vector_ok);
+        }
+        CGPTX_LAUNCH_CHECK();
+        return CGPTX_OK;
+    });
+    if (status) return status;
+    hipLaunchKernelGGL(mean_reduce_kernel, dim3(1), dim3(256), 0, stream, loss, row_loss, r,
+                       1.0f / static_cast<float>(rows));
+    CGPTX_LAUNCH_CHECK();
+    return CGPTX_OK;
+}
+
+}  // namespace
+}  // namespace cgptx
+
+extern "C" int cgptx_cross_entropy_forward_backward(float* loss, void* gradient, const void* logits,
+                                                    const uint32_t* targets, size_t rows, size_t vocab,
+                                                    float gradient_scale, int dtype, cgptx_stream stream) {
+    return cgptx::run(loss, gradient, logits, targets, rows, vocab, gradient_scale, dtype,
+                      static_cast<hipStream_t>(stream), true, "cross_entropy_forward_backward");
+}
+
+extern "C" int cgptx_cross_entropy_forward(float* loss, const void* logits, const uint32_t* targets, size_t rows,
+                                           size_t vocab, int dtype, cgptx_stream stream) {
+    return cgptx::run(loss, nullptr, logits, targets, rows, vocab, 1.0f, dtype, static_cast<hipStream_t>(stream),
+                      false, "cross_entropy_forward");
+}

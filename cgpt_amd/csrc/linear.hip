@@ -1,0 +1,112 @@
+// linear_forward / linear_backward on top of the MFMA contraction kernels.
+//
+// Reference interfaces: include/ops/linear.h (Y = X·Wᵀ + b) and
+// include/ops/backward/linear_backward.h:36-46 (dX = dY·W, dW = dYᵀ·X,
+// db = Σ_rows dY), CPU arithmetic src/ops/cpu/backward/linear_backward_cpu.cpp:131-165.
+#include "gemm.hpp"
+#include "reduce.hpp"
+
+#include <limits>
+
+namespace cgptx {
+namespace {
+
+int validate(const char* name, std::size_t rows, std::size_t in_features, std::size_t out_features, int dtype) {
+    if (!valid_dtype(dtype)) return fail(CGPTX_INVALID_ARGUMENT, std::string(name) + ": unsupported dtype");
+    if (rows == 0 || in_features == 0 || out_features == 0)
+        return fail(CGPTX_INVALID_ARGUMENT, std::string(name) + ": empty shape");
+    constexpr std::size_t i32max = std::numeric_limits<int>::max();
+    if (rows > i32max || in_features > i32max || out_features > i32max)
+        return fail(CGPTX_OVERFLOW, std::string(name) + ": dimension exceeds int range");
+    return CGPTX_OK;
+}
+
+}  // namespace
+}  // namespace cgptx
+
+extern "C" int cgptx_linear_forward(void* output, const void* input, const void* weight, const void* bias,
+                                    size_t rows, size_t in_features, size_t out_features, int dtype,
+                                    cgptx_stream stream) {
+    using namespace cgptx;
+    if (int s = validate("linear_forward", rows, in_features, out_features, dtype)) return s;
+    if (output == nullptr || input == nullptr || weight == nullptr)
+        return fail(CGPTX_INVALID_ARGUMENT, "linear_forward: null tensor");
+    GemmArgs g;
+    g.a = input;
+    g.b = weight;
+    g.c = output;
+    g.bias = bias;
+    g.m = rows;
+    g.n = out_features;
+    g.k = in_features;
+    g.lda = in_features;
+    g.ldb = in_features;
+    g.ldc = out_features;
+    g.dtype = dtype;
+    return gemm(g, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int cgptx_linear_backward(void* grad_input, void* grad_weight, void* grad_bias, const void* grad_output,
+                                     const void* input, const void* weight, size_t rows, size_t in_features,
+                                     size_t out_features, int accumulate_input, int accumulate_weight,
+                                     int accumulate_bias, int dtype, cgptx_stream stream_) {
+    using namespace cgptx;
+    if (int s = validate("linear_backward", rows, in_features, out_features, dtype)) return s;
+    if (grad_output == nullptr || (grad_input != nullptr && weight == nullptr) ||
+        (grad_weight != nullptr && input == nullptr))
+        return fail(CGPTX_INVALID_ARGUMENT, "linear_backward: null tensor");
+    auto stream = static_cast<hipStream_t>(stream_);
+    if (grad_input != nullptr) {  // dX[rows, in] = dY[rows, out] · W[out, in]
+        GemmArgs g;
+        g.a = grad_output;
+        g.b = weight;
+        g.c = grad_input;
+        g.m = rows;
+        g.n = in_features;
+        g.k = out_features;
+        g.lda = out_features;
+        g.ldb = in_features;
+        g.ldc = in_features;
+        g.b_k_contiguous = false;
+        g.accumulate = accumulate_input != 0;
+        g.dtype = dtype;
+        if (int s = gemm(g, stream)) return s;
+    }
+    if (grad_weight != nullptr) {  // dW[out, in] = dYᵀ[out, rows] · X[rows, in]
+        GemmArgs g;
+        g.a = grad_output;
+        g.b = input;
+        g.c = grad_weight;
+        g.m = out_features;
+        g.n = in_features;
+        g.k = rows;
+        g.lda = out_features;
+        g.ldb = in_features;
+        g.ldc = in_features;
+        g.a_k_contiguous = false;
+        g.b_k_contiguous = false;
+        g.accumulate = accumulate_weight != 0;
+        g.dtype = dtype;
+        if (int s = gemm(g, stream)) return s;
+    }
+    if (grad_bias != nullptr) {  // db[out] = Σ_rows dY
+        const int cols = static_cast<int>(out_features);
+        const int slices = rows < 256 ? 1 : (rows < 65536 ? 64 : 256);
+        const long rows_per_slice = (static_cast<long>(rows) + slices - 1) / slices;
+        void* mem = nullptr;
+        if (int s = scratch(stream, static_cast<std::size_t>(slices) * out_features * sizeof(float), &mem)) return s;
+        auto* partial = static_cast<float*>(mem);
+        const int col_blocks = (cols + kWave - 1) / kWave;
+        return dispatch_dtype(dtype, [&]<typename T>() -> int {
+            hipLaunchKernelGGL((column_sum_partial_kernel<T>), dim3(col_blocks, slices), dim3(kReduceThreads), 0,
+                               stream, partial, static_cast<const T*>(grad_output), static_cast<long>(rows), cols,
+                               rows_per_slice);
+            CGPTX_LAUNCH_CHECK();
+            hipLaunchKernelGGL((column_partial_reduce_kernel<T>), dim3(col_blocks), dim3(kReduceThreads), 0, stream,
+                               static_cast<T*>(grad_bias), partial, slices, cols, accumulate_bias != 0 ? 1 : 0);
+            CGPTX_LAUNCH_CHECK();
+            return CGPTX_OK;
+        });
+    }
+    return CGPTX_OK;
+}

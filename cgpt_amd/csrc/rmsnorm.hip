@@ -1,0 +1,348 @@
+// RMSNorm forward and backward for gfx950.
+//
+// Backward (reference semantics: src/ops/cpu/backward/rmsnorm_backward_cpu.cpp:86-133,
+// CUDA dispatch src/ops/backward/rmsnorm_backward.cu:445-547):
+//   r = 1/sqrt(mean(x^2)+eps);  c = (sum_j dy_j w_j x_j) r^3 / H
+//   dx = dy w r - x c;          dgamma_j = sum_rows dy x r
+//
+// Fast path: one pass over x and dy. A wavefront owns 64/LPR rows at a time
+// (LPR lanes per row, 128-bit accesses), keeps the row in registers between the
+// reduction and the dx store, and accumulates its dgamma columns in registers.
+// Per-block dgamma partials go to scratch and a second small kernel sums them in
+// a fixed order, so the result does not depend on scheduling. HBM traffic is
+// read x + read dy + write dx (+ partials, ~2% at 32768x1024).
+//
+// Generic path (any H, any alignment): row kernel with a second, cache-served
+// read, then a column kernel over saved 1/rms.
+#include "common.hpp"
+#include "reduce.hpp"
+
+#include <cmath>
+#include <limits>
+
+namespace cgptx {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kWavesPerBlock = kThreads / kWave;
+
+// ------------------------------------------------------------------ fast path
+template <typename T, int LPR, int K, bool Backward>
+__global__ __launch_bounds__(kThreads) void rmsnorm_rows_kernel(
+    T* __restrict__ out,            // dx (backward) or y (forward)
+    float* __restrict__ partial,    // [gridDim.x, H] dgamma partials (backward)
+    const T* __restrict__ dy,       // backward only
+    const T* __restrict__ x, const T* __restrict__ w, int rows, int hidden, float inv_hidden, float eps) {
+    constexpr int VEC = kVec128<T>;
+    constexpr int RPW = kWave / LPR;  // rows per wavefront iteration
+    using F = vec_t<float, VEC>;
+
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    const int sub = lane % LPR;   // lane within the row
+    const int rsel = lane / LPR;  // which of the RPW rows
+
+    F wv[K];
+    F acc[K];
+    bool live[K];
+#pragma unroll
+    for (int c = 0; c < K; ++c) {
+        const int col = (c * LPR + sub) * VEC;
+        live[c] = col < hidden;
+        wv[c] = live[c] ? vec_to_f32<T, VEC>(load_vec<T, VEC>(w + col)) : F(0.0f);
+        acc[c] = F(0.0f);
+    }
+
+    const int groups = (rows + RPW - 1) / RPW;
+    const int wave_global = blockIdx.x * kWavesPerBlock + wave;
+    const int wave_count = gridDim.x * kWavesPerBlock;
+    for (int g = wave_global; g < groups; g += wave_count) {
+        const int row = g * RPW + rsel;
+        const bool row_live = row < rows;
+        const std::size_t base = static_cast<std::size_t>(row) * hidden;
+        F xv[K], gv[K];
+#pragma unroll
+        for (int c = 0; c < K; ++c) {
+            const int col = (c * LPR + sub) * VEC;
+            if (row_live && live[c]) {
+                xv[c] = vec_to_f32<T, VEC>(load_vec<T, VEC>(x + base + col));
+                if constexpr (Backward) gv[c] = vec_to_f32<T, VEC>(load_vec<T, VEC>(dy + base + col));
+            } else {
+                xv[c] = F(0.0f);
+                if constexpr (Backward) gv[c] = F(0.0f);
+            }
+        }
+        float ss = 0.0f, dd = 0.0f;
+#pragma unroll
+        for (int c = 0; c < K; ++c) {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                ss = fmaf(xv[c][e], xv[c][e], ss);
+                if constexpr (Backward) dd = fmaf(gv[c][e] * wv[c][e], xv[c][e], dd);
+            }
+        }
+        ss = wave_sum<LPR>(ss);
+        const float inv = 1.0f / sqrtf(ss * inv_hidden + eps);
+        if constexpr (Backward) {
+            dd = wave_sum<LPR>(dd);
+            const float corr = dd * inv * inv * inv * inv_hidden;
+#pragma unroll
+            for (int c = 0; c < K; ++c) {
+                F r;
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    r[e] = gv[c][e] * wv[c][e] * inv - xv[c][e] * corr;
+                    acc[c][e] = fmaf(gv[c][e], xv[c][e] * inv, acc[c][e]);
+                }
+                const int col = (c * LPR + sub) * VEC;
+                if (row_live && live[c]) store_vec<T, VEC>(out + base + col, vec_from_f32<T, VEC>(r));
+            }
+        } else {
+#pragma unroll
+            for (int c = 0; c < K; ++c) {
+                F r;
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) r[e] = xv[c][e] * inv * wv[c][e];
+                const int col = (c * LPR + sub) * VEC;
+                if (row_live && live[c]) store_vec<T, VEC>(out + base + col, vec_from_f32<T, VEC>(r));
+            }
+        }
+    }
+
+    if constexpr (Backward) {
+        // Fold the RPW row slots of the wavefront, then the block's wavefronts.
+        __shared__ float stage[kWavesPerBlock][LPR * K * VEC];
+#pragma unroll
+        for (int c = 0; c < K; ++c) {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                float v = acc[c][e];
+#pragma unroll
+                for (int offset = LPR; offset < kWave; offset <<= 1) v += __shfl_xor(v, offset, kWave);
+                if (rsel == 0) stage[wave][(c * LPR + sub) * VEC + e] = v;
+            }
+        }
+        __syncthreads();
+        for (int col = threadIdx.x; col < hidden; col += kThreads) {
+            float v = 0.0f;
+#pragma unroll
+            for (int s = 0; s < kWavesPerBlock; ++s) v += stage[s][col];
+            partial[static_cast<std::size_t>(blockIdx.x) * hidden + col] = v;
+        }
+    }
+}
+
+// --------------------------------------------------------------- generic path
+template <typename T, bool Backward>
+__global__ __launch_bounds__(kThreads) void rmsnorm_row_generic_kernel(
+    T* __restrict__ out, float* __restrict__ inv_rms, const T* __restrict__ dy, const T* __restrict__ x,
+    const T* __restrict__ w, int rows, int hidden, float inv_hidden, float eps) {
+    __shared__ float red[2][kWavesPerBlock];
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    for (int row = blockIdx.x; row < rows; row += gridDim.x) {
+        const std::size_t base = static_cast<std::size_t>(row) * hidden;
+        float ss = 0.0f, dd = 0.0f;
+        for (int col = threadIdx.x; col < hidden; col += kThreads) {
+            const float xv = to_f32(x[base + col]);
+            ss = fmaf(xv, xv, ss);
+            if constexpr (Backward) dd = fmaf(to_f32(dy[base + col]) * to_f32(w[col]), xv, dd);
+        }
+        ss = wave_sum(ss);
+        dd = wave_sum(dd);
+        __syncthreads();  // protects red[] against the previous iteration's readers
+        if (lane == 0) {
+            red[0][wave] = ss;
+            red[1][wave] = dd;
+        }
+        __syncthreads();
+        ss = 0.0f;
+        dd = 0.0f;
+#pragma unroll
+        for (int s = 0; s < kWavesPerBlock; ++s) {
+            ss += red[0][s];
+            dd += red[1][s];
+        }
+        const float inv = 1.0f / sqrtf(ss * inv_hidden + eps);
+        if constexpr (Backward) {
+            const float corr = dd * inv * inv * inv * inv_hidden;
+            if (threadIdx.x == 0) inv_rms[row] = inv;
+            for (int col = threadIdx.x; col < hidden; col += kThreads) {
+                out[base + col] = from_f32<T>(to_f32(dy[base + col]) * to_f32(w[col]) * inv -
+                                              to_f32(x[base + col]) * corr);
+            }
+        } else {
+            for (int col = threadIdx.x; col < hidden; col += kThreads) {
+                out[base + col] = from_f32<T>(to_f32(x[base + col]) * inv * to_f32(w[col]));
+            }
+        }
+    }
+}
+
+// partial[blockIdx.y, col] = sum over this block's row slice of dy*x*inv_rms.
+template <typename T>
+__global__ __launch_bounds__(kThreads) void rmsnorm_dgamma_generic_kernel(
+    float* __restrict__ partial, const T* __restrict__ dy, const T* __restrict__ x,
+    const float* __restrict__ inv_rms, int rows, int hidden, int rows_per_slice) {
+    __shared__ float stage[kWavesPerBlock][kWave];
+    const int lane = threadIdx.x & (kWave - 1);
+    const int slice = threadIdx.x / kWave;
+    const int col = blockIdx.x * kWave + lane;
+    const int row_begin = blockIdx.y * rows_per_slice;
+    const int row_end = min(rows, row_begin + rows_per_slice);
+    float v = 0.0f;
+    if (col < hidden) {
+        for (int row = row_begin + slice; row < row_end; row += kWavesPerBlock) {
+            const std::size_t index = static_cast<std::size_t>(row) * hidden + col;
+            v = fmaf(to_f32(dy[index]), to_f32(x[index]) * inv_rms[row], v);
+        }
+    }
+    stage[slice][lane] = v;
+    __syncthreads();
+    if (slice == 0 && col < hidden) {
+        float total = 0.0f;
+#pragma unroll
+        for (int s = 0; s < kWavesPerBlock; ++s) total += stage[s][lane];
+        partial[static_cast<std::size_t>(blockIdx.y) * hidden + col] = total;
+    }
+}
+
+// ------------------------------------------------------------------- dispatch
+struct FastShape {
+    int lpr = 0;
+    int k = 0;
+};
+
+template <typename T>
+FastShape pick_fast_shape(int hidden) {
+    constexpr int VEC = kVec128<T>;
+    if (hidden % VEC != 0) return {};
+    const int vecs = hidden / VEC;
+    if (vecs <= 16) return {16, 1};
+    if (vecs <= 32) return {32, 1};
+    if (vecs <= 64) return {64, 1};
+    if (vecs <= 128) return {64, 2};
+    if (vecs <= 256) return {64, 4};
+    return {};
+}
+
+template <typename T, bool Backward>
+int launch_fast(const FastShape shape, T* out, float* partial, const T* dy, const T* x, const T* w, int rows,
+                int hidden, float eps, int blocks, hipStream_t stream) {
+    const float inv_hidden = 1.0f / static_cast<float>(hidden);
+#define CGPTX_RMS_CASE(L, KK)                                                                             \
+    if (shape.lpr == L && shape.k == KK) {                                                                \
+        hipLaunchKernelGGL((rmsnorm_rows_kernel<T, L, KK, Backward>), dim3(blocks), dim3(kThreads), 0,   \
+                           stream, out, partial, dy, x, w, rows, hidden, inv_hidden, eps);                \
+        return CGPTX_OK;                                                                                  \
+    }
+    CGPTX_RMS_CASE(16, 1)
+    CGPTX_RMS_CASE(32, 1)
+    CGPTX_RMS_CASE(64, 1)
+    CGPTX_RMS_CASE(64, 2)
+    CGPTX_RMS_CASE(64, 4)
+#undef CGPTX_RMS_CASE
+    return fail(CGPTX_RUNTIME, "rmsnorm: no kernel for shape");
+}
+
+int fast_blocks(const FastShape shape, int rows) {
+    const int rpw = kWave / shape.lpr;
+    const long groups = (static_cast<long>(rows) + rpw - 1) / rpw;
+    const long wanted = (groups + kWavesPerBlock - 1) / kWavesPerBlock;
+    const long cap = static_cast<long>(compute_units()) * 4;
+    return static_cast<int>(wanted < cap ? wanted : cap);
+}
+
+int validate(const void* a, const void* b, const void* c, std::size_t rows, std::size_t hidden, float eps, int dtype,
+             const char* name) {
+    if (!valid_dtype(dtype)) return fail(CGPTX_INVALID_ARGUMENT, std::string(name) + ": unsupported dtype");
+    if (!std::isfinite(eps) || eps <= 0.0f)
+        return fail(CGPTX_INVALID_ARGUMENT, std::string(name) + ": epsilon must be finite and positive");
+    if (a == nullptr || b == nullptr || c == nullptr)
+        return fail(CGPTX_INVALID_ARGUMENT, std::string(name) + ": null tensor");
+    if (rows == 0 || hidden == 0) return fail(CGPTX_INVALID_ARGUMENT, std::string(name) + ": empty shape");
+    if (rows > static_cast<std::size_t>(std::numeric_limits<int>::max()) ||
+        hidden > static_cast<std::size_t>(std::numeric_limits<int>::max()))
+        return fail(CGPTX_INVALID_ARGUMENT, std::string(name) + ": dimensions exceed supported range");
+    return CGPTX_OK;
+}
+
+}  // namespace
+}  // namespace cgptx
+
+extern "C" int cgptx_rmsnorm_backward(void* grad_input, void* grad_weight, const void* grad_output, const void* input,
+                                      const void* weight, size_t rows, size_t hidden, float epsilon, int dtype,
+                                      cgptx_stream stream_) {
+    using namespace cgptx;
+    if (int s = validate(grad_input, grad_output, input, rows, hidden, epsilon, dtype, "rmsnorm_backward")) return s;
+    if (grad_weight == nullptr || weight == nullptr)
+        return fail(CGPTX_INVALID_ARGUMENT, "rmsnorm_backward: null weight tensor");
+    auto stream = static_cast<hipStream_t>(stream_);
+    const int r = static_cast<int>(rows), h = static_cast<int>(hidden);
+    return dispatch_dtype(dtype, [&]<typename T>() -> int {
+        auto* dx = static_cast<T*>(grad_input);
+        auto* dw = static_cast<T*>(grad_weight);
+        auto* dy = static_cast<const T*>(grad_output);
+        auto* x = static_cast<const T*>(input);
+        auto* w = static_cast<const T*>(weight);
+        const FastShape shape = pick_fast_shape<T>(h);
+        const bool aligned = is_aligned16(dx) && is_aligned16(dy) && is_aligned16(x) && is_aligned16(w);
+        const int reduce_blocks = (h + kWave - 1) / kWave;
+        if (shape.lpr != 0 && aligned) {
+            const int blocks = fast_blocks(shape, r);
+            void* mem = nullptr;
+            if (int s = scratch(stream, static_cast<std::size_t>(blocks) * hidden * sizeof(float), &mem)) return s;
+            auto* partial = static_cast<float*>(mem);
+            if (int s = launch_fast<T, true>(shape, dx, partial, dy, x, w, r, h, epsilon, blocks, stream)) return s;
+            CGPTX_LAUNCH_CHECK();
+            hipLaunchKernelGGL((column_partial_reduce_kernel<T>), dim3(reduce_blocks), dim3(kThreads), 0, stream, dw,
+                               partial, blocks, h, 0);
+            CGPTX_LAUNCH_CHECK();
+            return CGPTX_OK;
+        }
+        const int slices = r < 256 ? 1 : (r < 65536 ? 64 : 256);
+        const int rows_per_slice = (r + slices - 1) / slices;
+        void* mem = nullptr;
+        const std::size_t inv_bytes = (rows * sizeof(float) + 255) & ~std::size_t{255};
+        if (int s = scratch(stream, inv_bytes + static_cast<std::size_t>(slices) * hidden * sizeof(float), &mem))
+            return s;
+        auto* inv_rms = static_cast<float*>(mem);
+        auto* partial = reinterpret_cast<float*>(static_cast<char*>(mem) + inv_bytes);
+        const int row_blocks = r < compute_units() * 8 ? r : compute_units() * 8;
+        hipLaunchKernelGGL((rmsnorm_row_generic_kernel<T, true>), dim3(row_blocks), dim3(kThreads), 0, stream, dx,
+                           inv_rms, dy, x, w, r, h, 1.0f / static_cast<float>(h), epsilon);
+        CGPTX_LAUNCH_CHECK();
+        hipLaunchKernelGGL((rmsnorm_dgamma_generic_kernel<T>), dim3(reduce_blocks, slices), dim3(kThreads), 0, stream,
+                           partial, dy, x, inv_rms, r, h, rows_per_slice);
+        CGPTX_LAUNCH_CHECK();
+        hipLaunchKernelGGL((column_partial_reduce_kernel<T>), dim3(reduce_blocks), dim3(kThreads), 0, stream, dw,
+                           partial, slices, h, 0);
+        CGPTX_LAUNCH_CHECK();
+        return CGPTX_OK;
+    });
+}
+
+extern "C" int cgptx_rmsnorm_forward(void* output, const void* input, const void* weight, size_t rows, size_t hidden,
+                                     float epsilon, int dtype, cgptx_stream stream_) {
+    using namespace cgptx;
+    if (int s = validate(output, input, weight, rows, hidden, epsilon, dtype, "rmsnorm_forward")) return s;
+    auto stream = static_cast<hipStream_t>(stream_);
+    const int r = static_cast<int>(rows), h = static_cast<int>(hidden);
+    return dispatch_dtype(dtype, [&]<typename T>() -> int {
+        auto* y = static_cast<T*>(output);
+        auto* x = static_cast<const T*>(input);
+        auto* w = static_cast<const T*>(weight);
+        const FastShape shape = pick_fast_shape<T>(h);
+        if (shape.lpr != 0 && is_aligned16(y) && is_aligned16(x) && is_aligned16(w)) {
+            const int blocks = fast_blocks(shape, r);
+            if (int s = launch_fast<T, false>(shape, y, nullptr, nullptr, x, w, r, h, epsilon, blocks, stream)) return s;
+            CGPTX_LAUNCH_CHECK();
+            return CGPTX_OK;
+        }
+        const int row_blocks = r < compute_units() * 8 ? r : compute_units() * 8;
+        hipLaunchKernelGGL((rmsnorm_row_generic_kernel<T, false>), dim3(row_blocks), dim3(kThreads), 0, stream, y,
+                           nullptr, nullptr, x, w, r, h, 1.0f / static_cast<float>(h), epsilon);
+        CGPTX_LAUNCH_CHECK();
+        return CGPTX_OK;
+    });
+}
