@@ -1,0 +1,145 @@
+"""GPU parity tests of linear_forward / linear_backward (MFMA contraction kernels and the plain
+fallback) against the CPU checker and float64 matmuls, through the C-ABI."""
+import numpy as np
+import pytest
+import torch
+
+from cgpt_amd import ops
+from oracle import cpu_ops, oracle64
+from tests.util import DTYPES, DTYPE_IDS, TOL, assert_close, randn, to_np
+
+pytestmark = pytest.mark.gpu
+
+
+def dev(t, device):
+    return t.to(device).contiguous()
+
+
+def test_linear_backward_known_answer_and_accumulation(device):
+    """tests/linear_backward_test.cu:20-45 (F32, 2x3)."""
+    x = torch.tensor([1, 2, 3, 4, 5, 6.0]).reshape(2, 3).to(device)
+    w = torch.tensor([1, 0, 2, -1, 3, 1.0]).reshape(2, 3).to(device)
+    dy = torch.tensor([2, -1, 3, 4.0]).reshape(2, 2).to(device)
+    gi, gw, gb = torch.zeros(2, 3, device=device), torch.zeros(2, 3, device=device), torch.zeros(2, device=device)
+    ops.linear_backward(gi, gw, gb, dy, x, w)
+    assert gi.reshape(-1).tolist() == [3, -3, 3, -1, 12, 10]
+    assert gw.reshape(-1).tolist() == [14, 19, 24, 15, 18, 21]
+    assert gb.tolist() == [5, 3]
+    options = ops.LinearBackwardOptions(accumulate_input=True, accumulate_weight=True, accumulate_bias=True)
+    ops.linear_backward(gi, gw, gb, dy, x, w, None, None, options)
+    assert gi.reshape(-1).tolist() == [6, -6, 6, -2, 24, 20]
+    assert gw.reshape(-1).tolist() == [28, 38, 48, 30, 36, 42]
+    assert gb.tolist() == [10, 6]
+
+
+def test_linear_backward_batched_f16_known_answer(device):
+    """tests/linear_backward_test.cu:47-58."""
+    f16 = torch.float16
+    x = torch.tensor([1, 2, 3, 4, 5, 6, 7, 8.0]).reshape(2, 2, 2).to(f16).to(device)
+    w = torch.tensor([1, 2, 3, 4, 5, 6.0]).reshape(3, 2).to(f16).to(device)
+    dy = torch.arange(1, 13, dtype=torch.float32).reshape(2, 2, 3).to(f16).to(device)
+    gi, gw, gb = torch.empty_like(x), torch.empty_like(w), torch.empty(3, dtype=f16, device=device)
+    ops.linear_backward(gi, gw, gb, dy, x, w)
+    assert np.abs(to_np(gi).reshape(-1) - [22, 28, 49, 64, 76, 100, 103, 136]).max() <= 0.1
+    assert np.abs(to_np(gw).reshape(-1) - [118, 140, 134, 160, 150, 180]).max() <= 0.2
+    assert np.abs(to_np(gb) - [22, 26, 30]).max() <= 0.1
+
+
+def check_against_float64(got, want64, dtype, what, terms):
+    """A dot product of `terms` rounded inputs: compare relative to the result's scale."""
+    scale = max(1.0, float(np.abs(want64).max()))
+    err = np.abs(to_np(got) - want64).max()
+    assert np.isfinite(to_np(got)).all()
+    assert err <= TOL[dtype] * scale, f"{what}: abs err {err:.3e} vs scale {scale:.3e}"
+
+
+SHAPES = [  # rows, in, out
+    (5, 7, 3), (33, 20, 17), (64, 64, 64), (128, 128, 256), (256, 192, 128), (136, 64, 72), (200, 256, 264),
+    (384, 1024, 256), (1024, 320, 1024),
+]
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=DTYPE_IDS)
+@pytest.mark.parametrize("rows,fin,fout", SHAPES)
+def test_linear_forward_backward_parity(device, rows, fin, fout, dtype):
+    x, w = randn((rows, fin), dtype, 1), randn((fout, fin), dtype, 2, 0.1)
+    dy, b = randn((rows, fout), dtype, 3), randn((fout,), dtype, 4)
+    dx_, dw_, ddy_, db_ = dev(x, device), dev(w, device), dev(dy, device), dev(b, device)
+
+    y = torch.empty(rows, fout, dtype=dtype, device=device)
+    ops.linear_forward(y, dx_, dw_, None, None, db_)
+    check_against_float64(y, oracle64.linear_forward(to_np(x), to_np(w), to_np(b)), dtype, "y", fin)
+
+    gi = torch.full((rows, fin), 5.0, dtype=dtype, device=device)
+    gw = torch.full((fout, fin), 5.0, dtype=dtype, device=device)
+    gb = torch.full((fout,), 5.0, dtype=dtype, device=device)
+    ops.linear_backward(gi, gw, gb, ddy_, dx_, dw_)
+    dx64, dw64, db64 = oracle64.linear_backward(to_np(dy), to_np(x), to_np(w))
+    check_against_float64(gi, dx64, dtype, "dX", fout)
+    check_against_float64(gw, dw64, dtype, "dW", rows)
+    check_against_float64(gb, db64, dtype, "db", rows)
+
+    if rows * fin * fout <= 256 * 192 * 128:  # the scalar CPU checker is O(rows*in*out)
+        ci, cw, cb = torch.empty_like(x), torch.empty_like(w), torch.empty_like(b)
+        cpu_ops.linear_backward(ci, cw, cb, dy, x, w)
+        check_against_float64(gi, to_np(ci), dtype, "dX vs checker", fout)
+        check_against_float64(gw, to_np(cw), dtype, "dW vs checker", rows)
+        check_against_float64(gb, to_np(cb), dtype, "db vs checker", rows)
+
+    # accumulate adds the same product onto what is there
+    before = (gi.clone(), gw.clone(), gb.clone())
+    options = ops.LinearBackwardOptions(accumulate_input=True, accumulate_weight=True, accumulate_bias=True)
+    ops.linear_backward(gi, gw, gb, ddy_, dx_, dw_, None, None, options)
+    check_against_float64(gi, to_np(before[0]) + dx64, dtype, "dX accumulate", fout)
+    check_against_float64(gw, to_np(before[1]) + dw64, dtype, "dW accumulate", rows)
+    check_against_float64(gb, to_np(before[2]) + db64, dtype, "db accumulate", rows)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+def test_linear_backward_integer_valued_inputs_are_exact(device, dtype):
+    """Small integers make every product and partial sum exactly representable: the MFMA path (incl. split-K
+    for dW) must return the exact integers whatever the summation order."""
+    rows, fin, fout = 2048, 256, 128
+    g = torch.Generator().manual_seed(5)
+    x = torch.randint(-2, 3, (rows, fin), generator=g).to(dtype)
+    w = torch.randint(-2, 3, (fout, fin), generator=g).to(dtype)
+    dy = torch.randint(-1, 2, (rows, fout), generator=g).to(dtype)
+    dx64, dw64, db64 = oracle64.linear_backward(to_np(dy), to_np(x), to_np(w))
+    gi = torch.empty(rows, fin, dtype=dtype, device=device)
+    gw = torch.empty(fout, fin, dtype=dtype, device=device)
+    ops.linear_backward(gi, gw, None, dev(dy, device), dev(x, device), dev(w, device))
+    assert np.array_equal(to_np(gi), to_np(torch.tensor(dx64).to(dtype)))
+    assert np.array_equal(to_np(gw), to_np(torch.tensor(dw64).to(dtype)))
+    y = torch.empty(rows, fout, dtype=dtype, device=device)
+    ops.linear_forward(y, dev(x, device), dev(w, device))
+    assert np.array_equal(to_np(y), to_np(torch.tensor(to_np(x) @ to_np(w).T).to(dtype)))
+
+
+def test_linear_backward_layer_shapes_of_the_104m_model(device):
+    """One layer's projection shapes at 4096 of the 32768 training rows (k/v 256x1024, q/o 1024x1024,
+    gate/up 2048x1024, down 1024x2048), bf16, against float64 matmuls, run twice bit-identically."""
+    dtype = torch.bfloat16
+    rows = 4096
+    for fout, fin in ((256, 1024), (1024, 1024), (2048, 1024), (1024, 2048)):
+        x, w, dy = randn((rows, fin), dtype, 6), randn((fout, fin), dtype, 7, 0.02), randn((rows, fout), dtype, 8)
+        dx64, dw64, _ = oracle64.linear_backward(to_np(dy), to_np(x), to_np(w))
+        outs = []
+        for _ in range(2):
+            gi = torch.empty(rows, fin, dtype=dtype, device=device)
+            gw = torch.empty(fout, fin, dtype=dtype, device=device)
+            ops.linear_backward(gi, gw, None, dev(dy, device), dev(x, device), dev(w, device))
+            outs.append((gi.cpu(), gw.cpu()))
+        assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
+        check_against_float64(outs[0][0], dx64, dtype, f"dX {fout}x{fin}", fout)
+        check_against_float64(outs[0][1], dw64, dtype, f"dW {fout}x{fin}", rows)
+
+
+def test_linear_argument_errors(device):
+    x, w, dy = torch.zeros(4, 8, device=device), torch.zeros(3, 8, device=device), torch.zeros(4, 3, device=device)
+    gi, gw, gb = torch.zeros_like(x), torch.zeros_like(w), torch.zeros(3, device=device)
+    with pytest.raises(ValueError):
+        ops.linear_backward(gi, gw, gb, torch.zeros(4, 4, device=device), x, w)
+    with pytest.raises(ValueError):
+        ops.linear_backward(gi, gw, gb, dy, x.half(), w)
+    with pytest.raises(ValueError):
+        ops.linear_backward(gi, torch.zeros(3, 7, device=device), gb, dy, x, w)
