@@ -1,0 +1,669 @@
+// Causal grouped-query flash attention for gfx950: forward with log-sum-exp,
+// and the backward (delta, dQ, dK/dV) on the matrix cores.
+//
+// Reference semantics: include/ops/attention.h:47-78, include/ops/backward/attention_backward.h:24-70,
+// formulas of src/ops/cpu/backward/attention_backward_cpu.cpp:206-280:
+//   P = exp(scale·QKᵀ − LSE) (key j visible to query i iff j <= offset + i when causal),
+//   delta = rowsum(dO∘O), dS = P∘(dO·Vᵀ − delta), dQ = scale·dS·K,
+//   dK = scale·Σ_{h in group} dSᵀ·Q, dV = Σ_{h in group} Pᵀ·dO.
+//
+// Layout idea shared by the three MFMA kernels (v_mfma_f32_32x32x16, 64 lanes):
+// the score tile is always produced so that the *stationary* index of the kernel
+// is the lane and the *streamed* index lives in the lane's 16 accumulator
+// registers. Row statistics (max, sum, LSE, delta) of the stationary index are then
+// lane-private scalars, and the converted accumulator registers are, as they are,
+// the k-operand of the second product (P·V, dS·K, Pᵀ·dO, dSᵀ·Q) — nothing is
+// written back to LDS between the two products. The other operand of the second
+// product needs the streamed index as its contraction index while the tile sits in
+// LDS with the head dimension contiguous; ds_read_b64_tr_b16 delivers exactly that
+// fragment (4 streamed rows x 16 head-dim columns per 16 lanes) in the same
+// {0-3, 8-11 | 4-7, 12-15} row order the accumulator registers have.
+//
+//   forward : block = 128 queries of one (batch, q-head), wave = 32 queries;
+//             streams 64-key K/V tiles through LDS; Sᵀ = K·Qᵀ, Oᵀ += Vᵀ·Pᵀ.
+//   dQ      : same shape; Sᵀ = K·Qᵀ, dPᵀ = V·dOᵀ, dQᵀ += Kᵀ·dSᵀ.
+//   dK/dV   : block = 128 keys of one (batch, kv-head), wave = 32 keys, K/V
+//             fragments live in registers; streams 64-query Q/dO tiles of every
+//             q-head of the group through LDS, so the group sum happens in the
+//             accumulators: no atomics, results independent of scheduling.
+//             S = Q·Kᵀ, dP = dO·Vᵀ, dVᵀ += dOᵀ·P, dKᵀ += Qᵀ·dS.
+// Causal tiles above the diagonal are skipped; ragged sequence ends are masked.
+#include "common.hpp"
+
+#include <cmath>
+#include <limits>
+
+namespace cgptx {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kBlockRows = 128;  // stationary rows per block (32 per wave)
+constexpr int kStream = 64;      // streamed rows per LDS tile
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+using acc_t = vec_t<float, 16>;
+using s16x4 = vec_t<short, 4>;
+
+template <typename T>
+struct Mma;
+template <>
+struct Mma<bf16_t> {
+    using frag = vec_t<bf16_t, 8>;
+    __device__ static __forceinline__ acc_t run(frag a, frag b, acc_t c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+    }
+};
+template <>
+struct Mma<f16_t> {
+    using frag = vec_t<f16_t, 8>;
+    __device__ static __forceinline__ acc_t run(frag a, frag b, acc_t c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+    }
+};
+
+struct Params {
+    void* out0;  // forward: O      | dq: dQ | dkv: dK
+    void* out1;  // forward: unused |        | dkv: dV
+    float* lse_out;
+    const void* q;
+    const void* k;
+    const void* v;
+    const void* dout;
+    const float* lse;
+    const float* delta;
+    int batch, qs, ks, hq, hkv, d;
+    float scale;
+    int causal, offset, accumulate;
+};
+
+template <int DP>
+constexpr int lds_stride() { return DP + 8; }
+
+// Cooperative load of a [rows_in_tile x DP] tile (row-major in LDS, stride DP+8) from a
+// [.., seq, heads, d] tensor: element (r, c) comes from base[(row0 + r) * row_stride + c].
+template <typename T, int ROWS, int DP>
+__device__ __forceinline__ void load_tile(T* lds, const T* base, long row_stride, int row0, int row_limit, int d) {
+    constexpr int kChunksPerRow = DP / 8;
+    constexpr int kChunks = ROWS * kChunksPerRow;
+    using chunk_t = vec_t<unsigned int, 4>;
+#pragma unroll
+    for (int c = threadIdx.x; c < kChunks; c += kThreads) {
+        const int r = c / kChunksPerRow, col = (c % kChunksPerRow) * 8;
+        chunk_t value(0u);
+        if (row0 + r < row_limit && col < d)
+            value = *reinterpret_cast<const chunk_t*>(base + static_cast<long>(row0 + r) * row_stride + col);
+        *reinterpret_cast<chunk_t*>(lds + r * lds_stride<DP>() + col) = value;
+    }
+}
+
+// Fragment with the head dimension as contraction index, read straight from LDS:
+// lane -> tile row (row0 + lane%32), elements d = 16*step + 8*(lane/32) .. +7.
+template <typename T, int DP>
+__device__ __forceinline__ typename Mma<T>::frag direct_frag(const T* lds, int row0, int step) {
+    const int lane = threadIdx.x & 63;
+    return *reinterpret_cast<const typename Mma<T>::frag*>(lds + (row0 + (lane & 31)) * lds_stride<DP>() + step * 16 +
+                                                            (lane >> 5) * 8);
+}
+
+// Same fragment taken from global memory (for the operand that stays in registers).
+template <typename T>
+__device__ __forceinline__ typename Mma<T>::frag global_frag(const T* row_ptr, bool live, int step, int d) {
+    const int lane = threadIdx.x & 63;
+    const int col = step * 16 + (lane >> 5) * 8;
+    using frag = typename Mma<T>::frag;
+    if (live && col < d) return *reinterpret_cast<const frag*>(row_ptr + col);
+    return frag(static_cast<T>(0.0f));
+}
+
+// Fragment with tile rows as contraction index (transposing LDS read): lane -> column
+// d0 + lane%32; elements = rows kbase + {0-3, 8-11} (lanes 0-31) or {4-7, 12-15} (lanes 32-63).
+template <typename T, int DP>
+__device__ __forceinline__ typename Mma<T>::frag transposed_frag(const T* lds, int kbase, int d0) {
+    const int lane = threadIdx.x & 63;
+    const int row = kbase + (lane >> 5) * 4 + ((lane & 15) >> 2);
+    const int col = d0 + ((lane >> 4) & 1) * 16 + (lane & 3) * 4;
+    const T* p = lds + row * lds_stride<DP>() + col;
+    using lds_ptr = __attribute__((address_space(3))) s16x4*;
+    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p));
+    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p + 8 * lds_stride<DP>()));
+    vec_t<short, 8> both;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        both[e] = lo[e];
+        both[4 + e] = hi[e];
+    }
+    return __builtin_bit_cast(typename Mma<T>::frag, both);
+}
+
+// Accumulator registers 8*step .. 8*step+7 as a 16-bit k-operand.
+template <typename T>
+__device__ __forceinline__ typename Mma<T>::frag acc_frag(const acc_t& acc, int step) {
+    vec_t<float, 8> f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) f[e] = acc[8 * step + e];
+    return vec_from_f32<T, 8>(f);
+}
+
+// Streamed index of accumulator register i: 8*(i/4) + 4*(lane/32) + i%4.
+__device__ __forceinline__ int acc_row(int i) { return 8 * (i >> 2) + 4 * ((threadIdx.x & 63) >> 5) + (i & 3); }
+
+// ------------------------------------------------------------------- forward
+template <typename T, int DP>
+__global__ __launch_bounds__(kThreads) void attention_forward_kernel(Params p) {
+    constexpr int STEPS = DP / 16, DT = DP / 32;
+    __shared__ __align__(16) T k_lds[kStream * lds_stride<DP>()];
+    __shared__ __align__(16) T v_lds[kStream * lds_stride<DP>()];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int b = blockIdx.z, h = blockIdx.y, kvh = h / (p.hq / p.hkv);
+    const int q_block = blockIdx.x * kBlockRows;
+    const int q_row = q_block + wave * 32 + (lane & 31);
+    const bool q_live = q_row < p.qs;
+    const long q_stride = static_cast<long>(p.hq) * p.d, kv_stride = static_cast<long>(p.hkv) * p.d;
+    const T* q_ptr = static_cast<const T*>(p.q) + (static_cast<long>(b) * p.qs + q_row) * q_stride + h * p.d;
+    const T* k_base = static_cast<const T*>(p.k) + static_cast<long>(b) * p.ks * kv_stride + kvh * p.d;
+    const T* v_base = static_cast<const T*>(p.v) + static_cast<long>(b) * p.ks * kv_stride + kvh * p.d;
+
+    typename Mma<T>::frag qf[STEPS];
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) qf[s] = global_frag<T>(q_ptr, q_live, s, p.d);
+
+    acc_t o[DT];
+#pragma unroll
+    for (int t = 0; t < DT; ++t) o[t] = acc_t(0.0f);
+    float m = -INFINITY, l = 0.0f;
+    const float scale2 = p.scale * kLog2e;
+    const int last_q_block = min(q_block + kBlockRows, p.qs) - 1;
+    const int k_end = p.causal ? min(p.ks, p.offset + last_q_block + 1) : p.ks;
+    const int wave_last_q = min(q_block + wave * 32 + 31, p.qs - 1);
+    const int q_limit = p.causal ? p.offset + q_row : p.ks;  // largest visible key of this lane's query
+
+    for (int k0 = 0; k0 < k_end; k0 += kStream) {
+        __syncthreads();
+        load_tile<T, kStream, DP>(k_lds, k_base, kv_stride, k0, p.ks, p.d);
+        load_tile<T, kStream, DP>(v_lds, v_base, kv_stride, k0, p.ks, p.d);
+        __syncthreads();
+        if (q_block + wave * 32 >= p.qs) continue;
+        if (p.causal && k0 > p.offset + wave_last_q) continue;
+        acc_t st[2];
+#pragma unroll
+        for (int sub = 0; sub < 2; ++sub) {
+            st[sub] = acc_t(0.0f);
+#pragma unroll
+            for (int s = 0; s < STEPS; ++s)
+                st[sub] = Mma<T>::run(direct_frag<T, DP>(k_lds, sub * 32, s), qf[s], st[sub]);
+        }
+        float tile_max = -INFINITY;
+#pragma unroll
+        for (int sub = 0; sub < 2; ++sub) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int key = k0 + sub * 32 + acc_row(i);
+                const bool visible = key < p.ks && key <= q_limit;
+                const float s = visible ? st[sub][i] * scale2 : -INFINITY;
+                st[sub][i] = s;
+                tile_max = fmaxf(tile_max, s);
+            }
+        }
+        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, kWave));
+        const float m_new = fmaxf(m, tile_max);
+        const float alpha = m_new == -INFINITY ? 1.0f : exp2f(m - m_new);
+        float tile_sum = 0.0f;
+#pragma unroll
+        for (int sub = 0; sub < 2; ++sub) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const float e = m_new == -INFINITY ? 0.0f : exp2f(st[sub][i] - m_new);
+                st[sub][i] = e;
+                tile_sum += e;
+            }
+        }
+        l = l * alpha + tile_sum;
+        m = m_new;
+#pragma unroll
+        for (int t = 0; t < DT; ++t) o[t] *= alpha;
+#pragma unroll
+        for (int sub = 0; sub < 2; ++sub) {
+#pragma unroll
+            for (int s = 0; s < 2; ++s) {
+                const typename Mma<T>::frag pf = acc_frag<T>(st[sub], s);
+#pragma unroll
+                for (int t = 0; t < DT; ++t)
+                    o[t] = Mma<T>::run(transposed_frag<T, DP>(v_lds, sub * 32 + s * 16, t * 32), pf, o[t]);
+            }
+        }
+    }
+    l += __shfl_xor(l, 32, kWave);
+    if (!q_live) return;
+    const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+    T* o_ptr = static_cast<T*>(p.out0) + (static_cast<long>(b) * p.qs + q_row) * q_stride + h * p.d;
+#pragma unroll
+    for (int t = 0; t < DT; ++t) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const int d0 = t * 32 + g * 8 + (lane >> 5) * 4;
+            if (d0 >= p.d) continue;
+            vec_t<float, 4> v;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] = o[t][4 * g + e] * inv;
+            store_vec<T, 4>(o_ptr + d0, vec_from_f32<T, 4>(v));
+        }
+    }
+    if (p.lse_out != nullptr && lane < 32)
+        p.lse_out[(static_cast<long>(b) * p.qs + q_row) * p.hq + h] = (m + log2f(l)) * kLn2;
+}
+
+// --------------------------------------------------------------------- delta
+// delta[b, t, h] = Σ_d dO·O, one group of LPR lanes per row, 128-bit loads.
+template <typename T, int LPR>
+__global__ __launch_bounds__(kThreads) void attention_delta_kernel(float* __restrict__ delta,
+                                                                  const T* __restrict__ dout,
+                                                                  const T* __restrict__ out, long rows, int d) {
+    const long row = (static_cast<long>(blockIdx.x) * kThreads + threadIdx.x) / LPR;
+    const int sub = threadIdx.x % LPR;
+    float sum = 0.0f;
+    if (row < rows && sub * 8 < d) {
+        const vec_t<float, 8> a = vec_to_f32<T, 8>(load_vec<T, 8>(dout + row * d + sub * 8));
+        const vec_t<float, 8> b = vec_to_f32<T, 8>(load_vec<T, 8>(out + row * d + sub * 8));
+#pragma unroll
+        for (int e = 0; e < 8; ++e) sum = fmaf(a[e], b[e], sum);
+    }
+    sum = wave_sum<LPR>(sum);
+    if (row < rows && sub == 0) delta[row] = sum;
+}
+
+// ------------------------------------------------------------------------ dQ
+template <typename T, int DP>
+__global__ __launch_bounds__(kThreads) void attention_dq_kernel(Params p) {
+    constexpr int STEPS = DP / 16, DT = DP / 32;
+    __shared__ __align__(16) T k_lds[kStream * lds_stride<DP>()];
+    __shared__ __align__(16) T v_lds[kStream * lds_stride<DP>()];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int b = blockIdx.z, h = blockIdx.y, kvh = h / (p.hq / p.hkv);
+    const int q_block = blockIdx.x * kBlockRows;
+    const int q_row = q_block + wave * 32 + (lane & 31);
+    const bool q_live = q_row < p.qs;
+    const long q_stride = static_cast<long>(p.hq) * p.d, kv_stride = static_cast<long>(p.hkv) * p.d;
+    const long q_offset = (static_cast<long>(b) * p.qs + q_row) * q_stride + h * p.d;
+    const T* k_base = static_cast<const T*>(p.k) + static_cast<long>(b) * p.ks * kv_stride + kvh * p.d;
+    const T* v_base = static_cast<const T*>(p.v) + static_cast<long>(b) * p.ks * kv_stride + kvh * p.d;
+
+    typename Mma<T>::frag qf[STEPS], dof[STEPS];
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) {
+        qf[s] = global_frag<T>(static_cast<const T*>(p.q) + q_offset, q_live, s, p.d);
+        dof[s] = global_frag<T>(static_cast<const T*>(p.dout) + q_offset, q_live, s, p.d);
+    }
+    const long stat_index = (static_cast<long>(b) * p.qs + q_row) * p.hq + h;
+    const float lse2 = q_live ? p.lse[stat_index] * kLog2e : 0.0f;
+    const float delta = q_live ? p.delta[stat_index] : 0.0f;
+
+    acc_t dq[DT];
+#pragma unroll
+    for (int t = 0; t < DT; ++t) dq[t] = acc_t(0.0f);
+    const float scale2 = p.scale * kLog2e;
+    const int last_q_block = min(q_block + kBlockRows, p.qs) - 1;
+    const int k_end = p.causal ? min(p.ks, p.offset + last_q_block + 1) : p.ks;
+    const int wave_last_q = min(q_block + wave * 32 + 31, p.qs - 1);
+    const int q_limit = p.causal ? p.offset + q_row : p.ks;
+
+    for (int k0 = 0; k0 < k_end; k0 += kStream) {
+        __syncthreads();
+        load_tile<T, kStream, DP>(k_lds, k_base, kv_stride, k0, p.ks, p.d);
+        load_tile<T, kStream, DP>(v_lds, v_base, kv_stride, k0, p.ks, p.d);
+        __syncthreads();
+        if (q_block + wave * 32 >= p.qs) continue;
+        if (p.causal && k0 > p.offset + wave_last_q) continue;
+#pragma unroll
+        for (int sub = 0; sub < 2; ++sub) {
+            acc_t st(0.0f), dpt(0.0f);
+#pragma unroll
+            for (int s = 0; s < STEPS; ++s) {
+                st = Mma<T>::run(direct_frag<T, DP>(k_lds, sub * 32, s), qf[s], st);
+                dpt = Mma<T>::run(direct_frag<T, DP>(v_lds, sub * 32, s), dof[s], dpt);
+            }
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int key = k0 + sub * 32 + acc_row(i);
+                const bool visible = q_live && key < p.ks && key <= q_limit;
+                const float prob = visible ? exp2f(st[i] * scale2 - lse2) : 0.0f;
+                st[i] = prob * (dpt[i] - delta);
+            }
+#pragma unroll
+            for (int s = 0; s < 2; ++s) {
+                const typename Mma<T>::frag dsf = acc_frag<T>(st, s);
+#pragma unroll
+                for (int t = 0; t < DT; ++t)
+                    dq[t] = Mma<T>::run(transposed_frag<T, DP>(k_lds, sub * 32 + s * 16, t * 32), dsf, dq[t]);
+            }
+        }
+    }
+    if (!q_live) return;
+    T* out = static_cast<T*>(p.out0) + q_offset;
+#pragma unroll
+    for (int t = 0; t < DT; ++t) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const int d0 = t * 32 + g * 8 + (lane >> 5) * 4;
+            if (d0 >= p.d) continue;
+            vec_t<float, 4> v;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] = dq[t][4 * g + e] * p.scale;
+            if (p.accumulate) v += vec_to_f32<T, 4>(load_vec<T, 4>(out + d0));
+            store_vec<T, 4>(out + d0, vec_from_f32<T, 4>(v));
+        }
+    }
+}
+
+// --------------------------------------------------------------------- dK/dV
+template <typename T, int DP>
+__global__ __launch_bounds__(kThreads) void attention_dkv_kernel(Params p) {
+    constexpr int STEPS = DP / 16, DT = DP / 32;
+    __shared__ __align__(16) T q_lds[kStream * lds_stride<DP>()];
+    __shared__ __align__(16) T do_lds[kStream * lds_stride<DP>()];
+    __shared__ float lse_lds[kStream];
+    __shared__ float delta_lds[kStream];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int b = blockIdx.z, kvh = blockIdx.y, group = p.hq / p.hkv;
+    const int k_block = blockIdx.x * kBlockRows;
+    const int k_row = k_block + wave * 32 + (lane & 31);
+    const bool k_live = k_row < p.ks;
+    const long q_stride = static_cast<long>(p.hq) * p.d, kv_stride = static_cast<long>(p.hkv) * p.d;
+    const long k_offset = (static_cast<long>(b) * p.ks + k_row) * kv_stride + kvh * p.d;
+
+    typename Mma<T>::frag kf[STEPS], vf[STEPS];
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) {
+        kf[s] = global_frag<T>(static_cast<const T*>(p.k) + k_offset, k_live, s, p.d);
+        vf[s] = global_frag<T>(static_cast<const T*>(p.v) + k_offset, k_live, s, p.d);
+    }
+    acc_t dk[DT], dv[DT];
+#pragma unroll
+    for (int t = 0; t < DT; ++t) {
+        dk[t] = acc_t(0.0f);
+        dv[t] = acc_t(0.0f);
+    }
+    const float scale2 = p.scale * kLog2e;
+    // First query that can see any key of this block / of this wave.
+    const int q_begin = p.causal ? max(0, k_block - p.offset) / kStream * kStream : 0;
+    const int wave_first_key = k_block + wave * 32;
+
+    for (int hg = 0; hg < group; ++hg) {
+        const int h = kvh * group + hg;
+        const T* q_base = static_cast<const T*>(p.q) + static_cast<long>(b) * p.qs * q_stride + h * p.d;
+        const T* do_base = static_cast<const T*>(p.dout) + static_cast<long>(b) * p.qs * q_stride + h * p.d;
+        for (int q0 = q_begin; q0 < p.qs; q0 += kStream) {
+            __syncthreads();
+            load_tile<T, kStream, DP>(q_lds, q_base, q_stride, q0, p.qs, p.d);
+            load_tile<T, kStream, DP>(do_lds, do_base, q_stride, q0, p.qs, p.d);
+            if (threadIdx.x < kStream) {
+                const int q = q0 + threadIdx.x;
+                const long index = (static_cast<long>(b) * p.qs + q) * p.hq + h;
+                lse_lds[threadIdx.x] = q < p.qs ? p.lse[index] * kLog2e : 0.0f;
+                delta_lds[threadIdx.x] = q < p.qs ? p.delta[index] : 0.0f;
+            }
+            __syncthreads();
+            if (wave_first_key >= p.ks) continue;
+            // every query of the tile sees at most keys <= offset + q0 + 63
+            if (p.causal && wave_first_key > p.offset + q0 + kStream - 1) continue;
+#pragma unroll
+            for (int sub = 0; sub < 2; ++sub) {
+                acc_t s_acc(0.0f), dp_acc(0.0f);
+#pragma unroll
+                for (int s = 0; s < STEPS; ++s) {
+                    s_acc = Mma<T>::run(direct_frag<T, DP>(q_lds, sub * 32, s), kf[s], s_acc);
+                    dp_acc = Mma<T>::run(direct_frag<T, DP>(do_lds, sub * 32, s), vf[s], dp_acc);
+                }
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const int local = sub * 32 + acc_row(i);
+                    const int q = q0 + local;
+                    const bool visible = k_live && q < p.qs && (!p.causal || k_row <= p.offset + q);
+                    const float prob = visible ? exp2f(s_acc[i] * scale2 - lse_lds[local]) : 0.0f;
+                    s_acc[i] = prob;
+                    dp_acc[i] = prob * (dp_acc[i] - delta_lds[local]);
+                }
+#pragma unroll
+                for (int s = 0; s < 2; ++s) {
+                    const typename Mma<T>::frag pf = acc_frag<T>(s_acc, s);
+                    const typename Mma<T>::frag dsf = acc_frag<T>(dp_acc, s);
+#pragma unroll
+                    for (int t = 0; t < DT; ++t) {
+                        dv[t] = Mma<T>::run(transposed_frag<T, DP>(do_lds, sub * 32 + s * 16, t * 32), pf, dv[t]);
+                        dk[t] = Mma<T>::run(transposed_frag<T, DP>(q_lds, sub * 32 + s * 16, t * 32), dsf, dk[t]);
+                    }
+                }
+            }
+        }
+    }
+    if (!k_live) return;
+    T* dk_out = static_cast<T*>(p.out0) + k_offset;
+    T* dv_out = static_cast<T*>(p.out1) + k_offset;
+#pragma unroll
+    for (int t = 0; t < DT; ++t) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const int d0 = t * 32 + g * 8 + (lane >> 5) * 4;
+            if (d0 >= p.d) continue;
+            vec_t<float, 4> a, c;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                a[e] = dk[t][4 * g + e] * p.scale;
+                c[e] = dv[t][4 * g + e];
+            }
+            if (p.accumulate) {
+                a += vec_to_f32<T, 4>(load_vec<T, 4>(dk_out + d0));
+                c += vec_to_f32<T, 4>(load_vec<T, 4>(dv_out + d0));
+            }
+            store_vec<T, 4>(dk_out + d0, vec_from_f32<T, 4>(a));
+            store_vec<T, 4>(dv_out + d0, vec_from_f32<T, 4>(c));
+        }
+    }
+}
+
+// ---------------------------------------------------------------------- host
+struct Shape {
+    std::size_t batch, qs, ks, hq, hkv, d;
+    float scale;
+    int causal;
+    std::size_t offset;
+    int dtype;
+};
+
+int validate(const char* name, const Shape& s) {
+    const std::string n(name);
+    if (s.dtype != CGPTX_F16 && s.dtype != CGPTX_BF16)
+        return fail(CGPTX_INVALID_ARGUMENT, n + ": only F16 and BF16 storage are supported by the MFMA kernels");
+    if (s.batch == 0 || s.qs == 0 || s.ks == 0 || s.hq == 0 || s.hkv == 0 || s.d == 0 || s.hq % s.hkv != 0)
+        return fail(CGPTX_INVALID_ARGUMENT, n + ": invalid tensors or options");
+    if (!std::isfinite(s.scale)) return fail(CGPTX_INVALID_ARGUMENT, n + ": attention scale must be finite");
+    if (s.causal && (s.offset > s.ks || s.qs > s.ks - s.offset))
+        return fail(CGPTX_INVALID_ARGUMENT, n + ": causal range exceeds the key sequence");
+    if (s.d % 8 != 0 || s.d > 128)
+        return fail(CGPTX_INVALID_ARGUMENT, n + ": head_dim must be a multiple of 8 up to 128");
+    constexpr std::size_t limit = 1u << 30;
+    if (s.batch > 65535 || s.qs > limit || s.ks > limit || s.hq > 65535 || s.offset > limit ||
+        s.hq * s.d > limit)
+        return fail(CGPTX_OVERFLOW, n + ": dimension exceeds the supported range");
+    return CGPTX_OK;
+}
+
+Params make_params(const Shape& s) {
+    Params p{};
+    p.batch = static_cast<int>(s.batch);
+    p.qs = static_cast<int>(s.qs);
+    p.ks = static_cast<int>(s.ks);
+    p.hq = static_cast<int>(s.hq);
+    p.hkv = static_cast<int>(s.hkv);
+    p.d = static_cast<int>(s.d);
+    p.scale = s.scale > 0.0f ? s.scale : 1.0f / std::sqrt(static_cast<float>(s.d));
+    p.causal = s.causal ? 1 : 0;
+    p.offset = static_cast<int>(s.offset);
+    return p;
+}
+
+template <typename Fn>
+int dispatch_head_dim(std::size_t d, Fn&& fn) {
+    if (d <= 32) return fn.template operator()<32>();
+    if (d <= 64) return fn.template operator()<64>();
+    return fn.template operator()<128>();
+}
+
+template <typename Fn>
+int dispatch_16bit(int dtype, Fn&& fn) {
+    return dtype == CGPTX_F16 ? fn.template operator()<f16_t>() : fn.template operator()<bf16_t>();
+}
+
+int launch_forward(const Shape& s, Params p, hipStream_t stream) {
+    const dim3 grid(static_cast<unsigned int>((s.qs + kBlockRows - 1) / kBlockRows), static_cast<unsigned int>(s.hq),
+                    static_cast<unsigned int>(s.batch));
+    return dispatch_16bit(s.dtype, [&]<typename T>() -> int {
+        return dispatch_head_dim(s.d, [&]<int DP>() -> int {
+            hipLaunchKernelGGL((attention_forward_kernel<T, DP>), grid, dim3(kThreads), 0, stream, p);
+            CGPTX_LAUNCH_CHECK();
+            return CGPTX_OK;
+        });
+    });
+}
+
+int launch_backward(const Shape& s, Params p, void* dq, void* dk, void* dv, const void* dout, const void* out,
+                    const float* lse, int accumulate, hipStream_t stream) {
+    const std::size_t rows = s.batch * s.qs * s.hq;
+    void* mem = nullptr;
+    if (int st = scratch(stream, rows * sizeof(float), &mem)) return st;
+    auto* delta = static_cast<float*>(mem);
+    p.dout = dout;
+    p.lse = lse;
+    p.delta = delta;
+    p.accumulate = accumulate;
+    return dispatch_16bit(s.dtype, [&]<typename T>() -> int {
+        const int lpr = s.d <= 32 ? 4 : (s.d <= 64 ? 8 : 16);
+        const unsigned int delta_blocks = static_cast<unsigned int>((rows * lpr + kThreads - 1) / kThreads);
+        auto* dout_t = static_cast<const T*>(dout);
+        auto* out_t = static_cast<const T*>(out);
+        const long r = static_cast<long>(rows);
+        const int d = static_cast<int>(s.d);
+        if (lpr == 4)
+            hipLaunchKernelGGL((attention_delta_kernel<T, 4>), dim3(delta_blocks), dim3(kThreads), 0, stream, delta,
+                               dout_t, out_t, r, d);
+        else if (lpr == 8)
+            hipLaunchKernelGGL((attention_delta_kernel<T, 8>), dim3(delta_blocks), dim3(kThreads), 0, stream, delta,
+                               dout_t, out_t, r, d);
+        else
+            hipLaunchKernelGGL((attention_delta_kernel<T, 16>), dim3(delta_blocks), dim3(kThreads), 0, stream, delta,
+                               dout_t, out_t, r, d);
+        CGPTX_LAUNCH_CHECK();
+        return dispatch_head_dim(s.d, [&]<int DP>() -> int {
+            Params pq = p;
+            pq.out0 = dq;
+            const dim3 q_grid(static_cast<unsigned int>((s.qs + kBlockRows - 1) / kBlockRows),
+                              static_cast<unsigned int>(s.hq), static_cast<unsigned int>(s.batch));
+            hipLaunchKernelGGL((attention_dq_kernel<T, DP>), q_grid, dim3(kThreads), 0, stream, pq);
+            CGPTX_LAUNCH_CHECK();
+            Params pk = p;
+            pk.out0 = dk;
+            pk.out1 = dv;
+            const dim3 k_grid(static_cast<unsigned int>((s.ks + kBlockRows - 1) / kBlockRows),
+                              static_cast<unsigned int>(s.hkv), static_cast<unsigned int>(s.batch));
+            hipLaunchKernelGGL((attention_dkv_kernel<T, DP>), k_grid, dim3(kThreads), 0, stream, pk);
+            CGPTX_LAUNCH_CHECK();
+            return CGPTX_OK;
+        });
+    });
+}
+
+bool aligned16_all(std::initializer_list<const void*> pointers) {
+    for (const void* ptr : pointers)
+        if (ptr != nullptr && !is_aligned16(ptr)) return false;
+    return true;
+}
+
+}  // namespace
+}  // namespace cgptx
+
+extern "C" int cgptx_flash_gqa_attention_forward(void* output, float* logsumexp, const void* query, const void* key,
+                                                 const void* value, size_t batch, size_t query_sequence,
+                                                 size_t kv_sequence, size_t query_heads, size_t kv_heads,
+                                                 size_t head_dim, float attention_scale, int causal,
+                                                 size_t query_position_offset, int dtype, cgptx_stream stream) {
+    using namespace cgptx;
+    const char* name = "flash_gqa_attention_forward";
+    const Shape s{batch, query_sequence, kv_sequence, query_heads, kv_heads, head_dim, attention_scale, causal,
+                  query_position_offset, dtype};
+    if (int st = validate(name, s)) return st;
+    if (output == nullptr || query == nullptr || key == nullptr || value == nullptr)
+        return fail(CGPTX_INVALID_ARGUMENT, std::string(name) + ": null tensor");
+    if (!aligned16_all({output, query, key, value}))
+        return fail(CGPTX_INVALID_ARGUMENT, std::string(name) + ": tensors must be 16-byte aligned");
+    Params p = make_params(s);
+    p.out0 = output;
+    p.lse_out = logsumexp;
+    p.q = query;
+    p.k = key;
+    p.v = value;
+    return launch_forward(s, p, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int cgptx_flash_gqa_attention_backward_with_lse(
+    void* grad_query, void* grad_key, void* grad_value, const void* grad_output, const void* output,
+    const float* logsumexp, const void* query, const void* key, const void* value, size_t batch,
+    size_t query_sequence, size_t kv_sequence, size_t query_heads, size_t kv_heads, size_t head_dim,
+    float attention_scale, int causal, size_t query_position_offset, int accumulate_grads, int dtype,
+    cgptx_stream stream) {
+    using namespace cgptx;
+    const char* name = "flash_gqa_attention_backward_with_lse";
+    const Shape s{batch, query_sequence, kv_sequence, query_heads, kv_heads, head_dim, attention_scale, causal,
+                  query_position_offset, dtype};
+    if (int st = validate(name, s)) return st;
+    if (grad_query == nullptr || grad_key == nullptr || grad_value == nullptr || grad_output == nullptr ||
+        output == nullptr || logsumexp == nullptr || query == nullptr || key == nullptr || value == nullptr)
+        return fail(CGPTX_INVALID_ARGUMENT, std::string(name) + ": null tensor");
+    if (!aligned16_all({grad_query, grad_key, grad_value, grad_output, output, query, key, value}))
+        return fail(CGPTX_INVALID_ARGUMENT, std::string(name) + ": tensors must be 16-byte aligned");
+    Params p = make_params(s);
+    p.q = query;
+    p.k = key;
+    p.v = value;
+    return launch_backward(s, p, grad_query, grad_key, grad_value, grad_output, output, logsumexp,
+                           accumulate_grads != 0, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int cgptx_flash_gqa_attention_backward(void* grad_query, void* grad_key, void* grad_value,
+                                                  const void* grad_output, const void* query, const void* key,
+                                                  const void* value, size_t batch, size_t query_sequence,
+                                                  size_t kv_sequence, size_t query_heads, size_t kv_heads,
+                                                  size_t head_dim, float attention_scale, int causal,
+                                                  size_t query_position_offset, int accumulate_grads, int dtype,
+                                                  cgptx_stream stream_) {
+    using namespace cgptx;
+    const char* name = "flash_gqa_attention_backward";
+    const Shape s{batch, query_sequence, kv_sequence, query_heads, kv_heads, head_dim, attention_scale, causal,
+                  query_position_offset, dtype};
+    if (int st = validate(name, s)) return st;
+    if (grad_query == nullptr || grad_key == nullptr || grad_value == nullptr || grad_output == nullptr ||
+        query == nullptr || key == nullptr || value == nullptr)
+        return fail(CGPTX_INVALID_ARGUMENT, std::string(name) + ": null tensor");
+    if (!aligned16_all({grad_query, grad_key, grad_value, grad_output, query, key, value}))
+        return fail(CGPTX_INVALID_ARGUMENT, std::string(name) + ": tensors must be 16-byte aligned");
+    auto stream = static_cast<hipStream_t>(stream_);
+    // Recompute the output and the log-sum-exp into scratch, then run the LSE path. The scratch
+    // block is laid out [delta | lse | output] so that launch_backward's request for the delta
+    // prefix returns the same base pointer.
+    const std::size_t rows = batch * query_sequence * query_heads;
+    const std::size_t stat_bytes = (rows * sizeof(float) + 255) & ~std::size_t{255};
+    const std::size_t out_bytes = rows * head_dim * 2;
+    void* mem = nullptr;
+    if (int st = scratch(stream, 2 * stat_bytes + out_bytes, &mem)) return st;
+    auto* lse = reinterpret_cast<float*>(static_cast<char*>(mem) + stat_bytes);
+    void* out = static_cast<char*>(mem) + 2 * stat_bytes;
+    Params p = make_params(s);
+    p.q = query;
+    p.k = key;
+    p.v = value;
+    Params fwd = p;
+    fwd.out0 = out;
+    fwd.lse_out = lse;
+    if (int st = launch_forward(s, fwd, stream)) return st;
+    return launch_backward(s, p, grad_query, grad_key, grad_value, grad_output, out, lse, accumulate_grads != 0,
+                           stream);
+}
