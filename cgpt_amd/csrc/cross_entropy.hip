@@ -11,7 +11,7 @@
 // read and one write of the logits. Per-row losses go to scratch and one block
 // adds them in a fixed order, where the reference uses a float atomicAdd
 // (src/ops/cross_entropy.cu:134-245).
-#include "common.hpp"
+#include "cross_entropy.hpp"
 
 #include <cmath>
 #include <limits>
@@ -49,8 +49,8 @@ __device__ __forceinline__ MaxSum block_combine(MaxSum v, MaxSum* stage) {
 
 template <typename T, bool WithGradient>
 __global__ __launch_bounds__(kThreads) void cross_entropy_row_kernel(float* __restrict__ row_loss,
-                                                                    T* __restrict__ gradient,
-                                                                    const T* __restrict__ logits,
+                                                                    T* gradient,  // may alias logits (in place)
+                                                                    const T* logits,
                                                                     const std::uint32_t* __restrict__ targets,
                                                                     unsigned int vocab, float factor,
                                                                     bool vector_ok) {
@@ -59,6 +59,9 @@ __global__ __launch_bounds__(kThreads) void cross_entropy_row_kernel(float* __re
     const std::size_t base = static_cast<std::size_t>(blockIdx.x) * vocab;
     const T* row = logits + base;
     const unsigned int vectors = vector_ok ? vocab / VEC : 0;
+    const std::uint32_t target = targets[blockIdx.x];
+    // Read before the barrier below: in-place use overwrites the row in pass 2.
+    const float target_logit = (threadIdx.x == 0 && target < vocab) ? to_f32(row[target]) : 0.0f;
 
     MaxSum acc{-INFINITY, 0.0f};
     for (unsigned int v = threadIdx.x; v < vectors; v += kThreads) {
@@ -84,10 +87,9 @@ __global__ __launch_bounds__(kThreads) void cross_entropy_row_kernel(float* __re
         if (acc.m != -INFINITY) acc.s += __expf(x - acc.m);
     }
     const MaxSum total = block_combine(acc, stage);
-    const std::uint32_t target = targets[blockIdx.x];
     if (threadIdx.x == 0) {
         float loss = 0.0f;
-        if (target < vocab) loss = __logf(total.s) + total.m - to_f32(row[target]);
+        if (target < vocab) loss = __logf(total.s) + total.m - target_logit;
         row_loss[blockIdx.x] = loss;
     }
     if constexpr (WithGradient) {
@@ -130,6 +132,33 @@ __global__ __launch_bounds__(256) void mean_reduce_kernel(float* __restrict__ lo
     if (threadIdx.x == 0) loss[0] = static_cast<float>(stage[0]) * inv_rows;
 }
 
+// Per-row pass: row_loss[r] and (optionally) the gradient, factor = gradient_scale / total_rows.
+int cross_entropy_rows(float* row_loss, void* gradient, const void* logits, const std::uint32_t* targets,
+                       std::size_t rows, std::size_t vocab, float factor, int dtype, hipStream_t stream) {
+    const auto r = static_cast<unsigned int>(rows), v = static_cast<unsigned int>(vocab);
+    const bool with_gradient = gradient != nullptr;
+    return dispatch_dtype(dtype, [&]<typename T>() -> int {
+        const bool vector_ok = vocab % kVec128<T> == 0 && is_aligned16(logits) &&
+                               (!with_gradient || is_aligned16(gradient));
+        if (with_gradient) {
+            hipLaunchKernelGGL((cross_entropy_row_kernel<T, true>), dim3(r), dim3(kThreads), 0, stream, row_loss,
+                               static_cast<T*>(gradient), static_cast<const T*>(logits), targets, v, factor, vector_ok);
+        } else {
+            hipLaunchKernelGGL((cross_entropy_row_kernel<T, false>), dim3(r), dim3(kThreads), 0, stream, row_loss,
+                               static_cast<T*>(nullptr), static_cast<const T*>(logits), targets, v, factor, vector_ok);
+        }
+        CGPTX_LAUNCH_CHECK();
+        return CGPTX_OK;
+    });
+}
+
+int mean_reduce(float* loss, const float* row_loss, std::size_t rows, hipStream_t stream) {
+    hipLaunchKernelGGL(mean_reduce_kernel, dim3(1), dim3(256), 0, stream, loss, row_loss,
+                       static_cast<unsigned int>(rows), 1.0f / static_cast<float>(rows));
+    CGPTX_LAUNCH_CHECK();
+    return CGPTX_OK;
+}
+
 namespace {
 
 int run(float* loss, void* gradient, const void* logits, const std::uint32_t* targets, std::size_t rows,
@@ -147,25 +176,10 @@ int run(float* loss, void* gradient, const void* logits, const std::uint32_t* ta
     if (int s = scratch(stream, rows * sizeof(float), &mem)) return s;
     auto* row_loss = static_cast<float*>(mem);
     const float factor = gradient_scale / static_cast<float>(rows);
-    const auto r = static_cast<unsigned int>(rows), v = static_cast<unsigned int>(vocab);
-    int status = dispatch_dtype(dtype, [&]<typename T>() -> int {
-        const bool vector_ok = vocab % kVec128<T> == 0 && is_aligned16(logits) &&
-                               (!with_gradient || is_aligned16(gradient));
-        if (with_gradient) {
-            hipLaunchKernelGGL((cross_entropy_row_kernel<T, true>), dim3(r), dim3(kThreads), 0, stream, row_loss,
-                               static_cast<T*>(gradient), static_cast<const T*>(logits), targets, v, factor, vector_ok);
-        } else {
-            hipLaunchKernelGGL((cross_entropy_row_kernel<T, false>), dim3(r), dim3(kThreads), 0, stream, row_loss,
-                               static_cast<T*>(nullptr), static_cast<const T*>(logits), targets, v, factor, vector_ok);
-        }
-        CGPTX_LAUNCH_CHECK();
-        return CGPTX_OK;
-    });
-    if (status) return status;
-    hipLaunchKernelGGL(mean_reduce_kernel, dim3(1), dim3(256), 0, stream, loss, row_loss, r,
-                       1.0f / static_cast<float>(rows));
-    CGPTX_LAUNCH_CHECK();
-    return CGPTX_OK;
+    if (int s = cross_entropy_rows(row_loss, with_gradient ? gradient : nullptr, logits, targets, rows, vocab, factor,
+                                   dtype, stream))
+        return s;
+    return mean_reduce(loss, row_loss, rows, stream);
 }
 
 }  // namespace

@@ -441,7 +441,7 @@ int run_typed(const GemmArgs& g, hipStream_t stream) {
         const long tiles = static_cast<long>(p.tiles_m) * p.tiles_n;
         const long want_blocks = static_cast<long>(compute_units()) * 2;
         int slices = 1;
-        if (tiles < want_blocks && k_tiles >= 16) {
+        if (!g.no_split && tiles < want_blocks && k_tiles >= 16) {
             slices = static_cast<int>(std::min<long>((want_blocks + tiles - 1) / tiles, k_tiles / 8));
             if (slices < 1) slices = 1;
         }

@@ -22,6 +22,7 @@ struct GemmArgs {
     bool b_k_contiguous = true;
     bool accumulate = false;
     bool c_is_f32 = false;
+    bool no_split = false;  // never use split-K scratch (the caller owns the arena)
     int dtype = CGPTX_BF16;
 };
 

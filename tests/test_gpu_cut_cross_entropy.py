@@ -1,0 +1,90 @@
+"""GPU parity tests of cut cross-entropy against the float64 statement (loss, dX, dC) and against the
+dense path it must be equivalent to: cross_entropy(X·Cᵀ) followed by linear_backward."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from cgpt_amd import ops
+from oracle import oracle64
+from tests.util import DTYPES, DTYPE_IDS, TOL, assert_close, randint, randn, to_np
+
+pytestmark = pytest.mark.gpu
+
+
+def run(device, x, c, targets, scale=1.0, accumulate=False, base=None):
+    loss = torch.zeros(1, device=device)
+    dx = torch.full_like(x, 3.0, device=device)
+    dc = torch.full_like(c, 3.0, device=device) if base is None else base.to(device).clone()
+    ops.cut_cross_entropy_forward_backward(loss, dx, dc, x.to(device), c.to(device), targets.to(device), x.shape[0],
+                                           None, scale, accumulate)
+    return loss.item(), dx, dc
+
+
+def test_reference_test_case(device):
+    """tests/cut_cross_entropy_test.cu:19-31 (F32, 2x2 input, 3 classes). Row 1 of dX and row 2 of dC are
+    compared with the reference's formula rather than its constants, which disagree with its own kernels
+    (see tests/test_oracle_pins.py::test_cut_cross_entropy_known_answer)."""
+    x = torch.tensor([[1, 2], [3, 4.0]])
+    c = torch.tensor([[1, 0], [0, 1], [1, 1.0]])
+    targets = torch.tensor([2, 0], dtype=torch.int32)
+    loss, dx, dc = run(device, x, c, targets)
+    e = math.exp
+    assert abs(loss - (math.log(e(1) + e(2) + e(3)) - 3 + math.log(e(3) + e(4) + e(7)) - 3) / 2) <= 2e-5
+    assert np.abs(to_np(dx)[0] - [-0.1223642, -0.0450153]).max() <= 2e-5
+    assert np.abs(to_np(dc)[:2].reshape(-1) - [-1.4295, -1.876, 0.193, 0.339]).max() <= 2e-3
+    l64, dx64, dc64 = oracle64.cut_cross_entropy(x.numpy(), c.numpy(), targets.numpy())
+    assert_close(dx, dx64, 1e-5, "dX")
+    assert_close(dc, dc64, 1e-5, "dC")
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=DTYPE_IDS)
+@pytest.mark.parametrize("rows,hidden,vocab", [(5, 7, 11), (64, 64, 128), (300, 128, 1000), (1024, 256, 4096)])
+def test_parity_with_float64(device, rows, hidden, vocab, dtype):
+    if dtype == torch.float32 and rows * hidden * vocab > 300 * 128 * 1000:
+        pytest.skip("fp32 storage runs on the plain contraction kernel; large shapes are covered in 16-bit")
+    x, c = randn((rows, hidden), dtype, 1), randn((vocab, hidden), dtype, 2, 0.05)
+    targets = randint(vocab, (rows,), 3)
+    l64, dx64, dc64 = oracle64.cut_cross_entropy(to_np(x), to_np(c), targets.numpy(), 1024.0)
+    loss, dx, dc = run(device, x, c, targets, 1024.0)
+    assert abs(loss - l64) <= (1e-4 if dtype == torch.float32 else 5e-3) * max(1.0, l64)
+    assert_close(dx, dx64, TOL[dtype] * max(1.0, np.abs(dx64).max()), "dX")
+    assert_close(dc, dc64, TOL[dtype] * max(1.0, np.abs(dc64).max()), "dC")
+    base = randn((vocab, hidden), dtype, 4)
+    _, _, dc2 = run(device, x, c, targets, 1024.0, True, base)
+    want = dc64 + to_np(base)
+    assert_close(dc2, want, TOL[dtype] * max(1.0, np.abs(want).max()), "dC accumulate")
+
+
+def test_equivalent_to_dense_cross_entropy_plus_linear_backward(device):
+    """Several row chunks (rows > the chunk derived from 128 MiB / vocab): bf16, [6000, 256] x [32000, 256]."""
+    dtype = torch.bfloat16
+    rows, hidden, vocab = 6000, 256, 32000
+    x, c = randn((rows, hidden), dtype, 5).to(device), randn((vocab, hidden), dtype, 6, 0.05).to(device)
+    targets = randint(vocab, (rows,), 7).to(device)
+    loss, dx, dc = run(device, x, c, targets, 1024.0)
+    logits = torch.empty(rows, vocab, dtype=dtype, device=device)
+    ops.linear_forward(logits, x, c)
+    dense_loss = torch.zeros(1, device=device)
+    grad = torch.empty_like(logits)
+    ops.cross_entropy_forward_backward(dense_loss, grad, logits, targets, rows, None, 1024.0)
+    dx2, dc2 = torch.empty_like(x), torch.empty_like(c)
+    ops.linear_backward(dx2, dc2, None, grad, x, c)
+    assert abs(loss - dense_loss.item()) <= 1e-5 * dense_loss.item()
+    assert_close(dx, dx2, TOL[dtype] * max(1.0, float(dx2.float().abs().max())), "dX vs dense path")
+    assert_close(dc, dc2, TOL[dtype] * max(1.0, float(dc2.float().abs().max())), "dC vs dense path")
+    again = run(device, x, c, targets, 1024.0)
+    assert again[0] == loss and torch.equal(again[1], dx) and torch.equal(again[2], dc)
+
+
+def test_argument_errors(device):
+    x, c = torch.zeros(4, 8, device=device), torch.zeros(5, 8, device=device)
+    t = torch.zeros(4, dtype=torch.int32, device=device)
+    loss = torch.zeros(1, device=device)
+    with pytest.raises(ValueError):
+        ops.cut_cross_entropy_forward_backward(loss, x.clone(), c.clone(), x, torch.zeros(5, 7, device=device), t, 4)
+    with pytest.raises(ValueError):
+        ops.cut_cross_entropy_forward_backward(loss, x.clone(), c.clone(), x, c, t, 3)
+    with pytest.raises(ValueError):
+        ops.cut_cross_entropy_forward_backward(loss.half(), x.clone(), c.clone(), x, c, t, 4)
