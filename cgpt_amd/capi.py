@@ -37,7 +37,15 @@ class AdamWEntry(ctypes.Structure):
                 ("second_moment", _vp), ("count", _sz), ("dtype", _i)]
 
 
-# name -> argtypes, in the order of include/cgptx.h
+class ModelConfig(ctypes.Structure):
+    """cgptx_model_config (include/cgptx_train.h)."""
+
+    _fields_ = [("vocabulary_size", _sz), ("num_layers", _sz), ("hidden_size", _sz), ("intermediate_size", _sz),
+                ("num_query_heads", _sz), ("num_kv_heads", _sz), ("head_dim", _sz), ("rotary_dim", _sz),
+                ("rms_epsilon", _f), ("rope_base", _f), ("dtype", _i)]
+
+
+# name -> argtypes, in the order of include/cgptx.h and include/cgptx_train.h
 PROTOTYPES = {
     "cgptx_release_scratch": [],
     "cgptx_rmsnorm_backward": [_vp, _vp, _vp, _vp, _vp, _sz, _sz, _f, _i, _vp],
@@ -66,7 +74,19 @@ PROTOTYPES = {
     "cgptx_embedding_forward": [_vp, _vp, _sz, _vp, _sz, _sz, _i, _vp],
     "cgptx_flash_gqa_attention_forward": [_vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz, _sz, _f, _i, _sz, _i, _vp],
     "cgptx_add": [_vp, _vp, _vp, _sz, _i, _vp],
+    "cgptx_model_create": [ctypes.POINTER(_vp), ctypes.POINTER(ModelConfig), _sz, _sz, _u64],
+    "cgptx_model_destroy": [_vp],
+    "cgptx_model_set_tokens": [_vp, _vp, _vp],
+    "cgptx_model_forward_backward": [_vp, _f, _i, _i, _vp],
+    "cgptx_model_optimizer_step": [_vp, ctypes.POINTER(AdamWOptions), _vp],
+    "cgptx_model_train_step": [_vp, ctypes.POINTER(AdamWOptions), _i, _i, _vp],
+    "cgptx_model_status": [_vp, ctypes.POINTER(_f), ctypes.POINTER(_i), ctypes.POINTER(_u64), _vp],
+    "cgptx_model_parameter": [_vp, _sz, ctypes.POINTER(ctypes.c_char_p), ctypes.POINTER(_vp), ctypes.POINTER(_vp),
+                              ctypes.POINTER(_sz)],
+    "cgptx_model_activation": [_vp, ctypes.c_char_p, ctypes.POINTER(_vp), ctypes.POINTER(_sz)],
 }
+
+SIZE_FUNCTIONS = {"cgptx_model_parameter_count": [_vp], "cgptx_model_num_parameters": [_vp]}
 
 STRING_FUNCTIONS = ("cgptx_last_error", "cgptx_version")
 
@@ -94,6 +114,9 @@ def lib() -> ctypes.CDLL:
             fn.restype = _i
         for name in STRING_FUNCTIONS:
             getattr(loaded, name).restype = ctypes.c_char_p
+        for name, argtypes in SIZE_FUNCTIONS.items():
+            getattr(loaded, name).argtypes = argtypes
+            getattr(loaded, name).restype = _sz
         _lib = loaded
     return _lib
 

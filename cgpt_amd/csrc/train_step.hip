@@ -1,0 +1,549 @@
+// The caller side of the hot path: a decoder model and its train step composed
+// from the cgptx_* operators, in the order of the reference's
+// transformer_model_forward/backward (src/core/transformer_model.cu:195-241, 336-381),
+// transformer_block_forward/backward (src/core/transformer_block.cu:405-611, 644-748)
+// and the training loop (train/train.cpp:536-556).
+//
+// Differences from the reference's glue, none of which changes a result:
+//   * no device-to-device copies: projections write straight into the buffers that
+//     the backward pass reads (q/k before QK-norm, the layer inputs), and the output
+//     projection's backward reads the incoming gradient in place;
+//   * the attention-norm output is kept instead of being recomputed in the backward;
+//   * bias gradients, which the reference computes into scratch and never uses
+//     (the model has no biases), are not computed;
+//   * forward + loss + backward are captured into one hipGraph after one eager run;
+//     every scratch request was sized by that eager run, so replay allocates nothing.
+#include "cgptx_train.h"
+#include "common.hpp"
+
+#include <cmath>
+#include <cstring>
+#include <string>
+#include <vector>
+
+namespace cgptx {
+namespace {
+
+// ---- deterministic host-side initialisation ----------------------------------
+inline std::uint64_t splitmix64(std::uint64_t x) {
+    x += 0x9E3779B97F4A7C15ull;
+    x = (x ^ (x >> 30)) * 0xBF58476D1CE4E5B9ull;
+    x = (x ^ (x >> 27)) * 0x94D049BB133111EBull;
+    return x ^ (x >> 31);
+}
+
+// Standard normal from (seed, tensor, index): Box–Muller on two counter-derived uniforms.
+inline float normal_at(std::uint64_t seed, std::uint64_t tensor, std::uint64_t index) {
+    const std::uint64_t a = splitmix64(seed ^ splitmix64(tensor * 0x100000001B3ull + 2 * index));
+    const std::uint64_t b = splitmix64(seed ^ splitmix64(tensor * 0x100000001B3ull + 2 * index + 1));
+    const double u1 = (static_cast<double>(a >> 11) + 1.0) / 9007199254740993.0;  // (0, 1)
+    const double u2 = static_cast<double>(b >> 11) / 9007199254740992.0;          // [0, 1)
+    return static_cast<float>(std::sqrt(-2.0 * std::log(u1)) * std::cos(6.283185307179586 * u2));
+}
+
+inline std::uint16_t to_bf16_bits(float x) {
+    std::uint32_t b;
+    std::memcpy(&b, &x, 4);
+    return static_cast<std::uint16_t>((b + 0x7fffu + ((b >> 16) & 1u)) >> 16);
+}
+
+inline std::uint16_t to_f16_bits(float x) {
+    const _Float16 h = static_cast<_Float16>(x);
+    std::uint16_t bits;
+    std::memcpy(&bits, &h, 2);
+    return bits;
+}
+
+void convert_to_storage(const std::vector<float>& src, int dtype, std::vector<unsigned char>& dst) {
+    if (dtype == CGPTX_F32) {
+        dst.resize(src.size() * 4);
+        std::memcpy(dst.data(), src.data(), dst.size());
+        return;
+    }
+    dst.resize(src.size() * 2);
+    auto* out = reinterpret_cast<std::uint16_t*>(dst.data());
+    for (std::size_t i = 0; i < src.size(); ++i) out[i] = dtype == CGPTX_BF16 ? to_bf16_bits(src[i]) : to_f16_bits(src[i]);
+}
+
+struct Parameter {
+    std::string name;
+    void* value = nullptr;
+    void* gradient = nullptr;
+    float* master = nullptr;
+    float* first = nullptr;
+    float* second = nullptr;
+    std::size_t count = 0;
+};
+
+struct LayerParameters {
+    Parameter attention_norm, q, k, q_norm, k_norm, v, o, ffn_norm, gate, up, down;
+};
+
+struct LayerActivations {
+    void *norm_a, *q_pre, *k_pre, *q, *k, *v, *attn_out, *norm_f, *gate, *up, *act;
+    float* lse;
+};
+
+}  // namespace
+}  // namespace cgptx
+
+struct cgptx_model {
+    cgptx_model_config config{};
+    std::size_t batch = 0, sequence = 0, rows = 0;
+    std::vector<void*> allocations;
+    cgptx::Parameter embedding, final_norm;
+    std::vector<cgptx::LayerParameters> layers;
+    std::vector<cgptx::LayerActivations> acts;
+    std::vector<void*> hidden;  // num_layers + 1 buffers [rows, hidden]
+    void* normalized = nullptr;
+    void* logits = nullptr;       // dense loss only, allocated on first use
+    void* grad_logits = nullptr;
+    void *cos_cache = nullptr, *sin_cache = nullptr;
+    std::uint32_t *tokens = nullptr, *targets = nullptr;
+    float* loss = nullptr;
+    // backward workspace
+    void *d_normalized = nullptr, *grad_a = nullptr, *grad_b = nullptr, *d_act = nullptr, *d_gate = nullptr,
+         *d_up = nullptr, *d_norm_in = nullptr, *d_residual = nullptr, *d_attn_out = nullptr, *d_q = nullptr,
+         *d_k = nullptr, *d_v = nullptr, *d_q_pre = nullptr, *d_k_pre = nullptr;
+    cgptx_adamw_workspace* optimizer = nullptr;
+    std::vector<cgptx_adamw_entry> entries;
+    // captured graph
+    hipGraphExec_t graph_exec = nullptr;
+    float graph_loss_scale = 0.0f;
+    int graph_loss_mode = -1;
+    hipStream_t graph_stream = nullptr;
+    bool warmed = false;
+    float warm_loss_scale = 0.0f;
+    int warm_loss_mode = -1;
+};
+
+namespace cgptx {
+namespace {
+
+int allocate(cgptx_model* m, void** out, std::size_t bytes) {
+    CGPTX_HIP(hipMalloc(out, bytes));
+    m->allocations.push_back(*out);
+    return CGPTX_OK;
+}
+
+template <typename P>
+int allocate_typed(cgptx_model* m, P** out, std::size_t bytes) {
+    void* p = nullptr;
+    if (int s = allocate(m, &p, bytes)) return s;
+    *out = static_cast<P*>(p);
+    return CGPTX_OK;
+}
+
+// kind: 0 = normal(0, stddev), 1 = ones
+int make_parameter(cgptx_model* m, Parameter& p, const std::string& name, std::size_t count, int kind, float stddev,
+                   std::uint64_t seed, std::uint64_t tensor_id) {
+    const std::size_t elem = dtype_size(m->config.dtype);
+    p.name = name;
+    p.count = count;
+    if (int s = allocate(m, &p.value, count * elem)) return s;
+    if (int s = allocate(m, &p.gradient, count * elem)) return s;
+    if (int s = allocate_typed(m, &p.master, count * sizeof(float))) return s;
+    if (int s = allocate_typed(m, &p.first, count * sizeof(float))) return s;
+    if (int s = allocate_typed(m, &p.second, count * sizeof(float))) return s;
+    std::vector<float> host(count);
+    if (kind == 1) {
+        for (auto& v : host) v = 1.0f;
+    } else {
+        for (std::size_t i = 0; i < count; ++i) host[i] = stddev * normal_at(seed, tensor_id, i);
+    }
+    std::vector<unsigned char> storage;
+    convert_to_storage(host, m->config.dtype, storage);
+    CGPTX_HIP(hipMemcpy(p.value, storage.data(), storage.size(), hipMemcpyHostToDevice));
+    // The master copy is the stored (rounded) parameter widened to fp32, as AdamWState::for_parameter does.
+    if (m->config.dtype != CGPTX_F32) {
+        const auto* bits = reinterpret_cast<const std::uint16_t*>(storage.data());
+        for (std::size_t i = 0; i < count; ++i) {
+            if (m->config.dtype == CGPTX_BF16) {
+                const std::uint32_t b = static_cast<std::uint32_t>(bits[i]) << 16;
+                std::memcpy(&host[i], &b, 4);
+            } else {
+                _Float16 h;
+                std::memcpy(&h, &bits[i], 2);
+                host[i] = static_cast<float>(h);
+            }
+        }
+    }
+    CGPTX_HIP(hipMemcpy(p.master, host.data(), count * sizeof(float), hipMemcpyHostToDevice));
+    CGPTX_HIP(hipMemset(p.first, 0, count * sizeof(float)));
+    CGPTX_HIP(hipMemset(p.second, 0, count * sizeof(float)));
+    CGPTX_HIP(hipMemset(p.gradient, 0, count * elem));
+    return CGPTX_OK;
+}
+
+void collect(cgptx_model* m, std::vector<Parameter*>& out) {
+    out.clear();
+    out.push_back(&m->embedding);
+    out.push_back(&m->final_norm);
+    for (auto& l : m->layers) {
+        for (Parameter* p : {&l.attention_norm, &l.q, &l.k, &l.q_norm, &l.k_norm, &l.v, &l.o, &l.ffn_norm, &l.gate,
+                             &l.up, &l.down})
+            out.push_back(p);
+    }
+}
+
+#define CGPTX_TRY(expr)                     \
+    do {                                    \
+        if (int status_ = (expr)) return status_; \
+    } while (0)
+
+int enqueue_forward_backward(cgptx_model* m, float loss_scale, int loss_mode, hipStream_t stream) {
+    const auto& c = m->config;
+    const int dt = c.dtype;
+    const std::size_t N = m->rows, H = c.hidden_size, I = c.intermediate_size;
+    const std::size_t HQ = c.num_query_heads, HKV = c.num_kv_heads, D = c.head_dim;
+    const std::size_t QW = HQ * D, KW = HKV * D;
+    const float eps = c.rms_epsilon;
+    auto* s = static_cast<cgptx_stream>(stream);
+
+    // ------------------------------------------------------------------ forward
+    CGPTX_TRY(cgptx_embedding_forward(m->hidden[0], m->tokens, N, m->embedding.value, c.vocabulary_size, H, dt, s));
+    for (std::size_t l = 0; l < c.num_layers; ++l) {
+        const auto& w = m->layers[l];
+        const auto& a = m->acts[l];
+        void* x = m->hidden[l];
+        void* out = m->hidden[l + 1];
+        CGPTX_TRY(cgptx_rmsnorm_forward(a.norm_a, x, w.attention_norm.value, N, H, eps, dt, s));
+        CGPTX_TRY(cgptx_linear_forward(a.q_pre, a.norm_a, w.q.value, nullptr, N, H, QW, dt, s));
+        CGPTX_TRY(cgptx_linear_forward(a.k_pre, a.norm_a, w.k.value, nullptr, N, H, KW, dt, s));
+        CGPTX_TRY(cgptx_linear_forward(a.v, a.norm_a, w.v.value, nullptr, N, H, KW, dt, s));
+        CGPTX_TRY(cgptx_rmsnorm_forward(a.q, a.q_pre, w.q_norm.value, N * HQ, D, eps, dt, s));
+        CGPTX_TRY(cgptx_rmsnorm_forward(a.k, a.k_pre, w.k_norm.value, N * HKV, D, eps, dt, s));
+        CGPTX_TRY(cgptx_rope_forward(a.q, a.k, m->cos_cache, m->sin_cache, m->batch, m->sequence, HQ, HKV, D,
+                                     c.rotary_dim, 0, m->sequence, dt, s));
+        CGPTX_TRY(cgptx_flash_gqa_attention_forward(a.attn_out, a.lse, a.q, a.k, a.v, m->batch, m->sequence,
+                                                    m->sequence, HQ, HKV, D, 0.0f, 1, 0, dt, s));
+        CGPTX_TRY(cgptx_linear_forward(m->d_residual, a.attn_out, w.o.value, nullptr, N, QW, H, dt, s));
+        CGPTX_TRY(cgptx_rmsnorm_forward(a.norm_f, x, w.ffn_norm.value, N, H, eps, dt, s));
+        CGPTX_TRY(cgptx_linear_forward(a.gate, a.norm_f, w.gate.value, nullptr, N, H, I, dt, s));
+        CGPTX_TRY(cgptx_linear_forward(a.up, a.norm_f, w.up.value, nullptr, N, H, I, dt, s));
+        CGPTX_TRY(cgptx_swiglu_forward(a.act, a.gate, a.up, N * I, dt, s));
+        CGPTX_TRY(cgptx_linear_forward(m->d_norm_in, a.act, w.down.value, nullptr, N, I, H, dt, s));
+        // out = x + attention_projection, then out += ffn_output (src/core/transformer_block.cu:594-595)
+        CGPTX_TRY(cgptx_add(out, x, m->d_residual, N * H, dt, s));
+        CGPTX_TRY(cgptx_add(out, out, m->d_norm_in, N * H, dt, s));
+    }
+    void* last = m->hidden[c.num_layers];
+    CGPTX_TRY(cgptx_rmsnorm_forward(m->normalized, last, m->final_norm.value, N, H, eps, dt, s));
+
+    // --------------------------------------------------------- loss + classifier
+    if (loss_mode == CGPTX_LOSS_CUT) {
+        CGPTX_TRY(cgptx_cut_cross_entropy_forward_backward(m->loss, m->d_normalized, m->embedding.gradient,
+                                                           m->normalized, m->embedding.value, m->targets, N, H,
+                                                           c.vocabulary_size, loss_scale, 0, dt, s));
+    } else {
+        CGPTX_TRY(cgptx_linear_forward(m->logits, m->normalized, m->embedding.value, nullptr, N, H,
+                                       c.vocabulary_size, dt, s));
+        CGPTX_TRY(cgptx_cross_entropy_forward_backward(m->loss, m->grad_logits, m->logits, m->targets, N,
+                                                       c.vocabulary_size, loss_scale, dt, s));
+        CGPTX_TRY(cgptx_linear_backward(m->d_normalized, m->embedding.gradient, nullptr, m->grad_logits,
+                                        m->normalized, m->embedding.value, N, H, c.vocabulary_size, 0, 0, 0, dt, s));
+    }
+
+    // ----------------------------------------------------------------- backward
+    void* current = m->grad_a;
+    void* previous = m->grad_b;
+    CGPTX_TRY(cgptx_rmsnorm_backward(current, m->final_norm.gradient, m->d_normalized, last, m->final_norm.value, N,
+                                     H, eps, dt, s));
+    for (std::size_t reverse = c.num_layers; reverse-- > 0;) {
+        const auto& w = m->layers[reverse];
+        const auto& a = m->acts[reverse];
+        void* x = m->hidden[reverse];
+        CGPTX_TRY(cgptx_linear_backward(m->d_act, w.down.gradient, nullptr, current, a.act, w.down.value, N, I, H, 0,
+                                        0, 0, dt, s));
+        CGPTX_TRY(cgptx_swiglu_backward(m->d_gate, m->d_up, m->d_act, a.gate, a.up, N * I, 0, 0, dt, s));
+        CGPTX_TRY(cgptx_linear_backward(m->d_norm_in, w.gate.gradient, nullptr, m->d_gate, a.norm_f, w.gate.value, N,
+                                        H, I, 0, 0, 0, dt, s));
+        CGPTX_TRY(cgptx_linear_backward(m->d_norm_in, w.up.gradient, nullptr, m->d_up, a.norm_f, w.up.value, N, H, I,
+                                        1, 0, 0, dt, s));
+        CGPTX_TRY(cgptx_rmsnorm_backward(m->d_residual, w.ffn_norm.gradient, m->d_norm_in, x, w.ffn_norm.value, N, H,
+                                         eps, dt, s));
+        CGPTX_TRY(cgptx_add(previous, current, m->d_residual, N * H, dt, s));
+        CGPTX_TRY(cgptx_linear_backward(m->d_attn_out, w.o.gradient, nullptr, current, a.attn_out, w.o.value, N, QW,
+                                        H, 0, 0, 0, dt, s));
+        CGPTX_TRY(cgptx_flash_gqa_attention_backward_with_lse(m->d_q, m->d_k, m->d_v, m->d_attn_out, a.attn_out,
+                                                              a.lse, a.q, a.k, a.v, m->batch, m->sequence,
+                                                              m->sequence, HQ, HKV, D, 0.0f, 1, 0, 0, dt, s));
+        CGPTX_TRY(cgptx_rope_backward(m->d_q_pre, m->d_k_pre, m->d_q, m->d_k, m->cos_cache, m->sin_cache, m->batch,
+                                      m->sequence, HQ, HKV, D, c.rotary_dim, 0, m->sequence, dt, s));
+        CGPTX_TRY(cgptx_rmsnorm_backward(m->d_q, w.q_norm.gradient, m->d_q_pre, a.q_pre, w.q_norm.value, N * HQ, D,
+                                         eps, dt, s));
+        CGPTX_TRY(cgptx_rmsnorm_backward(m->d_k, w.k_norm.gradient, m->d_k_pre, a.k_pre, w.k_norm.value, N * HKV, D,
+                                         eps, dt, s));
+        CGPTX_TRY(cgptx_linear_backward(m->d_norm_in, w.q.gradient, nullptr, m->d_q, a.norm_a, w.q.value, N, H, QW, 0,
+                                        0, 0, dt, s));
+        CGPTX_TRY(cgptx_linear_backward(m->d_norm_in, w.k.gradient, nullptr, m->d_k, a.norm_a, w.k.value, N, H, KW, 1,
+                                        0, 0, dt, s));
+        CGPTX_TRY(cgptx_linear_backward(m->d_norm_in, w.v.gradient, nullptr, m->d_v, a.norm_a, w.v.value, N, H, KW, 1,
+                                        0, 0, dt, s));
+        CGPTX_TRY(cgptx_rmsnorm_backward(m->d_residual, w.attention_norm.gradient, m->d_norm_in, x,
+                                         w.attention_norm.value, N, H, eps, dt, s));
+        CGPTX_TRY(cgptx_add(previous, previous, m->d_residual, N * H, dt, s));
+        std::swap(current, previous);
+    }
+    // Tied embedding: the classifier gradient is already in place; add the lookup's gradient
+    // (src/core/transformer_model.cu:375-380).
+    CGPTX_TRY(cgptx_embedding_backward(m->embedding.gradient, current, m->tokens, N, c.vocabulary_size, H, 1, 1, dt, s));
+    return CGPTX_OK;
+}
+
+int validate_config(const cgptx_model_config& c, std::size_t batch, std::size_t sequence) {
+    if (!valid_dtype(c.dtype)) return fail(CGPTX_INVALID_ARGUMENT, "model: unsupported dtype");
+    if (c.vocabulary_size == 0 || c.num_layers == 0 || c.hidden_size == 0 || c.intermediate_size == 0 ||
+        c.num_query_heads == 0 || c.num_kv_heads == 0 || c.head_dim == 0 || batch == 0 || sequence == 0)
+        return fail(CGPTX_INVALID_ARGUMENT, "model: every dimension must be positive");
+    if (c.num_query_heads % c.num_kv_heads != 0)
+        return fail(CGPTX_INVALID_ARGUMENT, "model: query heads must be a multiple of kv heads");
+    if (c.num_query_heads * c.head_dim != c.hidden_size)
+        return fail(CGPTX_INVALID_ARGUMENT, "model: hidden_size must equal num_query_heads * head_dim");
+    const std::size_t rotary = c.rotary_dim == 0 ? c.head_dim : c.rotary_dim;
+    if ((rotary & 1) != 0 || rotary > c.head_dim || (c.head_dim & 1) != 0)
+        return fail(CGPTX_INVALID_ARGUMENT, "model: head_dim and rotary_dim must be even, rotary_dim <= head_dim");
+    if (!std::isfinite(c.rms_epsilon) || c.rms_epsilon <= 0.0f || !std::isfinite(c.rope_base) || c.rope_base <= 0.0f)
+        return fail(CGPTX_INVALID_ARGUMENT, "model: invalid epsilon or rope base");
+    return CGPTX_OK;
+}
+
+}  // namespace
+}  // namespace cgptx
+
+extern "C" int cgptx_model_destroy(cgptx_model* m) {
+    if (m == nullptr) return CGPTX_OK;
+    (void)hipDeviceSynchronize();
+    if (m->graph_exec != nullptr) (void)hipGraphExecDestroy(m->graph_exec);
+    if (m->optimizer != nullptr) (void)cgptx_adamw_workspace_destroy(m->optimizer);
+    for (void* p : m->allocations) (void)hipFree(p);
+    delete m;
+    return CGPTX_OK;
+}
+
+extern "C" int cgptx_model_create(cgptx_model** out, const cgptx_model_config* config, size_t batch, size_t sequence,
+                                  uint64_t seed) {
+    using namespace cgptx;
+    if (out == nullptr || config == nullptr) return fail(CGPTX_INVALID_ARGUMENT, "model_create: null argument");
+    if (int s = validate_config(*config, batch, sequence)) return s;
+    auto* m = new cgptx_model();
+    m->config = *config;
+    if (m->config.rotary_dim == 0) m->config.rotary_dim = m->config.head_dim;
+    m->batch = batch;
+    m->sequence = sequence;
+    m->rows = batch * sequence;
+    const auto& c = m->config;
+    const std::size_t elem = dtype_size(c.dtype);
+    const std::size_t N = m->rows, H = c.hidden_size, I = c.intermediate_size;
+    const std::size_t QW = c.num_query_heads * c.head_dim, KW = c.num_kv_heads * c.head_dim;
+    const float stddev = 0.02f;
+    const float residual_stddev = stddev / std::sqrt(2.0f * static_cast<float>(c.num_layers));
+    auto build = [&]() -> int {
+        CGPTX_TRY(make_parameter(m, m->embedding, "model.embed_tokens.weight", c.vocabulary_size * H, 0, stddev, seed, 0));
+        CGPTX_TRY(make_parameter(m, m->final_norm, "model.norm.weight", H, 1, 0.0f, seed, 1));
+        m->layers.resize(c.num_layers);
+        m->acts.resize(c.num_layers);
+        for (std::size_t l = 0; l < c.num_layers; ++l) {
+            auto& w = m->layers[l];
+            const std::string prefix = "model.layers." + std::to_string(l) + ".";
+            const std::uint64_t id = 2 + l * 11;
+            CGPTX_TRY(make_parameter(m, w.attention_norm, prefix + "input_layernorm.weight", H, 1, 0, seed, id));
+            CGPTX_TRY(make_parameter(m, w.q, prefix + "self_attn.q_proj.weight", QW * H, 0, stddev, seed, id + 1));
+            CGPTX_TRY(make_parameter(m, w.k, prefix + "self_attn.k_proj.weight", KW * H, 0, stddev, seed, id + 2));
+            CGPTX_TRY(make_parameter(m, w.q_norm, prefix + "self_attn.q_norm.weight", c.head_dim, 1, 0, seed, id + 3));
+            CGPTX_TRY(make_parameter(m, w.k_norm, prefix + "self_attn.k_norm.weight", c.head_dim, 1, 0, seed, id + 4));
+            CGPTX_TRY(make_parameter(m, w.v, prefix + "self_attn.v_proj.weight", KW * H, 0, stddev, seed, id + 5));
+            CGPTX_TRY(make_parameter(m, w.o, prefix + "self_attn.o_proj.weight", H * QW, 0, residual_stddev, seed, id + 6));
+            CGPTX_TRY(make_parameter(m, w.ffn_norm, prefix + "post_attention_layernorm.weight", H, 1, 0, seed, id + 7));
+            CGPTX_TRY(make_parameter(m, w.gate, prefix + "mlp.gate_proj.weight", I * H, 0, stddev, seed, id + 8));
+            CGPTX_TRY(make_parameter(m, w.up, prefix + "mlp.up_proj.weight", I * H, 0, stddev, seed, id + 9));
+            CGPTX_TRY(make_parameter(m, w.down, prefix + "mlp.down_proj.weight", H * I, 0, residual_stddev, seed, id + 10));
+            auto& a = m->acts[l];
+            CGPTX_TRY(allocate(m, &a.norm_a, N * H * elem));
+            CGPTX_TRY(allocate(m, &a.q_pre, N * QW * elem));
+            CGPTX_TRY(allocate(m, &a.k_pre, N * KW * elem));
+            CGPTX_TRY(allocate(m, &a.q, N * QW * elem));
+            CGPTX_TRY(allocate(m, &a.k, N * KW * elem));
+            CGPTX_TRY(allocate(m, &a.v, N * KW * elem));
+            CGPTX_TRY(allocate(m, &a.attn_out, N * QW * elem));
+            CGPTX_TRY(allocate_typed(m, &a.lse, N * c.num_query_heads * sizeof(float)));
+            CGPTX_TRY(allocate(m, &a.norm_f, N * H * elem));
+            CGPTX_TRY(allocate(m, &a.gate, N * I * elem));
+            CGPTX_TRY(allocate(m, &a.up, N * I * elem));
+            CGPTX_TRY(allocate(m, &a.act, N * I * elem));
+        }
+        m->hidden.resize(c.num_layers + 1);
+        for (auto& h : m->hidden) CGPTX_TRY(allocate(m, &h, N * H * elem));
+        CGPTX_TRY(allocate(m, &m->normalized, N * H * elem));
+        CGPTX_TRY(allocate_typed(m, &m->tokens, N * sizeof(std::uint32_t)));
+        CGPTX_TRY(allocate_typed(m, &m->targets, N * sizeof(std::uint32_t)));
+        CGPTX_HIP(hipMemset(m->tokens, 0, N * sizeof(std::uint32_t)));
+        CGPTX_HIP(hipMemset(m->targets, 0, N * sizeof(std::uint32_t)));
+        CGPTX_TRY(allocate_typed(m, &m->loss, 256));
+        CGPTX_HIP(hipMemset(m->loss, 0, 256));
+        for (void** p : {&m->d_normalized, &m->grad_a, &m->grad_b, &m->d_norm_in, &m->d_residual})
+            CGPTX_TRY(allocate(m, p, N * H * elem));
+        for (void** p : {&m->d_act, &m->d_gate, &m->d_up}) CGPTX_TRY(allocate(m, p, N * I * elem));
+        for (void** p : {&m->d_attn_out, &m->d_q, &m->d_q_pre}) CGPTX_TRY(allocate(m, p, N * QW * elem));
+        for (void** p : {&m->d_k, &m->d_v, &m->d_k_pre}) CGPTX_TRY(allocate(m, p, N * KW * elem));
+        // Rotary cache: theta = pos / base^(2i/rotary), cos/sin in float, stored in the model dtype
+        // (train/train.cpp:322-333).
+        const std::size_t pairs = c.rotary_dim / 2;
+        std::vector<float> cosine(sequence * pairs), sine(sequence * pairs);
+        for (std::size_t pos = 0; pos < sequence; ++pos) {
+            for (std::size_t i = 0; i < pairs; ++i) {
+                const float theta = static_cast<float>(pos) /
+                                    std::pow(c.rope_base, 2.0f * static_cast<float>(i) / static_cast<float>(c.rotary_dim));
+                cosine[pos * pairs + i] = std::cos(theta);
+                sine[pos * pairs + i] = std::sin(theta);
+            }
+        }
+        std::vector<unsigned char> storage;
+        CGPTX_TRY(allocate(m, &m->cos_cache, sequence * pairs * elem));
+        CGPTX_TRY(allocate(m, &m->sin_cache, sequence * pairs * elem));
+        convert_to_storage(cosine, c.dtype, storage);
+        CGPTX_HIP(hipMemcpy(m->cos_cache, storage.data(), storage.size(), hipMemcpyHostToDevice));
+        convert_to_storage(sine, c.dtype, storage);
+        CGPTX_HIP(hipMemcpy(m->sin_cache, storage.data(), storage.size(), hipMemcpyHostToDevice));
+        CGPTX_TRY(cgptx_adamw_workspace_create(&m->optimizer));
+        std::vector<Parameter*> all;
+        collect(m, all);
+        for (Parameter* p : all)
+            m->entries.push_back({p->value, p->gradient, p->master, p->first, p->second, p->count, c.dtype});
+        return CGPTX_OK;
+    };
+    if (int s = build()) {
+        const std::string message = cgptx_last_error();
+        cgptx_model_destroy(m);
+        return fail(s, message);
+    }
+    *out = m;
+    return CGPTX_OK;
+}
+
+extern "C" int cgptx_model_set_tokens(cgptx_model* m, const uint32_t* inputs, const uint32_t* targets) {
+    using namespace cgptx;
+    if (m == nullptr || inputs == nullptr || targets == nullptr)
+        return fail(CGPTX_INVALID_ARGUMENT, "model_set_tokens: null argument");
+    CGPTX_HIP(hipDeviceSynchronize());
+    CGPTX_HIP(hipMemcpy(m->tokens, inputs, m->rows * sizeof(std::uint32_t), hipMemcpyHostToDevice));
+    CGPTX_HIP(hipMemcpy(m->targets, targets, m->rows * sizeof(std::uint32_t), hipMemcpyHostToDevice));
+    return CGPTX_OK;
+}
+
+extern "C" int cgptx_model_forward_backward(cgptx_model* m, float loss_scale, int loss_mode, int use_graph,
+                                            cgptx_stream stream_) {
+    using namespace cgptx;
+    if (m == nullptr) return fail(CGPTX_INVALID_ARGUMENT, "model_forward_backward: null model");
+    if (!std::isfinite(loss_scale) || loss_scale <= 0.0f)
+        return fail(CGPTX_INVALID_ARGUMENT, "model_forward_backward: loss scale must be finite and positive");
+    if (loss_mode != CGPTX_LOSS_DENSE && loss_mode != CGPTX_LOSS_CUT)
+        return fail(CGPTX_INVALID_ARGUMENT, "model_forward_backward: unknown loss mode");
+    auto stream = static_cast<hipStream_t>(stream_);
+    if (loss_mode == CGPTX_LOSS_DENSE && m->logits == nullptr) {
+        const std::size_t bytes = m->rows * m->config.vocabulary_size * dtype_size(m->config.dtype);
+        if (int s = allocate(m, &m->logits, bytes)) return s;
+        if (int s = allocate(m, &m->grad_logits, bytes)) return s;
+    }
+    if (!use_graph) return enqueue_forward_backward(m, loss_scale, loss_mode, stream);
+    if (stream == nullptr)
+        return fail(CGPTX_INVALID_ARGUMENT, "model_forward_backward: graph capture needs a non-default stream");
+    const bool have_graph = m->graph_exec != nullptr && m->graph_loss_scale == loss_scale &&
+                            m->graph_loss_mode == loss_mode && m->graph_stream == stream;
+    if (have_graph) {
+        CGPTX_HIP(hipGraphLaunch(m->graph_exec, stream));
+        return CGPTX_OK;
+    }
+    // Eager run first: it sizes every scratch arena and does this call's work. Then record the
+    // same sequence for the following calls.
+    if (int s = enqueue_forward_backward(m, loss_scale, loss_mode, stream)) return s;
+    CGPTX_HIP(hipStreamSynchronize(stream));
+    if (m->graph_exec != nullptr) {
+        CGPTX_HIP(hipGraphExecDestroy(m->graph_exec));
+        m->graph_exec = nullptr;
+    }
+    CGPTX_HIP(hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal));
+    const int status = enqueue_forward_backward(m, loss_scale, loss_mode, stream);
+    hipGraph_t graph = nullptr;
+    const hipError_t end = hipStreamEndCapture(stream, &graph);
+    if (status != CGPTX_OK) {
+        if (graph != nullptr) (void)hipGraphDestroy(graph);
+        return status;
+    }
+    CGPTX_HIP(end);
+    const hipError_t inst = hipGraphInstantiate(&m->graph_exec, graph, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(graph);
+    CGPTX_HIP(inst);
+    m->graph_loss_scale = loss_scale;
+    m->graph_loss_mode = loss_mode;
+    m->graph_stream = stream;
+    return CGPTX_OK;
+}
+
+extern "C" int cgptx_model_optimizer_step(cgptx_model* m, const cgptx_adamw_options* options, cgptx_stream stream) {
+    using namespace cgptx;
+    if (m == nullptr) return fail(CGPTX_INVALID_ARGUMENT, "model_optimizer_step: null model");
+    return cgptx_adamw_step_many_async(m->optimizer, m->entries.data(), m->entries.size(), options, 0, stream);
+}
+
+extern "C" int cgptx_model_train_step(cgptx_model* m, const cgptx_adamw_options* options, int loss_mode,
+                                      int use_graph, cgptx_stream stream) {
+    using namespace cgptx;
+    if (m == nullptr || options == nullptr) return fail(CGPTX_INVALID_ARGUMENT, "model_train_step: null argument");
+    if (int s = cgptx_model_forward_backward(m, options->loss_scale, loss_mode, use_graph, stream)) return s;
+    return cgptx_model_optimizer_step(m, options, stream);
+}
+
+extern "C" int cgptx_model_status(cgptx_model* m, float* loss, int* all_finite, uint64_t* step,
+                                  cgptx_stream stream_) {
+    using namespace cgptx;
+    if (m == nullptr || loss == nullptr || all_finite == nullptr || step == nullptr)
+        return fail(CGPTX_INVALID_ARGUMENT, "model_status: null argument");
+    auto stream = static_cast<hipStream_t>(stream_);
+    CGPTX_HIP(hipStreamSynchronize(stream));
+    CGPTX_HIP(hipMemcpy(loss, m->loss, sizeof(float), hipMemcpyDeviceToHost));
+    return cgptx_adamw_check(m->optimizer, all_finite, step, stream_);
+}
+
+extern "C" size_t cgptx_model_parameter_count(const cgptx_model* m) { return m == nullptr ? 0 : m->entries.size(); }
+
+extern "C" int cgptx_model_parameter(const cgptx_model* m, size_t index, const char** name, void** parameter,
+                                     void** gradient, size_t* count) {
+    using namespace cgptx;
+    if (m == nullptr || index >= m->entries.size())
+        return fail(CGPTX_INVALID_ARGUMENT, "model_parameter: index out of range");
+    std::vector<Parameter*> all;
+    collect(const_cast<cgptx_model*>(m), all);
+    if (name != nullptr) *name = all[index]->name.c_str();
+    if (parameter != nullptr) *parameter = all[index]->value;
+    if (gradient != nullptr) *gradient = all[index]->gradient;
+    if (count != nullptr) *count = all[index]->count;
+    return CGPTX_OK;
+}
+
+extern "C" size_t cgptx_model_num_parameters(const cgptx_model* m) {
+    if (m == nullptr) return 0;
+    size_t total = 0;
+    for (const auto& e : m->entries) total += e.count;
+    return total;
+}
+
+extern "C" int cgptx_model_activation(const cgptx_model* m, const char* name, void** data, size_t* count) {
+    using namespace cgptx;
+    if (m == nullptr || name == nullptr || data == nullptr || count == nullptr)
+        return fail(CGPTX_INVALID_ARGUMENT, "model_activation: null argument");
+    const std::string n(name);
+    const std::size_t NH = m->rows * m->config.hidden_size;
+    if (n == "normalized") { *data = m->normalized; *count = NH; return CGPTX_OK; }
+    if (n == "loss") { *data = m->loss; *count = 1; return CGPTX_OK; }
+    if (n == "logits" && m->logits != nullptr) {
+        *data = m->logits;
+        *count = m->rows * m->config.vocabulary_size;
+        return CGPTX_OK;
+    }
+    if (n.rfind("hidden.", 0) == 0) {
+        const std::size_t l = std::stoul(n.substr(7));
+        if (l < m->hidden.size()) { *data = m->hidden[l]; *count = NH; return CGPTX_OK; }
+    }
+    return fail(CGPTX_INVALID_ARGUMENT, "model_activation: unknown activation " + n);
+}

@@ -1,0 +1,84 @@
+/*
+ * cgptx_train.h — C-ABI of the caller side of the hot path: one decoder model
+ * (weights, gradients, AdamW state, activations) and its train step, composed
+ * from the operators of cgptx.h in the order the reference composes them:
+ *   forward   src/core/transformer_model.cu:195-241, src/core/transformer_block.cu:405-611
+ *   backward  src/core/transformer_model.cu:336-381, src/core/transformer_block.cu:644-748
+ *   step      train/train.cpp:536-556 (forward + loss + backward replayed from one
+ *             captured graph, AdamW enqueued after it)
+ * The block is the reference's parallel-residual block with per-head QK-norm:
+ *   out = x + Wo·Attn(rope(norm_q(Wq·n_a)), rope(norm_k(Wk·n_a)), Wv·n_a) + Wd·swiglu(Wg·n_f, Wu·n_f),
+ *   n_a = RMSNorm_a(x), n_f = RMSNorm_f(x); embeddings are tied to the classifier.
+ */
+#ifndef CGPTX_TRAIN_H
+#define CGPTX_TRAIN_H
+
+#include "cgptx.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* TransformerModelOptions + TransformerBlockOptions (include/core/transformer_model.h,
+ * include/core/transformer_block.h); the 104m preset is train/train.cpp:146-148. */
+typedef struct cgptx_model_config {
+    size_t vocabulary_size;
+    size_t num_layers;
+    size_t hidden_size;
+    size_t intermediate_size;
+    size_t num_query_heads;
+    size_t num_kv_heads;
+    size_t head_dim;
+    size_t rotary_dim;
+    float rms_epsilon;
+    float rope_base;   /* 10000 in train/train.cpp:326 */
+    int dtype;         /* storage dtype of weights, activations and gradients */
+} cgptx_model_config;
+
+enum { CGPTX_LOSS_DENSE = 0, CGPTX_LOSS_CUT = 1 };
+
+typedef struct cgptx_model cgptx_model;
+
+/* Allocates everything for a fixed [batch, sequence] step and initialises the weights from
+ * `seed` with a counter-based generator: N(0, 0.02), o/down projections N(0, 0.02/sqrt(2L)),
+ * norm weights 1 (the distribution of src/core/weight_initialization.cu:158-179). */
+int cgptx_model_create(cgptx_model** model, const cgptx_model_config* config, size_t batch, size_t sequence,
+                       uint64_t seed);
+int cgptx_model_destroy(cgptx_model* model);
+
+/* Copies `batch*sequence` input and target ids from host memory into the model's graph-stable
+ * device buffers (data::upload_batch, src/data/dataset_loader.cpp:145-166). Synchronous. */
+int cgptx_model_set_tokens(cgptx_model* model, const uint32_t* inputs, const uint32_t* targets);
+
+/* Enqueues forward + loss + backward on `stream` (gradient of loss·loss_scale). With use_graph
+ * the sequence is captured on first use (after one eager run) and replayed afterwards. */
+int cgptx_model_forward_backward(cgptx_model* model, float loss_scale, int loss_mode, int use_graph,
+                                 cgptx_stream stream);
+
+/* Enqueues the global-norm AdamW update over all parameters (adamw_step_many_async). */
+int cgptx_model_optimizer_step(cgptx_model* model, const cgptx_adamw_options* options, cgptx_stream stream);
+
+/* forward_backward followed by optimizer_step. */
+int cgptx_model_train_step(cgptx_model* model, const cgptx_adamw_options* options, int loss_mode, int use_graph,
+                           cgptx_stream stream);
+
+/* Synchronises `stream`; returns the last loss, whether all optimizer steps since the previous
+ * call saw finite gradients, and the optimizer step count (adamw_check). */
+int cgptx_model_status(cgptx_model* model, float* loss, int* all_finite, uint64_t* step, cgptx_stream stream);
+
+/* Number of parameter tensors and, per index, name / device pointers / element count. Names follow
+ * the checkpoint names of src/core/huggingface_export.cpp:362-378 where one exists. */
+size_t cgptx_model_parameter_count(const cgptx_model* model);
+int cgptx_model_parameter(const cgptx_model* model, size_t index, const char** name, void** parameter,
+                          void** gradient, size_t* count);
+/* Total number of parameters (tied embedding counted once). */
+size_t cgptx_model_num_parameters(const cgptx_model* model);
+
+/* Device pointer to a named saved activation of the last forward ("hidden.<l>", "logits" ...);
+ * used by tests. Returns INVALID_ARGUMENT for unknown names. */
+int cgptx_model_activation(const cgptx_model* model, const char* name, void** data, size_t* count);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CGPTX_TRAIN_H */

@@ -1,0 +1,219 @@
+"""The composed train step: the float64 composition is pinned by finite differences (CPU), then
+the GPU step (eager and hipGraph replay, dense and cut loss) is compared with it."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import model64
+from tests.util import to_np
+
+TINY = dict(vocab=50, layers=2, hidden=32, inter=48, hq=4, hkv=2, d=8, eps=1e-5)
+
+
+def random_params(cfg, rng, scale=0.3):
+    H, I, QW, KW = cfg["hidden"], cfg["inter"], cfg["hq"] * cfg["d"], cfg["hkv"] * cfg["d"]
+    layers = []
+    for _ in range(cfg["layers"]):
+        layers.append({
+            "attention_norm": 1 + 0.1 * rng.normal(size=H), "q": scale * rng.normal(size=(QW, H)),
+            "k": scale * rng.normal(size=(KW, H)), "q_norm": 1 + 0.1 * rng.normal(size=cfg["d"]),
+            "k_norm": 1 + 0.1 * rng.normal(size=cfg["d"]), "v": scale * rng.normal(size=(KW, H)),
+            "o": scale * rng.normal(size=(H, QW)), "ffn_norm": 1 + 0.1 * rng.normal(size=H),
+            "gate": scale * rng.normal(size=(I, H)), "up": scale * rng.normal(size=(I, H)),
+            "down": scale * rng.normal(size=(H, I)),
+        })
+    return {"embedding": scale * rng.normal(size=(cfg["vocab"], H)), "final_norm": 1 + 0.1 * rng.normal(size=H),
+            "layers": layers}
+
+
+def test_float64_composition_matches_finite_differences():
+    """Pins oracle/model64.py: its analytic gradients equal central differences of its own loss,
+    for a sample of entries of every parameter tensor (incl. the tied embedding, which receives
+    both the classifier and the lookup gradient)."""
+    cfg = dict(TINY, layers=2)
+    rng = np.random.default_rng(0)
+    params = random_params(cfg, rng)
+    tokens = rng.integers(0, cfg["vocab"], size=(2, 5))
+    targets = rng.integers(0, cfg["vocab"], size=(2, 5))
+    tokens[0, 1] = tokens[0, 3]  # a repeated id
+    loss, grads, _ = model64.forward_backward(params, tokens, targets, cfg)
+    assert np.isfinite(loss)
+
+    def check(array, grad, name):
+        flat = array.reshape(-1)
+        for idx in rng.choice(flat.size, size=min(6, flat.size), replace=False):
+            old = flat[idx]
+            flat[idx] = old + 1e-6
+            hi = model64.loss_only(params, tokens, targets, cfg)
+            flat[idx] = old - 1e-6
+            lo = model64.loss_only(params, tokens, targets, cfg)
+            flat[idx] = old
+            fd = (hi - lo) / 2e-6
+            assert abs(fd - grad.reshape(-1)[idx]) <= 1e-6 + 1e-5 * abs(fd), (name, idx, fd, grad.reshape(-1)[idx])
+
+    check(params["embedding"], grads["embedding"], "embedding")
+    check(params["final_norm"], grads["final_norm"], "final_norm")
+    for l, (w, g) in enumerate(zip(params["layers"], grads["layers"])):
+        for key in model64.LAYER_KEYS:
+            check(w[key], g[key], f"layer{l}.{key}")
+    # the embedding row of a token that is used twice and is also a target gets all three contributions
+    used = tokens[0, 1]
+    assert np.abs(grads["embedding"][used]).max() > 0
+
+
+# --------------------------------------------------------------------------------- GPU
+def torch_round(dtype):
+    def rnd(a):
+        return torch.from_numpy(np.asarray(a, dtype=np.float64)).to(torch.float32).to(dtype).to(torch.float64).numpy()
+    return rnd
+
+
+def build(device, dtype, batch, seq, cfg, seed=3):
+    from cgpt_amd.model import Model, ModelConfig
+
+    config = ModelConfig(vocabulary_size=cfg["vocab"], num_layers=cfg["layers"], hidden_size=cfg["hidden"],
+                         intermediate_size=cfg["inter"], num_query_heads=cfg["hq"], num_kv_heads=cfg["hkv"],
+                         head_dim=cfg["d"], rotary_dim=cfg["d"], rms_epsilon=cfg["eps"], dtype=dtype)
+    return Model(config, batch, seq, seed=seed, device=device)
+
+
+def params_from_model(model, cfg):
+    """Reads the library's (rounded) weights back as the float64 parameter structure."""
+    H, I, QW, KW, D = cfg["hidden"], cfg["inter"], cfg["hq"] * cfg["d"], cfg["hkv"] * cfg["d"], cfg["d"]
+    shapes = {"attention_norm": (H,), "q": (QW, H), "k": (KW, H), "q_norm": (D,), "k_norm": (D,), "v": (KW, H),
+              "o": (H, QW), "ffn_norm": (H,), "gate": (I, H), "up": (I, H), "down": (H, I)}
+    names = {"input_layernorm.weight": "attention_norm", "self_attn.q_proj.weight": "q",
+             "self_attn.k_proj.weight": "k", "self_attn.q_norm.weight": "q_norm", "self_attn.k_norm.weight": "k_norm",
+             "self_attn.v_proj.weight": "v", "self_attn.o_proj.weight": "o",
+             "post_attention_layernorm.weight": "ffn_norm", "mlp.gate_proj.weight": "gate",
+             "mlp.up_proj.weight": "up", "mlp.down_proj.weight": "down"}
+    params = {"layers": [dict() for _ in range(cfg["layers"])]}
+    grads = {"layers": [dict() for _ in range(cfg["layers"])]}
+    for name, p, g in model.parameters():
+        if name == "model.embed_tokens.weight":
+            params["embedding"], grads["embedding"] = to_np(p).reshape(cfg["vocab"], H), g
+        elif name == "model.norm.weight":
+            params["final_norm"], grads["final_norm"] = to_np(p), g
+        else:
+            _, _, layer, rest = name.split(".", 3)
+            key = names[rest]
+            params["layers"][int(layer)][key] = to_np(p).reshape(shapes[key])
+            grads["layers"][int(layer)][key] = g
+    return params, grads
+
+
+def compare_gradients(got, want, tol, loss_scale):
+    def one(g, w, name):
+        w = np.asarray(w).reshape(-1)
+        scale = max(np.abs(w).max(), 1e-3 * loss_scale)
+        err = np.abs(to_np(g) - w).max() / scale
+        assert np.isfinite(to_np(g)).all(), name
+        assert err <= tol, f"{name}: error {err:.3e} of the tensor's scale"
+    one(got["embedding"], want["embedding"], "embedding")
+    one(got["final_norm"], want["final_norm"], "final_norm")
+    for l, (g, w) in enumerate(zip(got["layers"], want["layers"])):
+        for key in model64.LAYER_KEYS:
+            one(g[key], w[key], f"layer{l}.{key}")
+
+
+MODEL_CFG = dict(vocab=96, layers=2, hidden=64, inter=128, hq=2, hkv=1, d=32, eps=1e-5)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+@pytest.mark.parametrize("loss_mode", [0, 1], ids=["dense", "cut"])
+def test_gpu_step_matches_float64_composition(device, dtype, loss_mode):
+    """Hidden 64, 2:1 heads of 32, T=24, B=2, two layers: every parameter gradient of the GPU step against
+    the float64 composition that rounds each operator output to the storage dtype where the GPU stores it.
+    Tolerance: 5e-2 of each tensor's largest gradient entry (2e-2 per operator, several operators deep)."""
+    cfg = MODEL_CFG
+    batch, seq, loss_scale = 2, 24, 64.0
+    model = build(device, dtype, batch, seq, cfg)
+    rng = np.random.default_rng(5)
+    tokens = rng.integers(0, cfg["vocab"], size=(batch, seq))
+    targets = rng.integers(0, cfg["vocab"], size=(batch, seq))
+    tokens[1, 2] = tokens[1, 7]
+    model.set_tokens(tokens, targets)
+    model.forward_backward(loss_scale, loss_mode, use_graph=False)
+    loss, _, _ = model.status()
+    params, grads = params_from_model(model, cfg)
+    want_loss, want, saved = model64.forward_backward(params, tokens, targets, cfg, loss_scale, torch_round(dtype))
+    assert abs(loss - want_loss) <= 2e-2 * want_loss
+    for l in range(cfg["layers"] + 1):
+        hidden = to_np(model.activation(f"hidden.{l}")).reshape(batch * seq, cfg["hidden"])
+        assert np.abs(hidden - saved["hidden"][l]).max() <= 4e-2 * max(1.0, np.abs(saved["hidden"][l]).max())
+    compare_gradients(grads, want, 5e-2, loss_scale)
+    model.close()
+
+
+@pytest.mark.gpu
+def test_graph_replay_equals_eager_and_losses_agree_between_modes(device):
+    cfg = MODEL_CFG
+    dtype = torch.bfloat16
+    batch, seq = 2, 40
+    rng = np.random.default_rng(6)
+    tokens = rng.integers(0, cfg["vocab"], size=(batch, seq))
+    targets = rng.integers(0, cfg["vocab"], size=(batch, seq))
+    stream = torch.cuda.Stream(device=device)
+    results = {}
+    for mode in (0, 1):
+        model = build(device, dtype, batch, seq, cfg)
+        model.set_tokens(tokens, targets)
+        model.forward_backward(1024.0, mode, use_graph=False, stream=stream)
+        loss_eager = model.status(stream)[0]
+        eager = [g.clone() for _, _, g in model.parameters()]
+        model.forward_backward(1024.0, mode, use_graph=True, stream=stream)   # eager run + capture
+        for replay in range(3):
+            for _, _, g in model.parameters():
+                g.zero_()
+            torch.cuda.synchronize()
+            model.forward_backward(1024.0, mode, use_graph=True, stream=stream)  # replay
+            loss_graph = model.status(stream)[0]
+            assert loss_graph == loss_eager
+            for (name, _, g), e in zip(model.parameters(), eager):
+                assert torch.equal(g, e), f"{name} differs on replay {replay}"
+        results[mode] = (loss_eager, eager)
+        model.close()
+    assert abs(results[0][0] - results[1][0]) <= 1e-3 * results[0][0]
+    for a, b in zip(results[0][1], results[1][1]):
+        scale = max(float(a.float().abs().max()), 1e-3)
+        assert float((a.float() - b.float()).abs().max()) <= 3e-2 * scale
+
+
+@pytest.mark.gpu
+def test_train_steps_reduce_the_loss_and_count_steps(device):
+    cfg = MODEL_CFG
+    from cgpt_amd.ops import AdamWOptions
+
+    model = build(device, torch.bfloat16, 4, 32, cfg)
+    rng = np.random.default_rng(7)
+    tokens = rng.integers(0, cfg["vocab"], size=(4, 32))
+    model.set_tokens(tokens, np.roll(tokens, -1, axis=1))
+    options = AdamWOptions(learning_rate=1e-2, beta1=0.9, beta2=0.95, weight_decay=0.1, loss_scale=1024.0,
+                           max_grad_norm=1.0)
+    stream = torch.cuda.Stream(device=device)
+    losses = []
+    for _ in range(30):
+        model.train_step(options, loss_mode=1, use_graph=True, stream=stream)
+        losses.append(model.status(stream))
+    assert all(finite for _, finite, _ in losses)
+    assert losses[-1][2] == 30
+    assert losses[-1][0] < 0.5 * losses[0][0]
+    assert abs(losses[0][0] - np.log(cfg["vocab"])) < 0.5   # random init: loss starts near ln(vocab)
+    model.close()
+
+
+@pytest.mark.gpu
+def test_model_argument_errors(device):
+    from cgpt_amd.model import Model, ModelConfig
+
+    with pytest.raises(ValueError):
+        Model(ModelConfig(num_query_heads=8, num_kv_heads=3), 1, 8, device=device)
+    with pytest.raises(ValueError):
+        Model(ModelConfig(hidden_size=1000), 1, 8, device=device)
+    model = build(device, torch.bfloat16, 1, 8, MODEL_CFG)
+    with pytest.raises(ValueError):
+        model.forward_backward(0.0, 1)
+    with pytest.raises(ValueError):
+        model.forward_backward(1.0, 1, use_graph=True, stream=0)   # capture needs a real stream
+    model.close()
