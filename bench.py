@@ -1,0 +1,174 @@
+#!/usr/bin/env python3
+"""Headline benchmark: train tokens/s of one full 104m step (forward + loss + backward + AdamW)
+at B=32, T=1024 on one MI355X, bf16 storage with fp32 accumulation, synthetic seeded token ids
+and random-init weights.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--loss cut|dense] [--no-cpu-baseline]
+
+Prints ONE JSON line. Besides the contract fields it carries
+  roofline     – the operator kind that takes the most time in the step (from HIP events
+                 recorded around every operator call of one eager pass on the launch stream):
+                 algorithmic FLOPs of its launches / their summed duration, against the
+                 2.5 PFLOP/s dense bf16 MFMA peak; plus the per-kind breakdown in milliseconds;
+  cpu_baseline – the float32 CPU restatement of the reference's operators (oracle/, "port")
+                 timed on this host on a bounded sample of the same workload.
+This run uses one GPU; --gpus above 1 exits with a message.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import sys
+import time
+
+import numpy as np
+
+PEAK_BF16_TFLOPS = 2500.0
+PEAK_HBM_GBS = 8000.0
+
+
+def op_work(cfg, batch, seq, loss_mode):
+    """Algorithmic FLOPs (MFMA-bound kinds) or HBM bytes (bandwidth-bound kinds) per step and kind."""
+    N, H, I, V, L = batch * seq, cfg.hidden_size, cfg.intermediate_size, cfg.vocabulary_size, cfg.num_layers
+    HQ, HKV, D = cfg.num_query_heads, cfg.num_kv_heads, cfg.head_dim
+    QW, KW = HQ * D, HKV * D
+    layer_weights = QW * H + 2 * KW * H + H * QW + 2 * I * H + H * I
+    linear = 2.0 * N * layer_weights * L
+    head = 2.0 * N * V * H
+    attention = 2.0 * batch * HQ * seq * seq * D / 2  # one causal matmul
+    e = 2  # bytes per 16-bit element
+    work = {
+        "gemm_fwd": ("mfma", linear + (head if loss_mode == "dense" else 0)),
+        "gemm_dx": ("mfma", linear + (head if loss_mode == "dense" else 0)),
+        "gemm_dw": ("mfma", linear + (head if loss_mode == "dense" else 0)),
+        "cut_ce": ("mfma", 3 * head),
+        "attn_fwd": ("mfma", 2 * attention * L),
+        "attn_bwd": ("mfma", 5 * attention * L),
+        "dense_ce": ("hbm", 2.0 * N * V * e),
+        "rmsnorm_fwd": ("hbm", (2 * N * H * 2 + N * (QW + KW) * 2) * e * L + 2 * N * H * e),
+        "rmsnorm_bwd": ("hbm", (2 * N * H * 3 + N * (QW + KW) * 3) * e * L + 3 * N * H * e),
+        "rope_fwd": ("hbm", N * (QW + KW) * 2 * e * L),
+        "rope_bwd": ("hbm", N * (QW + KW) * 2 * e * L),
+        "swiglu_fwd": ("hbm", N * I * 3 * e * L),
+        "swiglu_bwd": ("hbm", N * I * 5 * e * L),
+        "add": ("hbm", N * H * 3 * e * 4 * L),
+        "embedding_fwd": ("hbm", N * H * 2 * e),
+        "embedding_bwd": ("hbm", N * H * 3 * e),
+    }
+    return work
+
+
+def cpu_baseline(seed):
+    """Times the CPU port on B=1, T=8 of the same 104m model (forward + loss + backward + AdamW)."""
+    from oracle import cpu_model, cpu_ops
+
+    cfg = dict(vocab=32000, layers=8, hidden=1024, inter=2048, hq=8, hkv=2, d=128, eps=1e-5)
+    batch, seq = 1, 8
+    seconds, loss = cpu_model.timed_train_step(cfg, batch, seq, seed)
+    return {"value": batch * seq / seconds, "unit": "tokens/s", "cores": cpu_ops.max_threads(), "kind": "port",
+            "sample": f"one full 104m train step (fwd+loss+bwd+AdamW, fp32) at B={batch}, T={seq}: "
+                      f"{seconds:.1f} s, loss {loss:.3f}; attention backward is cubic in T on this path, "
+                      "so the rate does not extrapolate to T=1024"}
+
+
+def main() -> int:
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=10)
+    parser.add_argument("--warmup", type=int, default=3)
+    parser.add_argument("--batch", type=int, default=32)
+    parser.add_argument("--seq", type=int, default=1024)
+    parser.add_argument("--loss", choices=["cut", "dense"], default="cut")
+    parser.add_argument("--no-graph", action="store_true")
+    parser.add_argument("--no-cpu-baseline", action="store_true")
+    parser.add_argument("--seed", type=int, default=0)
+    args = parser.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this build runs on one GPU; --gpus {args.gpus} is not supported "
+              "(no collectives are part of the measured path)", file=sys.stderr)
+        return 2
+
+    import torch
+
+    from cgpt_amd.model import LOSS_CUT, LOSS_DENSE, Model, ModelConfig
+    from cgpt_amd.ops import AdamWOptions
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 3
+    device = torch.device("cuda:0")
+    cfg = ModelConfig()  # the reference's 104m preset
+    model = Model(cfg, args.batch, args.seq, seed=args.seed, device=device)
+    rng = np.random.default_rng(args.seed)
+    model.set_tokens(rng.integers(0, cfg.vocabulary_size, size=(args.batch, args.seq)),
+                     rng.integers(0, cfg.vocabulary_size, size=(args.batch, args.seq)))
+    options = AdamWOptions(learning_rate=3e-4, beta1=0.9, beta2=0.95, epsilon=1e-8, weight_decay=0.1,
+                           loss_scale=1024.0, max_grad_norm=1.0)
+    loss_mode = LOSS_CUT if args.loss == "cut" else LOSS_DENSE
+    stream = torch.cuda.Stream(device=device)
+    use_graph = not args.no_graph
+
+    for _ in range(args.warmup):
+        model.train_step(options, loss_mode, use_graph, stream)
+    first_loss, finite, _ = model.status(stream)
+    torch.cuda.synchronize()
+    start = time.perf_counter()
+    for _ in range(args.steps):
+        model.train_step(options, loss_mode, use_graph, stream)
+    stream.synchronize()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - start
+    last_loss, finite_after, steps_done = model.status(stream)
+    tokens = args.batch * args.seq
+    ms_per_step = elapsed / max(args.steps, 1) * 1e3
+
+    breakdown = model.profile(options.loss_scale, loss_mode, stream)
+    work = op_work(cfg, args.batch, args.seq, args.loss)
+    dominant = max(breakdown, key=breakdown.get)
+    bound, amount = work[dominant]
+    seconds = breakdown[dominant] * 1e-3
+    if bound == "mfma":
+        achieved, peak, unit = amount / seconds / 1e12, PEAK_BF16_TFLOPS, "TFLOP/s"
+    else:
+        achieved, peak, unit = amount / seconds / 1e9, PEAK_HBM_GBS, "GB/s"
+    per_kind = {}
+    for kind, ms in sorted(breakdown.items(), key=lambda kv: -kv[1]):
+        b, amt = work[kind]
+        rate = amt / (ms * 1e-3) / (1e12 if b == "mfma" else 1e9)
+        per_kind[kind] = {"ms": round(ms, 3), "rate": round(rate, 1), "unit": "TFLOP/s" if b == "mfma" else "GB/s",
+                          "frac": round(rate / (PEAK_BF16_TFLOPS if b == "mfma" else PEAK_HBM_GBS), 4)}
+
+    result = {
+        "metric": "train tokens/sec, 104m fwd+bwd+AdamW B=32 T=1024",
+        "value": tokens * args.steps / elapsed,
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": f"full 104m train step (embedding, 8 blocks, {args.loss} cross-entropy, backward, "
+                               f"AdamW), B={args.batch}, T={args.seq}, hipGraph={'on' if use_graph else 'off'}",
+                   "parameters": model.num_parameters, "global_batch": args.batch, "seq_len": args.seq,
+                   "loss_scale": 1024.0},
+        "loss_first": first_loss, "loss_last": last_loss, "all_finite": bool(finite and finite_after),
+        "optimizer_steps": steps_done,
+        "roofline": {"bound": bound, "achieved": achieved, "peak": peak, "unit": unit, "frac": achieved / peak,
+                     "traffic": None, "kernel": dominant,
+                     "note": "algorithmic work of all launches of this operator kind in one step / their summed "
+                             "duration (HIP events around each call on the launch stream, one eager pass)",
+                     "breakdown": per_kind},
+    }
+    model.close()
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(args.seed)
+    print(json.dumps(result))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -84,9 +84,12 @@ PROTOTYPES = {
     "cgptx_model_parameter": [_vp, _sz, ctypes.POINTER(ctypes.c_char_p), ctypes.POINTER(_vp), ctypes.POINTER(_vp),
                               ctypes.POINTER(_sz)],
     "cgptx_model_activation": [_vp, ctypes.c_char_p, ctypes.POINTER(_vp), ctypes.POINTER(_sz)],
+    "cgptx_model_profile": [_vp, _f, _i, _vp],
+    "cgptx_model_profile_entry": [_vp, _sz, ctypes.POINTER(ctypes.c_char_p), ctypes.POINTER(_f)],
 }
 
-SIZE_FUNCTIONS = {"cgptx_model_parameter_count": [_vp], "cgptx_model_num_parameters": [_vp]}
+SIZE_FUNCTIONS = {"cgptx_model_parameter_count": [_vp], "cgptx_model_num_parameters": [_vp],
+                  "cgptx_model_profile_count": [_vp]}
 
 STRING_FUNCTIONS = ("cgptx_last_error", "cgptx_version")
 

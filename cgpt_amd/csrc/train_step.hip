@@ -112,9 +112,14 @@ struct cgptx_model {
     float graph_loss_scale = 0.0f;
     int graph_loss_mode = -1;
     hipStream_t graph_stream = nullptr;
-    bool warmed = false;
-    float warm_loss_scale = 0.0f;
-    int warm_loss_mode = -1;
+    // optional per-operator timing of one eager pass
+    struct Timed {
+        const char* label;
+        hipEvent_t start, stop;
+    };
+    bool profiling = false;
+    std::vector<Timed> timed;
+    std::vector<std::pair<std::string, float>> profile;  // label, milliseconds (summed per label)
 };
 
 namespace cgptx {
@@ -191,6 +196,34 @@ void collect(cgptx_model* m, std::vector<Parameter*>& out) {
         if (int status_ = (expr)) return status_; \
     } while (0)
 
+// Runs one operator call; when profiling, brackets it with events on the same stream.
+#define CGPTX_OP(label, expr)                                                   \
+    do {                                                                        \
+        cgptx_model::Timed t_{label, nullptr, nullptr};                         \
+        if (m->profiling) {                                                     \
+            CGPTX_HIP(hipEventCreate(&t_.start));                               \
+            CGPTX_HIP(hipEventCreate(&t_.stop));                                \
+            CGPTX_HIP(hipEventRecord(t_.start, stream));                        \
+        }                                                                       \
+        if (int status_ = (expr)) return status_;                               \
+        if (m->profiling) {                                                     \
+            CGPTX_HIP(hipEventRecord(t_.stop, stream));                         \
+            m->timed.push_back(t_);                                             \
+        }                                                                       \
+    } while (0)
+
+// linear_backward as two single-kernel calls so that each can be timed on its own.
+int linear_backward_split(cgptx_model* m, void* dx, void* dw, const void* dy, const void* x, const void* w,
+                          std::size_t rows, std::size_t in_features, std::size_t out_features, int accumulate_input,
+                          int dt, hipStream_t stream) {
+    auto* s = static_cast<cgptx_stream>(stream);
+    CGPTX_OP("gemm_dx", cgptx_linear_backward(dx, nullptr, nullptr, dy, x, w, rows, in_features, out_features,
+                                              accumulate_input, 0, 0, dt, s));
+    CGPTX_OP("gemm_dw", cgptx_linear_backward(nullptr, dw, nullptr, dy, x, w, rows, in_features, out_features, 0, 0,
+                                              0, dt, s));
+    return CGPTX_OK;
+}
+
 int enqueue_forward_backward(cgptx_model* m, float loss_scale, int loss_mode, hipStream_t stream) {
     const auto& c = m->config;
     const int dt = c.dtype;
@@ -201,93 +234,85 @@ int enqueue_forward_backward(cgptx_model* m, float loss_scale, int loss_mode, hi
     auto* s = static_cast<cgptx_stream>(stream);
 
     // ------------------------------------------------------------------ forward
-    CGPTX_TRY(cgptx_embedding_forward(m->hidden[0], m->tokens, N, m->embedding.value, c.vocabulary_size, H, dt, s));
+    CGPTX_OP("embedding_fwd", cgptx_embedding_forward(m->hidden[0], m->tokens, N, m->embedding.value, c.vocabulary_size, H, dt, s));
     for (std::size_t l = 0; l < c.num_layers; ++l) {
         const auto& w = m->layers[l];
         const auto& a = m->acts[l];
         void* x = m->hidden[l];
         void* out = m->hidden[l + 1];
-        CGPTX_TRY(cgptx_rmsnorm_forward(a.norm_a, x, w.attention_norm.value, N, H, eps, dt, s));
-        CGPTX_TRY(cgptx_linear_forward(a.q_pre, a.norm_a, w.q.value, nullptr, N, H, QW, dt, s));
-        CGPTX_TRY(cgptx_linear_forward(a.k_pre, a.norm_a, w.k.value, nullptr, N, H, KW, dt, s));
-        CGPTX_TRY(cgptx_linear_forward(a.v, a.norm_a, w.v.value, nullptr, N, H, KW, dt, s));
-        CGPTX_TRY(cgptx_rmsnorm_forward(a.q, a.q_pre, w.q_norm.value, N * HQ, D, eps, dt, s));
-        CGPTX_TRY(cgptx_rmsnorm_forward(a.k, a.k_pre, w.k_norm.value, N * HKV, D, eps, dt, s));
-        CGPTX_TRY(cgptx_rope_forward(a.q, a.k, m->cos_cache, m->sin_cache, m->batch, m->sequence, HQ, HKV, D,
+        CGPTX_OP("rmsnorm_fwd", cgptx_rmsnorm_forward(a.norm_a, x, w.attention_norm.value, N, H, eps, dt, s));
+        CGPTX_OP("gemm_fwd", cgptx_linear_forward(a.q_pre, a.norm_a, w.q.value, nullptr, N, H, QW, dt, s));
+        CGPTX_OP("gemm_fwd", cgptx_linear_forward(a.k_pre, a.norm_a, w.k.value, nullptr, N, H, KW, dt, s));
+        CGPTX_OP("gemm_fwd", cgptx_linear_forward(a.v, a.norm_a, w.v.value, nullptr, N, H, KW, dt, s));
+        CGPTX_OP("rmsnorm_fwd", cgptx_rmsnorm_forward(a.q, a.q_pre, w.q_norm.value, N * HQ, D, eps, dt, s));
+        CGPTX_OP("rmsnorm_fwd", cgptx_rmsnorm_forward(a.k, a.k_pre, w.k_norm.value, N * HKV, D, eps, dt, s));
+        CGPTX_OP("rope_fwd", cgptx_rope_forward(a.q, a.k, m->cos_cache, m->sin_cache, m->batch, m->sequence, HQ, HKV, D,
                                      c.rotary_dim, 0, m->sequence, dt, s));
-        CGPTX_TRY(cgptx_flash_gqa_attention_forward(a.attn_out, a.lse, a.q, a.k, a.v, m->batch, m->sequence,
+        CGPTX_OP("attn_fwd", cgptx_flash_gqa_attention_forward(a.attn_out, a.lse, a.q, a.k, a.v, m->batch, m->sequence,
                                                     m->sequence, HQ, HKV, D, 0.0f, 1, 0, dt, s));
-        CGPTX_TRY(cgptx_linear_forward(m->d_residual, a.attn_out, w.o.value, nullptr, N, QW, H, dt, s));
-        CGPTX_TRY(cgptx_rmsnorm_forward(a.norm_f, x, w.ffn_norm.value, N, H, eps, dt, s));
-        CGPTX_TRY(cgptx_linear_forward(a.gate, a.norm_f, w.gate.value, nullptr, N, H, I, dt, s));
-        CGPTX_TRY(cgptx_linear_forward(a.up, a.norm_f, w.up.value, nullptr, N, H, I, dt, s));
-        CGPTX_TRY(cgptx_swiglu_forward(a.act, a.gate, a.up, N * I, dt, s));
-        CGPTX_TRY(cgptx_linear_forward(m->d_norm_in, a.act, w.down.value, nullptr, N, I, H, dt, s));
+        CGPTX_OP("gemm_fwd", cgptx_linear_forward(m->d_residual, a.attn_out, w.o.value, nullptr, N, QW, H, dt, s));
+        CGPTX_OP("rmsnorm_fwd", cgptx_rmsnorm_forward(a.norm_f, x, w.ffn_norm.value, N, H, eps, dt, s));
+        CGPTX_OP("gemm_fwd", cgptx_linear_forward(a.gate, a.norm_f, w.gate.value, nullptr, N, H, I, dt, s));
+        CGPTX_OP("gemm_fwd", cgptx_linear_forward(a.up, a.norm_f, w.up.value, nullptr, N, H, I, dt, s));
+        CGPTX_OP("swiglu_fwd", cgptx_swiglu_forward(a.act, a.gate, a.up, N * I, dt, s));
+        CGPTX_OP("gemm_fwd", cgptx_linear_forward(m->d_norm_in, a.act, w.down.value, nullptr, N, I, H, dt, s));
         // out = x + attention_projection, then out += ffn_output (src/core/transformer_block.cu:594-595)
-        CGPTX_TRY(cgptx_add(out, x, m->d_residual, N * H, dt, s));
-        CGPTX_TRY(cgptx_add(out, out, m->d_norm_in, N * H, dt, s));
+        CGPTX_OP("add", cgptx_add(out, x, m->d_residual, N * H, dt, s));
+        CGPTX_OP("add", cgptx_add(out, out, m->d_norm_in, N * H, dt, s));
     }
     void* last = m->hidden[c.num_layers];
-    CGPTX_TRY(cgptx_rmsnorm_forward(m->normalized, last, m->final_norm.value, N, H, eps, dt, s));
+    CGPTX_OP("rmsnorm_fwd", cgptx_rmsnorm_forward(m->normalized, last, m->final_norm.value, N, H, eps, dt, s));
 
     // --------------------------------------------------------- loss + classifier
     if (loss_mode == CGPTX_LOSS_CUT) {
-        CGPTX_TRY(cgptx_cut_cross_entropy_forward_backward(m->loss, m->d_normalized, m->embedding.gradient,
+        CGPTX_OP("cut_ce", cgptx_cut_cross_entropy_forward_backward(m->loss, m->d_normalized, m->embedding.gradient,
                                                            m->normalized, m->embedding.value, m->targets, N, H,
                                                            c.vocabulary_size, loss_scale, 0, dt, s));
     } else {
-        CGPTX_TRY(cgptx_linear_forward(m->logits, m->normalized, m->embedding.value, nullptr, N, H,
+        CGPTX_OP("gemm_fwd", cgptx_linear_forward(m->logits, m->normalized, m->embedding.value, nullptr, N, H,
                                        c.vocabulary_size, dt, s));
-        CGPTX_TRY(cgptx_cross_entropy_forward_backward(m->loss, m->grad_logits, m->logits, m->targets, N,
+        CGPTX_OP("dense_ce", cgptx_cross_entropy_forward_backward(m->loss, m->grad_logits, m->logits, m->targets, N,
                                                        c.vocabulary_size, loss_scale, dt, s));
-        CGPTX_TRY(cgptx_linear_backward(m->d_normalized, m->embedding.gradient, nullptr, m->grad_logits,
-                                        m->normalized, m->embedding.value, N, H, c.vocabulary_size, 0, 0, 0, dt, s));
+        CGPTX_TRY(linear_backward_split(m, m->d_normalized, m->embedding.gradient, m->grad_logits, m->normalized, m->embedding.value, N, H, c.vocabulary_size, 0, dt, stream));
     }
 
     // ----------------------------------------------------------------- backward
     void* current = m->grad_a;
     void* previous = m->grad_b;
-    CGPTX_TRY(cgptx_rmsnorm_backward(current, m->final_norm.gradient, m->d_normalized, last, m->final_norm.value, N,
+    CGPTX_OP("rmsnorm_bwd", cgptx_rmsnorm_backward(current, m->final_norm.gradient, m->d_normalized, last, m->final_norm.value, N,
                                      H, eps, dt, s));
     for (std::size_t reverse = c.num_layers; reverse-- > 0;) {
         const auto& w = m->layers[reverse];
         const auto& a = m->acts[reverse];
         void* x = m->hidden[reverse];
-        CGPTX_TRY(cgptx_linear_backward(m->d_act, w.down.gradient, nullptr, current, a.act, w.down.value, N, I, H, 0,
-                                        0, 0, dt, s));
-        CGPTX_TRY(cgptx_swiglu_backward(m->d_gate, m->d_up, m->d_act, a.gate, a.up, N * I, 0, 0, dt, s));
-        CGPTX_TRY(cgptx_linear_backward(m->d_norm_in, w.gate.gradient, nullptr, m->d_gate, a.norm_f, w.gate.value, N,
-                                        H, I, 0, 0, 0, dt, s));
-        CGPTX_TRY(cgptx_linear_backward(m->d_norm_in, w.up.gradient, nullptr, m->d_up, a.norm_f, w.up.value, N, H, I,
-                                        1, 0, 0, dt, s));
-        CGPTX_TRY(cgptx_rmsnorm_backward(m->d_residual, w.ffn_norm.gradient, m->d_norm_in, x, w.ffn_norm.value, N, H,
+        CGPTX_TRY(linear_backward_split(m, m->d_act, w.down.gradient, current, a.act, w.down.value, N, I, H, 0, dt, stream));
+        CGPTX_OP("swiglu_bwd", cgptx_swiglu_backward(m->d_gate, m->d_up, m->d_act, a.gate, a.up, N * I, 0, 0, dt, s));
+        CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.gate.gradient, m->d_gate, a.norm_f, w.gate.value, N, H, I, 0, dt, stream));
+        CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.up.gradient, m->d_up, a.norm_f, w.up.value, N, H, I, 1, dt, stream));
+        CGPTX_OP("rmsnorm_bwd", cgptx_rmsnorm_backward(m->d_residual, w.ffn_norm.gradient, m->d_norm_in, x, w.ffn_norm.value, N, H,
                                          eps, dt, s));
-        CGPTX_TRY(cgptx_add(previous, current, m->d_residual, N * H, dt, s));
-        CGPTX_TRY(cgptx_linear_backward(m->d_attn_out, w.o.gradient, nullptr, current, a.attn_out, w.o.value, N, QW,
-                                        H, 0, 0, 0, dt, s));
-        CGPTX_TRY(cgptx_flash_gqa_attention_backward_with_lse(m->d_q, m->d_k, m->d_v, m->d_attn_out, a.attn_out,
+        CGPTX_OP("add", cgptx_add(previous, current, m->d_residual, N * H, dt, s));
+        CGPTX_TRY(linear_backward_split(m, m->d_attn_out, w.o.gradient, current, a.attn_out, w.o.value, N, QW, H, 0, dt, stream));
+        CGPTX_OP("attn_bwd", cgptx_flash_gqa_attention_backward_with_lse(m->d_q, m->d_k, m->d_v, m->d_attn_out, a.attn_out,
                                                               a.lse, a.q, a.k, a.v, m->batch, m->sequence,
                                                               m->sequence, HQ, HKV, D, 0.0f, 1, 0, 0, dt, s));
-        CGPTX_TRY(cgptx_rope_backward(m->d_q_pre, m->d_k_pre, m->d_q, m->d_k, m->cos_cache, m->sin_cache, m->batch,
+        CGPTX_OP("rope_bwd", cgptx_rope_backward(m->d_q_pre, m->d_k_pre, m->d_q, m->d_k, m->cos_cache, m->sin_cache, m->batch,
                                       m->sequence, HQ, HKV, D, c.rotary_dim, 0, m->sequence, dt, s));
-        CGPTX_TRY(cgptx_rmsnorm_backward(m->d_q, w.q_norm.gradient, m->d_q_pre, a.q_pre, w.q_norm.value, N * HQ, D,
+        CGPTX_OP("rmsnorm_bwd", cgptx_rmsnorm_backward(m->d_q, w.q_norm.gradient, m->d_q_pre, a.q_pre, w.q_norm.value, N * HQ, D,
                                          eps, dt, s));
-        CGPTX_TRY(cgptx_rmsnorm_backward(m->d_k, w.k_norm.gradient, m->d_k_pre, a.k_pre, w.k_norm.value, N * HKV, D,
+        CGPTX_OP("rmsnorm_bwd", cgptx_rmsnorm_backward(m->d_k, w.k_norm.gradient, m->d_k_pre, a.k_pre, w.k_norm.value, N * HKV, D,
                                          eps, dt, s));
-        CGPTX_TRY(cgptx_linear_backward(m->d_norm_in, w.q.gradient, nullptr, m->d_q, a.norm_a, w.q.value, N, H, QW, 0,
-                                        0, 0, dt, s));
-        CGPTX_TRY(cgptx_linear_backward(m->d_norm_in, w.k.gradient, nullptr, m->d_k, a.norm_a, w.k.value, N, H, KW, 1,
-                                        0, 0, dt, s));
-        CGPTX_TRY(cgptx_linear_backward(m->d_norm_in, w.v.gradient, nullptr, m->d_v, a.norm_a, w.v.value, N, H, KW, 1,
-                                        0, 0, dt, s));
-        CGPTX_TRY(cgptx_rmsnorm_backward(m->d_residual, w.attention_norm.gradient, m->d_norm_in, x,
+        CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.q.gradient, m->d_q, a.norm_a, w.q.value, N, H, QW, 0, dt, stream));
+        CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.k.gradient, m->d_k, a.norm_a, w.k.value, N, H, KW, 1, dt, stream));
+        CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.v.gradient, m->d_v, a.norm_a, w.v.value, N, H, KW, 1, dt, stream));
+        CGPTX_OP("rmsnorm_bwd", cgptx_rmsnorm_backward(m->d_residual, w.attention_norm.gradient, m->d_norm_in, x,
                                          w.attention_norm.value, N, H, eps, dt, s));
-        CGPTX_TRY(cgptx_add(previous, previous, m->d_residual, N * H, dt, s));
+        CGPTX_OP("add", cgptx_add(previous, previous, m->d_residual, N * H, dt, s));
         std::swap(current, previous);
     }
     // Tied embedding: the classifier gradient is already in place; add the lookup's gradient
     // (src/core/transformer_model.cu:375-380).
-    CGPTX_TRY(cgptx_embedding_backward(m->embedding.gradient, current, m->tokens, N, c.vocabulary_size, H, 1, 1, dt, s));
+    CGPTX_OP("embedding_bwd", cgptx_embedding_backward(m->embedding.gradient, current, m->tokens, N, c.vocabulary_size, H, 1, 1, dt, s));
     return CGPTX_OK;
 }
 
@@ -503,6 +528,47 @@ extern "C" int cgptx_model_status(cgptx_model* m, float* loss, int* all_finite, 
     CGPTX_HIP(hipStreamSynchronize(stream));
     CGPTX_HIP(hipMemcpy(loss, m->loss, sizeof(float), hipMemcpyDeviceToHost));
     return cgptx_adamw_check(m->optimizer, all_finite, step, stream_);
+}
+
+extern "C" int cgptx_model_profile(cgptx_model* m, float loss_scale, int loss_mode, cgptx_stream stream_) {
+    using namespace cgptx;
+    if (m == nullptr) return fail(CGPTX_INVALID_ARGUMENT, "model_profile: null model");
+    auto stream = static_cast<hipStream_t>(stream_);
+    if (int s = cgptx_model_forward_backward(m, loss_scale, loss_mode, 0, stream_)) return s;  // sizes scratch
+    CGPTX_HIP(hipStreamSynchronize(stream));
+    m->profiling = true;
+    m->timed.clear();
+    const int status = enqueue_forward_backward(m, loss_scale, loss_mode, stream);
+    m->profiling = false;
+    CGPTX_HIP(hipStreamSynchronize(stream));
+    m->profile.clear();
+    for (auto& t : m->timed) {
+        float ms = 0.0f;
+        if (status == CGPTX_OK) (void)hipEventElapsedTime(&ms, t.start, t.stop);
+        (void)hipEventDestroy(t.start);
+        (void)hipEventDestroy(t.stop);
+        bool found = false;
+        for (auto& entry : m->profile) {
+            if (entry.first == t.label) {
+                entry.second += ms;
+                found = true;
+            }
+        }
+        if (!found) m->profile.emplace_back(t.label, ms);
+    }
+    m->timed.clear();
+    return status;
+}
+
+extern "C" size_t cgptx_model_profile_count(const cgptx_model* m) { return m == nullptr ? 0 : m->profile.size(); }
+
+extern "C" int cgptx_model_profile_entry(const cgptx_model* m, size_t index, const char** label, float* milliseconds) {
+    using namespace cgptx;
+    if (m == nullptr || index >= m->profile.size() || label == nullptr || milliseconds == nullptr)
+        return fail(CGPTX_INVALID_ARGUMENT, "model_profile_entry: index out of range");
+    *label = m->profile[index].first.c_str();
+    *milliseconds = m->profile[index].second;
+    return CGPTX_OK;
 }
 
 extern "C" size_t cgptx_model_parameter_count(const cgptx_model* m) { return m == nullptr ? 0 : m->entries.size(); }

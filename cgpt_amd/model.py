@@ -121,3 +121,13 @@ class Model:
         capi.call("cgptx_model_activation", self._handle, name.encode(), ctypes.byref(p), ctypes.byref(n))
         dtype = torch.float32 if name == "loss" else self.config.dtype
         return _as_tensor(p.value, n.value, dtype, self.device)
+
+    def profile(self, loss_scale=1.0, loss_mode=LOSS_CUT, stream=None):
+        """One eager pass with events around every operator call: {operator kind: milliseconds}."""
+        capi.call("cgptx_model_profile", self._handle, loss_scale, loss_mode, _stream(stream))
+        out = {}
+        for i in range(capi.lib().cgptx_model_profile_count(self._handle)):
+            label, ms = ctypes.c_char_p(), ctypes.c_float()
+            capi.call("cgptx_model_profile_entry", self._handle, i, ctypes.byref(label), ctypes.byref(ms))
+            out[label.value.decode()] = ms.value
+        return out

@@ -66,6 +66,13 @@ int cgptx_model_train_step(cgptx_model* model, const cgptx_adamw_options* option
  * call saw finite gradients, and the optimizer step count (adamw_check). */
 int cgptx_model_status(cgptx_model* model, float* loss, int* all_finite, uint64_t* step, cgptx_stream stream);
 
+/* Runs one eager forward + loss + backward with HIP events around every operator call on
+ * `stream` and keeps the time per operator kind ("gemm_fwd", "gemm_dx", "gemm_dw", "attn_fwd",
+ * "attn_bwd", "rmsnorm_bwd", ...), summed over the calls of that kind. Synchronises. */
+int cgptx_model_profile(cgptx_model* model, float loss_scale, int loss_mode, cgptx_stream stream);
+size_t cgptx_model_profile_count(const cgptx_model* model);
+int cgptx_model_profile_entry(const cgptx_model* model, size_t index, const char** label, float* milliseconds);
+
 /* Number of parameter tensors and, per index, name / device pointers / element count. Names follow
  * the checkpoint names of src/core/huggingface_export.cpp:362-378 where one exists. */
 size_t cgptx_model_parameter_count(const cgptx_model* model);

@@ -106,8 +106,9 @@ def compare_gradients(got, want, tol, loss_scale):
     def one(g, w, name):
         w = np.asarray(w).reshape(-1)
         scale = max(np.abs(w).max(), 1e-3 * loss_scale)
-        err = np.abs(to_np(g) - w).max() / scale
-        assert np.isfinite(to_np(g)).all(), name
+        got_flat = to_np(g).reshape(-1)
+        err = np.abs(got_flat - w).max() / scale
+        assert np.isfinite(got_flat).all(), name
         assert err <= tol, f"{name}: error {err:.3e} of the tensor's scale"
     one(got["embedding"], want["embedding"], "embedding")
     one(got["final_norm"], want["final_norm"], "final_norm")
@@ -217,3 +218,25 @@ def test_model_argument_errors(device):
     with pytest.raises(ValueError):
         model.forward_backward(1.0, 1, use_graph=True, stream=0)   # capture needs a real stream
     model.close()
+
+
+def test_cpu_float32_step_matches_float64_composition():
+    """oracle/cpu_model.py (the CPU baseline that bench.py times) against oracle/model64.py on a tiny model."""
+    from oracle import cpu_model
+
+    cfg = dict(TINY)
+    w = cpu_model.make_weights(cfg, seed=1)
+    for lw in w["layers"]:
+        for key in lw:
+            if lw[key].dim() == 2:
+                lw[key].mul_(10.0)   # make the gradients large enough to compare
+    w["embedding"].mul_(10.0)
+    g = torch.Generator().manual_seed(2)
+    tokens = torch.randint(0, cfg["vocab"], (2, 6), generator=g)
+    targets = torch.randint(0, cfg["vocab"], (2, 6), generator=g)
+    params = {"embedding": to_np(w["embedding"]), "final_norm": to_np(w["final_norm"]),
+              "layers": [{k: to_np(v) for k, v in lw.items()} for lw in w["layers"]]}
+    loss, grads = cpu_model.train_step(w, tokens, targets, cfg, 8.0)
+    want_loss, want, _ = model64.forward_backward(params, tokens.numpy(), targets.numpy(), cfg, 8.0)
+    assert abs(loss - want_loss) <= 1e-5 * want_loss
+    compare_gradients(grads, want, 1e-4, 8.0)
