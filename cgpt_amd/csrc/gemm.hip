@@ -40,6 +40,7 @@
 #include "gemm.hpp"
 
 #include <algorithm>
+#include <cstdlib>
 #include <limits>
 
 namespace cgptx {
@@ -97,11 +98,11 @@ struct DirectTile {
         for (int i = 0; i < kChunks; ++i) {
             const int chunk = threadIdx.x + i * kThreads;
             const int row = chunk >> 3, kc = chunk & 7;
-            if (row0 + row < row_limit) {
-                regs[i] = *reinterpret_cast<const u32x4*>(base + static_cast<long>(row0 + row) * ld + k0 + kc * 8);
-            } else {
-                regs[i] = u32x4(0u);
-            }
+            // Rows past the edge are clamped to the last valid row instead of being predicated: they
+            // only feed C rows/columns that are never stored, and a branch-free loop lets the loads
+            // stay in flight across the MFMAs of the current tile.
+            const int safe = min(row0 + row, row_limit - 1);
+            regs[i] = *reinterpret_cast<const u32x4*>(base + static_cast<long>(safe) * ld + k0 + kc * 8);
         }
     }
     template <typename T>
@@ -130,16 +131,14 @@ struct TransposedTile {
 #pragma unroll
         for (int i = 0; i < kPerThread; ++i) {
             const int task = task_of(i);
-            const int kg = task / (COLS / 8), nc = task % (COLS / 8);
-            const bool live = task < kTasks && col0 + nc * 8 < col_limit;
+            const int safe_task = min(task, kTasks - 1);
+            const int kg = safe_task / (COLS / 8), nc = safe_task % (COLS / 8);
+            // Column blocks past the edge are clamped (see DirectTile::load); col_limit is a multiple of 8.
+            const int safe_col = min(col0 + nc * 8, col_limit - 8);
 #pragma unroll
             for (int r = 0; r < 8; ++r) {
-                if (live) {
-                    regs[i][r] = *reinterpret_cast<const u32x4*>(base + static_cast<long>(k0 + kg * 8 + r) * ld +
-                                                                 col0 + nc * 8);
-                } else {
-                    regs[i][r] = u32x4(0u);
-                }
+                regs[i][r] = *reinterpret_cast<const u32x4*>(base + static_cast<long>(k0 + kg * 8 + r) * ld +
+                                                             safe_col);
             }
         }
     }
@@ -174,8 +173,9 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     T* smem = reinterpret_cast<T*>(smem_raw);
     constexpr int kATile = BM * kLdsStride, kBTile = BN * kLdsStride;
-    T* a_lds[2] = {smem, smem + kATile + kBTile};
-    T* b_lds[2] = {smem + kATile, smem + 2 * kATile + kBTile};
+    // Stage s holds [A tile | B tile] at smem + s * kStage. Offsets are added to the one shared base
+    // so that every access is provably an LDS access (ds_read/ds_write, counted by lgkmcnt only).
+    constexpr int kStage = kATile + kBTile;
 
     // XCD-contiguous, grouped tile order.
     const int total = p.tiles_m * p.tiles_n;
@@ -209,8 +209,8 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
         if constexpr (B_K) b_direct.load(B, p.ldb, n0, p.n, k0); else b_trans.load(B, p.ldb, n0, p.n, k0);
     };
     auto store_tiles = [&](int buf) {
-        if constexpr (A_K) a_direct.store(a_lds[buf]); else a_trans.store(a_lds[buf]);
-        if constexpr (B_K) b_direct.store(b_lds[buf]); else b_trans.store(b_lds[buf]);
+        if constexpr (A_K) a_direct.store(smem + buf * kStage); else a_trans.store(smem + buf * kStage);
+        if constexpr (B_K) b_direct.store(smem + buf * kStage + kATile); else b_trans.store(smem + buf * kStage + kATile);
     };
 
     const int lane = threadIdx.x & (kWave - 1);
@@ -233,19 +233,29 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
         const int buf = (kt - kt_begin) & 1;
         const bool more = kt + 1 < kt_end;
         if (more) load_tiles(kt + 1);
-        const T* as = a_lds[buf] + (wm * WM + frag_row) * kLdsStride + frag_k;
-        const T* bs = b_lds[buf] + (wn * WN + frag_row) * kLdsStride + frag_k;
+        const T* as = smem + buf * kStage + (wm * WM + frag_row) * kLdsStride + frag_k;
+        const T* bs = smem + buf * kStage + kATile + (wn * WN + frag_row) * kLdsStride + frag_k;
+        // Fragments of K sub-step kk+1 are requested before the MFMAs of sub-step kk are issued.
+        frag_t af[2][TM], bf[2][TN];
+#pragma unroll
+        for (int i = 0; i < TM; ++i) af[0][i] = *reinterpret_cast<const frag_t*>(as + i * 32 * kLdsStride);
+#pragma unroll
+        for (int j = 0; j < TN; ++j) bf[0][j] = *reinterpret_cast<const frag_t*>(bs + j * 32 * kLdsStride);
 #pragma unroll
         for (int kk = 0; kk < kBK / 16; ++kk) {
-            frag_t af[TM], bf[TN];
+            const int cur = kk & 1, nxt = cur ^ 1;
+            if (kk + 1 < kBK / 16) {
 #pragma unroll
-            for (int i = 0; i < TM; ++i) af[i] = *reinterpret_cast<const frag_t*>(as + i * 32 * kLdsStride + kk * 16);
+                for (int i = 0; i < TM; ++i)
+                    af[nxt][i] = *reinterpret_cast<const frag_t*>(as + i * 32 * kLdsStride + (kk + 1) * 16);
 #pragma unroll
-            for (int j = 0; j < TN; ++j) bf[j] = *reinterpret_cast<const frag_t*>(bs + j * 32 * kLdsStride + kk * 16);
+                for (int j = 0; j < TN; ++j)
+                    bf[nxt][j] = *reinterpret_cast<const frag_t*>(bs + j * 32 * kLdsStride + (kk + 1) * 16);
+            }
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
-                for (int j = 0; j < TN; ++j) acc[i][j] = Mfma<T>::run(bf[j], af[i], acc[i][j]);
+                for (int j = 0; j < TN; ++j) acc[i][j] = Mfma<T>::run(bf[cur][j], af[cur][i], acc[i][j]);
         }
         if (more) store_tiles(buf ^ 1);
         __syncthreads();
@@ -401,6 +411,46 @@ int launch_layout(const KernelArgs& p, bool a_k, bool b_k, int slices, hipStream
     return fail(CGPTX_RUNTIME, "gemm: unsupported operand layout");
 }
 
+// CGPTX_GEMM_TILE=128|256 pins the tile size (for experiments); anything else = automatic.
+int forced_tile() {
+    static const int value = [] {
+        const char* text = std::getenv("CGPTX_GEMM_TILE");
+        if (text == nullptr) return 0;
+        const int v = std::atoi(text);
+        return (v == 128 || v == 256) ? v : 0;
+    }();
+    return value;
+}
+
+template <typename T, int BM, int BN>
+int run_config(const GemmArgs& g, KernelArgs p, hipStream_t stream) {
+    p.tiles_m = (p.m + BM - 1) / BM;
+    p.tiles_n = (p.n + BN - 1) / BN;
+    const int k_tiles = p.k / kBK;
+    const long tiles = static_cast<long>(p.tiles_m) * p.tiles_n;
+    const long want_blocks = static_cast<long>(compute_units()) * (BM == 256 ? 1 : 2);
+    int slices = 1;
+    if (!g.no_split && tiles < want_blocks && k_tiles >= 16) {
+        slices = static_cast<int>(std::min<long>((want_blocks + tiles - 1) / tiles, k_tiles / 8));
+        if (slices < 1) slices = 1;
+    }
+    p.k_tiles_per_slice = (k_tiles + slices - 1) / slices;
+    slices = (k_tiles + p.k_tiles_per_slice - 1) / p.k_tiles_per_slice;
+    if (slices == 1) return launch_layout<T, BM, BN, false>(p, g.a_k_contiguous, g.b_k_contiguous, 1, stream);
+    void* mem = nullptr;
+    if (int s = scratch(stream, static_cast<std::size_t>(slices) * g.m * g.n * sizeof(float), &mem)) return s;
+    KernelArgs split = p;
+    split.c = mem;
+    if (int s = launch_layout<T, BM, BN, true>(split, g.a_k_contiguous, g.b_k_contiguous, slices, stream)) return s;
+    const long quads = static_cast<long>(p.m) * (p.n / 4);
+    const long blocks = std::min<long>((quads + kThreads - 1) / kThreads, static_cast<long>(compute_units()) * 8);
+    hipLaunchKernelGGL((splitk_reduce_kernel<T>), dim3(static_cast<unsigned int>(blocks)), dim3(kThreads), 0, stream,
+                       g.c, static_cast<const float*>(mem), static_cast<const T*>(g.bias), p.m, p.n, p.ldc, slices,
+                       p.accumulate, p.c_f32);
+    CGPTX_LAUNCH_CHECK();
+    return CGPTX_OK;
+}
+
 template <typename T>
 int run_typed(const GemmArgs& g, hipStream_t stream) {
     KernelArgs p{};
@@ -434,31 +484,13 @@ int run_typed(const GemmArgs& g, hipStream_t stream) {
         return CGPTX_OK;
     }
     if constexpr (!std::is_same_v<T, float>) {
-        constexpr int BM = 128, BN = 128;
-        p.tiles_m = (p.m + BM - 1) / BM;
-        p.tiles_n = (p.n + BN - 1) / BN;
-        const int k_tiles = p.k / kBK;
-        const long tiles = static_cast<long>(p.tiles_m) * p.tiles_n;
-        const long want_blocks = static_cast<long>(compute_units()) * 2;
-        int slices = 1;
-        if (!g.no_split && tiles < want_blocks && k_tiles >= 16) {
-            slices = static_cast<int>(std::min<long>((want_blocks + tiles - 1) / tiles, k_tiles / 8));
-            if (slices < 1) slices = 1;
-        }
-        p.k_tiles_per_slice = (k_tiles + slices - 1) / slices;
-        slices = (k_tiles + p.k_tiles_per_slice - 1) / p.k_tiles_per_slice;
-        if (slices == 1) return launch_layout<T, BM, BN, false>(p, g.a_k_contiguous, g.b_k_contiguous, 1, stream);
-        void* mem = nullptr;
-        if (int s = scratch(stream, static_cast<std::size_t>(slices) * g.m * g.n * sizeof(float), &mem)) return s;
-        KernelArgs split = p;
-        split.c = mem;
-        if (int s = launch_layout<T, BM, BN, true>(split, g.a_k_contiguous, g.b_k_contiguous, slices, stream)) return s;
-        const long quads = static_cast<long>(p.m) * (p.n / 4);
-        const long blocks = std::min<long>((quads + kThreads - 1) / kThreads, static_cast<long>(compute_units()) * 8);
-        hipLaunchKernelGGL((splitk_reduce_kernel<T>), dim3(static_cast<unsigned int>(blocks)), dim3(kThreads), 0,
-                           stream, g.c, static_cast<const float*>(mem), static_cast<const T*>(g.bias), p.m, p.n,
-                           p.ldc, slices, p.accumulate, p.c_f32);
-        CGPTX_LAUNCH_CHECK();
+        // 256x256 tiles (one block per CU, 64 MFMAs per wavefront and K step) when they still give
+        // every CU a tile; otherwise 128x128 tiles, with K split when even those are too few.
+        const long big_tiles = static_cast<long>((g.m + 255) / 256) * static_cast<long>((g.n + 255) / 256);
+        const int forced = forced_tile();
+        const bool big = forced == 256 || (forced == 0 && big_tiles * 5 >= static_cast<long>(compute_units()) * 4);
+        if (big) return run_config<T, 256, 256>(g, p, stream);
+        return run_config<T, 128, 128>(g, p, stream);
     }
     return CGPTX_OK;
 }
