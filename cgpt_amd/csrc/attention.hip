@@ -80,22 +80,47 @@ struct Params {
 template <int DP>
 constexpr int lds_stride() { return DP + 8; }
 
-// Cooperative load of a [rows_in_tile x DP] tile (row-major in LDS, stride DP+8) from a
-// [.., seq, heads, d] tensor: element (r, c) comes from base[(row0 + r) * row_stride + c].
+// Register-staged copy of a [ROWS x DP] tile of a [.., seq, heads, d] tensor into LDS (row-major,
+// stride DP+8): element (r, c) comes from base[(row0 + r) * row_stride + c]. load() only issues
+// the 128-bit global loads (rows past the end are clamped to a valid address and zeroed by a
+// select, so there is no branch and the loads stay in flight); store() writes them to LDS later,
+// after the MFMAs of the previous tile.
 template <typename T, int ROWS, int DP>
-__device__ __forceinline__ void load_tile(T* lds, const T* base, long row_stride, int row0, int row_limit, int d) {
-    constexpr int kChunksPerRow = DP / 8;
-    constexpr int kChunks = ROWS * kChunksPerRow;
+struct TileRegs {
+    static constexpr int kChunksPerRow = DP / 8;
+    static constexpr int kPerThread = ROWS * kChunksPerRow / kThreads;
     using chunk_t = vec_t<unsigned int, 4>;
+    chunk_t regs[kPerThread];
+    int row0_ = 0, row_limit_ = 0, d_ = 0;
+
+    __device__ __forceinline__ void load(const T* base, long row_stride, int row0, int row_limit, int d) {
+        row0_ = row0;
+        row_limit_ = row_limit;
+        d_ = d;
 #pragma unroll
-    for (int c = threadIdx.x; c < kChunks; c += kThreads) {
-        const int r = c / kChunksPerRow, col = (c % kChunksPerRow) * 8;
-        chunk_t value(0u);
-        if (row0 + r < row_limit && col < d)
-            value = *reinterpret_cast<const chunk_t*>(base + static_cast<long>(row0 + r) * row_stride + col);
-        *reinterpret_cast<chunk_t*>(lds + r * lds_stride<DP>() + col) = value;
+        for (int i = 0; i < kPerThread; ++i) {
+            const int c = threadIdx.x + i * kThreads;
+            const int r = c / kChunksPerRow, col = (c % kChunksPerRow) * 8;
+            const int safe_row = min(row0 + r, row_limit - 1);
+            const int safe_col = min(col, d - 8);
+            regs[i] = *reinterpret_cast<const chunk_t*>(base + static_cast<long>(safe_row) * row_stride + safe_col);
+        }
     }
-}
+    // The zeroing of out-of-range chunks happens here, not in load(), so that nothing waits for
+    // the loaded data before the tile is actually needed.
+    __device__ __forceinline__ void store(T* lds) const {
+#pragma unroll
+        for (int i = 0; i < kPerThread; ++i) {
+            const int c = threadIdx.x + i * kThreads;
+            const int r = c / kChunksPerRow, col = (c % kChunksPerRow) * 8;
+            const bool live = row0_ + r < row_limit_ && col < d_;
+            chunk_t value;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) value[e] = live ? regs[i][e] : 0u;
+            *reinterpret_cast<chunk_t*>(lds + r * lds_stride<DP>() + col) = value;
+        }
+    }
+};
 
 // Fragment with the head dimension as contraction index, read straight from LDS:
 // lane -> tile row (row0 + lane%32), elements d = 16*step + 8*(lane/32) .. +7.
@@ -178,20 +203,32 @@ __global__ __launch_bounds__(kThreads) void attention_forward_kernel(Params p) {
     const int wave_last_q = min(q_block + wave * 32 + 31, p.qs - 1);
     const int q_limit = p.causal ? p.offset + q_row : p.ks;  // largest visible key of this lane's query
 
+    TileRegs<T, kStream, DP> k_regs, v_regs;
+    if (k_end > 0) {
+        k_regs.load(k_base, kv_stride, 0, p.ks, p.d);
+        v_regs.load(v_base, kv_stride, 0, p.ks, p.d);
+    }
     for (int k0 = 0; k0 < k_end; k0 += kStream) {
+        __syncthreads();  // every wavefront is done reading the previous tile
+        k_regs.store(k_lds);
+        v_regs.store(v_lds);
         __syncthreads();
-        load_tile<T, kStream, DP>(k_lds, k_base, kv_stride, k0, p.ks, p.d);
-        load_tile<T, kStream, DP>(v_lds, v_base, kv_stride, k0, p.ks, p.d);
-        __syncthreads();
+        if (k0 + kStream < k_end) {  // next tile's loads fly during this tile's MFMAs
+            k_regs.load(k_base, kv_stride, k0 + kStream, p.ks, p.d);
+            v_regs.load(v_base, kv_stride, k0 + kStream, p.ks, p.d);
+        }
         if (q_block + wave * 32 >= p.qs) continue;
         if (p.causal && k0 > p.offset + wave_last_q) continue;
         acc_t st[2];
 #pragma unroll
         for (int sub = 0; sub < 2; ++sub) {
             st[sub] = acc_t(0.0f);
+            typename Mma<T>::frag ka[STEPS];  // all LDS reads first, then the MFMA chain
 #pragma unroll
-            for (int s = 0; s < STEPS; ++s)
-                st[sub] = Mma<T>::run(direct_frag<T, DP>(k_lds, sub * 32, s), qf[s], st[sub]);
+            for (int s = 0; s < STEPS; ++s) ka[s] = direct_frag<T, DP>(k_lds, sub * 32, s);
+            __builtin_amdgcn_sched_barrier(0);  // keep the reads ahead of the MFMA chain
+#pragma unroll
+            for (int s = 0; s < STEPS; ++s) st[sub] = Mma<T>::run(ka[s], qf[s], st[sub]);
         }
         float tile_max = -INFINITY;
 #pragma unroll
@@ -227,9 +264,12 @@ __global__ __launch_bounds__(kThreads) void attention_forward_kernel(Params p) {
 #pragma unroll
             for (int s = 0; s < 2; ++s) {
                 const typename Mma<T>::frag pf = acc_frag<T>(st[sub], s);
+                typename Mma<T>::frag vt[DT];
 #pragma unroll
-                for (int t = 0; t < DT; ++t)
-                    o[t] = Mma<T>::run(transposed_frag<T, DP>(v_lds, sub * 32 + s * 16, t * 32), pf, o[t]);
+                for (int t = 0; t < DT; ++t) vt[t] = transposed_frag<T, DP>(v_lds, sub * 32 + s * 16, t * 32);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int t = 0; t < DT; ++t) o[t] = Mma<T>::run(vt[t], pf, o[t]);
             }
         }
     }
@@ -307,20 +347,36 @@ __global__ __launch_bounds__(kThreads) void attention_dq_kernel(Params p) {
     const int wave_last_q = min(q_block + wave * 32 + 31, p.qs - 1);
     const int q_limit = p.causal ? p.offset + q_row : p.ks;
 
+    TileRegs<T, kStream, DP> k_regs, v_regs;
+    if (k_end > 0) {
+        k_regs.load(k_base, kv_stride, 0, p.ks, p.d);
+        v_regs.load(v_base, kv_stride, 0, p.ks, p.d);
+    }
     for (int k0 = 0; k0 < k_end; k0 += kStream) {
+        __syncthreads();  // every wavefront is done reading the previous tile
+        k_regs.store(k_lds);
+        v_regs.store(v_lds);
         __syncthreads();
-        load_tile<T, kStream, DP>(k_lds, k_base, kv_stride, k0, p.ks, p.d);
-        load_tile<T, kStream, DP>(v_lds, v_base, kv_stride, k0, p.ks, p.d);
-        __syncthreads();
+        if (k0 + kStream < k_end) {  // next tile's loads fly during this tile's MFMAs
+            k_regs.load(k_base, kv_stride, k0 + kStream, p.ks, p.d);
+            v_regs.load(v_base, kv_stride, k0 + kStream, p.ks, p.d);
+        }
         if (q_block + wave * 32 >= p.qs) continue;
         if (p.causal && k0 > p.offset + wave_last_q) continue;
 #pragma unroll
         for (int sub = 0; sub < 2; ++sub) {
             acc_t st(0.0f), dpt(0.0f);
+            typename Mma<T>::frag ka[STEPS], va[STEPS];  // all LDS reads first, then two independent MFMA chains
 #pragma unroll
             for (int s = 0; s < STEPS; ++s) {
-                st = Mma<T>::run(direct_frag<T, DP>(k_lds, sub * 32, s), qf[s], st);
-                dpt = Mma<T>::run(direct_frag<T, DP>(v_lds, sub * 32, s), dof[s], dpt);
+                ka[s] = direct_frag<T, DP>(k_lds, sub * 32, s);
+                va[s] = direct_frag<T, DP>(v_lds, sub * 32, s);
+            }
+            __builtin_amdgcn_sched_barrier(0);  // keep the reads ahead of the MFMA chains
+#pragma unroll
+            for (int s = 0; s < STEPS; ++s) {
+                st = Mma<T>::run(ka[s], qf[s], st);
+                dpt = Mma<T>::run(va[s], dof[s], dpt);
             }
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
@@ -332,9 +388,12 @@ __global__ __launch_bounds__(kThreads) void attention_dq_kernel(Params p) {
 #pragma unroll
             for (int s = 0; s < 2; ++s) {
                 const typename Mma<T>::frag dsf = acc_frag<T>(st, s);
+                typename Mma<T>::frag kt[DT];
 #pragma unroll
-                for (int t = 0; t < DT; ++t)
-                    dq[t] = Mma<T>::run(transposed_frag<T, DP>(k_lds, sub * 32 + s * 16, t * 32), dsf, dq[t]);
+                for (int t = 0; t < DT; ++t) kt[t] = transposed_frag<T, DP>(k_lds, sub * 32 + s * 16, t * 32);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int t = 0; t < DT; ++t) dq[t] = Mma<T>::run(kt[t], dsf, dq[t]);
             }
         }
     }
@@ -388,49 +447,83 @@ __global__ __launch_bounds__(kThreads) void attention_dkv_kernel(Params p) {
     const int q_begin = p.causal ? max(0, k_block - p.offset) / kStream * kStream : 0;
     const int wave_first_key = k_block + wave * 32;
 
-    for (int hg = 0; hg < group; ++hg) {
-        const int h = kvh * group + hg;
-        const T* q_base = static_cast<const T*>(p.q) + static_cast<long>(b) * p.qs * q_stride + h * p.d;
-        const T* do_base = static_cast<const T*>(p.dout) + static_cast<long>(b) * p.qs * q_stride + h * p.d;
-        for (int q0 = q_begin; q0 < p.qs; q0 += kStream) {
-            __syncthreads();
-            load_tile<T, kStream, DP>(q_lds, q_base, q_stride, q0, p.qs, p.d);
-            load_tile<T, kStream, DP>(do_lds, do_base, q_stride, q0, p.qs, p.d);
+    // The (head of the group, query tile) pairs form one flat sequence so that the next tile can be
+    // prefetched across the head boundary.
+    const int tiles_per_head = q_begin < p.qs ? (p.qs - q_begin + kStream - 1) / kStream : 0;
+    const int total_tiles = tiles_per_head * group;
+    const T* q_batch = static_cast<const T*>(p.q) + static_cast<long>(b) * p.qs * q_stride;
+    const T* do_batch = static_cast<const T*>(p.dout) + static_cast<long>(b) * p.qs * q_stride;
+    TileRegs<T, kStream, DP> q_regs, do_regs;
+    float lse_reg = 0.0f, delta_reg = 0.0f;
+    auto prefetch = [&](int tile) {
+        const int h = kvh * group + tile / tiles_per_head;
+        const int q0 = q_begin + (tile % tiles_per_head) * kStream;
+        q_regs.load(q_batch + h * p.d, q_stride, q0, p.qs, p.d);
+        do_regs.load(do_batch + h * p.d, q_stride, q0, p.qs, p.d);
+        if (threadIdx.x < kStream) {
+            const int q = min(q0 + static_cast<int>(threadIdx.x), p.qs - 1);
+            const long index = (static_cast<long>(b) * p.qs + q) * p.hq + h;
+            lse_reg = p.lse[index] * kLog2e;
+            delta_reg = p.delta[index];
+        }
+    };
+    if (total_tiles > 0) prefetch(0);
+    for (int tile = 0; tile < total_tiles; ++tile) {
+        {
+            const int q0 = q_begin + (tile % tiles_per_head) * kStream;
+            __syncthreads();  // every wavefront is done reading the previous tile
+            q_regs.store(q_lds);
+            do_regs.store(do_lds);
             if (threadIdx.x < kStream) {
-                const int q = q0 + threadIdx.x;
-                const long index = (static_cast<long>(b) * p.qs + q) * p.hq + h;
-                lse_lds[threadIdx.x] = q < p.qs ? p.lse[index] * kLog2e : 0.0f;
-                delta_lds[threadIdx.x] = q < p.qs ? p.delta[index] : 0.0f;
+                lse_lds[threadIdx.x] = lse_reg;
+                delta_lds[threadIdx.x] = delta_reg;
             }
             __syncthreads();
+            if (tile + 1 < total_tiles) prefetch(tile + 1);
             if (wave_first_key >= p.ks) continue;
             // every query of the tile sees at most keys <= offset + q0 + 63
             if (p.causal && wave_first_key > p.offset + q0 + kStream - 1) continue;
 #pragma unroll
             for (int sub = 0; sub < 2; ++sub) {
                 acc_t s_acc(0.0f), dp_acc(0.0f);
+                typename Mma<T>::frag qa[STEPS], da[STEPS];  // all LDS reads first, then two MFMA chains
 #pragma unroll
                 for (int s = 0; s < STEPS; ++s) {
-                    s_acc = Mma<T>::run(direct_frag<T, DP>(q_lds, sub * 32, s), kf[s], s_acc);
-                    dp_acc = Mma<T>::run(direct_frag<T, DP>(do_lds, sub * 32, s), vf[s], dp_acc);
+                    qa[s] = direct_frag<T, DP>(q_lds, sub * 32, s);
+                    da[s] = direct_frag<T, DP>(do_lds, sub * 32, s);
+                }
+                __builtin_amdgcn_sched_barrier(0);  // keep the reads ahead of the MFMA chains
+#pragma unroll
+                for (int s = 0; s < STEPS; ++s) {
+                    s_acc = Mma<T>::run(qa[s], kf[s], s_acc);
+                    dp_acc = Mma<T>::run(da[s], vf[s], dp_acc);
                 }
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
                     const int local = sub * 32 + acc_row(i);
                     const int q = q0 + local;
                     const bool visible = k_live && q < p.qs && (!p.causal || k_row <= p.offset + q);
-                    const float prob = visible ? exp2f(s_acc[i] * scale2 - lse_lds[local]) : 0.0f;
+                    const float lse_q = lse_lds[local], delta_q = delta_lds[local];  // unconditional reads
+                    const float e = exp2f(s_acc[i] * scale2 - lse_q);
+                    const float prob = visible ? e : 0.0f;
                     s_acc[i] = prob;
-                    dp_acc[i] = prob * (dp_acc[i] - delta_lds[local]);
+                    dp_acc[i] = prob * (dp_acc[i] - delta_q);
                 }
 #pragma unroll
                 for (int s = 0; s < 2; ++s) {
                     const typename Mma<T>::frag pf = acc_frag<T>(s_acc, s);
                     const typename Mma<T>::frag dsf = acc_frag<T>(dp_acc, s);
+                    typename Mma<T>::frag dot[DT], qt[DT];
 #pragma unroll
                     for (int t = 0; t < DT; ++t) {
-                        dv[t] = Mma<T>::run(transposed_frag<T, DP>(do_lds, sub * 32 + s * 16, t * 32), pf, dv[t]);
-                        dk[t] = Mma<T>::run(transposed_frag<T, DP>(q_lds, sub * 32 + s * 16, t * 32), dsf, dk[t]);
+                        dot[t] = transposed_frag<T, DP>(do_lds, sub * 32 + s * 16, t * 32);
+                        qt[t] = transposed_frag<T, DP>(q_lds, sub * 32 + s * 16, t * 32);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int t = 0; t < DT; ++t) {
+                        dv[t] = Mma<T>::run(dot[t], pf, dv[t]);
+                        dk[t] = Mma<T>::run(qt[t], dsf, dk[t]);
                     }
                 }
             }

@@ -62,10 +62,10 @@ extern "C" int cgptx_cut_cross_entropy_forward_backward(float* loss, void* input
         return fail(CGPTX_OVERFLOW, std::string(name) + ": dimension exceeds int range");
     auto stream = static_cast<hipStream_t>(stream_);
     const std::size_t elem = dtype_size(dtype);
-    // Chunk so that the logits scratch stays near 128 MiB (it then lives in the 256 MB
-    // last-level cache between the three kernels that touch it).
-    std::size_t chunk = (std::size_t{128} << 20) / (vocab * elem);
-    chunk = std::max<std::size_t>(128, chunk / 128 * 128);
+    // Chunk so that the logits scratch stays near 512 MiB whatever the number of rows, while each
+    // chunk still gives the three contractions enough tiles to fill the chip (8192 rows at V=32000).
+    std::size_t chunk = (std::size_t{512} << 20) / (vocab * elem);
+    chunk = std::max<std::size_t>(256, chunk / 256 * 256);
     chunk = std::min(chunk, rows);
     const std::size_t loss_bytes = (rows * sizeof(float) + 255) & ~std::size_t{255};
     const std::size_t acc_bytes = (vocab * hidden * sizeof(float) + 255) & ~std::size_t{255};

@@ -24,8 +24,9 @@
 //   * Global loads of tile t+1 are issued before the MFMAs of tile t and land in
 //     the other LDS buffer afterwards: one barrier per K step.
 //   * MFMA is issued as (B-fragment, A-fragment), so a lane ends up holding four
-//     consecutive n for one m per accumulator group and stores 8 B (16-bit C) or
-//     16 B (fp32 C) per store.
+//     consecutive n for one m per accumulator group; the finished tile is staged in
+//     LDS as fp32 and written out row by row (512 contiguous bytes per wavefront
+//     store), with bias / accumulate added in fp32 and one rounding to the dtype.
 //   * Block ids are remapped so that the 8 XCDs (blocks are dealt round-robin to
 //     them) each walk a contiguous range of tiles, and tiles are ordered in groups
 //     of 8 tile-rows so that the tiles resident on one XCD share A and B panels in
@@ -132,7 +133,10 @@ struct TransposedTile {
         for (int i = 0; i < kPerThread; ++i) {
             const int task = task_of(i);
             const int safe_task = min(task, kTasks - 1);
-            const int kg = safe_task / (COLS / 8), nc = safe_task % (COLS / 8);
+            // Eight adjacent lanes take the eight k-groups of one column block: their 16-byte loads
+            // fill one 128-byte line per k row, and their LDS stores below fall in one contiguous
+            // 128-byte row segment (no bank conflicts).
+            const int kg = safe_task % (kBK / 8), nc = safe_task / (kBK / 8);
             // Column blocks past the edge are clamped (see DirectTile::load); col_limit is a multiple of 8.
             const int safe_col = min(col0 + nc * 8, col_limit - 8);
 #pragma unroll
@@ -148,7 +152,7 @@ struct TransposedTile {
         for (int i = 0; i < kPerThread; ++i) {
             const int task = task_of(i);
             if (task >= kTasks) continue;
-            const int kg = task / (COLS / 8), nc = task % (COLS / 8);
+            const int kg = task % (kBK / 8), nc = task / (kBK / 8);
 #pragma unroll
             for (int j = 0; j < 8; ++j) {  // output row: column nc*8 + j, k = kg*8 .. kg*8+7
                 u32x4 out;
@@ -261,43 +265,65 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
         __syncthreads();
     }
 
-    // Epilogue. acc[i][j][4g+e] holds C[m, n] with m = lane%32, n = 8g + 4*(lane/32) + e.
+    // Epilogue. acc[i][j][4g+e] holds C[m, n] with m = lane%32, n = 8g + 4*(lane/32) + e. The tile
+    // goes through LDS (fp32, row stride BN+4 so that the 16 lanes of a ds_write_b128 pass hit 16
+    // different bank groups) and leaves it row by row, so that a wavefront stores 512 contiguous
+    // bytes of C per instruction instead of 32 separate 16-byte pieces. Rounding to the storage
+    // dtype still happens once, after bias and accumulate were added in fp32.
+    constexpr int kStageStride = BN + 4;
+    constexpr int kSmemBytes = 2 * (BM + BN) * kLdsStride * static_cast<int>(sizeof(T));
+    constexpr int kPassRows = (BM * kStageStride * 4 <= kSmemBytes) ? BM : BM / 2;
+    constexpr int kPasses = BM / kPassRows;
+    static_assert(kPassRows * kStageStride * 4 <= kSmemBytes, "epilogue staging does not fit in LDS");
+    static_assert(kPasses == 1 || kPassRows == WM, "a pass must be one row of wavefronts");
+    float* stage = reinterpret_cast<float*>(smem_raw);
     const int m_lane = lane & 31, n_lane = (lane >> 5) * 4;
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
-        const int m = m0 + wm * WM + i * 32 + m_lane;
-        if (m >= p.m) continue;
+    for (int pass = 0; pass < kPasses; ++pass) {
+        if (kPasses == 1 || wm == pass) {
+            const int row_base = kPasses == 1 ? wm * WM : 0;
 #pragma unroll
-        for (int j = 0; j < TN; ++j) {
+            for (int i = 0; i < TM; ++i) {
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const int n = n0 + wn * WN + j * 32 + g * 8 + n_lane;
-                if (n >= p.n) continue;
-                vec_t<float, 4> v;
+                for (int j = 0; j < TN; ++j) {
 #pragma unroll
-                for (int e = 0; e < 4; ++e) v[e] = acc[i][j][4 * g + e];
-                if constexpr (SPLIT) {
-                    float* out = static_cast<float*>(p.c) +
-                                 (static_cast<long>(blockIdx.y) * p.m + m) * static_cast<long>(p.n) + n;
-                    *reinterpret_cast<vec_t<float, 4>*>(out) = v;
-                } else {
-                    if (p.bias != nullptr) {
-                        const vec_t<float, 4> bv =
-                            vec_to_f32<T, 4>(load_vec<T, 4>(static_cast<const T*>(p.bias) + n));
-                        v += bv;
-                    }
-                    if (p.c_f32) {
-                        float* out = static_cast<float*>(p.c) + static_cast<long>(m) * p.ldc + n;
-                        if (p.accumulate) v += *reinterpret_cast<const vec_t<float, 4>*>(out);
-                        *reinterpret_cast<vec_t<float, 4>*>(out) = v;
-                    } else {
-                        T* out = static_cast<T*>(p.c) + static_cast<long>(m) * p.ldc + n;
-                        if (p.accumulate) v += vec_to_f32<T, 4>(load_vec<T, 4>(out));
-                        store_vec<T, 4>(out, vec_from_f32<T, 4>(v));
+                    for (int g = 0; g < 4; ++g) {
+                        vec_t<float, 4> v;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) v[e] = acc[i][j][4 * g + e];
+                        const int row = row_base + i * 32 + m_lane;
+                        const int col = wn * WN + j * 32 + g * 8 + n_lane;
+                        *reinterpret_cast<vec_t<float, 4>*>(stage + row * kStageStride + col) = v;
                     }
                 }
             }
         }
+        __syncthreads();
+        constexpr int kChunksPerRow = BN / 4;
+        constexpr int kChunks = kPassRows * kChunksPerRow;
+        for (int c = threadIdx.x; c < kChunks; c += kThreads) {
+            const int r = c / kChunksPerRow, col = (c % kChunksPerRow) * 4;
+            const int m = m0 + pass * kPassRows + r, n = n0 + col;
+            if (m >= p.m || n >= p.n) continue;
+            vec_t<float, 4> v = *reinterpret_cast<const vec_t<float, 4>*>(stage + r * kStageStride + col);
+            if constexpr (SPLIT) {
+                float* out = static_cast<float*>(p.c) +
+                             (static_cast<long>(blockIdx.y) * p.m + m) * static_cast<long>(p.n) + n;
+                *reinterpret_cast<vec_t<float, 4>*>(out) = v;
+            } else {
+                if (p.bias != nullptr) v += vec_to_f32<T, 4>(load_vec<T, 4>(static_cast<const T*>(p.bias) + n));
+                if (p.c_f32) {
+                    float* out = static_cast<float*>(p.c) + static_cast<long>(m) * p.ldc + n;
+                    if (p.accumulate) v += *reinterpret_cast<const vec_t<float, 4>*>(out);
+                    *reinterpret_cast<vec_t<float, 4>*>(out) = v;
+                } else {
+                    T* out = static_cast<T*>(p.c) + static_cast<long>(m) * p.ldc + n;
+                    if (p.accumulate) v += vec_to_f32<T, 4>(load_vec<T, 4>(out));
+                    store_vec<T, 4>(out, vec_from_f32<T, 4>(v));
+                }
+            }
+        }
+        if (pass + 1 < kPasses) __syncthreads();
     }
 }
 
