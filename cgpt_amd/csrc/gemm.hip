@@ -13,16 +13,18 @@
 //     and walks K in steps of 64. Each wavefront owns (BM/2) x (BN/2) and issues
 //     v_mfma_f32_32x32x16 (bf16 or f16), so every LDS fragment read feeds
 //     (BM/64)·(BN/64) MFMAs.
-//   * Both operands are staged in LDS k-contiguous with a row stride of 72
-//     elements (144 B): the 16 rows a quarter-wavefront reads with one
-//     ds_read_b128 then fall in 16 distinct bank groups.
+//   * A k-contiguous operand is staged in LDS with a row stride of 72 elements
+//     (144 B): the rows a ds_read_b128 fragment read touches then fall in distinct
+//     bank groups.
 //   * Operands that are not k-contiguous in memory (dX's weight, both dW
-//     operands) are transposed in registers on their way to LDS: a thread loads
-//     an 8(k) x 8(n) block with eight coalesced 128-bit loads, regroups it with
-//     v_perm_b32 into eight k-contiguous 128-bit rows and stores those. No
-//     separate transpose pass over HBM and no 16-bit LDS accesses.
-//   * Global loads of tile t+1 are issued before the MFMAs of tile t and land in
-//     the other LDS buffer afterwards: one barrier per K step.
+//     operands) are copied to LDS as they are (coalesced 128-bit loads and
+//     stores) and transposed by the LDS read itself (ds_read_b64_tr_b16): no
+//     separate transpose pass over HBM, no VALU shuffles, no 16-bit LDS accesses.
+//   * The K loop is a software pipeline with one barrier per K step whose issue
+//     order is pinned with sched_group_barrier: LDS fragment reads, the LDS
+//     stores of the next tile and the global loads of the tile after it are
+//     spread between the MFMAs they overlap with, and the loop has no
+//     data-dependent branch (edges are clamped, not predicated).
 //   * MFMA is issued as (B-fragment, A-fragment), so a lane ends up holding four
 //     consecutive n for one m per accumulator group; the finished tile is staged in
 //     LDS as fp32 and written out row by row (512 contiguous bytes per wavefront
@@ -41,6 +43,7 @@
 #include "gemm.hpp"
 
 #include <algorithm>
+#include <type_traits>
 #include <cstdlib>
 #include <limits>
 
@@ -87,16 +90,37 @@ struct KernelArgs {
     int c_f32;
 };
 
-// ---- k-contiguous operand: rows x 64 tile, 128-bit chunks ---------------------
-template <int ROWS>
-struct DirectTile {
-    static constexpr int kChunks = ROWS * (kBK / 8) / kThreads;  // per thread
-    u32x4 regs[kChunks];
+// Instruction classes of __builtin_amdgcn_sched_group_barrier.
+constexpr int kSchedMfma = 0x008, kSchedVmemRead = 0x020, kSchedDsRead = 0x100, kSchedDsWrite = 0x200;
 
-    template <typename T>
+template <int MASK, int COUNT>
+__device__ __forceinline__ void sched_group() {
+    if constexpr (COUNT > 0) __builtin_amdgcn_sched_group_barrier(MASK, COUNT, 0);
+}
+// Asks the scheduler for MFMAS matrix instructions with EXTRA0 instructions of class CLASS0 and EXTRA1 of
+// class CLASS1 spread evenly between them, so that their issue slots fall in the shadow of an MFMA.
+template <int MFMAS, int CLASS0, int EXTRA0, int CLASS1, int EXTRA1, int I = 0>
+__device__ __forceinline__ void sched_interleave() {
+    if constexpr (I < MFMAS) {
+        sched_group<kSchedMfma, 1>();
+        sched_group<CLASS0, ((I + 1) * EXTRA0) / MFMAS - (I * EXTRA0) / MFMAS>();
+        sched_group<CLASS1, ((I + 1) * EXTRA1) / MFMAS - (I * EXTRA1) / MFMAS>();
+        sched_interleave<MFMAS, CLASS0, EXTRA0, CLASS1, EXTRA1, I + 1>();
+    }
+}
+
+// ---- operand stored [ROWS, K] (k-contiguous): ROWS x 64 slab, LDS rows of 72 elements ---------
+template <typename T, int ROWS>
+struct KTile {
+    using frag_t = typename Mfma<T>::frag;
+    static constexpr int kLoads = ROWS * (kBK / 8) / kThreads;  // 128-bit chunks per thread
+    static constexpr int kElems = ROWS * kLdsStride;
+    static constexpr int kFragReads = 1;  // LDS instructions per fragment
+    u32x4 regs[kLoads];
+
     __device__ __forceinline__ void load(const T* base, long ld, int row0, int row_limit, int k0) {
 #pragma unroll
-        for (int i = 0; i < kChunks; ++i) {
+        for (int i = 0; i < kLoads; ++i) {
             const int chunk = threadIdx.x + i * kThreads;
             const int row = chunk >> 3, kc = chunk & 7;
             // Rows past the edge are clamped to the last valid row instead of being predicated: they
@@ -106,80 +130,98 @@ struct DirectTile {
             regs[i] = *reinterpret_cast<const u32x4*>(base + static_cast<long>(safe) * ld + k0 + kc * 8);
         }
     }
-    template <typename T>
     __device__ __forceinline__ void store(T* lds) const {
 #pragma unroll
-        for (int i = 0; i < kChunks; ++i) {
+        for (int i = 0; i < kLoads; ++i) {
             const int chunk = threadIdx.x + i * kThreads;
             const int row = chunk >> 3, kc = chunk & 7;
             *reinterpret_cast<u32x4*>(lds + row * kLdsStride + kc * 8) = regs[i];
         }
     }
+    // Per-lane part of a fragment address: row lane%32 of a 32-row block, k group lane/32.
+    __device__ __forceinline__ static int lane_offset(int lane) { return (lane & 31) * kLdsStride + (lane >> 5) * 8; }
+    // Fragment of rows block0 .. block0+31, K sub-step kk (16 values of k, 8 per lane).
+    __device__ __forceinline__ static frag_t frag(const T* lane_base, int block0, int kk) {
+        return *reinterpret_cast<const frag_t*>(lane_base + block0 * kLdsStride + kk * 16);
+    }
 };
 
-// ---- n-contiguous operand: 64(k) x COLS tile, transposed in registers ---------
-template <int COLS, int THREAD_SHIFT>
-struct TransposedTile {
-    static constexpr int kTasks = (kBK / 8) * (COLS / 8);
-    static constexpr int kPerThread = (kTasks + kThreads - 1) / kThreads;
-    u32x4 regs[kPerThread][8];
+// ---- operand stored [K, COLS] (n-contiguous): 64 x COLS slab kept in that order in LDS ---------
+// The transpose happens on the way out of LDS: ds_read_b64_tr_b16 hands lane n of a 16-lane group
+// the four k-values of column n from a 4(k) x 16(n) block, so two of them build the 8-k fragment of
+// one column. Rows are padded by 32 elements (64 B): the four k rows that 32 lanes read then start
+// 16 banks apart and the read is conflict-free; the row-contiguous 128-bit stores are anyway.
+template <typename T, int COLS>
+struct NTile {
+    using frag_t = typename Mfma<T>::frag;
+    static constexpr int kStride = COLS + 32;
+    static constexpr int kChunksPerRow = COLS / 8;
+    static constexpr int kLoads = kBK * kChunksPerRow / kThreads;
+    static constexpr int kElems = kBK * kStride;
+    static constexpr int kFragReads = 2;
+    u32x4 regs[kLoads];
 
-    __device__ __forceinline__ static int task_of(int i) {
-        return ((threadIdx.x + THREAD_SHIFT) & (kThreads - 1)) + i * kThreads;
-    }
-    template <typename T>
     __device__ __forceinline__ void load(const T* base, long ld, int col0, int col_limit, int k0) {
 #pragma unroll
-        for (int i = 0; i < kPerThread; ++i) {
-            const int task = task_of(i);
-            const int safe_task = min(task, kTasks - 1);
-            // Eight adjacent lanes take the eight k-groups of one column block: their 16-byte loads
-            // fill one 128-byte line per k row, and their LDS stores below fall in one contiguous
-            // 128-byte row segment (no bank conflicts).
-            const int kg = safe_task % (kBK / 8), nc = safe_task / (kBK / 8);
-            // Column blocks past the edge are clamped (see DirectTile::load); col_limit is a multiple of 8.
-            const int safe_col = min(col0 + nc * 8, col_limit - 8);
-#pragma unroll
-            for (int r = 0; r < 8; ++r) {
-                regs[i][r] = *reinterpret_cast<const u32x4*>(base + static_cast<long>(k0 + kg * 8 + r) * ld +
-                                                             safe_col);
-            }
+        for (int i = 0; i < kLoads; ++i) {
+            const int chunk = threadIdx.x + i * kThreads;
+            const int row = chunk / kChunksPerRow, cc = chunk % kChunksPerRow;
+            // Column blocks past the edge are clamped (see KTile::load); col_limit is a multiple of 8.
+            const int safe_col = min(col0 + cc * 8, col_limit - 8);
+            regs[i] = *reinterpret_cast<const u32x4*>(base + static_cast<long>(k0 + row) * ld + safe_col);
         }
     }
-    template <typename T>
     __device__ __forceinline__ void store(T* lds) const {
 #pragma unroll
-        for (int i = 0; i < kPerThread; ++i) {
-            const int task = task_of(i);
-            if (task >= kTasks) continue;
-            const int kg = task % (kBK / 8), nc = task / (kBK / 8);
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {  // output row: column nc*8 + j, k = kg*8 .. kg*8+7
-                u32x4 out;
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const unsigned int lo = regs[i][2 * q][j >> 1];
-                    const unsigned int hi = regs[i][2 * q + 1][j >> 1];
-                    out[q] = (j & 1) ? __builtin_amdgcn_perm(hi, lo, 0x07060302u)
-                                     : __builtin_amdgcn_perm(hi, lo, 0x05040100u);
-                }
-                *reinterpret_cast<u32x4*>(lds + (nc * 8 + j) * kLdsStride + kg * 8) = out;
-            }
+        for (int i = 0; i < kLoads; ++i) {
+            const int chunk = threadIdx.x + i * kThreads;
+            const int row = chunk / kChunksPerRow, cc = chunk % kChunksPerRow;
+            *reinterpret_cast<u32x4*>(lds + row * kStride + cc * 8) = regs[i];
         }
     }
+    // Lane i of a 16-lane group addresses k row i/4, columns 4*(i%4) .. +3 of the group's 4 x 16
+    // block; groups 0/1 take columns 0-15/16-31 of the fragment, lanes 32-63 the k values 8-15.
+    __device__ __forceinline__ static int lane_offset(int lane) {
+        return ((lane >> 5) * 8 + ((lane & 15) >> 2)) * kStride + ((lane >> 4) & 1) * 16 + (lane & 3) * 4;
+    }
+    __device__ __forceinline__ static frag_t frag(const T* lane_base, int block0, int kk) {
+        using s16x4 = vec_t<short, 4>;
+        using lds_ptr = __attribute__((address_space(3))) s16x4*;
+        const T* q = lane_base + kk * 16 * kStride + block0;
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(q));
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(q + 4 * kStride));
+        vec_t<short, 8> both;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            both[e] = lo[e];
+            both[4 + e] = hi[e];
+        }
+        return __builtin_bit_cast(frag_t, both);
+    }
+};
+
+template <typename T, int BM, int BN, bool A_K, bool B_K>
+struct TileLayout {
+    using ATile = std::conditional_t<A_K, KTile<T, BM>, NTile<T, BM>>;
+    using BTile = std::conditional_t<B_K, KTile<T, BN>, NTile<T, BN>>;
+    static constexpr int kStage = ATile::kElems + BTile::kElems;  // elements per LDS stage: [A | B]
+    static constexpr int kSmemBytes = 2 * kStage * static_cast<int>(sizeof(T));
 };
 
 template <typename T, int BM, int BN, bool A_K, bool B_K, bool SPLIT>
 __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
     using frag_t = typename Mfma<T>::frag;
+    using Layout = TileLayout<T, BM, BN, A_K, B_K>;
+    using ATile = typename Layout::ATile;
+    using BTile = typename Layout::BTile;
     constexpr int WM = BM / 2, WN = BN / 2;
     constexpr int TM = WM / 32, TN = WN / 32;
     extern __shared__ __align__(16) unsigned char smem_raw[];
     T* smem = reinterpret_cast<T*>(smem_raw);
-    constexpr int kATile = BM * kLdsStride, kBTile = BN * kLdsStride;
     // Stage s holds [A tile | B tile] at smem + s * kStage. Offsets are added to the one shared base
     // so that every access is provably an LDS access (ds_read/ds_write, counted by lgkmcnt only).
-    constexpr int kStage = kATile + kBTile;
+    constexpr int kStage = Layout::kStage;
+    constexpr int kATile = ATile::kElems;
 
     // XCD-contiguous, grouped tile order.
     const int total = p.tiles_m * p.tiles_n;
@@ -198,29 +240,29 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
     const int k_tiles_total = p.k / kBK;
     const int kt_begin = blockIdx.y * p.k_tiles_per_slice;
     const int kt_end = min(k_tiles_total, kt_begin + p.k_tiles_per_slice);
+    const int count = kt_end - kt_begin;
 
     const T* A = static_cast<const T*>(p.a);
     const T* B = static_cast<const T*>(p.b);
 
-    DirectTile<BM> a_direct;
-    DirectTile<BN> b_direct;
-    TransposedTile<BM, 0> a_trans;
-    TransposedTile<BN, (A_K ? 0 : kThreads / 2)> b_trans;
-
+    ATile a_regs;
+    BTile b_regs;
+    // Tiles past the end of the slice reload the last one (it is stored but never multiplied), which
+    // keeps the K loop free of data-dependent branches.
     auto load_tiles = [&](int kt) {
-        const int k0 = kt * kBK;
-        if constexpr (A_K) a_direct.load(A, p.lda, m0, p.m, k0); else a_trans.load(A, p.lda, m0, p.m, k0);
-        if constexpr (B_K) b_direct.load(B, p.ldb, n0, p.n, k0); else b_trans.load(B, p.ldb, n0, p.n, k0);
+        const int k0 = min(kt, kt_end - 1) * kBK;
+        a_regs.load(A, p.lda, m0, p.m, k0);
+        b_regs.load(B, p.ldb, n0, p.n, k0);
     };
     auto store_tiles = [&](int buf) {
-        if constexpr (A_K) a_direct.store(smem + buf * kStage); else a_trans.store(smem + buf * kStage);
-        if constexpr (B_K) b_direct.store(smem + buf * kStage + kATile); else b_trans.store(smem + buf * kStage + kATile);
+        a_regs.store(smem + buf * kStage);
+        b_regs.store(smem + buf * kStage + kATile);
     };
 
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x / kWave;
     const int wm = wave >> 1, wn = wave & 1;
-    const int frag_row = lane & 31, frag_k = (lane >> 5) * 8;
+    const int a_lane = ATile::lane_offset(lane), b_lane = BTile::lane_offset(lane);
 
     acc_t acc[TM][TN];
 #pragma unroll
@@ -228,42 +270,63 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
 #pragma unroll
         for (int j = 0; j < TN; ++j) acc[i][j] = acc_t(0.0f);
 
-    if (kt_begin < kt_end) {
+    frag_t af[2][TM], bf[2][TN];
+    auto read_frags = [&](int set, int buf, int kk) {
+        const T* as = smem + buf * kStage + a_lane;
+        const T* bs = smem + buf * kStage + kATile + b_lane;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) af[set][i] = ATile::frag(as, wm * WM + i * 32, kk);
+#pragma unroll
+        for (int j = 0; j < TN; ++j) bf[set][j] = BTile::frag(bs, wn * WN + j * 32, kk);
+    };
+    auto multiply = [&](int set) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) acc[i][j] = Mfma<T>::run(bf[set][j], af[set][i], acc[i][j]);
+    };
+
+    // Software pipeline over K tiles t = 0 .. count-1 (tile t lives in LDS stage t%2), four K
+    // sub-steps of 16 per tile:
+    //   sub-steps 0,1  MFMAs ‖ LDS reads of the next sub-step's fragments
+    //   sub-step  2    MFMAs ‖ fragments of sub-step 3 ‖ registers of tile t+1 -> stage (t+1)%2
+    //   barrier        tile t+1 visible; nobody reads stage t%2 any more
+    //   sub-step  3    MFMAs ‖ fragments of tile t+1, sub-step 0 ‖ global loads of tile t+2
+    // so LDS latency, the barrier and most of the global latency sit in the shadow of MFMAs.
+    constexpr int kMfmas = TM * TN;
+    constexpr int kFragReads = TM * ATile::kFragReads + TN * BTile::kFragReads;
+    constexpr int kTileLoads = ATile::kLoads + BTile::kLoads;
+    static_assert(kBK == 64, "the pipeline below is written for four K sub-steps");
+    if (count > 0) {
         load_tiles(kt_begin);
         store_tiles(0);
+        load_tiles(kt_begin + 1);
+        __syncthreads();
+        read_frags(0, 0, 0);
+        for (int t = 0; t < count; ++t) {
+            const int buf = t & 1;
+            read_frags(1, buf, 1);
+            multiply(0);
+            read_frags(0, buf, 2);
+            multiply(1);
+            read_frags(1, buf, 3);
+            store_tiles(buf ^ 1);
+            multiply(0);
+            sched_interleave<kMfmas, kSchedDsRead, kFragReads, 0, 0>();
+            sched_interleave<kMfmas, kSchedDsRead, kFragReads, 0, 0>();
+            // LDS stores may not move above the (possibly aliasing) fragment reads issued before them:
+            // reads go with the first MFMAs of the sub-step, stores with the rest.
+            sched_interleave<kMfmas / 2, kSchedDsRead, kFragReads, 0, 0>();
+            sched_interleave<kMfmas - kMfmas / 2, kSchedDsWrite, kTileLoads, 0, 0>();
+            __builtin_amdgcn_sched_barrier(0);
+            __syncthreads();
+            read_frags(0, buf ^ 1, 0);
+            load_tiles(kt_begin + t + 2);
+            multiply(1);
+            sched_interleave<kMfmas, kSchedDsRead, kFragReads, kSchedVmemRead, kTileLoads>();
+        }
     }
     __syncthreads();
-    for (int kt = kt_begin; kt < kt_end; ++kt) {
-        const int buf = (kt - kt_begin) & 1;
-        const bool more = kt + 1 < kt_end;
-        if (more) load_tiles(kt + 1);
-        const T* as = smem + buf * kStage + (wm * WM + frag_row) * kLdsStride + frag_k;
-        const T* bs = smem + buf * kStage + kATile + (wn * WN + frag_row) * kLdsStride + frag_k;
-        // Fragments of K sub-step kk+1 are requested before the MFMAs of sub-step kk are issued.
-        frag_t af[2][TM], bf[2][TN];
-#pragma unroll
-        for (int i = 0; i < TM; ++i) af[0][i] = *reinterpret_cast<const frag_t*>(as + i * 32 * kLdsStride);
-#pragma unroll
-        for (int j = 0; j < TN; ++j) bf[0][j] = *reinterpret_cast<const frag_t*>(bs + j * 32 * kLdsStride);
-#pragma unroll
-        for (int kk = 0; kk < kBK / 16; ++kk) {
-            const int cur = kk & 1, nxt = cur ^ 1;
-            if (kk + 1 < kBK / 16) {
-#pragma unroll
-                for (int i = 0; i < TM; ++i)
-                    af[nxt][i] = *reinterpret_cast<const frag_t*>(as + i * 32 * kLdsStride + (kk + 1) * 16);
-#pragma unroll
-                for (int j = 0; j < TN; ++j)
-                    bf[nxt][j] = *reinterpret_cast<const frag_t*>(bs + j * 32 * kLdsStride + (kk + 1) * 16);
-            }
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-#pragma unroll
-                for (int j = 0; j < TN; ++j) acc[i][j] = Mfma<T>::run(bf[cur][j], af[cur][i], acc[i][j]);
-        }
-        if (more) store_tiles(buf ^ 1);
-        __syncthreads();
-    }
 
     // Epilogue. acc[i][j][4g+e] holds C[m, n] with m = lane%32, n = 8g + 4*(lane/32) + e. The tile
     // goes through LDS (fp32, row stride BN+4 so that the 16 lanes of a ds_write_b128 pass hit 16
@@ -271,7 +334,7 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
     // bytes of C per instruction instead of 32 separate 16-byte pieces. Rounding to the storage
     // dtype still happens once, after bias and accumulate were added in fp32.
     constexpr int kStageStride = BN + 4;
-    constexpr int kSmemBytes = 2 * (BM + BN) * kLdsStride * static_cast<int>(sizeof(T));
+    constexpr int kSmemBytes = Layout::kSmemBytes;
     constexpr int kPassRows = (BM * kStageStride * 4 <= kSmemBytes) ? BM : BM / 2;
     constexpr int kPasses = BM / kPassRows;
     static_assert(kPassRows * kStageStride * 4 <= kSmemBytes, "epilogue staging does not fit in LDS");
@@ -414,7 +477,7 @@ __global__ __launch_bounds__(kGenericTile* kGenericTile / 4) void gemm_generic_k
 // ------------------------------------------------------------------- host side
 template <typename T, int BM, int BN, bool A_K, bool B_K, bool SPLIT>
 int launch_mfma(const KernelArgs& p, int slices, hipStream_t stream) {
-    constexpr std::size_t smem = 2 * static_cast<std::size_t>(BM + BN) * kLdsStride * sizeof(T);
+    constexpr std::size_t smem = TileLayout<T, BM, BN, A_K, B_K>::kSmemBytes;
     auto kernel = gemm_mfma_kernel<T, BM, BN, A_K, B_K, SPLIT>;
     static bool configured = false;
     if (!configured) {
