@@ -554,6 +554,268 @@ __global__ __launch_bounds__(kThreads) void attention_dkv_kernel(Params p) {
     }
 }
 
+// ============================================================================================
+// Head dimensions 65..128 (padded width 128): the streamed tiles go from global memory straight
+// into LDS with buffer_load ... lds — no staging registers, no LDS stores, no address arithmetic in
+// the loop (one loop-invariant per-lane offset, the tile position is a scalar offset), rows past
+// the end of the sequence and columns past head_dim zero-filled by the buffer's range check. Two
+// LDS stages, one barrier per tile, two blocks per CU so that one block's softmax runs under the
+// other's MFMAs.
+//
+// A wavefront-wide LDS-direct load writes 64 x 16 B contiguously, so LDS rows are exactly 256 B
+// and cannot be padded. Instead the 16-byte chunk c of tile row r is kept at chunk position
+// c ^ swizzle(r), swizzle(r) = (r%4)*4 + (r/4)%4: the 16 rows a ds_read_b128 fragment read touches
+// hit 16 different chunk positions, and the 4 rows x 64 B a ds_read_b64_tr_b16 touches hit four
+// different 64-byte windows — both conflict-free. The lane that owns LDS slot (r, c') simply fetches
+// global chunk c' ^ swizzle(r).
+constexpr int kWideDim = 128;
+constexpr int kWideTile = kStream * kWideDim;  // elements of one 64 x 128 tile (16 KiB)
+
+constexpr int kSchedMfma = 0x008, kSchedDsRead = 0x100;
+template <int CLASS, int COUNT>
+__device__ __forceinline__ void sched_group() {
+    if constexpr (COUNT > 0) __builtin_amdgcn_sched_group_barrier(CLASS, COUNT, 0);
+}
+// LEAD LDS reads up front, then MFMAS matrix instructions with the remaining READS - LEAD reads
+// spread between the first ones of them.
+template <int MFMAS, int READS, int LEAD, int I = 0>
+__device__ __forceinline__ void sched_reads_under_mfmas() {
+    if constexpr (I == 0) sched_group<kSchedDsRead, LEAD>();
+    if constexpr (I < MFMAS) {
+        constexpr int kRest = READS - LEAD;
+        constexpr int kSpan = MFMAS - 2;  // the last two MFMAs need no further reads
+        constexpr int kDone = I < kSpan ? (I * kRest) / kSpan : kRest;
+        constexpr int kNext = I + 1 < kSpan ? ((I + 1) * kRest) / kSpan : kRest;
+        sched_group<kSchedMfma, 1>();
+        sched_group<kSchedDsRead, kNext - kDone>();
+        sched_reads_under_mfmas<MFMAS, READS, LEAD, I + 1>();
+    }
+}
+
+__device__ __forceinline__ int swizzle(int row) { return ((row & 3) << 2) | ((row >> 2) & 3); }
+
+using lds_void_ptr = __attribute__((address_space(3))) void*;
+
+// Where a lane's 16 bytes of a streamed tile come from: rows r0 + 16 i (i = 0..3) of the tile go
+// through the four loads of wavefront w, lane l owning LDS slot (row 4w + l/16, chunk l%16).
+struct TileSource {
+    __amdgpu_buffer_rsrc_t rsrc;
+    int voffset;    // bytes, loop-invariant
+    int row_bytes;  // bytes between consecutive sequence positions
+};
+
+template <typename T>
+__device__ __forceinline__ TileSource make_source(const T* base, long row_stride, int rows, int d, int wave) {
+    const int lane = threadIdx.x & 63;
+    TileSource s;
+    s.row_bytes = static_cast<int>(row_stride * sizeof(T));
+    const int bytes = static_cast<int>(((rows - 1) * row_stride + d) * sizeof(T));
+    s.rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(base), 0, bytes, 0x00020000);
+    const int r = wave * 4 + (lane >> 4);
+    const int chunk = (lane & 15) ^ swizzle(r);
+    // Chunks beyond head_dim get an offset past every valid byte: the load then returns zeros.
+    s.voffset = chunk * 8 < d ? r * s.row_bytes + chunk * 16 : (1 << 30);
+    return s;
+}
+
+template <typename T>
+__device__ __forceinline__ void stream_tile(const TileSource& s, int row0, T* tile, int wave) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(s.rsrc, (lds_void_ptr)(tile + (i * 16 + wave * 4) * kWideDim), 16,
+                                                 s.voffset, (row0 + i * 16) * s.row_bytes, 0, 0);
+}
+
+// Element offset (within a 32-row block of a swizzled tile) of the lane's ds_read_b128 fragment:
+// row lane%32, head-dim elements 16*step + 8*(lane/32) .. +7.
+__device__ __forceinline__ int wide_direct_offset(int lane, int step) {
+    const int row = lane & 31;
+    return row * kWideDim + (((2 * step + (lane >> 5)) ^ swizzle(row)) * 8);
+}
+// Element offset (within a 16-row block) of the lane's ds_read_b64_tr_b16 address for head-dim
+// columns 32t .. 32t+31: rows {0-3 | 4-7} (+8 for the second read), see transposed_frag.
+__device__ __forceinline__ int wide_transposed_offset(int lane, int t, int second) {
+    const int row = (lane >> 5) * 4 + ((lane & 15) >> 2) + second * 8;
+    const int chunk = t * 4 + ((lane >> 4) & 1) * 2 + ((lane & 3) >> 1);
+    return row * kWideDim + ((chunk ^ swizzle(row)) * 8) + (lane & 1) * 4;
+}
+template <typename T>
+__device__ __forceinline__ typename Mma<T>::frag wide_transposed_frag(const T* block, int first, int second) {
+    using lds_ptr = __attribute__((address_space(3))) s16x4*;
+    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(block + first));
+    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(block + second));
+    vec_t<short, 8> both;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        both[e] = lo[e];
+        both[4 + e] = hi[e];
+    }
+    return __builtin_bit_cast(typename Mma<T>::frag, both);
+}
+
+// Exchange between lane l and lane l^32.
+__device__ __forceinline__ float other_half(float v) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float((threadIdx.x & 32) ? r[0] : r[1]);
+}
+
+template <typename T>
+__global__ __launch_bounds__(kThreads, 2) void attention_forward_wide_kernel(Params p) {
+    using frag = typename Mma<T>::frag;
+    constexpr int STEPS = kWideDim / 16, DT = kWideDim / 32;
+    __shared__ __align__(1024) T lds[4 * kWideTile];  // [stage][K | V]
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int b = blockIdx.z, h = blockIdx.y, kvh = h / (p.hq / p.hkv);
+    const int q_block = (gridDim.x - 1 - blockIdx.x) * kBlockRows;  // blocks with the most key tiles start first
+    const int q_row = q_block + wave * 32 + (lane & 31);
+    const bool q_live = q_row < p.qs;
+    const long q_stride = static_cast<long>(p.hq) * p.d, kv_stride = static_cast<long>(p.hkv) * p.d;
+    const T* q_ptr = static_cast<const T*>(p.q) + (static_cast<long>(b) * p.qs + q_row) * q_stride + h * p.d;
+    const long kv_offset = static_cast<long>(b) * p.ks * kv_stride + kvh * p.d;
+    const TileSource k_src = make_source(static_cast<const T*>(p.k) + kv_offset, kv_stride, p.ks, p.d, wave);
+    const TileSource v_src = make_source(static_cast<const T*>(p.v) + kv_offset, kv_stride, p.ks, p.d, wave);
+
+    const int last_q_block = min(q_block + kBlockRows, p.qs) - 1;
+    const int k_end = p.causal ? min(p.ks, p.offset + last_q_block + 1) : p.ks;
+    const int tiles = (k_end + kStream - 1) / kStream;
+    if (tiles > 0) {
+        stream_tile(k_src, 0, lds, wave);
+        stream_tile(v_src, 0, lds + kWideTile, wave);
+    }
+
+    frag qf[STEPS];
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) qf[s] = global_frag<T>(q_ptr, q_live, s, p.d);
+    int k_off[STEPS], v_off[DT][2];
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) k_off[s] = wide_direct_offset(lane, s);
+#pragma unroll
+    for (int t = 0; t < DT; ++t) {
+        v_off[t][0] = wide_transposed_offset(lane, t, 0);
+        v_off[t][1] = wide_transposed_offset(lane, t, 1);
+    }
+
+    acc_t o[DT];
+#pragma unroll
+    for (int t = 0; t < DT; ++t) o[t] = acc_t(0.0f);
+    // The running maximum m is kept on the raw scores (the scale is positive, so it commutes with
+    // max); probabilities are exp2(s*scale2 - m*scale2), one FMA and one v_exp_f32 per score.
+    float m = -INFINITY, l = 0.0f;
+    const float scale2 = p.scale * kLog2e;
+    const int wave_first_q = q_block + wave * 32;
+    const int wave_last_q = min(wave_first_q + 31, p.qs - 1);
+    const bool wave_live = wave_first_q < p.qs;
+    const int q_limit = p.causal ? p.offset + q_row : p.ks;  // largest visible key of this lane's query
+    // Tiles whose last key is visible to the wave's first query need no masking at all.
+    const int clear_limit = p.causal ? min(p.ks - 1, p.offset + wave_first_q) : p.ks - 1;
+
+    for (int j = 0; j < tiles; ++j) {
+        const int k0 = j * kStream;
+        const T* k_tile = lds + (j & 1) * 2 * kWideTile;
+        const T* v_tile = k_tile + kWideTile;
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wavefront's part of tile j is in LDS
+        __syncthreads();                     // ... and everybody else's; stage (j+1)%2 is free
+        if (j + 1 < tiles) {
+            T* next = lds + ((j + 1) & 1) * 2 * kWideTile;
+            stream_tile(k_src, k0 + kStream, next, wave);
+            stream_tile(v_src, k0 + kStream, next + kWideTile, wave);
+        }
+        if (!wave_live || (p.causal && k0 > p.offset + wave_last_q)) continue;
+
+        acc_t st[2] = {acc_t(0.0f), acc_t(0.0f)};
+        {
+            frag ka[2][STEPS];
+#pragma unroll
+            for (int s = 0; s < STEPS; ++s) {
+                ka[0][s] = *reinterpret_cast<const frag*>(k_tile + k_off[s]);
+                ka[1][s] = *reinterpret_cast<const frag*>(k_tile + 32 * kWideDim + k_off[s]);
+            }
+#pragma unroll
+            for (int s = 0; s < STEPS; ++s) {
+                st[0] = Mma<T>::run(ka[0][s], qf[s], st[0]);
+                st[1] = Mma<T>::run(ka[1][s], qf[s], st[1]);
+            }
+            sched_reads_under_mfmas<2 * STEPS, 2 * STEPS, 4>();
+        }
+        __builtin_amdgcn_sched_barrier(0);
+
+        if (k0 + kStream - 1 > clear_limit) {
+            // key = k0 + 32 sub + 8 (i/4) + 4 (lane/32) + i%4 is visible iff key <= min(q_limit, ks-1):
+            // one comparison of a per-lane bound with a literal per score.
+            const int bound = min(q_limit, p.ks - 1) - k0 - 4 * (lane >> 5);
+            asm volatile("" ::: "memory");  // keeps the masking out of the common path (no if-conversion)
+#pragma unroll
+            for (int sub = 0; sub < 2; ++sub)
+#pragma unroll
+                for (int i = 0; i < 16; ++i)
+                    st[sub][i] = (sub * 32 + 8 * (i >> 2) + (i & 3) <= bound) ? st[sub][i] : -INFINITY;
+        }
+        float tile_max = fmaxf(st[0][0], st[1][0]);
+#pragma unroll
+        for (int i = 1; i < 16; ++i) tile_max = fmaxf(tile_max, fmaxf(st[0][i], st[1][i]));
+        tile_max = fmaxf(tile_max, other_half(tile_max));
+        const float m_new = fmaxf(m, tile_max);
+        const float mb = m_new == -INFINITY ? 0.0f : m_new * scale2;
+        const float alpha = __builtin_amdgcn_exp2f(m * scale2 - mb);
+        float tile_sum = 0.0f;
+#pragma unroll
+        for (int sub = 0; sub < 2; ++sub)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const float e = __builtin_amdgcn_exp2f(fmaf(st[sub][i], scale2, -mb));
+                st[sub][i] = e;
+                tile_sum += e;
+            }
+        l = l * alpha + tile_sum;
+        m = m_new;
+        if (__any(alpha != 1.0f)) {  // the maximum moved for some query of the wavefront
+#pragma unroll
+            for (int t = 0; t < DT; ++t) o[t] *= alpha;
+        }
+        __builtin_amdgcn_sched_barrier(0);
+
+        {
+            frag pf[2][2], vt[2][2][DT];
+#pragma unroll
+            for (int sub = 0; sub < 2; ++sub)
+#pragma unroll
+                for (int s = 0; s < 2; ++s) {
+                    pf[sub][s] = acc_frag<T>(st[sub], s);
+                    const T* block = v_tile + (sub * 32 + s * 16) * kWideDim;
+#pragma unroll
+                    for (int t = 0; t < DT; ++t) vt[sub][s][t] = wide_transposed_frag<T>(block, v_off[t][0], v_off[t][1]);
+                }
+#pragma unroll
+            for (int sub = 0; sub < 2; ++sub)
+#pragma unroll
+                for (int s = 0; s < 2; ++s)
+#pragma unroll
+                    for (int t = 0; t < DT; ++t) o[t] = Mma<T>::run(vt[sub][s][t], pf[sub][s], o[t]);
+            sched_reads_under_mfmas<4 * DT, 8 * DT, 8>();
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    l += other_half(l);
+    if (!q_live) return;
+    const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+    T* o_ptr = static_cast<T*>(p.out0) + (static_cast<long>(b) * p.qs + q_row) * q_stride + h * p.d;
+#pragma unroll
+    for (int t = 0; t < DT; ++t) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const int d0 = t * 32 + g * 8 + (lane >> 5) * 4;
+            if (d0 >= p.d) continue;
+            vec_t<float, 4> v;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] = o[t][4 * g + e] * inv;
+            store_vec<T, 4>(o_ptr + d0, vec_from_f32<T, 4>(v));
+        }
+    }
+    if (p.lse_out != nullptr && lane < 32)
+        p.lse_out[(static_cast<long>(b) * p.qs + q_row) * p.hq + h] = (m * scale2 + log2f(l)) * kLn2;
+}
+
 // ---------------------------------------------------------------------- host
 struct Shape {
     std::size_t batch, qs, ks, hq, hkv, d;
@@ -595,6 +857,13 @@ Params make_params(const Shape& s) {
     return p;
 }
 
+// The LDS-direct kernels cover head dimensions 65..128 and address K/V (and Q/dO) of one batch
+// element with 32-bit byte offsets.
+bool wide_path(const Shape& s) {
+    constexpr std::size_t limit = std::size_t{1} << 30;
+    return s.d > 64 && s.ks * s.hkv * s.d * 2 < limit && s.qs * s.hq * s.d * 2 < limit;
+}
+
 template <typename Fn>
 int dispatch_head_dim(std::size_t d, Fn&& fn) {
     if (d <= 32) return fn.template operator()<32>();
@@ -611,6 +880,11 @@ int launch_forward(const Shape& s, Params p, hipStream_t stream) {
     const dim3 grid(static_cast<unsigned int>((s.qs + kBlockRows - 1) / kBlockRows), static_cast<unsigned int>(s.hq),
                     static_cast<unsigned int>(s.batch));
     return dispatch_16bit(s.dtype, [&]<typename T>() -> int {
+        if (wide_path(s)) {
+            hipLaunchKernelGGL((attention_forward_wide_kernel<T>), grid, dim3(kThreads), 0, stream, p);
+            CGPTX_LAUNCH_CHECK();
+            return CGPTX_OK;
+        }
         return dispatch_head_dim(s.d, [&]<int DP>() -> int {
             hipLaunchKernelGGL((attention_forward_kernel<T, DP>), grid, dim3(kThreads), 0, stream, p);
             CGPTX_LAUNCH_CHECK();
