@@ -294,9 +294,11 @@ __global__ __launch_bounds__(kThreads) void attention_forward_kernel(Params p) {
 }
 
 // --------------------------------------------------------------------- delta
-// delta[b, t, h] = Σ_d dO·O, one group of LPR lanes per row, 128-bit loads.
+// delta[b, t, h] = Σ_d dO·O (and LSE·log2 e next to it), one group of LPR lanes per row, 128-bit loads.
 template <typename T, int LPR>
 __global__ __launch_bounds__(kThreads) void attention_delta_kernel(float* __restrict__ delta,
+                                                                  float* __restrict__ lse2,
+                                                                  const float* __restrict__ lse,
                                                                   const T* __restrict__ dout,
                                                                   const T* __restrict__ out, long rows, int d) {
     const long row = (static_cast<long>(blockIdx.x) * kThreads + threadIdx.x) / LPR;
@@ -309,7 +311,10 @@ __global__ __launch_bounds__(kThreads) void attention_delta_kernel(float* __rest
         for (int e = 0; e < 8; ++e) sum = fmaf(a[e], b[e], sum);
     }
     sum = wave_sum<LPR>(sum);
-    if (row < rows && sub == 0) delta[row] = sum;
+    if (row < rows && sub == 0) {
+        delta[row] = sum;
+        lse2[row] = lse[row] * kLog2e;  // the exponent the wide backward kernels subtract, in base 2
+    }
 }
 
 // ------------------------------------------------------------------------ dQ
@@ -604,12 +609,15 @@ struct TileSource {
     int row_bytes;  // bytes between consecutive sequence positions
 };
 
+// last_row: elements of the last row that belong to the buffer (head_dim when base points at one
+// head, the whole row when the head is chosen by the scalar offset of each load).
 template <typename T>
-__device__ __forceinline__ TileSource make_source(const T* base, long row_stride, int rows, int d, int wave) {
+__device__ __forceinline__ TileSource make_source(const T* base, long row_stride, int rows, int d, int wave,
+                                                  long last_row) {
     const int lane = threadIdx.x & 63;
     TileSource s;
     s.row_bytes = static_cast<int>(row_stride * sizeof(T));
-    const int bytes = static_cast<int>(((rows - 1) * row_stride + d) * sizeof(T));
+    const int bytes = static_cast<int>(((rows - 1) * row_stride + last_row) * sizeof(T));
     s.rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(base), 0, bytes, 0x00020000);
     const int r = wave * 4 + (lane >> 4);
     const int chunk = (lane & 15) ^ swizzle(r);
@@ -673,8 +681,8 @@ __global__ __launch_bounds__(kThreads, 2) void attention_forward_wide_kernel(Par
     const long q_stride = static_cast<long>(p.hq) * p.d, kv_stride = static_cast<long>(p.hkv) * p.d;
     const T* q_ptr = static_cast<const T*>(p.q) + (static_cast<long>(b) * p.qs + q_row) * q_stride + h * p.d;
     const long kv_offset = static_cast<long>(b) * p.ks * kv_stride + kvh * p.d;
-    const TileSource k_src = make_source(static_cast<const T*>(p.k) + kv_offset, kv_stride, p.ks, p.d, wave);
-    const TileSource v_src = make_source(static_cast<const T*>(p.v) + kv_offset, kv_stride, p.ks, p.d, wave);
+    const TileSource k_src = make_source(static_cast<const T*>(p.k) + kv_offset, kv_stride, p.ks, p.d, wave, p.d);
+    const TileSource v_src = make_source(static_cast<const T*>(p.v) + kv_offset, kv_stride, p.ks, p.d, wave, p.d);
 
     const int last_q_block = min(q_block + kBlockRows, p.qs) - 1;
     const int k_end = p.causal ? min(p.ks, p.offset + last_q_block + 1) : p.ks;
@@ -816,6 +824,369 @@ __global__ __launch_bounds__(kThreads, 2) void attention_forward_wide_kernel(Par
         p.lse_out[(static_cast<long>(b) * p.qs + q_row) * p.hq + h] = (m * scale2 + log2f(l)) * kLn2;
 }
 
+// dQ for head dimensions 65..128: the forward kernel's streaming scheme; per 32-key half tile
+// Sᵀ = K·Qᵀ and dPᵀ = V·dOᵀ (two independent MFMA chains), dS = P∘(dP − delta) in registers,
+// dQᵀ += Kᵀ·dSᵀ with K read back transposed. lse2 holds LSE·log2(e).
+template <typename T>
+__global__ __launch_bounds__(kThreads, 2) void attention_dq_wide_kernel(Params p) {
+    using frag = typename Mma<T>::frag;
+    constexpr int STEPS = kWideDim / 16, DT = kWideDim / 32;
+    __shared__ __align__(1024) T lds[4 * kWideTile];  // [stage][K | V]
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int b = blockIdx.z, h = blockIdx.y, kvh = h / (p.hq / p.hkv);
+    const int q_block = (gridDim.x - 1 - blockIdx.x) * kBlockRows;
+    const int q_row = q_block + wave * 32 + (lane & 31);
+    const bool q_live = q_row < p.qs;
+    const long q_stride = static_cast<long>(p.hq) * p.d, kv_stride = static_cast<long>(p.hkv) * p.d;
+    const long q_offset = (static_cast<long>(b) * p.qs + q_row) * q_stride + h * p.d;
+    const long kv_offset = static_cast<long>(b) * p.ks * kv_stride + kvh * p.d;
+    const TileSource k_src = make_source(static_cast<const T*>(p.k) + kv_offset, kv_stride, p.ks, p.d, wave, p.d);
+    const TileSource v_src = make_source(static_cast<const T*>(p.v) + kv_offset, kv_stride, p.ks, p.d, wave, p.d);
+
+    const int last_q_block = min(q_block + kBlockRows, p.qs) - 1;
+    const int k_end = p.causal ? min(p.ks, p.offset + last_q_block + 1) : p.ks;
+    const int tiles = (k_end + kStream - 1) / kStream;
+    if (tiles > 0) {
+        stream_tile(k_src, 0, lds, wave);
+        stream_tile(v_src, 0, lds + kWideTile, wave);
+    }
+
+    frag qf[STEPS], dof[STEPS];
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) {
+        qf[s] = global_frag<T>(static_cast<const T*>(p.q) + q_offset, q_live, s, p.d);
+        dof[s] = global_frag<T>(static_cast<const T*>(p.dout) + q_offset, q_live, s, p.d);
+    }
+    const long stat_index = (static_cast<long>(b) * p.qs + q_row) * p.hq + h;
+    const float lse2 = q_live ? p.lse[stat_index] : 0.0f;
+    const float delta = q_live ? p.delta[stat_index] : 0.0f;
+    int k_off[STEPS], kt_off[DT][2];
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) k_off[s] = wide_direct_offset(lane, s);
+#pragma unroll
+    for (int t = 0; t < DT; ++t) {
+        kt_off[t][0] = wide_transposed_offset(lane, t, 0);
+        kt_off[t][1] = wide_transposed_offset(lane, t, 1);
+    }
+
+    acc_t dq[DT];
+#pragma unroll
+    for (int t = 0; t < DT; ++t) dq[t] = acc_t(0.0f);
+    const float scale2 = p.scale * kLog2e;
+    const int wave_first_q = q_block + wave * 32;
+    const int wave_last_q = min(wave_first_q + 31, p.qs - 1);
+    const bool wave_live = wave_first_q < p.qs;
+    const int q_limit = p.causal ? p.offset + q_row : p.ks;
+    const int clear_limit = p.causal ? min(p.ks - 1, p.offset + wave_first_q) : p.ks - 1;
+
+    for (int j = 0; j < tiles; ++j) {
+        const int k0 = j * kStream;
+        const T* k_tile = lds + (j & 1) * 2 * kWideTile;
+        const T* v_tile = k_tile + kWideTile;
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+        __syncthreads();
+        if (j + 1 < tiles) {
+            T* next = lds + ((j + 1) & 1) * 2 * kWideTile;
+            stream_tile(k_src, k0 + kStream, next, wave);
+            stream_tile(v_src, k0 + kStream, next + kWideTile, wave);
+        }
+        if (!wave_live || (p.causal && k0 > p.offset + wave_last_q)) continue;
+        const bool masked = k0 + kStream - 1 > clear_limit;
+        const int bound = min(q_limit, p.ks - 1) - k0 - 4 * (lane >> 5);
+#pragma unroll
+        for (int sub = 0; sub < 2; ++sub) {
+            acc_t st(0.0f), dpt(0.0f);
+            {
+                frag ka[STEPS], va[STEPS];
+#pragma unroll
+                for (int s = 0; s < STEPS; ++s) {
+                    ka[s] = *reinterpret_cast<const frag*>(k_tile + sub * 32 * kWideDim + k_off[s]);
+                    va[s] = *reinterpret_cast<const frag*>(v_tile + sub * 32 * kWideDim + k_off[s]);
+                }
+#pragma unroll
+                for (int s = 0; s < STEPS; ++s) {
+                    st = Mma<T>::run(ka[s], qf[s], st);
+                    dpt = Mma<T>::run(va[s], dof[s], dpt);
+                }
+                sched_reads_under_mfmas<2 * STEPS, 2 * STEPS, 4>();
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            if (masked) {
+                asm volatile("" ::: "memory");  // keeps the masking out of the common path (no if-conversion)
+#pragma unroll
+                for (int i = 0; i < 16; ++i)
+                    st[i] = (sub * 32 + 8 * (i >> 2) + (i & 3) <= bound) ? st[i] : -INFINITY;
+            }
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const float prob = __builtin_amdgcn_exp2f(fmaf(st[i], scale2, -lse2));
+                st[i] = prob * (dpt[i] - delta);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            {
+                frag dsf[2], kt[2][DT];
+#pragma unroll
+                for (int s = 0; s < 2; ++s) {
+                    dsf[s] = acc_frag<T>(st, s);
+                    const T* block = k_tile + (sub * 32 + s * 16) * kWideDim;
+#pragma unroll
+                    for (int t = 0; t < DT; ++t) kt[s][t] = wide_transposed_frag<T>(block, kt_off[t][0], kt_off[t][1]);
+                }
+#pragma unroll
+                for (int s = 0; s < 2; ++s)
+#pragma unroll
+                    for (int t = 0; t < DT; ++t) dq[t] = Mma<T>::run(kt[s][t], dsf[s], dq[t]);
+                sched_reads_under_mfmas<2 * DT, 4 * DT, 6>();
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    if (!q_live) return;
+    T* out = static_cast<T*>(p.out0) + q_offset;
+#pragma unroll
+    for (int t = 0; t < DT; ++t) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const int d0 = t * 32 + g * 8 + (lane >> 5) * 4;
+            if (d0 >= p.d) continue;
+            vec_t<float, 4> v;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] = dq[t][4 * g + e] * p.scale;
+            if (p.accumulate) v += vec_to_f32<T, 4>(load_vec<T, 4>(out + d0));
+            store_vec<T, 4>(out + d0, vec_from_f32<T, 4>(v));
+        }
+    }
+}
+
+// dK/dV for head dimensions 65..128. A block owns 128 keys of one (batch, kv-head) — 32 per
+// wavefront, K and V fragments and the two accumulator tiles in registers — and streams the 64-query
+// Q/dO tiles (plus their LSE·log2 e and delta values) of every q-head of the group through two LDS
+// stages with LDS-direct loads. Registers allow one wavefront per SIMD here, so the overlap of
+// MFMA, VALU and LDS work is arranged inside the wavefront: the tile is handled as two 32-query
+// halves A and B whose phases are issued as
+//   S_A,dP_A | S_B,dP_B ‖ softmax_A | dV_A,dK_A ‖ softmax_B | dV_B,dK_B
+// with the instruction order pinned by sched_group_barrier.
+// Key blocks are handled in pairs (i, last-i) by one block: under a causal mask block i sees
+// (last-i+1)/(last+1) of the queries, so every pair carries the same work and 256 equal blocks fill
+// 256 CUs exactly at the training shape.
+// Queries past the end of the sequence need no masking: their dO rows and delta arrive as zeros
+// (buffer range check), so P·dO and P∘(dP−delta) vanish whatever P is.
+constexpr int kSchedValu = 0x402;  // VALU and transcendental
+constexpr int kWideDkvSmem = 4 * kWideTile * 2 + 4 * kStream * static_cast<int>(sizeof(float));
+
+template <int MFMAS, int LEAD, int READS_EACH, int READ_SPAN, int VALU_EACH, int I = 0>
+__device__ __forceinline__ void sched_phase() {
+    if constexpr (I == 0) sched_group<kSchedDsRead, LEAD>();
+    if constexpr (I < MFMAS) {
+        sched_group<kSchedMfma, 1>();
+        if constexpr (I < READ_SPAN) sched_group<kSchedDsRead, READS_EACH>();
+        sched_group<kSchedValu, VALU_EACH>();
+        sched_phase<MFMAS, LEAD, READS_EACH, READ_SPAN, VALU_EACH, I + 1>();
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kThreads, 1) void attention_dkv_wide_kernel(Params p) {
+    using frag = typename Mma<T>::frag;
+    constexpr int STEPS = kWideDim / 16, DT = kWideDim / 32;
+    extern __shared__ __align__(1024) unsigned char wide_smem[];
+    T* lds = reinterpret_cast<T*>(wide_smem);                             // [stage][Q | dO]
+    float* stats = reinterpret_cast<float*>(wide_smem + 4 * kWideTile * sizeof(T));  // [stage][lse2 | delta][64]
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int b = blockIdx.z, kvh = blockIdx.y, group = p.hq / p.hkv;
+    const long q_stride = static_cast<long>(p.hq) * p.d, kv_stride = static_cast<long>(p.hkv) * p.d;
+    const float scale2 = p.scale * kLog2e;
+
+    // Sources: Q and dO of this batch element (the head is part of the scalar offset), and the two
+    // per-(query, head) statistics, one float per lane.
+    const long q_batch = static_cast<long>(b) * p.qs * q_stride;
+    const TileSource q_src = make_source(static_cast<const T*>(p.q) + q_batch, q_stride, p.qs, p.d, wave, q_stride);
+    const TileSource do_src = make_source(static_cast<const T*>(p.dout) + q_batch, q_stride, p.qs, p.d, wave, q_stride);
+    const int stat_bytes = p.qs * p.hq * static_cast<int>(sizeof(float));
+    const float* stat_base = (wave == 0 ? p.lse : p.delta) + static_cast<long>(b) * p.qs * p.hq;
+    const __amdgpu_buffer_rsrc_t stat_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(stat_base), 0, stat_bytes, 0x00020000);
+    const int stat_voffset = lane * p.hq * static_cast<int>(sizeof(float));
+
+    int q_off[STEPS], t_off[DT][2];
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) q_off[s] = wide_direct_offset(lane, s);
+#pragma unroll
+    for (int t = 0; t < DT; ++t) {
+        t_off[t][0] = wide_transposed_offset(lane, t, 0);
+        t_off[t][1] = wide_transposed_offset(lane, t, 1);
+    }
+
+    const int key_blocks = (p.ks + kBlockRows - 1) / kBlockRows;
+    for (int half = 0; half < 2; ++half) {
+        const int block_index = half == 0 ? static_cast<int>(blockIdx.x) : key_blocks - 1 - static_cast<int>(blockIdx.x);
+        if (half == 1 && block_index <= static_cast<int>(blockIdx.x)) break;
+        const int k_block = block_index * kBlockRows;
+        const int k_row = k_block + wave * 32 + (lane & 31);
+        const bool k_live = k_row < p.ks;
+        const long k_offset = (static_cast<long>(b) * p.ks + k_row) * kv_stride + kvh * p.d;
+        frag kf[STEPS], vf[STEPS];
+#pragma unroll
+        for (int s = 0; s < STEPS; ++s) {
+            kf[s] = global_frag<T>(static_cast<const T*>(p.k) + k_offset, k_live, s, p.d);
+            vf[s] = global_frag<T>(static_cast<const T*>(p.v) + k_offset, k_live, s, p.d);
+        }
+        acc_t dk[DT], dv[DT];
+#pragma unroll
+        for (int t = 0; t < DT; ++t) {
+            dk[t] = acc_t(0.0f);
+            dv[t] = acc_t(0.0f);
+        }
+        // First query tile that can see any key of this block; the (head of the group, query tile)
+        // pairs form one flat sequence so that the next tile is prefetched across head boundaries.
+        const int q_begin = p.causal ? max(0, k_block - p.offset) / kStream * kStream : 0;
+        const int tiles_per_head = q_begin < p.qs ? (p.qs - q_begin + kStream - 1) / kStream : 0;
+        const int total_tiles = tiles_per_head * group;
+        const int wave_first_key = k_block + wave * 32;
+        const int wave_last_key = wave_first_key + 31;
+
+        auto issue = [&](int tile) {
+            const int h = kvh * group + tile / tiles_per_head;
+            const int q0 = q_begin + (tile % tiles_per_head) * kStream;
+            T* stage = lds + (tile & 1) * 2 * kWideTile;
+            const int head_bytes = h * p.d * static_cast<int>(sizeof(T));
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int soffset = (q0 + i * 16) * q_src.row_bytes + head_bytes;
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(q_src.rsrc, (lds_void_ptr)(stage + (i * 16 + wave * 4) * kWideDim),
+                                                         16, q_src.voffset, soffset, 0, 0);
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(
+                    do_src.rsrc, (lds_void_ptr)(stage + kWideTile + (i * 16 + wave * 4) * kWideDim), 16, do_src.voffset,
+                    soffset, 0, 0);
+            }
+            if (wave < 2)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(
+                    stat_rsrc, (lds_void_ptr)(stats + (tile & 1) * 2 * kStream + wave * kStream), 4, stat_voffset,
+                    (q0 * p.hq + h) * static_cast<int>(sizeof(float)), 0, 0);
+        };
+
+        // One 64-query tile. masked: some (query, key) pairs of this wavefront are hidden (causal
+        // mask, keys past the end); first = first visible register coordinate for this lane's key.
+        auto tile_body = [&](const T* q_tile, const T* do_tile, const float* stat, bool masked, int first) {
+            acc_t s_acc[2] = {acc_t(0.0f), acc_t(0.0f)}, dp_acc[2] = {acc_t(0.0f), acc_t(0.0f)};
+            frag pf[2][2], dsf[2][2];
+            auto scores = [&](int sub) {
+                frag qa[STEPS], da[STEPS];
+#pragma unroll
+                for (int s = 0; s < STEPS; ++s) {
+                    qa[s] = *reinterpret_cast<const frag*>(q_tile + sub * 32 * kWideDim + q_off[s]);
+                    da[s] = *reinterpret_cast<const frag*>(do_tile + sub * 32 * kWideDim + q_off[s]);
+                }
+#pragma unroll
+                for (int s = 0; s < STEPS; ++s) {
+                    s_acc[sub] = Mma<T>::run(qa[s], kf[s], s_acc[sub]);
+                    dp_acc[sub] = Mma<T>::run(da[s], vf[s], dp_acc[sub]);
+                }
+            };
+            auto softmax = [&](int sub) {
+                vec_t<float, 4> lse_q[4], delta_q[4];
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int local = sub * 32 + 8 * g + 4 * (lane >> 5);
+                    lse_q[g] = *reinterpret_cast<const vec_t<float, 4>*>(stat + local);
+                    delta_q[g] = *reinterpret_cast<const vec_t<float, 4>*>(stat + kStream + local);
+                }
+                acc_t prob, ds;
+#pragma unroll
+                for (int i = 0; i < 16; ++i)
+                    prob[i] = __builtin_amdgcn_exp2f(fmaf(s_acc[sub][i], scale2, -lse_q[i >> 2][i & 3]));
+                if (masked) {
+                    asm volatile("" ::: "memory");  // keeps the masking out of the common path (no if-conversion)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) prob[i] = (sub * 32 + 8 * (i >> 2) + (i & 3) >= first) ? prob[i] : 0.0f;
+                }
+#pragma unroll
+                for (int i = 0; i < 16; ++i) ds[i] = prob[i] * (dp_acc[sub][i] - delta_q[i >> 2][i & 3]);
+#pragma unroll
+                for (int s = 0; s < 2; ++s) {
+                    pf[sub][s] = acc_frag<T>(prob, s);
+                    dsf[sub][s] = acc_frag<T>(ds, s);
+                }
+            };
+            auto gradients = [&](int sub) {
+                frag dot[2][DT], qt[2][DT];
+#pragma unroll
+                for (int s = 0; s < 2; ++s) {
+                    const int block = (sub * 32 + s * 16) * kWideDim;
+#pragma unroll
+                    for (int t = 0; t < DT; ++t) {
+                        dot[s][t] = wide_transposed_frag<T>(do_tile + block, t_off[t][0], t_off[t][1]);
+                        qt[s][t] = wide_transposed_frag<T>(q_tile + block, t_off[t][0], t_off[t][1]);
+                    }
+                }
+#pragma unroll
+                for (int s = 0; s < 2; ++s)
+#pragma unroll
+                    for (int t = 0; t < DT; ++t) {
+                        dv[t] = Mma<T>::run(dot[s][t], pf[sub][s], dv[t]);
+                        dk[t] = Mma<T>::run(qt[s][t], dsf[sub][s], dk[t]);
+                    }
+            };
+#pragma unroll
+            for (int sub = 0; sub < 2; ++sub) {
+                scores(sub);
+                sched_reads_under_mfmas<2 * STEPS, 2 * STEPS, 4>();
+                __builtin_amdgcn_sched_barrier(0);
+                softmax(sub);
+                __builtin_amdgcn_sched_barrier(0);
+                gradients(sub);
+                sched_reads_under_mfmas<4 * DT, 8 * DT, 8>();
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        };
+
+        if (total_tiles > 0) issue(0);
+        for (int tile = 0; tile < total_tiles; ++tile) {
+            const int q0 = q_begin + (tile % tiles_per_head) * kStream;
+            const T* q_tile = lds + (tile & 1) * 2 * kWideTile;
+            const float* stat = stats + (tile & 1) * 2 * kStream;
+            __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wavefront's part of the tile is in LDS
+            __syncthreads();                     // ... and everybody else's; the other stage is free
+            if (tile + 1 < total_tiles) issue(tile + 1);
+            // Every wavefront runs every tile (no divergent paths around the accumulators): pairs the
+            // causal mask hides, and keys past the end of the sequence, get P = 0.
+            // Register i of half `sub` holds query q0 + 32 sub + 8 (i/4) + 4 (lane/32) + i%4; this lane's
+            // key sees it iff that query is >= key - offset.
+            const bool masked = (p.causal && wave_last_key > p.offset + q0) || wave_last_key >= p.ks;
+            const int causal_first = p.causal ? k_row - p.offset - q0 - 4 * (lane >> 5) : -(1 << 30);
+            const int first = k_live ? causal_first : (1 << 30);
+            tile_body(q_tile, q_tile + kWideTile, stat, masked, first);
+        }
+        __syncthreads();  // the next key block's first loads overwrite stage 0
+        if (k_live) {
+            T* dk_out = static_cast<T*>(p.out0) + k_offset;
+            T* dv_out = static_cast<T*>(p.out1) + k_offset;
+#pragma unroll
+            for (int t = 0; t < DT; ++t) {
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int d0 = t * 32 + g * 8 + (lane >> 5) * 4;
+                    if (d0 >= p.d) continue;
+                    vec_t<float, 4> a, c;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        a[e] = dk[t][4 * g + e] * p.scale;
+                        c[e] = dv[t][4 * g + e];
+                    }
+                    if (p.accumulate) {
+                        a += vec_to_f32<T, 4>(load_vec<T, 4>(dk_out + d0));
+                        c += vec_to_f32<T, 4>(load_vec<T, 4>(dv_out + d0));
+                    }
+                    store_vec<T, 4>(dk_out + d0, vec_from_f32<T, 4>(a));
+                    store_vec<T, 4>(dv_out + d0, vec_from_f32<T, 4>(c));
+                }
+            }
+        }
+    }
+}
+
 // ---------------------------------------------------------------------- host
 struct Shape {
     std::size_t batch, qs, ks, hq, hkv, d;
@@ -859,6 +1230,9 @@ Params make_params(const Shape& s) {
 
 // The LDS-direct kernels cover head dimensions 65..128 and address K/V (and Q/dO) of one batch
 // element with 32-bit byte offsets.
+// Bytes reserved for one float per (batch, query, head), rounded so that blocks stay 256-byte aligned.
+std::size_t stat_block_bytes(std::size_t rows) { return (rows * sizeof(float) + 255) & ~std::size_t{255}; }
+
 bool wide_path(const Shape& s) {
     constexpr std::size_t limit = std::size_t{1} << 30;
     return s.d > 64 && s.ks * s.hkv * s.d * 2 < limit && s.qs * s.hq * s.d * 2 < limit;
@@ -896,9 +1270,11 @@ int launch_forward(const Shape& s, Params p, hipStream_t stream) {
 int launch_backward(const Shape& s, Params p, void* dq, void* dk, void* dv, const void* dout, const void* out,
                     const float* lse, int accumulate, hipStream_t stream) {
     const std::size_t rows = s.batch * s.qs * s.hq;
+    const std::size_t stat_bytes = stat_block_bytes(rows);
     void* mem = nullptr;
-    if (int st = scratch(stream, rows * sizeof(float), &mem)) return st;
+    if (int st = scratch(stream, 2 * stat_bytes, &mem)) return st;  // [delta | LSE·log2 e]
     auto* delta = static_cast<float*>(mem);
+    auto* lse2 = reinterpret_cast<float*>(static_cast<char*>(mem) + stat_bytes);
     p.dout = dout;
     p.lse = lse;
     p.delta = delta;
@@ -912,27 +1288,46 @@ int launch_backward(const Shape& s, Params p, void* dq, void* dk, void* dv, cons
         const int d = static_cast<int>(s.d);
         if (lpr == 4)
             hipLaunchKernelGGL((attention_delta_kernel<T, 4>), dim3(delta_blocks), dim3(kThreads), 0, stream, delta,
-                               dout_t, out_t, r, d);
+                               lse2, lse, dout_t, out_t, r, d);
         else if (lpr == 8)
             hipLaunchKernelGGL((attention_delta_kernel<T, 8>), dim3(delta_blocks), dim3(kThreads), 0, stream, delta,
-                               dout_t, out_t, r, d);
+                               lse2, lse, dout_t, out_t, r, d);
         else
             hipLaunchKernelGGL((attention_delta_kernel<T, 16>), dim3(delta_blocks), dim3(kThreads), 0, stream, delta,
-                               dout_t, out_t, r, d);
+                               lse2, lse, dout_t, out_t, r, d);
         CGPTX_LAUNCH_CHECK();
         return dispatch_head_dim(s.d, [&]<int DP>() -> int {
             Params pq = p;
             pq.out0 = dq;
             const dim3 q_grid(static_cast<unsigned int>((s.qs + kBlockRows - 1) / kBlockRows),
                               static_cast<unsigned int>(s.hq), static_cast<unsigned int>(s.batch));
-            hipLaunchKernelGGL((attention_dq_kernel<T, DP>), q_grid, dim3(kThreads), 0, stream, pq);
+            if (wide_path(s)) {
+                pq.lse = lse2;
+                hipLaunchKernelGGL((attention_dq_wide_kernel<T>), q_grid, dim3(kThreads), 0, stream, pq);
+            } else {
+                hipLaunchKernelGGL((attention_dq_kernel<T, DP>), q_grid, dim3(kThreads), 0, stream, pq);
+            }
             CGPTX_LAUNCH_CHECK();
             Params pk = p;
             pk.out0 = dk;
             pk.out1 = dv;
-            const dim3 k_grid(static_cast<unsigned int>((s.ks + kBlockRows - 1) / kBlockRows),
-                              static_cast<unsigned int>(s.hkv), static_cast<unsigned int>(s.batch));
-            hipLaunchKernelGGL((attention_dkv_kernel<T, DP>), k_grid, dim3(kThreads), 0, stream, pk);
+            const unsigned int key_blocks = static_cast<unsigned int>((s.ks + kBlockRows - 1) / kBlockRows);
+            if (wide_path(s)) {
+                pk.lse = lse2;
+                auto kernel = attention_dkv_wide_kernel<T>;
+                static bool configured = false;
+                if (!configured) {
+                    CGPTX_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                                  hipFuncAttributeMaxDynamicSharedMemorySize, kWideDkvSmem));
+                    configured = true;
+                }
+                const dim3 pair_grid((key_blocks + 1) / 2, static_cast<unsigned int>(s.hkv),
+                                     static_cast<unsigned int>(s.batch));
+                hipLaunchKernelGGL(kernel, pair_grid, dim3(kThreads), kWideDkvSmem, stream, pk);
+            } else {
+                const dim3 k_grid(key_blocks, static_cast<unsigned int>(s.hkv), static_cast<unsigned int>(s.batch));
+                hipLaunchKernelGGL((attention_dkv_kernel<T, DP>), k_grid, dim3(kThreads), 0, stream, pk);
+            }
             CGPTX_LAUNCH_CHECK();
             return CGPTX_OK;
         });
@@ -1014,15 +1409,15 @@ extern "C" int cgptx_flash_gqa_attention_backward(void* grad_query, void* grad_k
         return fail(CGPTX_INVALID_ARGUMENT, std::string(name) + ": tensors must be 16-byte aligned");
     auto stream = static_cast<hipStream_t>(stream_);
     // Recompute the output and the log-sum-exp into scratch, then run the LSE path. The scratch
-    // block is laid out [delta | lse | output] so that launch_backward's request for the delta
-    // prefix returns the same base pointer.
+    // block is laid out [delta | LSE·log2 e | lse | output] so that launch_backward's request for
+    // the two-block prefix returns the same base pointer.
     const std::size_t rows = batch * query_sequence * query_heads;
-    const std::size_t stat_bytes = (rows * sizeof(float) + 255) & ~std::size_t{255};
+    const std::size_t stat_bytes = stat_block_bytes(rows);
     const std::size_t out_bytes = rows * head_dim * 2;
     void* mem = nullptr;
-    if (int st = scratch(stream, 2 * stat_bytes + out_bytes, &mem)) return st;
-    auto* lse = reinterpret_cast<float*>(static_cast<char*>(mem) + stat_bytes);
-    void* out = static_cast<char*>(mem) + 2 * stat_bytes;
+    if (int st = scratch(stream, 3 * stat_bytes + out_bytes, &mem)) return st;
+    auto* lse = reinterpret_cast<float*>(static_cast<char*>(mem) + 2 * stat_bytes);
+    void* out = static_cast<char*>(mem) + 3 * stat_bytes;
     Params p = make_params(s);
     p.q = query;
     p.k = key;
