@@ -89,6 +89,10 @@ CASES = [
     dict(b=1, qs=33, ks=33, hq=3, hkv=3, d=24),                        # head_dim below the tile width
     dict(b=3, qs=1, ks=1, hq=2, hkv=1, d=128),                         # a single token
     dict(b=1, qs=130, ks=130, hq=4, hkv=1, d=128, scale=0.05),
+    dict(b=1, qs=300, ks=300, hq=4, hkv=2, d=96),                      # padded columns on the 65..128 path, 3 key blocks
+    dict(b=1, qs=100, ks=260, hq=2, hkv=1, d=128, causal=False),       # non-causal on the 65..128 path, qs != ks
+    dict(b=1, qs=90, ks=150, hq=4, hkv=2, d=72, off=60, scale=0.3),    # offset on the 65..128 path
+    dict(b=2, qs=520, ks=520, hq=2, hkv=2, d=128),                     # 5 key blocks: pairs (0,4), (1,3) and 2 alone
 ]
 
 
