@@ -10,21 +10,21 @@
 //
 // Design
 //   * 256 threads = 4 wavefronts in a 2x2 grid; a block owns a BM x BN tile of C
-//     and walks K in steps of 64. Each wavefront owns (BM/2) x (BN/2) and issues
+//     and walks K in steps of 32. Each wavefront owns (BM/2) x (BN/2) and issues
 //     v_mfma_f32_32x32x16 (bf16 or f16), so every LDS fragment read feeds
 //     (BM/64)·(BN/64) MFMAs.
-//   * A k-contiguous operand is staged in LDS with a row stride of 72 elements
-//     (144 B): the rows a ds_read_b128 fragment read touches then fall in distinct
-//     bank groups.
-//   * Operands that are not k-contiguous in memory (dX's weight, both dW
-//     operands) are copied to LDS as they are (coalesced 128-bit loads and
-//     stores) and transposed by the LDS read itself (ds_read_b64_tr_b16): no
-//     separate transpose pass over HBM, no VALU shuffles, no 16-bit LDS accesses.
-//   * The K loop is a software pipeline with one barrier per K step whose issue
-//     order is pinned with sched_group_barrier: LDS fragment reads, the LDS
-//     stores of the next tile and the global loads of the tile after it are
-//     spread between the MFMAs they overlap with, and the loop has no
-//     data-dependent branch (edges are clamped, not predicated).
+//   * Operand tiles go global -> LDS with buffer_load ... lds (no staging registers, no
+//     LDS stores, one loop-invariant per-lane offset) into a ring of five LDS stages:
+//     one being multiplied, up to three K tiles in flight, one being refilled. LDS rows
+//     cannot be padded that way; a chunk swizzle keeps the fragment reads conflict-free.
+//   * Operands that are not k-contiguous in memory (dX's weight, both dW operands) sit
+//     in LDS as they are in memory and are transposed by the LDS read itself
+//     (ds_read_b64_tr_b16): no transpose pass over HBM, no VALU shuffles.
+//   * The K loop is a software pipeline with one barrier per K step whose issue order is
+//     pinned with sched_group_barrier: fragment reads are spread between the MFMAs they
+//     overlap with, the wait for the next K tile sits in the middle of the step, and the
+//     loop has no data-dependent branch (edges are clamped or zero-filled by the
+//     buffer range check, never predicated).
 //   * MFMA is issued as (B-fragment, A-fragment), so a lane ends up holding four
 //     consecutive n for one m per accumulator group; the finished tile is staged in
 //     LDS as fp32 and written out row by row (512 contiguous bytes per wavefront
@@ -37,7 +37,7 @@
 //     fp32 partial tiles go to scratch and a second kernel adds them in slice order
 //     (deterministic), applying accumulate and the dtype conversion.
 //
-// Shapes the MFMA path does not cover (K not a multiple of 64, leading dimensions
+// Shapes the MFMA path does not cover (K not a multiple of 32, leading dimensions
 // or pointers not 16-byte aligned, fp32 storage) run on a plain LDS-tiled fp32
 // kernel with the same semantics.
 #include "gemm.hpp"
@@ -51,8 +51,9 @@ namespace cgptx {
 namespace {
 
 constexpr int kThreads = 256;
-constexpr int kBK = 64;          // K step per LDS tile
-constexpr int kLdsStride = 72;   // elements per LDS row (64 + 8 padding)
+constexpr int kWaves = kThreads / kWave;
+constexpr int kBK = 32;          // K step per LDS stage
+constexpr int kStages = 5;       // LDS stages: one being multiplied, up to three in flight, one being refilled
 constexpr int kXcds = 8;
 constexpr int kGroupRows = 8;    // tile-rows per L2 locality group
 
@@ -91,7 +92,7 @@ struct KernelArgs {
 };
 
 // Instruction classes of __builtin_amdgcn_sched_group_barrier.
-constexpr int kSchedMfma = 0x008, kSchedVmemRead = 0x020, kSchedDsRead = 0x100, kSchedDsWrite = 0x200;
+constexpr int kSchedMfma = 0x008, kSchedDsRead = 0x100;
 
 template <int MASK, int COUNT>
 __device__ __forceinline__ void sched_group() {
@@ -109,87 +110,139 @@ __device__ __forceinline__ void sched_interleave() {
     }
 }
 
-// ---- operand stored [ROWS, K] (k-contiguous): ROWS x 64 slab, LDS rows of 72 elements ---------
+// s_waitcnt immediate that waits until at most `count` vector-memory operations are outstanding
+// (and for nothing else).
+constexpr int vmcnt_immediate(int count) { return (count & 15) | ((count >> 4) << 14) | 0x0F70; }
+
+// Buffer descriptor (raw buffer, range-checked) over `bytes` bytes starting at base.
+__device__ __forceinline__ u32x4 make_rsrc(const void* base, long bytes) {
+    const unsigned long address = reinterpret_cast<unsigned long>(base);
+    const long limit = 0xFFFFFFFFl;
+    u32x4 words;
+    words[0] = static_cast<unsigned int>(address);
+    words[1] = static_cast<unsigned int>(address >> 32) & 0xFFFFu;  // stride 0
+    words[2] = static_cast<unsigned int>(bytes < limit ? bytes : limit);
+    words[3] = 0x00020000u;
+    return words;
+}
+
+// One wavefront-wide 16-byte-per-lane load from a buffer straight into LDS: lane l's bytes land at
+// lds_address + 16 l. Written as assembly on purpose: the compiler would order every later LDS
+// read after *all* outstanding loads of this kind (vmcnt(0)), which defeats keeping several K tiles
+// in flight; the kernel counts its loads itself (vmcnt_immediate). M0 is used by nothing else here.
+__device__ __forceinline__ void load_to_lds(const u32x4& rsrc, unsigned int lds_address, int voffset,
+                                            unsigned int soffset) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :
+                 : "s"(lds_address), "v"(voffset), "s"(rsrc), "s"(soffset));
+}
+
+template <typename T>
+__device__ __forceinline__ unsigned int lds_address_of(const T* p) {
+    return static_cast<unsigned int>(reinterpret_cast<unsigned long>((__attribute__((address_space(3))) const T*)(p)));
+}
+
+// Operand tiles travel global -> LDS with buffer_load ... lds: a wavefront-wide load drops
+// 64 x 16 B contiguously into LDS, no staging registers and no LDS stores, and the only per-lane
+// address is a loop-invariant byte offset (the K position is a scalar offset). LDS rows therefore
+// cannot be padded; bank conflicts are avoided by storing 16-byte chunk c of a row at chunk
+// position c ^ swizzle(row) — the lane that owns an LDS slot fetches the matching global chunk.
+
+// ---- operand stored [ROWS, K] (k-contiguous): ROWS x 32 slab, LDS rows of 64 B ----------------
+// One load instruction covers 16 rows; wavefront w issues the loads of row groups w, w+4, ...
+// swizzle(row) = (row/4)%4: the 16 rows a quarter-wavefront reads with ds_read_b128 then hit the
+// 16 different 16-byte positions of a 256-byte bank period.
 template <typename T, int ROWS>
 struct KTile {
     using frag_t = typename Mfma<T>::frag;
-    static constexpr int kLoads = ROWS * (kBK / 8) / kThreads;  // 128-bit chunks per thread
-    static constexpr int kElems = ROWS * kLdsStride;
-    static constexpr int kFragReads = 1;  // LDS instructions per fragment
-    u32x4 regs[kLoads];
+    static constexpr int kElems = ROWS * kBK;
+    static constexpr int kLoads = ROWS / 16 / kWaves;  // load instructions per wavefront and tile
+    static constexpr int kFragReads = 1;               // LDS instructions per fragment
+    static constexpr int kOffsets = 2;                 // per-lane fragment offsets: one per K sub-step
 
-    __device__ __forceinline__ void load(const T* base, long ld, int row0, int row_limit, int k0) {
+    u32x4 rsrc;
+    int voffset;
+    unsigned int group_bytes;  // 16 rows further in global memory
+
+    // base: element (row0, 0) of the operand; rows past rows_left only feed C rows that are never
+    // stored (they read zeros or whatever follows, never out of the allocation's last row).
+    __device__ __forceinline__ void init(const T* base, long ld, int rows_left, int k_total) {
+        const int lane = threadIdx.x & (kWave - 1);
+        rsrc = make_rsrc(base, (static_cast<long>(rows_left - 1) * ld + k_total) * static_cast<long>(sizeof(T)));
+        const int row = lane >> 2;
+        voffset = static_cast<int>(row * ld * sizeof(T)) + (((lane & 3) ^ ((row >> 2) & 3)) * 16);
+        group_bytes = static_cast<unsigned int>(16 * ld * sizeof(T));
+    }
+    __device__ __forceinline__ void issue(T* tile, int k0, int wave) const {
 #pragma unroll
         for (int i = 0; i < kLoads; ++i) {
-            const int chunk = threadIdx.x + i * kThreads;
-            const int row = chunk >> 3, kc = chunk & 7;
-            // Rows past the edge are clamped to the last valid row instead of being predicated: they
-            // only feed C rows/columns that are never stored, and a branch-free loop lets the loads
-            // stay in flight across the MFMAs of the current tile.
-            const int safe = min(row0 + row, row_limit - 1);
-            regs[i] = *reinterpret_cast<const u32x4*>(base + static_cast<long>(safe) * ld + k0 + kc * 8);
+            const int group = i * kWaves + wave;
+            load_to_lds(rsrc, lds_address_of(tile + group * 16 * kBK), voffset,
+                        group * group_bytes + k0 * static_cast<unsigned int>(sizeof(T)));
         }
     }
-    __device__ __forceinline__ void store(T* lds) const {
-#pragma unroll
-        for (int i = 0; i < kLoads; ++i) {
-            const int chunk = threadIdx.x + i * kThreads;
-            const int row = chunk >> 3, kc = chunk & 7;
-            *reinterpret_cast<u32x4*>(lds + row * kLdsStride + kc * 8) = regs[i];
-        }
+    // Element offset of the lane's fragment within a 32-row block, K sub-step kk: row lane%32,
+    // k = 16 kk + 8 (lane/32) .. +7.
+    __device__ __forceinline__ static int lane_offset(int lane, int /*block0*/, int kk) {
+        return (lane & 31) * kBK + (((kk * 2 + (lane >> 5)) ^ ((lane >> 2) & 3)) * 8);
     }
-    // Per-lane part of a fragment address: row lane%32 of a 32-row block, k group lane/32.
-    __device__ __forceinline__ static int lane_offset(int lane) { return (lane & 31) * kLdsStride + (lane >> 5) * 8; }
-    // Fragment of rows block0 .. block0+31, K sub-step kk (16 values of k, 8 per lane).
-    __device__ __forceinline__ static frag_t frag(const T* lane_base, int block0, int kk) {
-        return *reinterpret_cast<const frag_t*>(lane_base + block0 * kLdsStride + kk * 16);
+    __device__ __forceinline__ static frag_t frag(const T* tile, int block0, int offset) {
+        return *reinterpret_cast<const frag_t*>(tile + block0 * kBK + offset);
     }
 };
 
-// ---- operand stored [K, COLS] (n-contiguous): 64 x COLS slab kept in that order in LDS ---------
+// ---- operand stored [K, COLS] (n-contiguous): 32 x COLS slab kept in that order in LDS ---------
 // The transpose happens on the way out of LDS: ds_read_b64_tr_b16 hands lane n of a 16-lane group
 // the four k-values of column n from a 4(k) x 16(n) block, so two of them build the 8-k fragment of
-// one column. Rows are padded by 32 elements (64 B): the four k rows that 32 lanes read then start
-// 16 banks apart and the read is conflict-free; the row-contiguous 128-bit stores are anyway.
+// one column. swizzle(k row) = 4*(row%4) on the chunk index: the four k rows that 32 lanes read sit
+// in four different 64-byte windows of the 256-byte bank period.
 template <typename T, int COLS>
 struct NTile {
     using frag_t = typename Mfma<T>::frag;
-    static constexpr int kStride = COLS + 32;
     static constexpr int kChunksPerRow = COLS / 8;
-    static constexpr int kLoads = kBK * kChunksPerRow / kThreads;
-    static constexpr int kElems = kBK * kStride;
+    static constexpr int kRowsPerLoad = 64 / kChunksPerRow;  // k rows one load instruction covers (2 or 4)
+    static constexpr int kElems = kBK * COLS;
+    static constexpr int kLoads = kBK / kRowsPerLoad / kWaves;
     static constexpr int kFragReads = 2;
-    u32x4 regs[kLoads];
+    static constexpr int kOffsets = COLS / 64;  // per-lane fragment offsets: one per 32-column block of a wavefront
 
-    __device__ __forceinline__ void load(const T* base, long ld, int col0, int col_limit, int k0) {
-#pragma unroll
-        for (int i = 0; i < kLoads; ++i) {
-            const int chunk = threadIdx.x + i * kThreads;
-            const int row = chunk / kChunksPerRow, cc = chunk % kChunksPerRow;
-            // Column blocks past the edge are clamped (see KTile::load); col_limit is a multiple of 8.
-            const int safe_col = min(col0 + cc * 8, col_limit - 8);
-            regs[i] = *reinterpret_cast<const u32x4*>(base + static_cast<long>(k0 + row) * ld + safe_col);
-        }
+    u32x4 rsrc;
+    int voffset;
+    unsigned int group_bytes;  // kRowsPerLoad k rows further in global memory
+
+    // base: element (0, col0) of the operand. Column chunks past cols_left are clamped to the last
+    // valid chunk: they only feed C columns that are never stored.
+    __device__ __forceinline__ void init(const T* base, long ld, int cols_left, int k_total, int wave) {
+        const int lane = threadIdx.x & (kWave - 1);
+        rsrc = make_rsrc(base, (static_cast<long>(k_total - 1) * ld + cols_left) * static_cast<long>(sizeof(T)));
+        const int row = lane / kChunksPerRow;                  // within the instruction's rows
+        const int k_row = (wave * kRowsPerLoad + row) & 3;     // low bits of the tile row (groups step by 4*kRowsPerLoad)
+        const int chunk = min((lane % kChunksPerRow) ^ (k_row << 2), cols_left / 8 - 1);
+        voffset = static_cast<int>(row * ld * sizeof(T)) + chunk * 16;
+        group_bytes = static_cast<unsigned int>(kRowsPerLoad * ld * sizeof(T));
     }
-    __device__ __forceinline__ void store(T* lds) const {
+    __device__ __forceinline__ void issue(T* tile, int k0, int wave) const {
 #pragma unroll
         for (int i = 0; i < kLoads; ++i) {
-            const int chunk = threadIdx.x + i * kThreads;
-            const int row = chunk / kChunksPerRow, cc = chunk % kChunksPerRow;
-            *reinterpret_cast<u32x4*>(lds + row * kStride + cc * 8) = regs[i];
+            const int group = i * kWaves + wave;
+            load_to_lds(rsrc, lds_address_of(tile + group * kRowsPerLoad * COLS), voffset,
+                        (group + k0 / kRowsPerLoad) * group_bytes);
         }
     }
     // Lane i of a 16-lane group addresses k row i/4, columns 4*(i%4) .. +3 of the group's 4 x 16
     // block; groups 0/1 take columns 0-15/16-31 of the fragment, lanes 32-63 the k values 8-15.
-    __device__ __forceinline__ static int lane_offset(int lane) {
-        return ((lane >> 5) * 8 + ((lane & 15) >> 2)) * kStride + ((lane >> 4) & 1) * 16 + (lane & 3) * 4;
+    // The offset is for K sub-step 0 and the first of the two reads; block0 is a multiple of 32.
+    __device__ __forceinline__ static int lane_offset(int lane, int block0, int /*kk*/) {
+        const int k_row = (lane >> 5) * 8 + ((lane & 15) >> 2);
+        const int chunk = ((block0 / 8) ^ ((k_row & 3) << 2)) + ((lane >> 4) & 1) * 2 + ((lane & 3) >> 1);
+        return k_row * COLS + chunk * 8 + (lane & 1) * 4;
     }
-    __device__ __forceinline__ static frag_t frag(const T* lane_base, int block0, int kk) {
+    __device__ __forceinline__ static frag_t frag(const T* tile, int kk, int offset) {
         using s16x4 = vec_t<short, 4>;
         using lds_ptr = __attribute__((address_space(3))) s16x4*;
-        const T* q = lane_base + kk * 16 * kStride + block0;
+        const T* q = tile + kk * 16 * COLS + offset;
         const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(q));
-        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(q + 4 * kStride));
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(q + 4 * COLS));
         vec_t<short, 8> both;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
@@ -205,7 +258,7 @@ struct TileLayout {
     using ATile = std::conditional_t<A_K, KTile<T, BM>, NTile<T, BM>>;
     using BTile = std::conditional_t<B_K, KTile<T, BN>, NTile<T, BN>>;
     static constexpr int kStage = ATile::kElems + BTile::kElems;  // elements per LDS stage: [A | B]
-    static constexpr int kSmemBytes = 2 * kStage * static_cast<int>(sizeof(T));
+    static constexpr int kSmemBytes = kStages * kStage * static_cast<int>(sizeof(T));
 };
 
 template <typename T, int BM, int BN, bool A_K, bool B_K, bool SPLIT>
@@ -216,10 +269,9 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
     using BTile = typename Layout::BTile;
     constexpr int WM = BM / 2, WN = BN / 2;
     constexpr int TM = WM / 32, TN = WN / 32;
-    extern __shared__ __align__(16) unsigned char smem_raw[];
+    extern __shared__ __align__(1024) unsigned char smem_raw[];
     T* smem = reinterpret_cast<T*>(smem_raw);
-    // Stage s holds [A tile | B tile] at smem + s * kStage. Offsets are added to the one shared base
-    // so that every access is provably an LDS access (ds_read/ds_write, counted by lgkmcnt only).
+    // Stage s holds [A tile | B tile] at smem + s * kStage.
     constexpr int kStage = Layout::kStage;
     constexpr int kATile = ATile::kElems;
 
@@ -242,27 +294,30 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
     const int kt_end = min(k_tiles_total, kt_begin + p.k_tiles_per_slice);
     const int count = kt_end - kt_begin;
 
-    const T* A = static_cast<const T*>(p.a);
-    const T* B = static_cast<const T*>(p.b);
-
-    ATile a_regs;
-    BTile b_regs;
-    // Tiles past the end of the slice reload the last one (it is stored but never multiplied), which
-    // keeps the K loop free of data-dependent branches.
-    auto load_tiles = [&](int kt) {
-        const int k0 = min(kt, kt_end - 1) * kBK;
-        a_regs.load(A, p.lda, m0, p.m, k0);
-        b_regs.load(B, p.ldb, n0, p.n, k0);
-    };
-    auto store_tiles = [&](int buf) {
-        a_regs.store(smem + buf * kStage);
-        b_regs.store(smem + buf * kStage + kATile);
-    };
-
     const int lane = threadIdx.x & (kWave - 1);
-    const int wave = threadIdx.x / kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const int wm = wave >> 1, wn = wave & 1;
-    const int a_lane = ATile::lane_offset(lane), b_lane = BTile::lane_offset(lane);
+
+    ATile a_src;
+    BTile b_src;
+    if constexpr (A_K) a_src.init(static_cast<const T*>(p.a) + static_cast<long>(m0) * p.lda, p.lda, p.m - m0, p.k);
+    else a_src.init(static_cast<const T*>(p.a) + m0, p.lda, p.m - m0, p.k, wave);
+    if constexpr (B_K) b_src.init(static_cast<const T*>(p.b) + static_cast<long>(n0) * p.ldb, p.ldb, p.n - n0, p.k);
+    else b_src.init(static_cast<const T*>(p.b) + n0, p.ldb, p.n - n0, p.k, wave);
+    // K tiles past the end of the slice reload the last one (never multiplied): the loop stays free
+    // of data-dependent branches and every wavefront always has the same number of loads in flight.
+    auto issue = [&](int t, int stage) {
+        const int k0 = min(kt_begin + t, kt_end - 1) * kBK;
+        a_src.issue(smem + stage * kStage, k0, wave);
+        b_src.issue(smem + stage * kStage + kATile, k0, wave);
+    };
+    constexpr int kTileLoads = ATile::kLoads + BTile::kLoads;  // per wavefront and K tile
+
+    int a_off[ATile::kOffsets], b_off[BTile::kOffsets];
+#pragma unroll
+    for (int i = 0; i < ATile::kOffsets; ++i) a_off[i] = ATile::lane_offset(lane, wm * WM + i * 32, i);
+#pragma unroll
+    for (int j = 0; j < BTile::kOffsets; ++j) b_off[j] = BTile::lane_offset(lane, wn * WN + j * 32, j);
 
     acc_t acc[TM][TN];
 #pragma unroll
@@ -271,13 +326,19 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
         for (int j = 0; j < TN; ++j) acc[i][j] = acc_t(0.0f);
 
     frag_t af[2][TM], bf[2][TN];
-    auto read_frags = [&](int set, int buf, int kk) {
-        const T* as = smem + buf * kStage + a_lane;
-        const T* bs = smem + buf * kStage + kATile + b_lane;
+    auto read_frags = [&](int set, int stage, int kk) {
+        const T* as = smem + stage * kStage;
+        const T* bs = as + kATile;
 #pragma unroll
-        for (int i = 0; i < TM; ++i) af[set][i] = ATile::frag(as, wm * WM + i * 32, kk);
+        for (int i = 0; i < TM; ++i) {
+            if constexpr (A_K) af[set][i] = ATile::frag(as, wm * WM + i * 32, a_off[kk]);
+            else af[set][i] = ATile::frag(as, kk, a_off[i]);
+        }
 #pragma unroll
-        for (int j = 0; j < TN; ++j) bf[set][j] = BTile::frag(bs, wn * WN + j * 32, kk);
+        for (int j = 0; j < TN; ++j) {
+            if constexpr (B_K) bf[set][j] = BTile::frag(bs, wn * WN + j * 32, b_off[kk]);
+            else bf[set][j] = BTile::frag(bs, kk, b_off[j]);
+        }
     };
     auto multiply = [&](int set) {
 #pragma unroll
@@ -286,46 +347,42 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
             for (int j = 0; j < TN; ++j) acc[i][j] = Mfma<T>::run(bf[set][j], af[set][i], acc[i][j]);
     };
 
-    // Software pipeline over K tiles t = 0 .. count-1 (tile t lives in LDS stage t%2), four K
-    // sub-steps of 16 per tile:
-    //   sub-steps 0,1  MFMAs ‖ LDS reads of the next sub-step's fragments
-    //   sub-step  2    MFMAs ‖ fragments of sub-step 3 ‖ registers of tile t+1 -> stage (t+1)%2
-    //   barrier        tile t+1 visible; nobody reads stage t%2 any more
-    //   sub-step  3    MFMAs ‖ fragments of tile t+1, sub-step 0 ‖ global loads of tile t+2
-    // so LDS latency, the barrier and most of the global latency sit in the shadow of MFMAs.
+    // Software pipeline over K tiles t = 0 .. count-1 (tile t lives in LDS stage t % kStages; tiles
+    // t+1 .. t+kStages-2 are in flight or landed), two K sub-steps of 16 per tile:
+    //   sub-step 0  MFMAs ‖ LDS reads of sub-step 1's fragments
+    //   wait        this wavefront's loads of tile t+1 have landed; barrier: everybody's have, and
+    //               nobody reads stage (t-1) % kStages any more
+    //   sub-step 1  MFMAs ‖ loads of tile t+kStages-1 into that stage ‖ fragments of tile t+1, sub-step 0
+    // so LDS latency and kStages-2 K tiles of global latency sit in the shadow of MFMAs.
     constexpr int kMfmas = TM * TN;
     constexpr int kFragReads = TM * ATile::kFragReads + TN * BTile::kFragReads;
-    constexpr int kTileLoads = ATile::kLoads + BTile::kLoads;
-    static_assert(kBK == 64, "the pipeline below is written for four K sub-steps");
+    static_assert(kBK == 32, "the pipeline below is written for two K sub-steps");
     if (count > 0) {
-        load_tiles(kt_begin);
-        store_tiles(0);
-        load_tiles(kt_begin + 1);
+#pragma unroll
+        for (int t = 0; t < kStages - 1; ++t) issue(t, t);
+        __builtin_amdgcn_s_waitcnt(vmcnt_immediate((kStages - 2) * kTileLoads));
         __syncthreads();
         read_frags(0, 0, 0);
+        int stage = 0;       // of tile t
+        int free_stage = kStages - 1;  // of tile t-1, refilled with tile t+kStages-1
         for (int t = 0; t < count; ++t) {
-            const int buf = t & 1;
-            read_frags(1, buf, 1);
-            multiply(0);
-            read_frags(0, buf, 2);
-            multiply(1);
-            read_frags(1, buf, 3);
-            store_tiles(buf ^ 1);
+            const int next_stage = stage + 1 == kStages ? 0 : stage + 1;
+            read_frags(1, stage, 1);
             multiply(0);
             sched_interleave<kMfmas, kSchedDsRead, kFragReads, 0, 0>();
-            sched_interleave<kMfmas, kSchedDsRead, kFragReads, 0, 0>();
-            // LDS stores may not move above the (possibly aliasing) fragment reads issued before them:
-            // reads go with the first MFMAs of the sub-step, stores with the rest.
-            sched_interleave<kMfmas / 2, kSchedDsRead, kFragReads, 0, 0>();
-            sched_interleave<kMfmas - kMfmas / 2, kSchedDsWrite, kTileLoads, 0, 0>();
             __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_s_waitcnt(vmcnt_immediate((kStages - 3) * kTileLoads));
             __syncthreads();
-            read_frags(0, buf ^ 1, 0);
-            load_tiles(kt_begin + t + 2);
+            issue(t + kStages - 1, free_stage);
+            read_frags(0, next_stage, 0);
             multiply(1);
-            sched_interleave<kMfmas, kSchedDsRead, kFragReads, kSchedVmemRead, kTileLoads>();
+            sched_interleave<kMfmas, kSchedDsRead, kFragReads, 0, 0>();
+            __builtin_amdgcn_sched_barrier(0);
+            free_stage = stage;
+            stage = next_stage;
         }
     }
+    __builtin_amdgcn_s_waitcnt(vmcnt_immediate(0));  // the staging below reuses LDS that loads may still target
     __syncthreads();
 
     // Epilogue. acc[i][j][4g+e] holds C[m, n] with m = lane%32, n = 8g + 4*(lane/32) + e. The tile
@@ -519,8 +576,8 @@ int run_config(const GemmArgs& g, KernelArgs p, hipStream_t stream) {
     const long tiles = static_cast<long>(p.tiles_m) * p.tiles_n;
     const long want_blocks = static_cast<long>(compute_units()) * (BM == 256 ? 1 : 2);
     int slices = 1;
-    if (!g.no_split && tiles < want_blocks && k_tiles >= 16) {
-        slices = static_cast<int>(std::min<long>((want_blocks + tiles - 1) / tiles, k_tiles / 8));
+    if (!g.no_split && tiles < want_blocks && k_tiles >= 32) {
+        slices = static_cast<int>(std::min<long>((want_blocks + tiles - 1) / tiles, k_tiles / 16));
         if (slices < 1) slices = 1;
     }
     p.k_tiles_per_slice = (k_tiles + slices - 1) / slices;
@@ -538,6 +595,15 @@ int run_config(const GemmArgs& g, KernelArgs p, hipStream_t stream) {
                        p.accumulate, p.c_f32);
     CGPTX_LAUNCH_CHECK();
     return CGPTX_OK;
+}
+
+// The streamed loads address an operand relative to the block's tile origin with 32-bit byte
+// offsets: a tile's rows (k-contiguous operand) or the whole K extent (n-contiguous operand).
+bool offsets_fit_32bit(const GemmArgs& g, std::size_t elem) {
+    constexpr std::size_t limit = (std::size_t{1} << 32) - (std::size_t{1} << 20);
+    const std::size_t a_span = g.a_k_contiguous ? (256 * g.lda + g.k) * elem : (g.k * g.lda + 256) * elem;
+    const std::size_t b_span = g.b_k_contiguous ? (256 * g.ldb + g.k) * elem : (g.k * g.ldb + 256) * elem;
+    return a_span < limit && b_span < limit;
 }
 
 template <typename T>
@@ -562,7 +628,7 @@ int run_typed(const GemmArgs& g, hipStream_t stream) {
         fast = g.k % kBK == 0 && g.lda % 8 == 0 && g.ldb % 8 == 0 && g.n % 8 == 0 && g.m % 8 == 0 &&
                is_aligned16(g.a) && is_aligned16(g.b) && (g.ldc * c_elem) % 16 == 0 && is_aligned16(g.c) &&
                (g.bias == nullptr || (reinterpret_cast<std::uintptr_t>(g.bias) & 7u) == 0) &&
-               !(!g.a_k_contiguous && g.b_k_contiguous);
+               !(!g.a_k_contiguous && g.b_k_contiguous) && offsets_fit_32bit(g, sizeof(T));
     }
     if (!fast) {
         const dim3 grid(static_cast<unsigned int>((g.n + kGenericTile - 1) / kGenericTile),
