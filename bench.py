@@ -46,12 +46,12 @@ def op_work(cfg, batch, seq, loss_mode):
         "attn_bwd": ("mfma", 5 * attention * L),
         "dense_ce": ("hbm", 2.0 * N * V * e),
         "rmsnorm_fwd": ("hbm", (2 * N * H * 2 + N * (QW + KW) * 2) * e * L + 2 * N * H * e),
-        "rmsnorm_bwd": ("hbm", (2 * N * H * 3 + N * (QW + KW) * 3) * e * L + 3 * N * H * e),
+        # the two hidden-wide norms of a block also read the residual gradient they are added to
+        "rmsnorm_bwd": ("hbm", (2 * N * H * 4 + N * (QW + KW) * 3) * e * L + 3 * N * H * e),
         "rope_fwd": ("hbm", N * (QW + KW) * 2 * e * L),
         "rope_bwd": ("hbm", N * (QW + KW) * 2 * e * L),
         "swiglu_fwd": ("hbm", N * I * 3 * e * L),
         "swiglu_bwd": ("hbm", N * I * 5 * e * L),
-        "add": ("hbm", N * H * 3 * e * 4 * L),
         "embedding_fwd": ("hbm", N * H * 2 * e),
         "embedding_bwd": ("hbm", N * H * 3 * e),
     }

@@ -99,6 +99,13 @@ int dispatch_dtype(int dtype, Fn&& fn) {
     }
 }
 
+// ---- fused variants used by the composed train step --------------------------
+// rmsnorm backward with grad_input = (norm gradient) + residual; residual may be null or alias
+// grad_input. Same validation and results as cgptx_rmsnorm_backward otherwise.
+int rmsnorm_backward_residual(void* grad_input, void* grad_weight, const void* grad_output, const void* input,
+                              const void* weight, const void* residual, std::size_t rows, std::size_t hidden,
+                              float epsilon, int dtype, hipStream_t stream);
+
 // ---- scratch arena ----------------------------------------------------------
 // Returns `bytes` of device scratch bound to (current device, stream), 256-byte
 // aligned. Grows by reallocation on eager calls; refuses to grow during capture.

@@ -62,9 +62,10 @@ extern "C" int cgptx_cut_cross_entropy_forward_backward(float* loss, void* input
         return fail(CGPTX_OVERFLOW, std::string(name) + ": dimension exceeds int range");
     auto stream = static_cast<hipStream_t>(stream_);
     const std::size_t elem = dtype_size(dtype);
-    // Chunk so that the logits scratch stays near 512 MiB whatever the number of rows, while each
-    // chunk still gives the three contractions enough tiles to fill the chip (8192 rows at V=32000).
-    std::size_t chunk = (std::size_t{512} << 20) / (vocab * elem);
+    // Chunk so that the logits scratch stays near 1 GiB whatever the number of rows, while each
+    // chunk still gives the three contractions enough 256x256 tiles to fill the chip (16384 rows at
+    // V=32000: the input-gradient contraction then has 64 x 4 tiles, one per CU).
+    std::size_t chunk = (std::size_t{1} << 30) / (vocab * elem);
     chunk = std::max<std::size_t>(256, chunk / 256 * 256);
     chunk = std::min(chunk, rows);
     const std::size_t loss_bytes = (rows * sizeof(float) + 255) & ~std::size_t{255};

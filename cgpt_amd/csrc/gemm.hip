@@ -83,8 +83,9 @@ struct KernelArgs {
     const void* b;
     void* c;            // T* (or float* when c_f32), or float partials when split
     const void* bias;
+    const void* residual;  // T*, row stride ldr, or null
     int m, n, k;
-    long lda, ldb, ldc;
+    long lda, ldb, ldc, ldr;
     int tiles_m, tiles_n;
     int k_tiles_per_slice;  // K tiles (of 64) handled by one blockIdx.y
     int accumulate;
@@ -432,6 +433,8 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
                 *reinterpret_cast<vec_t<float, 4>*>(out) = v;
             } else {
                 if (p.bias != nullptr) v += vec_to_f32<T, 4>(load_vec<T, 4>(static_cast<const T*>(p.bias) + n));
+                if (p.residual != nullptr)
+                    v += vec_to_f32<T, 4>(load_vec<T, 4>(static_cast<const T*>(p.residual) + static_cast<long>(m) * p.ldr + n));
                 if (p.c_f32) {
                     float* out = static_cast<float*>(p.c) + static_cast<long>(m) * p.ldc + n;
                     if (p.accumulate) v += *reinterpret_cast<const vec_t<float, 4>*>(out);
@@ -520,6 +523,7 @@ __global__ __launch_bounds__(kGenericTile* kGenericTile / 4) void gemm_generic_k
             if (m >= p.m || n >= p.n) continue;
             float v = acc[i][j];
             if (p.bias != nullptr) v += to_f32(static_cast<const T*>(p.bias)[n]);
+            if (p.residual != nullptr) v += to_f32(static_cast<const T*>(p.residual)[static_cast<long>(m) * p.ldr + n]);
             if (p.c_f32) {
                 float* out = static_cast<float*>(p.c) + m * p.ldc + n;
                 *out = p.accumulate ? v + *out : v;
@@ -576,7 +580,7 @@ int run_config(const GemmArgs& g, KernelArgs p, hipStream_t stream) {
     const long tiles = static_cast<long>(p.tiles_m) * p.tiles_n;
     const long want_blocks = static_cast<long>(compute_units()) * (BM == 256 ? 1 : 2);
     int slices = 1;
-    if (!g.no_split && tiles < want_blocks && k_tiles >= 32) {
+    if (!g.no_split && g.residual == nullptr && tiles < want_blocks && k_tiles >= 32) {
         slices = static_cast<int>(std::min<long>((want_blocks + tiles - 1) / tiles, k_tiles / 16));
         if (slices < 1) slices = 1;
     }
@@ -613,6 +617,8 @@ int run_typed(const GemmArgs& g, hipStream_t stream) {
     p.b = g.b;
     p.c = g.c;
     p.bias = g.bias;
+    p.residual = g.residual;
+    p.ldr = static_cast<long>(g.ldr);
     p.m = static_cast<int>(g.m);
     p.n = static_cast<int>(g.n);
     p.k = static_cast<int>(g.k);
@@ -628,6 +634,7 @@ int run_typed(const GemmArgs& g, hipStream_t stream) {
         fast = g.k % kBK == 0 && g.lda % 8 == 0 && g.ldb % 8 == 0 && g.n % 8 == 0 && g.m % 8 == 0 &&
                is_aligned16(g.a) && is_aligned16(g.b) && (g.ldc * c_elem) % 16 == 0 && is_aligned16(g.c) &&
                (g.bias == nullptr || (reinterpret_cast<std::uintptr_t>(g.bias) & 7u) == 0) &&
+               (g.residual == nullptr || ((reinterpret_cast<std::uintptr_t>(g.residual) & 7u) == 0 && g.ldr % 4 == 0)) &&
                !(!g.a_k_contiguous && g.b_k_contiguous) && offsets_fit_32bit(g, sizeof(T));
     }
     if (!fast) {

@@ -9,15 +9,17 @@ namespace cgptx {
 //   a_k_contiguous: A is stored [M, K] (row stride lda) — otherwise [K, M].
 //   b_k_contiguous: B is stored [N, K] (row stride ldb) — otherwise [K, N].
 // C is row-major [M, N] with row stride ldc, in the storage dtype of A and B
-// (or fp32 when c_is_f32). accumulate adds into C. bias (optional, [N], storage
+// (or fp32 when c_is_f32). accumulate adds into C. residual (optional, [M, N], storage dtype, row
+// stride ldr, may be C itself) is added elementwise. bias (optional, [N], storage
 // dtype) is added to every row after the product.
 struct GemmArgs {
     const void* a = nullptr;
     const void* b = nullptr;
     void* c = nullptr;
     const void* bias = nullptr;
+    const void* residual = nullptr;
     std::size_t m = 0, n = 0, k = 0;
-    std::size_t lda = 0, ldb = 0, ldc = 0;
+    std::size_t lda = 0, ldb = 0, ldc = 0, ldr = 0;
     bool a_k_contiguous = true;
     bool b_k_contiguous = true;
     bool accumulate = false;

@@ -39,6 +39,48 @@ __global__ __launch_bounds__(kReduceThreads) void column_partial_reduce_kernel(
 }
 
 
+// First level for many parts: block (x, y) of a (column groups, slices) grid folds the parts of
+// slice y for its 64 columns into second[y, col]; column_partial_reduce_kernel over the `slices`
+// rows of `second` finishes. (A single launch whose last block finishes would need device-scope
+// fences, which cost more here than the second launch.)
+static __global__ __launch_bounds__(kReduceThreads) void column_partial_fold_kernel(float* __restrict__ second,
+                                                                            const float* __restrict__ partial,
+                                                                            int parts, int hidden) {
+    __shared__ float stage[kReduceWaves][kWave];
+    const int lane = threadIdx.x & (kWave - 1);
+    const int slice = threadIdx.x / kWave;
+    const int col = blockIdx.x * kWave + lane;
+    const int slices = gridDim.y;
+    const int chunk = (parts + slices - 1) / slices;
+    const int begin = blockIdx.y * chunk;
+    const int end = begin + chunk < parts ? begin + chunk : parts;
+    float v0 = 0.0f, v1 = 0.0f;
+    if (col < hidden) {
+        int p = begin + slice;
+        for (; p + kReduceWaves < end; p += 2 * kReduceWaves) {
+            v0 += partial[static_cast<std::size_t>(p) * hidden + col];
+            v1 += partial[static_cast<std::size_t>(p + kReduceWaves) * hidden + col];
+        }
+        if (p < end) v0 += partial[static_cast<std::size_t>(p) * hidden + col];
+    }
+    stage[slice][lane] = v0 + v1;
+    __syncthreads();
+    if (slice == 0 && col < hidden) {
+        float v = 0.0f;
+#pragma unroll
+        for (int s = 0; s < kReduceWaves; ++s) v += stage[s][lane];
+        second[static_cast<std::size_t>(blockIdx.y) * hidden + col] = v;
+    }
+}
+
+// Slices for the kernel above: enough blocks to fill the chip, at least sixteen parts each.
+inline int wide_reduce_slices(int parts, int hidden, int units) {
+    const int groups = (hidden + kWave - 1) / kWave;
+    int slices = 2 * units / groups;
+    if (slices > parts / 16) slices = parts / 16;
+    return slices < 1 ? 1 : slices;
+}
+
 // partial[blockIdx.y, col] = Σ over this block's row slice of in[row, col] (fp32).
 template <typename T>
 __global__ __launch_bounds__(kReduceThreads) void column_sum_partial_kernel(float* __restrict__ partial,

@@ -29,9 +29,10 @@ constexpr int kWavesPerBlock = kThreads / kWave;
 // ------------------------------------------------------------------ fast path
 template <typename T, int LPR, int K, bool Backward>
 __global__ __launch_bounds__(kThreads) void rmsnorm_rows_kernel(
-    T* __restrict__ out,            // dx (backward) or y (forward)
+    T* out,                         // dx (backward) or y (forward)
     float* __restrict__ partial,    // [gridDim.x, H] dgamma partials (backward)
     const T* __restrict__ dy,       // backward only
+    const T* residual,              // backward only, optional: added to dx (may be out itself)
     const T* __restrict__ x, const T* __restrict__ w, int rows, int hidden, float inv_hidden, float eps) {
     constexpr int VEC = kVec128<T>;
     constexpr int RPW = kWave / LPR;  // rows per wavefront iteration
@@ -95,7 +96,10 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_rows_kernel(
                     acc[c][e] = fmaf(gv[c][e], xv[c][e] * inv, acc[c][e]);
                 }
                 const int col = (c * LPR + sub) * VEC;
-                if (row_live && live[c]) store_vec<T, VEC>(out + base + col, vec_from_f32<T, VEC>(r));
+                if (row_live && live[c]) {
+                    if (residual != nullptr) r += vec_to_f32<T, VEC>(load_vec<T, VEC>(residual + base + col));
+                    store_vec<T, VEC>(out + base + col, vec_from_f32<T, VEC>(r));
+                }
             }
         } else {
 #pragma unroll
@@ -227,13 +231,13 @@ FastShape pick_fast_shape(int hidden) {
 }
 
 template <typename T, bool Backward>
-int launch_fast(const FastShape shape, T* out, float* partial, const T* dy, const T* x, const T* w, int rows,
-                int hidden, float eps, int blocks, hipStream_t stream) {
+int launch_fast(const FastShape shape, T* out, float* partial, const T* dy, const T* residual, const T* x, const T* w,
+                int rows, int hidden, float eps, int blocks, hipStream_t stream) {
     const float inv_hidden = 1.0f / static_cast<float>(hidden);
 #define CGPTX_RMS_CASE(L, KK)                                                                             \
     if (shape.lpr == L && shape.k == KK) {                                                                \
         hipLaunchKernelGGL((rmsnorm_rows_kernel<T, L, KK, Backward>), dim3(blocks), dim3(kThreads), 0,   \
-                           stream, out, partial, dy, x, w, rows, hidden, inv_hidden, eps);                \
+                           stream, out, partial, dy, residual, x, w, rows, hidden, inv_hidden, eps);                \
         return CGPTX_OK;                                                                                  \
     }
     CGPTX_RMS_CASE(16, 1)
@@ -268,35 +272,45 @@ int validate(const void* a, const void* b, const void* c, std::size_t rows, std:
 }
 
 }  // namespace
-}  // namespace cgptx
 
-extern "C" int cgptx_rmsnorm_backward(void* grad_input, void* grad_weight, const void* grad_output, const void* input,
-                                      const void* weight, size_t rows, size_t hidden, float epsilon, int dtype,
-                                      cgptx_stream stream_) {
-    using namespace cgptx;
+int rmsnorm_backward_residual(void* grad_input, void* grad_weight, const void* grad_output, const void* input,
+                              const void* weight, const void* residual, std::size_t rows, std::size_t hidden,
+                              float epsilon, int dtype, hipStream_t stream) {
     if (int s = validate(grad_input, grad_output, input, rows, hidden, epsilon, dtype, "rmsnorm_backward")) return s;
     if (grad_weight == nullptr || weight == nullptr)
         return fail(CGPTX_INVALID_ARGUMENT, "rmsnorm_backward: null weight tensor");
-    auto stream = static_cast<hipStream_t>(stream_);
     const int r = static_cast<int>(rows), h = static_cast<int>(hidden);
     return dispatch_dtype(dtype, [&]<typename T>() -> int {
         auto* dx = static_cast<T*>(grad_input);
+        auto* res = static_cast<const T*>(residual);
         auto* dw = static_cast<T*>(grad_weight);
         auto* dy = static_cast<const T*>(grad_output);
         auto* x = static_cast<const T*>(input);
         auto* w = static_cast<const T*>(weight);
         const FastShape shape = pick_fast_shape<T>(h);
-        const bool aligned = is_aligned16(dx) && is_aligned16(dy) && is_aligned16(x) && is_aligned16(w);
+        const bool aligned = is_aligned16(dx) && is_aligned16(dy) && is_aligned16(x) && is_aligned16(w) && is_aligned16(res);
         const int reduce_blocks = (h + kWave - 1) / kWave;
         if (shape.lpr != 0 && aligned) {
             const int blocks = fast_blocks(shape, r);
+            const int slices = wide_reduce_slices(blocks, h, compute_units());
             void* mem = nullptr;
-            if (int s = scratch(stream, static_cast<std::size_t>(blocks) * hidden * sizeof(float), &mem)) return s;
+            const std::size_t partial_bytes = static_cast<std::size_t>(blocks) * hidden * sizeof(float);
+            if (int s = scratch(stream, partial_bytes + static_cast<std::size_t>(slices) * hidden * sizeof(float), &mem))
+                return s;
             auto* partial = static_cast<float*>(mem);
-            if (int s = launch_fast<T, true>(shape, dx, partial, dy, x, w, r, h, epsilon, blocks, stream)) return s;
+            if (int s = launch_fast<T, true>(shape, dx, partial, dy, res, x, w, r, h, epsilon, blocks, stream)) return s;
             CGPTX_LAUNCH_CHECK();
-            hipLaunchKernelGGL((column_partial_reduce_kernel<T>), dim3(reduce_blocks), dim3(kThreads), 0, stream, dw,
-                               partial, blocks, h, 0);
+            if (slices > 1) {
+                auto* second = reinterpret_cast<float*>(static_cast<char*>(mem) + partial_bytes);
+                hipLaunchKernelGGL(column_partial_fold_kernel, dim3(reduce_blocks, slices), dim3(kThreads), 0, stream,
+                                   second, partial, blocks, h);
+                CGPTX_LAUNCH_CHECK();
+                hipLaunchKernelGGL((column_partial_reduce_kernel<T>), dim3(reduce_blocks), dim3(kThreads), 0, stream, dw,
+                                   second, slices, h, 0);
+            } else {
+                hipLaunchKernelGGL((column_partial_reduce_kernel<T>), dim3(reduce_blocks), dim3(kThreads), 0, stream, dw,
+                                   partial, blocks, h, 0);
+            }
             CGPTX_LAUNCH_CHECK();
             return CGPTX_OK;
         }
@@ -318,8 +332,18 @@ extern "C" int cgptx_rmsnorm_backward(void* grad_input, void* grad_weight, const
         hipLaunchKernelGGL((column_partial_reduce_kernel<T>), dim3(reduce_blocks), dim3(kThreads), 0, stream, dw,
                            partial, slices, h, 0);
         CGPTX_LAUNCH_CHECK();
+        if (res != nullptr) return cgptx_add(dx, dx, res, rows * hidden, dtype, stream);
         return CGPTX_OK;
     });
+}
+
+}  // namespace cgptx
+
+extern "C" int cgptx_rmsnorm_backward(void* grad_input, void* grad_weight, const void* grad_output, const void* input,
+                                      const void* weight, size_t rows, size_t hidden, float epsilon, int dtype,
+                                      cgptx_stream stream) {
+    return cgptx::rmsnorm_backward_residual(grad_input, grad_weight, grad_output, input, weight, nullptr, rows, hidden,
+                                            epsilon, dtype, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int cgptx_rmsnorm_forward(void* output, const void* input, const void* weight, size_t rows, size_t hidden,
@@ -335,7 +359,7 @@ extern "C" int cgptx_rmsnorm_forward(void* output, const void* input, const void
         const FastShape shape = pick_fast_shape<T>(h);
         if (shape.lpr != 0 && is_aligned16(y) && is_aligned16(x) && is_aligned16(w)) {
             const int blocks = fast_blocks(shape, r);
-            if (int s = launch_fast<T, false>(shape, y, nullptr, nullptr, x, w, r, h, epsilon, blocks, stream)) return s;
+            if (int s = launch_fast<T, false>(shape, y, nullptr, nullptr, nullptr, x, w, r, h, epsilon, blocks, stream)) return s;
             CGPTX_LAUNCH_CHECK();
             return CGPTX_OK;
         }

@@ -15,6 +15,7 @@
 //     every scratch request was sized by that eager run, so replay allocates nothing.
 #include "cgptx_train.h"
 #include "common.hpp"
+#include "gemm.hpp"
 
 #include <cmath>
 #include <cstring>
@@ -103,7 +104,7 @@ struct cgptx_model {
     float* loss = nullptr;
     // backward workspace
     void *d_normalized = nullptr, *grad_a = nullptr, *grad_b = nullptr, *d_act = nullptr, *d_gate = nullptr,
-         *d_up = nullptr, *d_norm_in = nullptr, *d_residual = nullptr, *d_attn_out = nullptr, *d_q = nullptr,
+         *d_up = nullptr, *d_norm_in = nullptr, *d_attn_out = nullptr, *d_q = nullptr,
          *d_k = nullptr, *d_v = nullptr, *d_q_pre = nullptr, *d_k_pre = nullptr;
     cgptx_adamw_workspace* optimizer = nullptr;
     std::vector<cgptx_adamw_entry> entries;
@@ -224,6 +225,28 @@ int linear_backward_split(cgptx_model* m, void* dx, void* dw, const void* dy, co
     return CGPTX_OK;
 }
 
+// Y = X·Wᵀ + residual (accumulate: + Y): the block's residual additions ride in the projection's
+// epilogue (fp32, one rounding) instead of taking two more passes over the hidden state.
+int linear_forward_residual(void* out, const void* in, const void* w, const void* residual, bool accumulate,
+                            std::size_t rows, std::size_t in_features, std::size_t out_features, int dt,
+                            hipStream_t stream) {
+    GemmArgs g;
+    g.a = in;
+    g.b = w;
+    g.c = out;
+    g.residual = residual;
+    g.m = rows;
+    g.n = out_features;
+    g.k = in_features;
+    g.lda = in_features;
+    g.ldb = in_features;
+    g.ldc = out_features;
+    g.ldr = out_features;
+    g.accumulate = accumulate;
+    g.dtype = dt;
+    return gemm(g, stream);
+}
+
 int enqueue_forward_backward(cgptx_model* m, float loss_scale, int loss_mode, hipStream_t stream) {
     const auto& c = m->config;
     const int dt = c.dtype;
@@ -250,15 +273,13 @@ int enqueue_forward_backward(cgptx_model* m, float loss_scale, int loss_mode, hi
                                      c.rotary_dim, 0, m->sequence, dt, s));
         CGPTX_OP("attn_fwd", cgptx_flash_gqa_attention_forward(a.attn_out, a.lse, a.q, a.k, a.v, m->batch, m->sequence,
                                                     m->sequence, HQ, HKV, D, 0.0f, 1, 0, dt, s));
-        CGPTX_OP("gemm_fwd", cgptx_linear_forward(m->d_residual, a.attn_out, w.o.value, nullptr, N, QW, H, dt, s));
+        // out = x + attention_projection, then out += ffn_output (src/core/transformer_block.cu:594-595)
+        CGPTX_OP("gemm_fwd", linear_forward_residual(out, a.attn_out, w.o.value, x, false, N, QW, H, dt, stream));
         CGPTX_OP("rmsnorm_fwd", cgptx_rmsnorm_forward(a.norm_f, x, w.ffn_norm.value, N, H, eps, dt, s));
         CGPTX_OP("gemm_fwd", cgptx_linear_forward(a.gate, a.norm_f, w.gate.value, nullptr, N, H, I, dt, s));
         CGPTX_OP("gemm_fwd", cgptx_linear_forward(a.up, a.norm_f, w.up.value, nullptr, N, H, I, dt, s));
         CGPTX_OP("swiglu_fwd", cgptx_swiglu_forward(a.act, a.gate, a.up, N * I, dt, s));
-        CGPTX_OP("gemm_fwd", cgptx_linear_forward(m->d_norm_in, a.act, w.down.value, nullptr, N, I, H, dt, s));
-        // out = x + attention_projection, then out += ffn_output (src/core/transformer_block.cu:594-595)
-        CGPTX_OP("add", cgptx_add(out, x, m->d_residual, N * H, dt, s));
-        CGPTX_OP("add", cgptx_add(out, out, m->d_norm_in, N * H, dt, s));
+        CGPTX_OP("gemm_fwd", linear_forward_residual(out, a.act, w.down.value, nullptr, true, N, I, H, dt, stream));
     }
     void* last = m->hidden[c.num_layers];
     CGPTX_OP("rmsnorm_fwd", cgptx_rmsnorm_forward(m->normalized, last, m->final_norm.value, N, H, eps, dt, s));
@@ -289,9 +310,10 @@ int enqueue_forward_backward(cgptx_model* m, float loss_scale, int loss_mode, hi
         CGPTX_OP("swiglu_bwd", cgptx_swiglu_backward(m->d_gate, m->d_up, m->d_act, a.gate, a.up, N * I, 0, 0, dt, s));
         CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.gate.gradient, m->d_gate, a.norm_f, w.gate.value, N, H, I, 0, dt, stream));
         CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.up.gradient, m->d_up, a.norm_f, w.up.value, N, H, I, 1, dt, stream));
-        CGPTX_OP("rmsnorm_bwd", cgptx_rmsnorm_backward(m->d_residual, w.ffn_norm.gradient, m->d_norm_in, x, w.ffn_norm.value, N, H,
-                                         eps, dt, s));
-        CGPTX_OP("add", cgptx_add(previous, current, m->d_residual, N * H, dt, s));
+        // The gradient of the residual stream collects the two norm branches as they are produced:
+        // previous = current + d(ffn branch), later previous += d(attention branch).
+        CGPTX_OP("rmsnorm_bwd", rmsnorm_backward_residual(previous, w.ffn_norm.gradient, m->d_norm_in, x, w.ffn_norm.value,
+                                                          current, N, H, eps, dt, stream));
         CGPTX_TRY(linear_backward_split(m, m->d_attn_out, w.o.gradient, current, a.attn_out, w.o.value, N, QW, H, 0, dt, stream));
         CGPTX_OP("attn_bwd", cgptx_flash_gqa_attention_backward_with_lse(m->d_q, m->d_k, m->d_v, m->d_attn_out, a.attn_out,
                                                               a.lse, a.q, a.k, a.v, m->batch, m->sequence,
@@ -305,9 +327,8 @@ int enqueue_forward_backward(cgptx_model* m, float loss_scale, int loss_mode, hi
         CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.q.gradient, m->d_q, a.norm_a, w.q.value, N, H, QW, 0, dt, stream));
         CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.k.gradient, m->d_k, a.norm_a, w.k.value, N, H, KW, 1, dt, stream));
         CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.v.gradient, m->d_v, a.norm_a, w.v.value, N, H, KW, 1, dt, stream));
-        CGPTX_OP("rmsnorm_bwd", cgptx_rmsnorm_backward(m->d_residual, w.attention_norm.gradient, m->d_norm_in, x,
-                                         w.attention_norm.value, N, H, eps, dt, s));
-        CGPTX_OP("add", cgptx_add(previous, previous, m->d_residual, N * H, dt, s));
+        CGPTX_OP("rmsnorm_bwd", rmsnorm_backward_residual(previous, w.attention_norm.gradient, m->d_norm_in, x,
+                                                          w.attention_norm.value, previous, N, H, eps, dt, stream));
         std::swap(current, previous);
     }
     // Tied embedding: the classifier gradient is already in place; add the lookup's gradient
@@ -406,7 +427,7 @@ extern "C" int cgptx_model_create(cgptx_model** out, const cgptx_model_config* c
         CGPTX_HIP(hipMemset(m->targets, 0, N * sizeof(std::uint32_t)));
         CGPTX_TRY(allocate_typed(m, &m->loss, 256));
         CGPTX_HIP(hipMemset(m->loss, 0, 256));
-        for (void** p : {&m->d_normalized, &m->grad_a, &m->grad_b, &m->d_norm_in, &m->d_residual})
+        for (void** p : {&m->d_normalized, &m->grad_a, &m->grad_b, &m->d_norm_in})
             CGPTX_TRY(allocate(m, p, N * H * elem));
         for (void** p : {&m->d_act, &m->d_gate, &m->d_up}) CGPTX_TRY(allocate(m, p, N * I * elem));
         for (void** p : {&m->d_attn_out, &m->d_q, &m->d_q_pre}) CGPTX_TRY(allocate(m, p, N * QW * elem));
