@@ -267,6 +267,39 @@ __global__ __launch_bounds__(kThreads) void swiglu_forward_kernel(T* __restrict_
     }
 }
 
+// Packed input [rows, 2*hidden] = [gate | up] (src/ops/swiglu.cu:152-170): out[r, c] =
+// silu(gate_up[r, c]) * gate_up[r, hidden + c].
+template <typename T>
+__global__ __launch_bounds__(kThreads) void swiglu_forward_packed_kernel(T* __restrict__ out,
+                                                                        const T* __restrict__ gate_up,
+                                                                        std::size_t rows, std::size_t hidden,
+                                                                        bool vector_ok) {
+    constexpr int VEC = kVec128<T>;
+    const std::size_t count = rows * hidden;
+    if (vector_ok) {
+        const std::size_t row_vectors = hidden / VEC;
+        const std::size_t vectors = rows * row_vectors;
+        for (std::size_t v = static_cast<std::size_t>(blockIdx.x) * kThreads + threadIdx.x; v < vectors;
+             v += static_cast<std::size_t>(gridDim.x) * kThreads) {
+            const std::size_t row = v / row_vectors, col = (v - row * row_vectors) * VEC;
+            const T* in = gate_up + row * 2 * hidden + col;
+            const vec_t<float, VEC> g = vec_to_f32<T, VEC>(load_vec<T, VEC>(in));
+            const vec_t<float, VEC> u = vec_to_f32<T, VEC>(load_vec<T, VEC>(in + hidden));
+            vec_t<float, VEC> r;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) r[e] = g[e] * sigmoid_f32(g[e]) * u[e];
+            store_vec<T, VEC>(out + row * hidden + col, vec_from_f32<T, VEC>(r));
+        }
+        return;
+    }
+    for (std::size_t i = static_cast<std::size_t>(blockIdx.x) * kThreads + threadIdx.x; i < count;
+         i += static_cast<std::size_t>(gridDim.x) * kThreads) {
+        const std::size_t row = i / hidden, col = i - row * hidden;
+        const float g = to_f32(gate_up[row * 2 * hidden + col]);
+        out[i] = from_f32<T>(g * sigmoid_f32(g) * to_f32(gate_up[row * 2 * hidden + hidden + col]));
+    }
+}
+
 template <typename T>
 int launch_swiglu_backward(T* grad_gate, T* grad_up, const T* grad_output, const T* gate, const T* up,
                            std::size_t count, std::size_t row_elems, std::size_t packed_row_stride, bool acc_gate,
@@ -392,6 +425,24 @@ extern "C" int cgptx_swiglu_forward(void* output, const void* gate, const void* 
         hipLaunchKernelGGL((swiglu_forward_kernel<T>), dim3(grid_for(count / kVec128<T> + 1)), dim3(kThreads), 0,
                            static_cast<hipStream_t>(stream), static_cast<T*>(output), static_cast<const T*>(gate),
                            static_cast<const T*>(up), count, vector_ok);
+        CGPTX_LAUNCH_CHECK();
+        return CGPTX_OK;
+    });
+}
+
+extern "C" int cgptx_swiglu_forward_packed(void* output, const void* gate_up, size_t rows, size_t hidden, int dtype,
+                                           cgptx_stream stream) {
+    using namespace cgptx;
+    if (!valid_dtype(dtype)) return fail(CGPTX_INVALID_ARGUMENT, "swiglu_forward: unsupported dtype");
+    if (output == nullptr || gate_up == nullptr || rows == 0 || hidden == 0)
+        return fail(CGPTX_INVALID_ARGUMENT, "swiglu_forward: null or empty tensor");
+    if (rows > std::numeric_limits<std::size_t>::max() / (2 * hidden))
+        return fail(CGPTX_OVERFLOW, "swiglu_forward: element count overflows");
+    return dispatch_dtype(dtype, [&]<typename T>() -> int {
+        const bool vector_ok = is_aligned16(output) && is_aligned16(gate_up) && hidden % kVec128<T> == 0;
+        hipLaunchKernelGGL((swiglu_forward_packed_kernel<T>), dim3(grid_for(rows * hidden / kVec128<T> + 1)),
+                           dim3(kThreads), 0, static_cast<hipStream_t>(stream), static_cast<T*>(output),
+                           static_cast<const T*>(gate_up), rows, hidden, vector_ok);
         CGPTX_LAUNCH_CHECK();
         return CGPTX_OK;
     });

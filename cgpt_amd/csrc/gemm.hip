@@ -647,10 +647,16 @@ int run_typed(const GemmArgs& g, hipStream_t stream) {
     }
     if constexpr (!std::is_same_v<T, float>) {
         // 256x256 tiles (one block per CU, 64 MFMAs per wavefront and K step) when they still give
-        // every CU a tile; otherwise 128x128 tiles, with K split when even those are too few.
+        // every CU a tile, or when K is long enough to be split across the idle CUs without the
+        // fp32 partial tiles outweighing the contraction (at least 8 tiles, so at most 32 slices);
+        // otherwise 128x128 tiles, with K split when even those are too few.
         const long big_tiles = static_cast<long>((g.m + 255) / 256) * static_cast<long>((g.n + 255) / 256);
         const int forced = forced_tile();
-        const bool big = forced == 256 || (forced == 0 && big_tiles * 5 >= static_cast<long>(compute_units()) * 4);
+        const long units = compute_units();
+        const bool fills = big_tiles * 5 >= units * 4;
+        const bool splits = !g.no_split && g.residual == nullptr && big_tiles >= 8 &&
+                            g.k / kBK >= static_cast<std::size_t>(32 * ((units + big_tiles - 1) / big_tiles));
+        const bool big = forced == 256 || (forced == 0 && (fills || splits));
         if (big) return run_config<T, 256, 256>(g, p, stream);
         return run_config<T, 128, 128>(g, p, stream);
     }

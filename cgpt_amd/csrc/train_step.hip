@@ -81,7 +81,7 @@ struct LayerParameters {
 };
 
 struct LayerActivations {
-    void *norm_a, *q_pre, *k_pre, *q, *k, *v, *attn_out, *norm_f, *gate, *up, *act;
+    void *norm_a, *q_pre, *k_pre, *q, *k, *v, *attn_out, *norm_f, *gate_up, *act;  // gate_up: [rows, 2I] = [gate | up]
     float* lse;
 };
 
@@ -103,8 +103,8 @@ struct cgptx_model {
     std::uint32_t *tokens = nullptr, *targets = nullptr;
     float* loss = nullptr;
     // backward workspace
-    void *d_normalized = nullptr, *grad_a = nullptr, *grad_b = nullptr, *d_act = nullptr, *d_gate = nullptr,
-         *d_up = nullptr, *d_norm_in = nullptr, *d_attn_out = nullptr, *d_q = nullptr,
+    void *d_normalized = nullptr, *grad_a = nullptr, *grad_b = nullptr, *d_act = nullptr, *d_gate_up = nullptr,
+         *d_norm_in = nullptr, *d_attn_out = nullptr, *d_q = nullptr,
          *d_k = nullptr, *d_v = nullptr, *d_q_pre = nullptr, *d_k_pre = nullptr;
     cgptx_adamw_workspace* optimizer = nullptr;
     std::vector<cgptx_adamw_entry> entries;
@@ -141,13 +141,22 @@ int allocate_typed(cgptx_model* m, P** out, std::size_t bytes) {
 }
 
 // kind: 0 = normal(0, stddev), 1 = ones
+// value_slot / gradient_slot: storage inside a larger block (weights that one contraction reads as a
+// single matrix), or null for an allocation of the parameter's own.
 int make_parameter(cgptx_model* m, Parameter& p, const std::string& name, std::size_t count, int kind, float stddev,
-                   std::uint64_t seed, std::uint64_t tensor_id) {
+                   std::uint64_t seed, std::uint64_t tensor_id, void* value_slot = nullptr,
+                   void* gradient_slot = nullptr) {
     const std::size_t elem = dtype_size(m->config.dtype);
     p.name = name;
     p.count = count;
-    if (int s = allocate(m, &p.value, count * elem)) return s;
-    if (int s = allocate(m, &p.gradient, count * elem)) return s;
+    p.value = value_slot;
+    p.gradient = gradient_slot;
+    if (p.value == nullptr) {
+        if (int s = allocate(m, &p.value, count * elem)) return s;
+    }
+    if (p.gradient == nullptr) {
+        if (int s = allocate(m, &p.gradient, count * elem)) return s;
+    }
     if (int s = allocate_typed(m, &p.master, count * sizeof(float))) return s;
     if (int s = allocate_typed(m, &p.first, count * sizeof(float))) return s;
     if (int s = allocate_typed(m, &p.second, count * sizeof(float))) return s;
@@ -276,9 +285,8 @@ int enqueue_forward_backward(cgptx_model* m, float loss_scale, int loss_mode, hi
         // out = x + attention_projection, then out += ffn_output (src/core/transformer_block.cu:594-595)
         CGPTX_OP("gemm_fwd", linear_forward_residual(out, a.attn_out, w.o.value, x, false, N, QW, H, dt, stream));
         CGPTX_OP("rmsnorm_fwd", cgptx_rmsnorm_forward(a.norm_f, x, w.ffn_norm.value, N, H, eps, dt, s));
-        CGPTX_OP("gemm_fwd", cgptx_linear_forward(a.gate, a.norm_f, w.gate.value, nullptr, N, H, I, dt, s));
-        CGPTX_OP("gemm_fwd", cgptx_linear_forward(a.up, a.norm_f, w.up.value, nullptr, N, H, I, dt, s));
-        CGPTX_OP("swiglu_fwd", cgptx_swiglu_forward(a.act, a.gate, a.up, N * I, dt, s));
+        CGPTX_OP("gemm_fwd", cgptx_linear_forward(a.gate_up, a.norm_f, w.gate.value, nullptr, N, H, 2 * I, dt, s));
+        CGPTX_OP("swiglu_fwd", cgptx_swiglu_forward_packed(a.act, a.gate_up, N, I, dt, s));
         CGPTX_OP("gemm_fwd", linear_forward_residual(out, a.act, w.down.value, nullptr, true, N, I, H, dt, stream));
     }
     void* last = m->hidden[c.num_layers];
@@ -307,9 +315,8 @@ int enqueue_forward_backward(cgptx_model* m, float loss_scale, int loss_mode, hi
         const auto& a = m->acts[reverse];
         void* x = m->hidden[reverse];
         CGPTX_TRY(linear_backward_split(m, m->d_act, w.down.gradient, current, a.act, w.down.value, N, I, H, 0, dt, stream));
-        CGPTX_OP("swiglu_bwd", cgptx_swiglu_backward(m->d_gate, m->d_up, m->d_act, a.gate, a.up, N * I, 0, 0, dt, s));
-        CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.gate.gradient, m->d_gate, a.norm_f, w.gate.value, N, H, I, 0, dt, stream));
-        CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.up.gradient, m->d_up, a.norm_f, w.up.value, N, H, I, 1, dt, stream));
+        CGPTX_OP("swiglu_bwd", cgptx_swiglu_backward_packed(m->d_gate_up, m->d_act, a.gate_up, N, I, 0, dt, s));
+        CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.gate.gradient, m->d_gate_up, a.norm_f, w.gate.value, N, H, 2 * I, 0, dt, stream));
         // The gradient of the residual stream collects the two norm branches as they are produced:
         // previous = current + d(ffn branch), later previous += d(attention branch).
         CGPTX_OP("rmsnorm_bwd", rmsnorm_backward_residual(previous, w.ffn_norm.gradient, m->d_norm_in, x, w.ffn_norm.value,
@@ -401,8 +408,16 @@ extern "C" int cgptx_model_create(cgptx_model** out, const cgptx_model_config* c
             CGPTX_TRY(make_parameter(m, w.v, prefix + "self_attn.v_proj.weight", KW * H, 0, stddev, seed, id + 5));
             CGPTX_TRY(make_parameter(m, w.o, prefix + "self_attn.o_proj.weight", H * QW, 0, residual_stddev, seed, id + 6));
             CGPTX_TRY(make_parameter(m, w.ffn_norm, prefix + "post_attention_layernorm.weight", H, 1, 0, seed, id + 7));
-            CGPTX_TRY(make_parameter(m, w.gate, prefix + "mlp.gate_proj.weight", I * H, 0, stddev, seed, id + 8));
-            CGPTX_TRY(make_parameter(m, w.up, prefix + "mlp.up_proj.weight", I * H, 0, stddev, seed, id + 9));
+            // gate and up share one [2I, H] block (values and gradients), so that the block's three
+            // contractions with them each run as one [.., 2I] product on the packed activations.
+            void *gate_up_value = nullptr, *gate_up_gradient = nullptr;
+            CGPTX_TRY(allocate(m, &gate_up_value, 2 * I * H * elem));
+            CGPTX_TRY(allocate(m, &gate_up_gradient, 2 * I * H * elem));
+            CGPTX_TRY(make_parameter(m, w.gate, prefix + "mlp.gate_proj.weight", I * H, 0, stddev, seed, id + 8,
+                                     gate_up_value, gate_up_gradient));
+            CGPTX_TRY(make_parameter(m, w.up, prefix + "mlp.up_proj.weight", I * H, 0, stddev, seed, id + 9,
+                                     static_cast<char*>(gate_up_value) + I * H * elem,
+                                     static_cast<char*>(gate_up_gradient) + I * H * elem));
             CGPTX_TRY(make_parameter(m, w.down, prefix + "mlp.down_proj.weight", H * I, 0, residual_stddev, seed, id + 10));
             auto& a = m->acts[l];
             CGPTX_TRY(allocate(m, &a.norm_a, N * H * elem));
@@ -414,8 +429,7 @@ extern "C" int cgptx_model_create(cgptx_model** out, const cgptx_model_config* c
             CGPTX_TRY(allocate(m, &a.attn_out, N * QW * elem));
             CGPTX_TRY(allocate_typed(m, &a.lse, N * c.num_query_heads * sizeof(float)));
             CGPTX_TRY(allocate(m, &a.norm_f, N * H * elem));
-            CGPTX_TRY(allocate(m, &a.gate, N * I * elem));
-            CGPTX_TRY(allocate(m, &a.up, N * I * elem));
+            CGPTX_TRY(allocate(m, &a.gate_up, N * 2 * I * elem));
             CGPTX_TRY(allocate(m, &a.act, N * I * elem));
         }
         m->hidden.resize(c.num_layers + 1);
@@ -429,7 +443,8 @@ extern "C" int cgptx_model_create(cgptx_model** out, const cgptx_model_config* c
         CGPTX_HIP(hipMemset(m->loss, 0, 256));
         for (void** p : {&m->d_normalized, &m->grad_a, &m->grad_b, &m->d_norm_in})
             CGPTX_TRY(allocate(m, p, N * H * elem));
-        for (void** p : {&m->d_act, &m->d_gate, &m->d_up}) CGPTX_TRY(allocate(m, p, N * I * elem));
+        CGPTX_TRY(allocate(m, &m->d_act, N * I * elem));
+        CGPTX_TRY(allocate(m, &m->d_gate_up, N * 2 * I * elem));
         for (void** p : {&m->d_attn_out, &m->d_q, &m->d_q_pre}) CGPTX_TRY(allocate(m, p, N * QW * elem));
         for (void** p : {&m->d_k, &m->d_v, &m->d_k_pre}) CGPTX_TRY(allocate(m, p, N * KW * elem));
         // Rotary cache: theta = pos / base^(2i/rotary), cos/sin in float, stored in the model dtype

@@ -487,9 +487,23 @@ def rope_forward(query, key, cos_cache, sin_cache, stream=None, rope_options: Ro
               _stream(stream))
 
 
-def swiglu_forward(output, gate, up, stream=None):
-    """include/ops/swiglu.h."""
+def swiglu_forward(output, gate, up=None, stream=None):
+    """include/ops/swiglu.h: (output, gate, up) or, with up omitted, (output, gate_up) with the
+    projections concatenated along the last dimension."""
     name = "swiglu_forward"
+    if up is None:
+        gate_up = gate
+        _require_device(name, output, gate_up)
+        _same_dtype(name, gate_up, output)
+        if gate_up.dim() == 0 or gate_up.shape[-1] % 2 != 0:
+            raise ValueError(f"{name}: the last gate_up dimension must be even")
+        hidden = gate_up.shape[-1] // 2
+        if output.dim() != gate_up.dim() or tuple(output.shape[:-1]) != tuple(gate_up.shape[:-1]) or \
+                output.shape[-1] != hidden:
+            raise ValueError(f"{name}: output shape must match gate_up except for its last dimension")
+        capi.call("cgptx_swiglu_forward_packed", _ptr(output), _ptr(gate_up), output.numel() // hidden, hidden,
+                  _code(gate_up), _stream(stream))
+        return
     _require_device(name, output, gate, up)
     _same_dtype(name, gate, output, up)
     if output.shape != gate.shape or up.shape != gate.shape:

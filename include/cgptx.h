@@ -235,6 +235,11 @@ int cgptx_rope_forward(void* query, void* key, const void* cos_cache,
 int cgptx_swiglu_forward(void* output, const void* gate, const void* up,
                          size_t count, int dtype, cgptx_stream stream);
 
+/* swiglu_forward (packed input [rows, 2*hidden] = [gate | up]) — include/ops/swiglu.h:33-37,
+ * src/ops/swiglu.cu:152-170. output is [rows, hidden]. */
+int cgptx_swiglu_forward_packed(void* output, const void* gate_up, size_t rows,
+                                size_t hidden, int dtype, cgptx_stream stream);
+
 /* linear_forward — include/ops/linear.h. Y[rows,out] = X[rows,in]·W[out,in]ᵀ (+ bias[out]).
  * bias may be NULL. */
 int cgptx_linear_forward(void* output, const void* input, const void* weight,

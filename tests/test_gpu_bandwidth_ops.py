@@ -230,6 +230,20 @@ def test_swiglu_forward_and_add_parity(device, dtype):
     assert torch.equal(dout.cpu(), out)
 
 
+@pytest.mark.parametrize("dtype", DTYPES, ids=DTYPE_IDS)
+@pytest.mark.parametrize("rows,hidden", [(7, 24), (64, 2048), (5, 13)])
+def test_swiglu_forward_packed_parity(device, rows, hidden, dtype):
+    """Concatenated [gate | up] input (include/ops/swiglu.h:33-37): same values as the two-tensor form."""
+    gu = randn((rows, 2 * hidden), dtype, 41)
+    out = torch.empty((rows, hidden), dtype=dtype)
+    cpu_ops.swiglu_forward(out, gu[:, :hidden].contiguous(), gu[:, hidden:].contiguous())
+    dout = torch.empty((rows, hidden), dtype=dtype, device=device)
+    ops.swiglu_forward(dout, dev(gu, device))
+    assert_close(dout, out, TOL[dtype], "packed swiglu forward")
+    with pytest.raises(ValueError):
+        ops.swiglu_forward(dout, dev(gu, device)[:, : 2 * hidden - 1].contiguous())
+
+
 def test_swiglu_argument_errors(device):
     a = torch.zeros(4, 4, device=device)
     with pytest.raises(ValueError):
