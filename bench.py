@@ -61,7 +61,7 @@ def op_work(cfg, batch, seq, loss_mode):
 
 # The kernel that takes the largest share of a step is the 256x256-tile contraction with both
 # operands k-contiguous (every forward projection and the classifier logits). Its roofline entry is
-# measured on the launch it is used for most: the gate/up projection, [N, H] x [I, H]^T.
+# measured on the launch it spends most time in: the fused gate/up projection, [N, H] x [2I, H]^T.
 PROBE_KERNEL = "gemm_mfma_kernel<bf16, 256, 256, A k-contiguous, B k-contiguous> (gate/up projection shape)"
 TRAFFIC_FILE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles",
                             "gemm_nt_256x256_gate_projection_pmc.txt")
@@ -71,7 +71,7 @@ def kernel_probe(torch, cfg, batch, seq, stream, launches, seed):
     """Average duration of one launch of the dominant kernel: HIP events on the launch stream."""
     from cgpt_amd import ops
 
-    rows, hidden, inter = batch * seq, cfg.hidden_size, cfg.intermediate_size
+    rows, hidden, inter = batch * seq, cfg.hidden_size, 2 * cfg.intermediate_size  # [gate; up] as one weight
     generator = torch.Generator(device="cuda").manual_seed(seed)
     x = torch.randn(rows, hidden, device="cuda", generator=generator).to(torch.bfloat16)
     w = (torch.randn(inter, hidden, device="cuda", generator=generator) * 0.02).to(torch.bfloat16)

@@ -78,6 +78,13 @@ struct Mfma<f16_t> {
 
 using u32x4 = vec_t<unsigned int, 4>;
 
+struct KernelSegments {
+    const void* ptr[3];
+    long ld[3];
+    int cols[3];
+    int count;
+};
+
 struct KernelArgs {
     const void* a;
     const void* b;
@@ -90,6 +97,7 @@ struct KernelArgs {
     int k_tiles_per_slice;  // K tiles (of 64) handled by one blockIdx.y
     int accumulate;
     int c_f32;
+    KernelSegments a_seg, c_seg;  // column segments of A (as stored) and of C; count 0 = one buffer
 };
 
 // Instruction classes of __builtin_amdgcn_sched_group_barrier.
@@ -161,9 +169,9 @@ struct KTile {
     static constexpr int kFragReads = 1;               // LDS instructions per fragment
     static constexpr int kOffsets = 2;                 // per-lane fragment offsets: one per K sub-step
 
-    u32x4 rsrc;
-    int voffset;
-    unsigned int group_bytes;  // 16 rows further in global memory
+    u32x4 rsrc = {0u, 0u, 0u, 0u};
+    int voffset = 0;
+    unsigned int group_bytes = 0;  // 16 rows further in global memory
 
     // base: element (row0, 0) of the operand; rows past rows_left only feed C rows that are never
     // stored (they read zeros or whatever follows, never out of the allocation's last row).
@@ -207,9 +215,9 @@ struct NTile {
     static constexpr int kFragReads = 2;
     static constexpr int kOffsets = COLS / 64;  // per-lane fragment offsets: one per 32-column block of a wavefront
 
-    u32x4 rsrc;
-    int voffset;
-    unsigned int group_bytes;  // kRowsPerLoad k rows further in global memory
+    u32x4 rsrc = {0u, 0u, 0u, 0u};
+    int voffset = 0;
+    unsigned int group_bytes = 0;  // kRowsPerLoad k rows further in global memory
 
     // base: element (0, col0) of the operand. Column chunks past cols_left are clamped to the last
     // valid chunk: they only feed C columns that are never stored.
@@ -299,17 +307,55 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const int wm = wave >> 1, wn = wave & 1;
 
-    ATile a_src;
+    // A may be given as up to three column segments in separate buffers. Stored [M, K]: the K range
+    // is segmented and the source changes along the K loop (boundaries a_end0 / a_end1). Stored
+    // [K, M]: the M range is segmented and this block's rows pick their buffer once.
+    ATile a_src, a_src1, a_src2;
     BTile b_src;
-    if constexpr (A_K) a_src.init(static_cast<const T*>(p.a) + static_cast<long>(m0) * p.lda, p.lda, p.m - m0, p.k);
-    else a_src.init(static_cast<const T*>(p.a) + m0, p.lda, p.m - m0, p.k, wave);
+    int a_end0 = std::numeric_limits<int>::max(), a_end1 = std::numeric_limits<int>::max();
+    if constexpr (A_K) {
+        if (p.a_seg.count == 0) {
+            a_src.init(static_cast<const T*>(p.a) + static_cast<long>(m0) * p.lda, p.lda, p.m - m0, p.k);
+        } else {
+            a_src.init(static_cast<const T*>(p.a_seg.ptr[0]) + static_cast<long>(m0) * p.a_seg.ld[0], p.a_seg.ld[0],
+                       p.m - m0, p.a_seg.cols[0]);
+            if (p.a_seg.count > 1) {
+                a_end0 = p.a_seg.cols[0];
+                a_src1.init(static_cast<const T*>(p.a_seg.ptr[1]) + static_cast<long>(m0) * p.a_seg.ld[1],
+                            p.a_seg.ld[1], p.m - m0, p.a_seg.cols[1]);
+            }
+            if (p.a_seg.count > 2) {
+                a_end1 = a_end0 + p.a_seg.cols[1];
+                a_src2.init(static_cast<const T*>(p.a_seg.ptr[2]) + static_cast<long>(m0) * p.a_seg.ld[2],
+                            p.a_seg.ld[2], p.m - m0, p.a_seg.cols[2]);
+            }
+        }
+    } else {
+        const T* base = static_cast<const T*>(p.a);
+        long ld = p.lda;
+        int first = 0, width = p.m;
+        if (p.a_seg.count > 0) {
+            int s = 0;
+            while (s + 1 < p.a_seg.count && m0 >= first + p.a_seg.cols[s]) first += p.a_seg.cols[s++];
+            base = static_cast<const T*>(p.a_seg.ptr[s]);
+            ld = p.a_seg.ld[s];
+            width = p.a_seg.cols[s];
+        }
+        a_src.init(base + (m0 - first), ld, width - (m0 - first), p.k, wave);
+    }
     if constexpr (B_K) b_src.init(static_cast<const T*>(p.b) + static_cast<long>(n0) * p.ldb, p.ldb, p.n - n0, p.k);
     else b_src.init(static_cast<const T*>(p.b) + n0, p.ldb, p.n - n0, p.k, wave);
     // K tiles past the end of the slice reload the last one (never multiplied): the loop stays free
     // of data-dependent branches and every wavefront always has the same number of loads in flight.
     auto issue = [&](int t, int stage) {
         const int k0 = min(kt_begin + t, kt_end - 1) * kBK;
-        a_src.issue(smem + stage * kStage, k0, wave);
+        if constexpr (A_K) {
+            if (k0 < a_end0) a_src.issue(smem + stage * kStage, k0, wave);
+            else if (k0 < a_end1) a_src1.issue(smem + stage * kStage, k0 - a_end0, wave);
+            else a_src2.issue(smem + stage * kStage, k0 - a_end1, wave);
+        } else {
+            a_src.issue(smem + stage * kStage, k0, wave);
+        }
         b_src.issue(smem + stage * kStage + kATile, k0, wave);
     };
     constexpr int kTileLoads = ATile::kLoads + BTile::kLoads;  // per wavefront and K tile
@@ -397,6 +443,18 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
     constexpr int kPasses = BM / kPassRows;
     static_assert(kPassRows * kStageStride * 4 <= kSmemBytes, "epilogue staging does not fit in LDS");
     static_assert(kPasses == 1 || kPassRows == WM, "a pass must be one row of wavefronts");
+    // C may be given as column segments too: this tile's columns then belong to one of them.
+    void* c_base = p.c;
+    long c_ld = p.ldc;
+    int c_col0 = n0, c_cols = p.n;
+    if (p.c_seg.count > 0) {
+        int s = 0, first = 0;
+        while (s + 1 < p.c_seg.count && n0 >= first + p.c_seg.cols[s]) first += p.c_seg.cols[s++];
+        c_base = const_cast<void*>(p.c_seg.ptr[s]);
+        c_ld = p.c_seg.ld[s];
+        c_col0 = n0 - first;
+        c_cols = p.c_seg.cols[s];
+    }
     float* stage = reinterpret_cast<float*>(smem_raw);
     const int m_lane = lane & 31, n_lane = (lane >> 5) * 4;
 #pragma unroll
@@ -424,8 +482,8 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
         constexpr int kChunks = kPassRows * kChunksPerRow;
         for (int c = threadIdx.x; c < kChunks; c += kThreads) {
             const int r = c / kChunksPerRow, col = (c % kChunksPerRow) * 4;
-            const int m = m0 + pass * kPassRows + r, n = n0 + col;
-            if (m >= p.m || n >= p.n) continue;
+            const int m = m0 + pass * kPassRows + r, n = n0 + col, c_col = c_col0 + col;
+            if (m >= p.m || c_col >= c_cols) continue;
             vec_t<float, 4> v = *reinterpret_cast<const vec_t<float, 4>*>(stage + r * kStageStride + col);
             if constexpr (SPLIT) {
                 float* out = static_cast<float*>(p.c) +
@@ -436,11 +494,11 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
                 if (p.residual != nullptr)
                     v += vec_to_f32<T, 4>(load_vec<T, 4>(static_cast<const T*>(p.residual) + static_cast<long>(m) * p.ldr + n));
                 if (p.c_f32) {
-                    float* out = static_cast<float*>(p.c) + static_cast<long>(m) * p.ldc + n;
+                    float* out = static_cast<float*>(c_base) + static_cast<long>(m) * c_ld + c_col;
                     if (p.accumulate) v += *reinterpret_cast<const vec_t<float, 4>*>(out);
                     *reinterpret_cast<vec_t<float, 4>*>(out) = v;
                 } else {
-                    T* out = static_cast<T*>(p.c) + static_cast<long>(m) * p.ldc + n;
+                    T* out = static_cast<T*>(c_base) + static_cast<long>(m) * c_ld + c_col;
                     if (p.accumulate) v += vec_to_f32<T, 4>(load_vec<T, 4>(out));
                     store_vec<T, 4>(out, vec_from_f32<T, 4>(v));
                 }
@@ -580,7 +638,7 @@ int run_config(const GemmArgs& g, KernelArgs p, hipStream_t stream) {
     const long tiles = static_cast<long>(p.tiles_m) * p.tiles_n;
     const long want_blocks = static_cast<long>(compute_units()) * (BM == 256 ? 1 : 2);
     int slices = 1;
-    if (!g.no_split && g.residual == nullptr && tiles < want_blocks && k_tiles >= 32) {
+    if (!g.no_split && g.residual == nullptr && g.c_segments.count == 0 && tiles < want_blocks && k_tiles >= 32) {
         slices = static_cast<int>(std::min<long>((want_blocks + tiles - 1) / tiles, k_tiles / 16));
         if (slices < 1) slices = 1;
     }
@@ -598,6 +656,29 @@ int run_config(const GemmArgs& g, KernelArgs p, hipStream_t stream) {
                        g.c, static_cast<const float*>(mem), static_cast<const T*>(g.bias), p.m, p.n, p.ldc, slices,
                        p.accumulate, p.c_f32);
     CGPTX_LAUNCH_CHECK();
+    return CGPTX_OK;
+}
+
+// Validates column segments (widths multiples of `granule` except the last, summing to `total`,
+// 16-byte aligned rows) and copies them into the kernel arguments.
+int copy_segments(const GemmSegments& in, std::size_t total, std::size_t granule, KernelSegments& out) {
+    out = KernelSegments{};
+    if (in.count == 0) return CGPTX_OK;
+    if (in.count < 0 || in.count > 3) return fail(CGPTX_INVALID_ARGUMENT, "gemm: one to three segments");
+    std::size_t sum = 0;
+    for (int s = 0; s < in.count; ++s) {
+        const bool last = s + 1 == in.count;
+        if (in.ptr[s] == nullptr || in.cols[s] == 0 || in.ld[s] < in.cols[s] || in.ld[s] % 8 != 0 || in.cols[s] % 8 != 0 ||
+            !is_aligned16(in.ptr[s]) || (!last && in.cols[s] % granule != 0) ||
+            in.cols[s] > static_cast<std::size_t>(std::numeric_limits<int>::max()))
+            return fail(CGPTX_INVALID_ARGUMENT, "gemm: malformed operand segment");
+        out.ptr[s] = in.ptr[s];
+        out.ld[s] = static_cast<long>(in.ld[s]);
+        out.cols[s] = static_cast<int>(in.cols[s]);
+        sum += in.cols[s];
+    }
+    if (sum != total) return fail(CGPTX_INVALID_ARGUMENT, "gemm: segments do not cover the operand");
+    out.count = in.count;
     return CGPTX_OK;
 }
 
@@ -627,16 +708,36 @@ int run_typed(const GemmArgs& g, hipStream_t stream) {
     p.ldc = static_cast<long>(g.ldc);
     p.accumulate = g.accumulate ? 1 : 0;
     p.c_f32 = g.c_is_f32 ? 1 : 0;
+    const bool segmented = g.a_segments.count > 0 || g.c_segments.count > 0;
+    if (segmented) {
+        if (int s = copy_segments(g.a_segments, g.a_k_contiguous ? g.k : g.m, g.a_k_contiguous ? kBK : 256, p.a_seg))
+            return s;
+        if (int s = copy_segments(g.c_segments, g.n, 256, p.c_seg)) return s;
+        if (g.c_segments.count > 0 && (g.c_is_f32 || g.residual != nullptr))
+            return fail(CGPTX_INVALID_ARGUMENT, "gemm: a segmented output takes neither fp32 storage nor a residual");
+        if (std::is_same_v<T, float>) return fail(CGPTX_INVALID_ARGUMENT, "gemm: segmented operands need 16-bit storage");
+    }
 
     bool fast = false;
     if constexpr (!std::is_same_v<T, float>) {
         const std::size_t c_elem = g.c_is_f32 ? 4 : sizeof(T);
+        GemmArgs whole = g;  // alignment of segmented operands was checked per segment
+        if (g.a_segments.count > 0) {
+            whole.a = g.a_segments.ptr[0];
+            whole.lda = g.a_segments.ld[0];
+        }
+        if (g.c_segments.count > 0) {
+            whole.c = const_cast<void*>(g.c_segments.ptr[0]);
+            whole.ldc = g.c_segments.ld[0];
+        }
+        const GemmArgs& g = whole;
         fast = g.k % kBK == 0 && g.lda % 8 == 0 && g.ldb % 8 == 0 && g.n % 8 == 0 && g.m % 8 == 0 &&
                is_aligned16(g.a) && is_aligned16(g.b) && (g.ldc * c_elem) % 16 == 0 && is_aligned16(g.c) &&
                (g.bias == nullptr || (reinterpret_cast<std::uintptr_t>(g.bias) & 7u) == 0) &&
                (g.residual == nullptr || ((reinterpret_cast<std::uintptr_t>(g.residual) & 7u) == 0 && g.ldr % 4 == 0)) &&
                !(!g.a_k_contiguous && g.b_k_contiguous) && offsets_fit_32bit(g, sizeof(T));
     }
+    if (!fast && segmented) return fail(CGPTX_INVALID_ARGUMENT, "gemm: segmented operands need the aligned MFMA path");
     if (!fast) {
         const dim3 grid(static_cast<unsigned int>((g.n + kGenericTile - 1) / kGenericTile),
                         static_cast<unsigned int>((g.m + kGenericTile - 1) / kGenericTile));
@@ -654,7 +755,7 @@ int run_typed(const GemmArgs& g, hipStream_t stream) {
         const int forced = forced_tile();
         const long units = compute_units();
         const bool fills = big_tiles * 5 >= units * 4;
-        const bool splits = !g.no_split && g.residual == nullptr && big_tiles >= 8 &&
+        const bool splits = !g.no_split && g.residual == nullptr && g.c_segments.count == 0 && big_tiles >= 8 &&
                             g.k / kBK >= static_cast<std::size_t>(32 * ((units + big_tiles - 1) / big_tiles));
         const bool big = forced == 256 || (forced == 0 && (fills || splits));
         if (big) return run_config<T, 256, 256>(g, p, stream);
@@ -666,7 +767,8 @@ int run_typed(const GemmArgs& g, hipStream_t stream) {
 }  // namespace
 
 int gemm(const GemmArgs& g, hipStream_t stream) {
-    if (g.a == nullptr || g.b == nullptr || g.c == nullptr || g.m == 0 || g.n == 0 || g.k == 0)
+    if ((g.a == nullptr && g.a_segments.count == 0) || g.b == nullptr || (g.c == nullptr && g.c_segments.count == 0) ||
+        g.m == 0 || g.n == 0 || g.k == 0)
         return fail(CGPTX_INVALID_ARGUMENT, "gemm: null or empty operand");
     constexpr std::size_t i32max = std::numeric_limits<int>::max();
     if (g.m > i32max || g.n > i32max || g.k > i32max)

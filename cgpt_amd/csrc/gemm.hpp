@@ -12,6 +12,15 @@ namespace cgptx {
 // (or fp32 when c_is_f32). accumulate adds into C. residual (optional, [M, N], storage dtype, row
 // stride ldr, may be C itself) is added elementwise. bias (optional, [N], storage
 // dtype) is added to every row after the product.
+// Up to three column ranges of one logical matrix that live in separate row-major buffers
+// (e.g. the query, key and value activations next to each other). count == 0: not used.
+struct GemmSegments {
+    const void* ptr[3] = {nullptr, nullptr, nullptr};
+    std::size_t ld[3] = {0, 0, 0};
+    std::size_t cols[3] = {0, 0, 0};
+    int count = 0;
+};
+
 struct GemmArgs {
     const void* a = nullptr;
     const void* b = nullptr;
@@ -26,6 +35,11 @@ struct GemmArgs {
     bool c_is_f32 = false;
     bool no_split = false;  // never use split-K scratch (the caller owns the arena)
     int dtype = CGPTX_BF16;
+    // Column segments of A as stored (its K range when k-contiguous, its M range otherwise) and of
+    // C (written through; not combined with split-K, residual or fp32 output). Segment widths are
+    // multiples of 256 (of 32 for a k-contiguous A) except the last; a and lda / c and ldc are
+    // ignored for a segmented operand.
+    GemmSegments a_segments, c_segments;
 };
 
 int gemm(const GemmArgs& args, hipStream_t stream);

@@ -256,6 +256,70 @@ int linear_forward_residual(void* out, const void* in, const void* w, const void
     return gemm(g, stream);
 }
 
+// The three buffers [rows, QW], [rows, KW], [rows, KW] as column segments of one [rows, QW + 2 KW] matrix.
+GemmSegments qkv_segments(const void* q, const void* k, const void* v, std::size_t QW, std::size_t KW) {
+    GemmSegments seg;
+    seg.count = 3;
+    seg.ptr[0] = q;
+    seg.ptr[1] = k;
+    seg.ptr[2] = v;
+    seg.ld[0] = seg.cols[0] = QW;
+    seg.ld[1] = seg.cols[1] = KW;
+    seg.ld[2] = seg.cols[2] = KW;
+    return seg;
+}
+
+// [q | k | v] = X·[Wq; Wk; Wv]ᵀ in one launch; qkv_weight is the shared [QW + 2 KW, H] block.
+int qkv_forward(void* q, void* k, void* v, const void* x, const void* qkv_weight, std::size_t rows, std::size_t H,
+                std::size_t QW, std::size_t KW, int dt, hipStream_t stream) {
+    GemmArgs g;
+    g.a = x;
+    g.b = qkv_weight;
+    g.c_segments = qkv_segments(q, k, v, QW, KW);
+    g.m = rows;
+    g.n = QW + 2 * KW;
+    g.k = H;
+    g.lda = H;
+    g.ldb = H;
+    g.dtype = dt;
+    return gemm(g, stream);
+}
+
+// dX = [dq | dk | dv]·[Wq; Wk; Wv] in one launch.
+int qkv_backward_input(void* dx, const void* dq, const void* dk, const void* dv, const void* qkv_weight,
+                       std::size_t rows, std::size_t H, std::size_t QW, std::size_t KW, int dt, hipStream_t stream) {
+    GemmArgs g;
+    g.a_segments = qkv_segments(dq, dk, dv, QW, KW);
+    g.b = qkv_weight;
+    g.c = dx;
+    g.m = rows;
+    g.n = H;
+    g.k = QW + 2 * KW;
+    g.ldb = H;
+    g.ldc = H;
+    g.b_k_contiguous = false;
+    g.dtype = dt;
+    return gemm(g, stream);
+}
+
+// [dWq; dWk; dWv] = [dq | dk | dv]ᵀ·X in one launch.
+int qkv_backward_weight(void* qkv_gradient, const void* dq, const void* dk, const void* dv, const void* x,
+                        std::size_t rows, std::size_t H, std::size_t QW, std::size_t KW, int dt, hipStream_t stream) {
+    GemmArgs g;
+    g.a_segments = qkv_segments(dq, dk, dv, QW, KW);
+    g.b = x;
+    g.c = qkv_gradient;
+    g.m = QW + 2 * KW;
+    g.n = H;
+    g.k = rows;
+    g.ldb = H;
+    g.ldc = H;
+    g.a_k_contiguous = false;
+    g.b_k_contiguous = false;
+    g.dtype = dt;
+    return gemm(g, stream);
+}
+
 int enqueue_forward_backward(cgptx_model* m, float loss_scale, int loss_mode, hipStream_t stream) {
     const auto& c = m->config;
     const int dt = c.dtype;
@@ -264,6 +328,8 @@ int enqueue_forward_backward(cgptx_model* m, float loss_scale, int loss_mode, hi
     const std::size_t QW = HQ * D, KW = HKV * D;
     const float eps = c.rms_epsilon;
     auto* s = static_cast<cgptx_stream>(stream);
+    // One launch for the q/k/v projections needs 16-bit storage and segment widths the tiles respect.
+    const bool fused_qkv = dt != CGPTX_F32 && QW % 256 == 0 && KW % 256 == 0 && H % 32 == 0 && N % 32 == 0;
 
     // ------------------------------------------------------------------ forward
     CGPTX_OP("embedding_fwd", cgptx_embedding_forward(m->hidden[0], m->tokens, N, m->embedding.value, c.vocabulary_size, H, dt, s));
@@ -273,9 +339,13 @@ int enqueue_forward_backward(cgptx_model* m, float loss_scale, int loss_mode, hi
         void* x = m->hidden[l];
         void* out = m->hidden[l + 1];
         CGPTX_OP("rmsnorm_fwd", cgptx_rmsnorm_forward(a.norm_a, x, w.attention_norm.value, N, H, eps, dt, s));
-        CGPTX_OP("gemm_fwd", cgptx_linear_forward(a.q_pre, a.norm_a, w.q.value, nullptr, N, H, QW, dt, s));
-        CGPTX_OP("gemm_fwd", cgptx_linear_forward(a.k_pre, a.norm_a, w.k.value, nullptr, N, H, KW, dt, s));
-        CGPTX_OP("gemm_fwd", cgptx_linear_forward(a.v, a.norm_a, w.v.value, nullptr, N, H, KW, dt, s));
+        if (fused_qkv) {
+            CGPTX_OP("gemm_fwd", qkv_forward(a.q_pre, a.k_pre, a.v, a.norm_a, w.q.value, N, H, QW, KW, dt, stream));
+        } else {
+            CGPTX_OP("gemm_fwd", cgptx_linear_forward(a.q_pre, a.norm_a, w.q.value, nullptr, N, H, QW, dt, s));
+            CGPTX_OP("gemm_fwd", cgptx_linear_forward(a.k_pre, a.norm_a, w.k.value, nullptr, N, H, KW, dt, s));
+            CGPTX_OP("gemm_fwd", cgptx_linear_forward(a.v, a.norm_a, w.v.value, nullptr, N, H, KW, dt, s));
+        }
         CGPTX_OP("rmsnorm_fwd", cgptx_rmsnorm_forward(a.q, a.q_pre, w.q_norm.value, N * HQ, D, eps, dt, s));
         CGPTX_OP("rmsnorm_fwd", cgptx_rmsnorm_forward(a.k, a.k_pre, w.k_norm.value, N * HKV, D, eps, dt, s));
         CGPTX_OP("rope_fwd", cgptx_rope_forward(a.q, a.k, m->cos_cache, m->sin_cache, m->batch, m->sequence, HQ, HKV, D,
@@ -331,9 +401,14 @@ int enqueue_forward_backward(cgptx_model* m, float loss_scale, int loss_mode, hi
                                          eps, dt, s));
         CGPTX_OP("rmsnorm_bwd", cgptx_rmsnorm_backward(m->d_k, w.k_norm.gradient, m->d_k_pre, a.k_pre, w.k_norm.value, N * HKV, D,
                                          eps, dt, s));
-        CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.q.gradient, m->d_q, a.norm_a, w.q.value, N, H, QW, 0, dt, stream));
-        CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.k.gradient, m->d_k, a.norm_a, w.k.value, N, H, KW, 1, dt, stream));
-        CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.v.gradient, m->d_v, a.norm_a, w.v.value, N, H, KW, 1, dt, stream));
+        if (fused_qkv) {
+            CGPTX_OP("gemm_dx", qkv_backward_input(m->d_norm_in, m->d_q, m->d_k, m->d_v, w.q.value, N, H, QW, KW, dt, stream));
+            CGPTX_OP("gemm_dw", qkv_backward_weight(w.q.gradient, m->d_q, m->d_k, m->d_v, a.norm_a, N, H, QW, KW, dt, stream));
+        } else {
+            CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.q.gradient, m->d_q, a.norm_a, w.q.value, N, H, QW, 0, dt, stream));
+            CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.k.gradient, m->d_k, a.norm_a, w.k.value, N, H, KW, 1, dt, stream));
+            CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.v.gradient, m->d_v, a.norm_a, w.v.value, N, H, KW, 1, dt, stream));
+        }
         CGPTX_OP("rmsnorm_bwd", rmsnorm_backward_residual(previous, w.attention_norm.gradient, m->d_norm_in, x,
                                                           w.attention_norm.value, previous, N, H, eps, dt, stream));
         std::swap(current, previous);
@@ -401,11 +476,19 @@ extern "C" int cgptx_model_create(cgptx_model** out, const cgptx_model_config* c
             const std::string prefix = "model.layers." + std::to_string(l) + ".";
             const std::uint64_t id = 2 + l * 11;
             CGPTX_TRY(make_parameter(m, w.attention_norm, prefix + "input_layernorm.weight", H, 1, 0, seed, id));
-            CGPTX_TRY(make_parameter(m, w.q, prefix + "self_attn.q_proj.weight", QW * H, 0, stddev, seed, id + 1));
-            CGPTX_TRY(make_parameter(m, w.k, prefix + "self_attn.k_proj.weight", KW * H, 0, stddev, seed, id + 2));
+            // q, k and v share one [QW + 2 KW, H] block (values and gradients): the three projections of
+            // the normalized input run as one contraction whose output columns go to three buffers.
+            char *qkv_value = nullptr, *qkv_gradient = nullptr;
+            CGPTX_TRY(allocate_typed(m, &qkv_value, (QW + 2 * KW) * H * elem));
+            CGPTX_TRY(allocate_typed(m, &qkv_gradient, (QW + 2 * KW) * H * elem));
+            CGPTX_TRY(make_parameter(m, w.q, prefix + "self_attn.q_proj.weight", QW * H, 0, stddev, seed, id + 1, qkv_value,
+                                     qkv_gradient));
+            CGPTX_TRY(make_parameter(m, w.k, prefix + "self_attn.k_proj.weight", KW * H, 0, stddev, seed, id + 2,
+                                     qkv_value + QW * H * elem, qkv_gradient + QW * H * elem));
             CGPTX_TRY(make_parameter(m, w.q_norm, prefix + "self_attn.q_norm.weight", c.head_dim, 1, 0, seed, id + 3));
             CGPTX_TRY(make_parameter(m, w.k_norm, prefix + "self_attn.k_norm.weight", c.head_dim, 1, 0, seed, id + 4));
-            CGPTX_TRY(make_parameter(m, w.v, prefix + "self_attn.v_proj.weight", KW * H, 0, stddev, seed, id + 5));
+            CGPTX_TRY(make_parameter(m, w.v, prefix + "self_attn.v_proj.weight", KW * H, 0, stddev, seed, id + 5,
+                                     qkv_value + (QW + KW) * H * elem, qkv_gradient + (QW + KW) * H * elem));
             CGPTX_TRY(make_parameter(m, w.o, prefix + "self_attn.o_proj.weight", H * QW, 0, residual_stddev, seed, id + 6));
             CGPTX_TRY(make_parameter(m, w.ffn_norm, prefix + "post_attention_layernorm.weight", H, 1, 0, seed, id + 7));
             // gate and up share one [2I, H] block (values and gradients), so that the block's three

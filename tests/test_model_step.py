@@ -120,15 +120,22 @@ def compare_gradients(got, want, tol, loss_scale):
 MODEL_CFG = dict(vocab=96, layers=2, hidden=64, inter=128, hq=2, hkv=1, d=32, eps=1e-5)
 
 
+# Heads of 128 with 256-wide q and k/v projections, 64 rows: the shape class in which the step runs the
+# q/k/v projections as one contraction over segmented operands and attention on its head_dim-128 kernels.
+WIDE_CFG = dict(vocab=96, layers=1, hidden=256, inter=128, hq=2, hkv=2, d=128, eps=1e-5)
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
 @pytest.mark.parametrize("loss_mode", [0, 1], ids=["dense", "cut"])
-def test_gpu_step_matches_float64_composition(device, dtype, loss_mode):
-    """Hidden 64, 2:1 heads of 32, T=24, B=2, two layers: every parameter gradient of the GPU step against
-    the float64 composition that rounds each operator output to the storage dtype where the GPU stores it.
+@pytest.mark.parametrize("shape", [(MODEL_CFG, 2, 24), (WIDE_CFG, 2, 32)], ids=["heads32", "heads128-fused-qkv"])
+def test_gpu_step_matches_float64_composition(device, dtype, loss_mode, shape):
+    """Hidden 64, 2:1 heads of 32, T=24, B=2, two layers (and the wide-head variant above): every parameter
+    gradient of the GPU step against the float64 composition that rounds each operator output to the storage
+    dtype where the GPU stores it.
     Tolerance: 5e-2 of each tensor's largest gradient entry (2e-2 per operator, several operators deep)."""
-    cfg = MODEL_CFG
-    batch, seq, loss_scale = 2, 24, 64.0
+    cfg, batch, seq = shape
+    loss_scale = 64.0
     model = build(device, dtype, batch, seq, cfg)
     rng = np.random.default_rng(5)
     tokens = rng.integers(0, cfg["vocab"], size=(batch, seq))
