@@ -53,7 +53,10 @@ namespace {
 constexpr int kThreads = 256;
 constexpr int kWaves = kThreads / kWave;
 constexpr int kBK = 32;          // K step per LDS stage
-constexpr int kStages = 5;       // LDS stages: one being multiplied, up to three in flight, one being refilled
+// LDS stages of a BM x BN block: one being multiplied, one being refilled, the rest in flight.
+// 256x256 blocks own a CU (5 x 32 KiB); 128x256 blocks run two per CU, so that one block's
+// epilogue (LDS staging, stores draining to HBM) overlaps the other block's MFMAs (3 x 24 KiB each).
+constexpr int stages_for(int bm, int bn) { return bm + bn == 384 ? 3 : 5; }
 constexpr int kXcds = 8;
 constexpr int kGroupRows = 8;    // tile-rows per L2 locality group
 
@@ -157,43 +160,50 @@ __device__ __forceinline__ unsigned int lds_address_of(const T* p) {
 // cannot be padded; bank conflicts are avoided by storing 16-byte chunk c of a row at chunk
 // position c ^ swizzle(row) — the lane that owns an LDS slot fetches the matching global chunk.
 
-// ---- operand stored [ROWS, K] (k-contiguous): ROWS x 32 slab, LDS rows of 64 B ----------------
-// One load instruction covers 16 rows; wavefront w issues the loads of row groups w, w+4, ...
-// swizzle(row) = (row/4)%4: the 16 rows a quarter-wavefront reads with ds_read_b128 then hit the
-// 16 different 16-byte positions of a 256-byte bank period.
+// ---- operand stored [ROWS, K] (k-contiguous): ROWS x kBK slab, unpadded LDS rows ---------------
+// One load instruction covers 1024 B = kRowsPerLoad rows; wavefront w issues the loads of row
+// groups w, w+4, ... The chunk swizzle is (row / rows per 256 B) mod chunks per row: the 16 rows a
+// quarter-wavefront reads with ds_read_b128 then hit the 16 different 16-byte positions of a
+// 256-byte bank period.
 template <typename T, int ROWS>
 struct KTile {
     using frag_t = typename Mfma<T>::frag;
+    static constexpr int kChunksPerRow = kBK / 8;
+    static constexpr int kRowsPerLoad = 64 / kChunksPerRow;
     static constexpr int kElems = ROWS * kBK;
-    static constexpr int kLoads = ROWS / 16 / kWaves;  // load instructions per wavefront and tile
-    static constexpr int kFragReads = 1;               // LDS instructions per fragment
-    static constexpr int kOffsets = 2;                 // per-lane fragment offsets: one per K sub-step
+    static constexpr int kLoads = ROWS / kRowsPerLoad / kWaves;  // load instructions per wavefront and tile
+    static constexpr int kFragReads = 1;                        // LDS instructions per fragment
+    static constexpr int kOffsets = kBK / 16;                   // per-lane fragment offsets: one per K sub-step
 
     u32x4 rsrc = {0u, 0u, 0u, 0u};
     int voffset = 0;
-    unsigned int group_bytes = 0;  // 16 rows further in global memory
+    unsigned int group_bytes = 0;  // kRowsPerLoad rows further in global memory
+
+    __device__ __forceinline__ static int swizzle(int row) { return (row / (128 / kBK)) % kChunksPerRow; }
 
     // base: element (row0, 0) of the operand; rows past rows_left only feed C rows that are never
     // stored (they read zeros or whatever follows, never out of the allocation's last row).
-    __device__ __forceinline__ void init(const T* base, long ld, int rows_left, int k_total) {
+    __device__ __forceinline__ void init(const T* base, long ld, int rows_left, int k_total, int wave) {
         const int lane = threadIdx.x & (kWave - 1);
         rsrc = make_rsrc(base, (static_cast<long>(rows_left - 1) * ld + k_total) * static_cast<long>(sizeof(T)));
-        const int row = lane >> 2;
-        voffset = static_cast<int>(row * ld * sizeof(T)) + (((lane & 3) ^ ((row >> 2) & 3)) * 16);
-        group_bytes = static_cast<unsigned int>(16 * ld * sizeof(T));
+        const int row = lane / kChunksPerRow;
+        // The tile row of this lane's slot is (i*4 + wave) * kRowsPerLoad + row; its swizzle does not depend on i.
+        voffset = static_cast<int>(row * ld * sizeof(T)) +
+                  (((lane % kChunksPerRow) ^ swizzle(wave * kRowsPerLoad + row)) * 16);
+        group_bytes = static_cast<unsigned int>(kRowsPerLoad * ld * sizeof(T));
     }
     __device__ __forceinline__ void issue(T* tile, int k0, int wave) const {
 #pragma unroll
         for (int i = 0; i < kLoads; ++i) {
             const int group = i * kWaves + wave;
-            load_to_lds(rsrc, lds_address_of(tile + group * 16 * kBK), voffset,
+            load_to_lds(rsrc, lds_address_of(tile + group * kRowsPerLoad * kBK), voffset,
                         group * group_bytes + k0 * static_cast<unsigned int>(sizeof(T)));
         }
     }
     // Element offset of the lane's fragment within a 32-row block, K sub-step kk: row lane%32,
     // k = 16 kk + 8 (lane/32) .. +7.
     __device__ __forceinline__ static int lane_offset(int lane, int /*block0*/, int kk) {
-        return (lane & 31) * kBK + (((kk * 2 + (lane >> 5)) ^ ((lane >> 2) & 3)) * 8);
+        return (lane & 31) * kBK + (((kk * 2 + (lane >> 5)) ^ swizzle(lane & 31)) * 8);
     }
     __device__ __forceinline__ static frag_t frag(const T* tile, int block0, int offset) {
         return *reinterpret_cast<const frag_t*>(tile + block0 * kBK + offset);
@@ -267,6 +277,7 @@ struct TileLayout {
     using ATile = std::conditional_t<A_K, KTile<T, BM>, NTile<T, BM>>;
     using BTile = std::conditional_t<B_K, KTile<T, BN>, NTile<T, BN>>;
     static constexpr int kStage = ATile::kElems + BTile::kElems;  // elements per LDS stage: [A | B]
+    static constexpr int kStages = stages_for(BM, BN);
     static constexpr int kSmemBytes = kStages * kStage * static_cast<int>(sizeof(T));
 };
 
@@ -282,6 +293,7 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
     T* smem = reinterpret_cast<T*>(smem_raw);
     // Stage s holds [A tile | B tile] at smem + s * kStage.
     constexpr int kStage = Layout::kStage;
+    constexpr int kStages = Layout::kStages;
     constexpr int kATile = ATile::kElems;
 
     // XCD-contiguous, grouped tile order.
@@ -315,19 +327,19 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
     int a_end0 = std::numeric_limits<int>::max(), a_end1 = std::numeric_limits<int>::max();
     if constexpr (A_K) {
         if (p.a_seg.count == 0) {
-            a_src.init(static_cast<const T*>(p.a) + static_cast<long>(m0) * p.lda, p.lda, p.m - m0, p.k);
+            a_src.init(static_cast<const T*>(p.a) + static_cast<long>(m0) * p.lda, p.lda, p.m - m0, p.k, wave);
         } else {
             a_src.init(static_cast<const T*>(p.a_seg.ptr[0]) + static_cast<long>(m0) * p.a_seg.ld[0], p.a_seg.ld[0],
-                       p.m - m0, p.a_seg.cols[0]);
+                       p.m - m0, p.a_seg.cols[0], wave);
             if (p.a_seg.count > 1) {
                 a_end0 = p.a_seg.cols[0];
                 a_src1.init(static_cast<const T*>(p.a_seg.ptr[1]) + static_cast<long>(m0) * p.a_seg.ld[1],
-                            p.a_seg.ld[1], p.m - m0, p.a_seg.cols[1]);
+                            p.a_seg.ld[1], p.m - m0, p.a_seg.cols[1], wave);
             }
             if (p.a_seg.count > 2) {
                 a_end1 = a_end0 + p.a_seg.cols[1];
                 a_src2.init(static_cast<const T*>(p.a_seg.ptr[2]) + static_cast<long>(m0) * p.a_seg.ld[2],
-                            p.a_seg.ld[2], p.m - m0, p.a_seg.cols[2]);
+                            p.a_seg.ld[2], p.m - m0, p.a_seg.cols[2], wave);
             }
         }
     } else {
@@ -343,7 +355,7 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
         }
         a_src.init(base + (m0 - first), ld, width - (m0 - first), p.k, wave);
     }
-    if constexpr (B_K) b_src.init(static_cast<const T*>(p.b) + static_cast<long>(n0) * p.ldb, p.ldb, p.n - n0, p.k);
+    if constexpr (B_K) b_src.init(static_cast<const T*>(p.b) + static_cast<long>(n0) * p.ldb, p.ldb, p.n - n0, p.k, wave);
     else b_src.init(static_cast<const T*>(p.b) + n0, p.ldb, p.n - n0, p.k, wave);
     // K tiles past the end of the slice reload the last one (never multiplied): the loop stays free
     // of data-dependent branches and every wavefront always has the same number of loads in flight.
@@ -395,15 +407,16 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
     };
 
     // Software pipeline over K tiles t = 0 .. count-1 (tile t lives in LDS stage t % kStages; tiles
-    // t+1 .. t+kStages-2 are in flight or landed), two K sub-steps of 16 per tile:
-    //   sub-step 0  MFMAs ‖ LDS reads of sub-step 1's fragments
+    // t+1 .. t+kStages-2 are in flight or landed), kBK/16 K sub-steps of 16 per tile:
+    //   all but the last sub-step  MFMAs ‖ LDS reads of the next sub-step's fragments
     //   wait        this wavefront's loads of tile t+1 have landed; barrier: everybody's have, and
     //               nobody reads stage (t-1) % kStages any more
-    //   sub-step 1  MFMAs ‖ loads of tile t+kStages-1 into that stage ‖ fragments of tile t+1, sub-step 0
+    //   last sub-step  MFMAs ‖ loads of tile t+kStages-1 into that stage ‖ fragments of tile t+1, sub-step 0
     // so LDS latency and kStages-2 K tiles of global latency sit in the shadow of MFMAs.
     constexpr int kMfmas = TM * TN;
     constexpr int kFragReads = TM * ATile::kFragReads + TN * BTile::kFragReads;
-    static_assert(kBK == 32, "the pipeline below is written for two K sub-steps");
+    constexpr int kSubSteps = kBK / 16;
+    static_assert(kSubSteps % 2 == 0, "fragment sets alternate per sub-step and must line up across tiles");
     if (count > 0) {
 #pragma unroll
         for (int t = 0; t < kStages - 1; ++t) issue(t, t);
@@ -414,10 +427,13 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
         int free_stage = kStages - 1;  // of tile t-1, refilled with tile t+kStages-1
         for (int t = 0; t < count; ++t) {
             const int next_stage = stage + 1 == kStages ? 0 : stage + 1;
-            read_frags(1, stage, 1);
-            multiply(0);
-            sched_interleave<kMfmas, kSchedDsRead, kFragReads, 0, 0>();
-            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int kk = 0; kk + 1 < kSubSteps; ++kk) {
+                read_frags((kk + 1) & 1, stage, kk + 1);
+                multiply(kk & 1);
+                sched_interleave<kMfmas, kSchedDsRead, kFragReads, 0, 0>();
+                __builtin_amdgcn_sched_barrier(0);
+            }
             __builtin_amdgcn_s_waitcnt(vmcnt_immediate((kStages - 3) * kTileLoads));
             __syncthreads();
             issue(t + kStages - 1, free_stage);
@@ -433,10 +449,11 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
     __syncthreads();
 
     // Epilogue. acc[i][j][4g+e] holds C[m, n] with m = lane%32, n = 8g + 4*(lane/32) + e. The tile
-    // goes through LDS (fp32, row stride BN+4 so that the 16 lanes of a ds_write_b128 pass hit 16
-    // different bank groups) and leaves it row by row, so that a wavefront stores 512 contiguous
-    // bytes of C per instruction instead of 32 separate 16-byte pieces. Rounding to the storage
-    // dtype still happens once, after bias and accumulate were added in fp32.
+    // goes through LDS and leaves it row by row, so that a wavefront stores whole contiguous row
+    // segments of C per instruction instead of 32 separate 16-byte pieces. When bias, residual or
+    // the old C are added (or the output is fp32 / a split-K partial), the staging is fp32 (row
+    // stride BN+4: the 16 lanes of a ds_write_b128 pass hit 16 different bank groups) and rounding
+    // to the storage dtype still happens once, after the additions.
     constexpr int kStageStride = BN + 4;
     constexpr int kSmemBytes = Layout::kSmemBytes;
     constexpr int kPassRows = (BM * kStageStride * 4 <= kSmemBytes) ? BM : BM / 2;
@@ -455,8 +472,56 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
         c_col0 = n0 - first;
         c_cols = p.c_seg.cols[s];
     }
-    float* stage = reinterpret_cast<float*>(smem_raw);
     const int m_lane = lane & 31, n_lane = (lane >> 5) * 4;
+    if constexpr (!SPLIT) {
+        if (p.bias == nullptr && p.residual == nullptr && !p.accumulate && !p.c_f32) {
+            // Nothing is added to the product: round in registers, stage the whole tile in the
+            // storage dtype (one pass, half the LDS traffic) and store 16 bytes per lane, eight
+            // chunks in flight per thread.
+            constexpr int kTileStride = BN + 8;
+            static_assert(BM * kTileStride * static_cast<int>(sizeof(T)) <= kSmemBytes, "tile staging does not fit in LDS");
+            T* tile = smem;
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+#pragma unroll
+                for (int j = 0; j < TN; ++j) {
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        vec_t<float, 4> v;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) v[e] = acc[i][j][4 * g + e];
+                        store_vec<T, 4>(tile + (wm * WM + i * 32 + m_lane) * kTileStride + wn * WN + j * 32 + g * 8 + n_lane,
+                                        vec_from_f32<T, 4>(v));
+                    }
+                }
+            }
+            __syncthreads();
+            constexpr int kChunksPerRow = BN / 8;
+            constexpr int kPerThread = BM * kChunksPerRow / kThreads;
+            constexpr int kUnroll = 8;
+            static_assert(kPerThread % kUnroll == 0, "copy-out unrolling");
+            T* out = static_cast<T*>(c_base);
+            for (int base = 0; base < kPerThread; base += kUnroll) {
+                u32x4 data[kUnroll];
+#pragma unroll
+                for (int u = 0; u < kUnroll; ++u) {
+                    const int c = (base + u) * kThreads + threadIdx.x;
+                    const int r = c / kChunksPerRow, col = (c % kChunksPerRow) * 8;
+                    data[u] = *reinterpret_cast<const u32x4*>(tile + r * kTileStride + col);
+                }
+#pragma unroll
+                for (int u = 0; u < kUnroll; ++u) {
+                    const int c = (base + u) * kThreads + threadIdx.x;
+                    const int r = c / kChunksPerRow, col = (c % kChunksPerRow) * 8;
+                    const int m = m0 + r, c_col = c_col0 + col;
+                    if (m < p.m && c_col < c_cols)
+                        *reinterpret_cast<u32x4*>(out + static_cast<long>(m) * c_ld + c_col) = data[u];
+                }
+            }
+            return;
+        }
+    }
+    float* stage = reinterpret_cast<float*>(smem_raw);
 #pragma unroll
     for (int pass = 0; pass < kPasses; ++pass) {
         if (kPasses == 1 || wm == pass) {
@@ -619,13 +684,13 @@ int launch_layout(const KernelArgs& p, bool a_k, bool b_k, int slices, hipStream
     return fail(CGPTX_RUNTIME, "gemm: unsupported operand layout");
 }
 
-// CGPTX_GEMM_TILE=128|256 pins the tile size (for experiments); anything else = automatic.
+// CGPTX_GEMM_TILE=128|256|384 pins the tile size (384 = 128x256; for experiments); anything else = automatic.
 int forced_tile() {
     static const int value = [] {
         const char* text = std::getenv("CGPTX_GEMM_TILE");
         if (text == nullptr) return 0;
         const int v = std::atoi(text);
-        return (v == 128 || v == 256) ? v : 0;
+        return (v == 128 || v == 256 || v == 384) ? v : 0;
     }();
     return value;
 }
@@ -758,6 +823,7 @@ int run_typed(const GemmArgs& g, hipStream_t stream) {
         const bool splits = !g.no_split && g.residual == nullptr && g.c_segments.count == 0 && big_tiles >= 8 &&
                             g.k / kBK >= static_cast<std::size_t>(32 * ((units + big_tiles - 1) / big_tiles));
         const bool big = forced == 256 || (forced == 0 && (fills || splits));
+        if (forced == 384) return run_config<T, 128, 256>(g, p, stream);
         if (big) return run_config<T, 256, 256>(g, p, stream);
         return run_config<T, 128, 128>(g, p, stream);
     }
