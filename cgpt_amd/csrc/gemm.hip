@@ -545,27 +545,40 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
         __syncthreads();
         constexpr int kChunksPerRow = BN / 4;
         constexpr int kChunks = kPassRows * kChunksPerRow;
-        for (int c = threadIdx.x; c < kChunks; c += kThreads) {
-            const int r = c / kChunksPerRow, col = (c % kChunksPerRow) * 4;
-            const int m = m0 + pass * kPassRows + r, n = n0 + col, c_col = c_col0 + col;
-            if (m >= p.m || c_col >= c_cols) continue;
-            vec_t<float, 4> v = *reinterpret_cast<const vec_t<float, 4>*>(stage + r * kStageStride + col);
-            if constexpr (SPLIT) {
-                float* out = static_cast<float*>(p.c) +
-                             (static_cast<long>(blockIdx.y) * p.m + m) * static_cast<long>(p.n) + n;
-                *reinterpret_cast<vec_t<float, 4>*>(out) = v;
-            } else {
-                if (p.bias != nullptr) v += vec_to_f32<T, 4>(load_vec<T, 4>(static_cast<const T*>(p.bias) + n));
-                if (p.residual != nullptr)
-                    v += vec_to_f32<T, 4>(load_vec<T, 4>(static_cast<const T*>(p.residual) + static_cast<long>(m) * p.ldr + n));
-                if (p.c_f32) {
-                    float* out = static_cast<float*>(c_base) + static_cast<long>(m) * c_ld + c_col;
-                    if (p.accumulate) v += *reinterpret_cast<const vec_t<float, 4>*>(out);
+        constexpr int kBatch = 4;  // LDS reads in flight per thread before the dependent global accesses
+        static_assert(kChunks % (kThreads * kBatch) == 0, "copy-out batching");
+        for (int first = threadIdx.x; first < kChunks; first += kThreads * kBatch) {
+            vec_t<float, 4> staged[kBatch];
+#pragma unroll
+            for (int u = 0; u < kBatch; ++u) {
+                const int c = first + u * kThreads;
+                staged[u] = *reinterpret_cast<const vec_t<float, 4>*>(stage + (c / kChunksPerRow) * kStageStride +
+                                                                      (c % kChunksPerRow) * 4);
+            }
+#pragma unroll
+            for (int u = 0; u < kBatch; ++u) {
+                const int c = first + u * kThreads;
+                const int r = c / kChunksPerRow, col = (c % kChunksPerRow) * 4;
+                const int m = m0 + pass * kPassRows + r, n = n0 + col, c_col = c_col0 + col;
+                if (m >= p.m || c_col >= c_cols) continue;
+                vec_t<float, 4> v = staged[u];
+                if constexpr (SPLIT) {
+                    float* out = static_cast<float*>(p.c) +
+                                 (static_cast<long>(blockIdx.y) * p.m + m) * static_cast<long>(p.n) + n;
                     *reinterpret_cast<vec_t<float, 4>*>(out) = v;
                 } else {
-                    T* out = static_cast<T*>(c_base) + static_cast<long>(m) * c_ld + c_col;
-                    if (p.accumulate) v += vec_to_f32<T, 4>(load_vec<T, 4>(out));
-                    store_vec<T, 4>(out, vec_from_f32<T, 4>(v));
+                    if (p.bias != nullptr) v += vec_to_f32<T, 4>(load_vec<T, 4>(static_cast<const T*>(p.bias) + n));
+                    if (p.residual != nullptr)
+                        v += vec_to_f32<T, 4>(load_vec<T, 4>(static_cast<const T*>(p.residual) + static_cast<long>(m) * p.ldr + n));
+                    if (p.c_f32) {
+                        float* out = static_cast<float*>(c_base) + static_cast<long>(m) * c_ld + c_col;
+                        if (p.accumulate) v += *reinterpret_cast<const vec_t<float, 4>*>(out);
+                        *reinterpret_cast<vec_t<float, 4>*>(out) = v;
+                    } else {
+                        T* out = static_cast<T*>(c_base) + static_cast<long>(m) * c_ld + c_col;
+                        if (p.accumulate) v += vec_to_f32<T, 4>(load_vec<T, 4>(out));
+                        store_vec<T, 4>(out, vec_from_f32<T, 4>(v));
+                    }
                 }
             }
         }
