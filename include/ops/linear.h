@@ -1,0 +1,41 @@
+// linear_forward — reference: include/ops/linear.h:10-45. Y[.., out] = X[.., in]·W[out, in]ᵀ (+ bias).
+#pragma once
+
+#include "core/gemm_context.h"
+#include "core/status.h"
+#include "core/tensor.h"
+
+struct LinearOptions {
+    ComputeType compute_type = ComputeType::TF32;         // accepted, not used: accumulation is fp32
+    std::size_t workspace_bytes = 32U * 1024U * 1024U;    // accepted, not used: scratch is the library's own
+};
+
+namespace cgptx_detail {
+inline void linear_forward_impl(Tensor& output, const Tensor& input, const Tensor& weight, const Tensor* bias,
+                                hipStream_t stream) {
+    const char* op = "linear_forward";
+    require_device(op, {&output, &input, &weight});
+    require_same_dtype(op, input, {&output, &weight});
+    if (weight.dim() != 2 || input.dim() == 0 || output.dim() != input.dim() || input.shape().back() != weight.size(1) ||
+        output.shape().back() != weight.size(0) || output.numel() / weight.size(0) != input.numel() / weight.size(1))
+        throw std::invalid_argument("linear_forward: incompatible tensors");
+    if (bias != nullptr) {
+        require_device(op, {bias});
+        require_same_dtype(op, input, {bias});
+        if (bias->numel() != weight.size(0)) throw std::invalid_argument("linear_forward: bias must have out_features elements");
+    }
+    check(cgptx_linear_forward(output.raw_data(), input.raw_data(), weight.raw_data(), bias ? bias->raw_data() : nullptr,
+                               input.numel() / weight.size(1), weight.size(1), weight.size(0), dtype_code(input.dtype()),
+                               stream));
+}
+}  // namespace cgptx_detail
+
+inline void linear_forward(Tensor& output, const Tensor& input, const Tensor& weight, const GemmContext&,
+                           hipStream_t stream = nullptr, const LinearOptions& = {}) {
+    cgptx_detail::linear_forward_impl(output, input, weight, nullptr, stream);
+}
+
+inline void linear_forward(Tensor& output, const Tensor& input, const Tensor& weight, const Tensor& bias,
+                           const GemmContext&, hipStream_t stream = nullptr, const LinearOptions& = {}) {
+    cgptx_detail::linear_forward_impl(output, input, weight, &bias, stream);
+}

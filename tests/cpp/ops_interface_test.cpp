@@ -1,0 +1,342 @@
+// Drives the C++ operator interface (include/ops/**, include/optim/adamw.h) the way the reference's
+// own test binaries drive theirs: same calls, same known answers, same exception types.
+// Known answers are the constants of the reference's tests, cited per case. Built with hipcc by
+// __graft_entry__.build(); run by tests/test_cpp_interface.py on the GPU.
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <functional>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "ops/attention.h"
+#include "ops/backward/attention_backward.h"
+#include "ops/backward/embedding_backward.h"
+#include "ops/backward/linear_backward.h"
+#include "ops/backward/rmsnorm_backward.h"
+#include "ops/backward/rope_backward.h"
+#include "ops/backward/swiglu_backward.h"
+#include "ops/cross_entropy.h"
+#include "ops/cut_cross_entropy.h"
+#include "ops/embedding.h"
+#include "ops/linear.h"
+#include "ops/rmsnorm.h"
+#include "ops/rope.h"
+#include "ops/swiglu.h"
+#include "optim/adamw.h"
+
+namespace {
+
+int failures = 0;
+
+void expect(bool ok, const std::string& what) {
+    if (!ok) {
+        ++failures;
+        std::printf("FAIL %s\n", what.c_str());
+    }
+}
+
+Tensor device_f32(std::vector<std::size_t> shape, const std::vector<float>& values) {
+    Tensor t(std::move(shape), DeviceType::GPU, Dtype::F32);
+    t.copy_raw_from_host({reinterpret_cast<const std::uint8_t*>(values.data()), values.size() * sizeof(float)});
+    return t;
+}
+
+std::vector<float> host_f32(const Tensor& t) {
+    if (hipDeviceSynchronize() != hipSuccess) throw std::runtime_error("synchronize failed");
+    std::vector<float> values(t.numel());
+    t.copy_raw_to_host({reinterpret_cast<std::uint8_t*>(values.data()), values.size() * sizeof(float)});
+    return values;
+}
+
+bool close(const std::vector<float>& got, const std::vector<float>& want, float tolerance) {
+    if (got.size() != want.size()) return false;
+    for (std::size_t i = 0; i < got.size(); ++i)
+        if (!(std::fabs(got[i] - want[i]) <= tolerance)) return false;
+    return true;
+}
+
+bpe::TokenId* device_ids(const std::vector<bpe::TokenId>& ids) {
+    bpe::TokenId* p = nullptr;
+    if (hipMalloc(reinterpret_cast<void**>(&p), ids.size() * sizeof(bpe::TokenId)) != hipSuccess)
+        throw std::runtime_error("hipMalloc failed");
+    embedding_upload_token_ids(p, ids);
+    return p;
+}
+
+template <typename E>
+bool throws(const std::function<void()>& call) {
+    try {
+        call();
+    } catch (const E&) {
+        return true;
+    } catch (...) {
+        return false;
+    }
+    return false;
+}
+
+// tests/linear_backward_test.cu:20-45 — integer-valued 2x3 case, then all three accumulate flags.
+void linear_backward_known_answers() {
+    GemmContext context;
+    Tensor x = device_f32({2, 3}, {1, 2, 3, 4, 5, 6}), w = device_f32({2, 3}, {1, 0, 2, -1, 3, 1});
+    Tensor dy = device_f32({2, 2}, {2, -1, 3, 4});
+    Tensor gi = Tensor::zeros({2, 3}), gw = Tensor::zeros({2, 3}), gb = Tensor::zeros({2});
+    linear_backward(gi, gw, gb, dy, x, w, context);
+    expect(close(host_f32(gi), {3, -3, 3, -1, 12, 10}, 0), "linear_backward dX");
+    expect(close(host_f32(gw), {14, 19, 24, 15, 18, 21}, 0), "linear_backward dW");
+    expect(close(host_f32(gb), {5, 3}, 0), "linear_backward db");
+    LinearBackwardOptions options;
+    options.accumulate_input = options.accumulate_weight = options.accumulate_bias = true;
+    linear_backward(gi, gw, gb, dy, x, w, context, nullptr, options);
+    expect(close(host_f32(gi), {6, -6, 6, -2, 24, 20}, 0), "linear_backward dX accumulated");
+    expect(close(host_f32(gw), {28, 38, 48, 30, 36, 42}, 0), "linear_backward dW accumulated");
+    expect(close(host_f32(gb), {10, 6}, 0), "linear_backward db accumulated");
+    Tensor y = Tensor::zeros({2, 2});
+    linear_forward(y, x, w, context);
+    expect(close(host_f32(y), {7, 8, 16, 17}, 0), "linear_forward");
+    Tensor wrong = Tensor::zeros({2, 4});
+    expect(throws<std::invalid_argument>([&] { linear_backward(wrong, gw, gb, dy, x, w, context); }),
+           "linear_backward shape mismatch -> invalid_argument");
+}
+
+// tests/cross_entropy_test.cu:33-63 — values, gradient scale 1024, target-count mismatch.
+void cross_entropy_known_answers() {
+    Tensor logits = device_f32({2, 3}, {1, 2, 3, 1, 1, 1});
+    bpe::TokenId* targets = device_ids({2, 0});
+    Tensor loss = Tensor::zeros({1}), grad = Tensor::zeros({2, 3});
+    cross_entropy_forward_backward(loss, grad, logits, targets, 2);
+    const float want = (std::log(std::exp(1.0f) + std::exp(2.0f) + std::exp(3.0f)) - 3.0f + std::log(3.0f)) / 2.0f;
+    expect(close(host_f32(loss), {want}, 1e-5f), "cross_entropy loss");
+    expect(close(host_f32(grad), {0.0450153f, 0.1223642f, -0.1673795f, -0.3333333f, 0.1666667f, 0.1666667f}, 1e-5f),
+           "cross_entropy gradient");
+    Tensor only = Tensor::zeros({1});
+    cross_entropy_forward(only, logits, targets, 2);
+    expect(close(host_f32(only), {want}, 1e-5f), "cross_entropy_forward loss");
+    Tensor zero_logits = Tensor::zeros({1, 2}), scaled = Tensor::zeros({1, 2});
+    bpe::TokenId* first = device_ids({0});
+    cross_entropy_forward_backward(loss, scaled, zero_logits, first, 1, nullptr, 1024.0f);
+    expect(close(host_f32(loss), {std::log(2.0f)}, 1e-6f), "cross_entropy loss at scale 1024");
+    expect(close(host_f32(scaled), {-512.0f, 512.0f}, 0), "cross_entropy gradient at scale 1024");
+    expect(throws<std::invalid_argument>([&] { cross_entropy_forward_backward(loss, grad, logits, targets, 1); }),
+           "cross_entropy target count mismatch -> invalid_argument");
+    (void)hipFree(targets);
+    (void)hipFree(first);
+}
+
+// tests/rope_test.cu:99-127 — cos/sin in {0, 1}, rotary_dim 2 of head_dim 4; forward undoes backward.
+void rope_known_answers() {
+    Tensor q = device_f32({1, 2, 2, 4}, {1, 2, 30, 40, 3, 4, 50, 60, 5, 6, 70, 80, 7, 8, 90, 100});
+    Tensor k = device_f32({1, 2, 1, 4}, {1, -2, 30, 40, 5, -6, 70, 80});
+    Tensor cosine = device_f32({2, 1}, {1, 0}), sine = device_f32({2, 1}, {0, 1});
+    Tensor gq = Tensor::zeros({1, 2, 2, 4}), gk = Tensor::zeros({1, 2, 1, 4});
+    RopeOptions options;
+    options.rotary_dim = 2;
+    rope_backward(gq, gk, q, k, cosine, sine, nullptr, options);
+    expect(close(host_f32(gq), {1, 2, 30, 40, 3, 4, 50, 60, 6, -5, 70, 80, 8, -7, 90, 100}, 1e-6f), "rope_backward query");
+    expect(close(host_f32(gk), {1, -2, 30, 40, -6, -5, 70, 80}, 1e-6f), "rope_backward key");
+    rope_forward(gq, gk, cosine, sine, nullptr, options);
+    expect(close(host_f32(gq), host_f32(q), 1e-6f) && close(host_f32(gk), host_f32(k), 1e-6f), "rope_forward inverts rope_backward");
+}
+
+// tests/embedding_test.cu:183-203 — repeated token ids; the table is cleared first.
+void embedding_known_answers() {
+    Tensor dy = device_f32({3, 4}, {1, 2, 3, 4, 0.5f, 1.5f, -1, 2, 7, 8, 9, 10});
+    bpe::TokenId* ids = device_ids({1, 1, 2});
+    Tensor gw = device_f32({3, 4}, std::vector<float>(12, 5.0f));
+    embedding_backward(gw, dy, ids, 3);
+    expect(close(host_f32(gw), {0, 0, 0, 0, 1.5f, 3.5f, 2, 6, 7, 8, 9, 10}, 0), "embedding_backward repeated ids");
+    Tensor table = device_f32({3, 2}, {1, 2, 3, 4, 5, 6}), rows = Tensor::zeros({3, 2});
+    embedding_forward(rows, ids, 3, table);
+    expect(close(host_f32(rows), {3, 4, 3, 4, 5, 6}, 0), "embedding_forward");
+    (void)hipFree(ids);
+}
+
+// tests/adamw_test.cu:21-57 — two plain steps; loss scale 4 with clipping to 1; skipped step on Inf.
+void adamw_known_answers() {
+    Tensor p = device_f32({2}, {1.0f, -2.0f}), g = device_f32({2}, {0.1f, -0.2f});
+    AdamWState state = AdamWState::for_parameter(p);
+    AdamWOptions options;
+    options.learning_rate = 0.1f;
+    options.weight_decay = 0.01f;
+    expect(adamw_step(p, g, state, options), "adamw first step applied");
+    expect(close(host_f32(p), {0.899f, -1.898f}, 2e-6f), "adamw parameter after step 1");
+    expect(close(host_f32(state.first_moment), {0.01f, -0.02f}, 2e-6f), "adamw first moment");
+    expect(close(host_f32(state.second_moment), {0.00001f, 0.00004f}, 2e-6f), "adamw second moment");
+    expect(adamw_step(p, g, state, options) && state.step == 2, "adamw second step applied");
+    expect(close(host_f32(p), {0.798101f, -1.796102f}, 2e-6f), "adamw parameter after step 2");
+
+    Tensor p2 = device_f32({2}, {1.0f, -1.0f}), g2 = device_f32({2}, {8.0f, 0.0f});
+    AdamWState state2 = AdamWState::for_parameter(p2);
+    AdamWOptions scaled;
+    scaled.learning_rate = 0.1f;
+    scaled.weight_decay = 0.0f;
+    scaled.loss_scale = 4.0f;
+    scaled.max_grad_norm = 1.0f;
+    expect(adamw_step(p2, g2, state2, scaled), "adamw scaled step applied");
+    expect(close(host_f32(p2), {0.9f, -1.0f}, 2e-6f), "adamw unscale + clip");
+    Tensor bad = device_f32({2}, {INFINITY, 0.0f});
+    expect(!adamw_step(p2, bad, state2, scaled) && state2.step == 1, "adamw skips a non-finite gradient");
+    expect(close(host_f32(p2), {0.9f, -1.0f}, 2e-6f), "adamw leaves the parameter on a skipped step");
+
+    // batched form: same numbers through adamw_step_many_async + adamw_check (tests/adamw_test.cu:70-91)
+    Tensor p3 = device_f32({2}, {1.0f, -2.0f});
+    AdamWState state3 = AdamWState::for_parameter(p3);
+    AdamWWorkspace workspace;
+    const AdamWBatchEntry entry{&p3, &g, &state3};
+    adamw_step_many_async({&entry, 1}, options, workspace);
+    expect(adamw_check(workspace) && state3.step == 1, "adamw batched step applied");
+    expect(close(host_f32(p3), {0.899f, -1.898f}, 2e-6f), "adamw batched parameter");
+    Tensor short_gradient = Tensor::zeros({1});
+    expect(throws<std::invalid_argument>([&] { (void)adamw_step(p, short_gradient, state, options); }),
+           "adamw size mismatch -> invalid_argument");
+}
+
+// tests/cut_cross_entropy_test.cu:19-31 — the loss closed form; gradients against the dense
+// composition cross_entropy(X·Cᵀ) + linear_backward, which the reference states as the definition.
+void cut_cross_entropy_matches_dense() {
+    GemmContext context;
+    Tensor x = device_f32({2, 2}, {1, 2, -1, 0.5f}), c = device_f32({3, 2}, {0.5f, -1, 1.5f, 0.25f, -0.75f, 2});
+    bpe::TokenId* targets = device_ids({2, 0});
+    Tensor loss = Tensor::zeros({1}), dx = Tensor::zeros({2, 2}), dc = Tensor::zeros({3, 2});
+    cut_cross_entropy_forward_backward(loss, dx, dc, x, c, targets, 2);
+    Tensor logits = Tensor::zeros({2, 3}), dense_loss = Tensor::zeros({1}), dlogits = Tensor::zeros({2, 3});
+    linear_forward(logits, x, c, context);
+    cross_entropy_forward_backward(dense_loss, dlogits, logits, targets, 2);
+    Tensor dx2 = Tensor::zeros({2, 2}), dc2 = Tensor::zeros({3, 2}), db = Tensor::zeros({3});
+    linear_backward(dx2, dc2, db, dlogits, x, c, context);
+    expect(close(host_f32(loss), host_f32(dense_loss), 1e-5f), "cut cross-entropy loss = dense loss");
+    expect(close(host_f32(dx), host_f32(dx2), 1e-5f), "cut cross-entropy dX = dense dX");
+    expect(close(host_f32(dc), host_f32(dc2), 1e-5f), "cut cross-entropy dC = dense dC");
+    (void)hipFree(targets);
+}
+
+// rmsnorm: closed form on a row (tests/rmsnorm_test.cu:268-322 states the same formulas) and
+// SwiGLU: separate and concatenated inputs agree (include/ops/swiglu.h:16-37).
+void rmsnorm_and_swiglu() {
+    const std::vector<float> xv = {1, -2, 3, 0.5f}, wv = {1, 0.5f, 2, -1}, dyv = {0.25f, -1, 0.5f, 2};
+    Tensor x = device_f32({1, 4}, xv), w = device_f32({4}, wv), dy = device_f32({1, 4}, dyv);
+    Tensor y = Tensor::zeros({1, 4}), dx = Tensor::zeros({1, 4}), dw = Tensor::zeros({4});
+    const float eps = 1e-5f;
+    rmsnorm_forward(y, x, w, eps);
+    rmsnorm_backward(dx, dw, dy, x, w, eps);
+    double ss = 0, dot = 0;
+    for (int i = 0; i < 4; ++i) ss += double(xv[i]) * xv[i];
+    const double r = 1.0 / std::sqrt(ss / 4 + eps);
+    for (int i = 0; i < 4; ++i) dot += double(dyv[i]) * wv[i] * xv[i];
+    std::vector<float> want_y(4), want_dx(4), want_dw(4);
+    for (int i = 0; i < 4; ++i) {
+        want_y[i] = float(xv[i] * r * wv[i]);
+        want_dx[i] = float(dyv[i] * wv[i] * r - xv[i] * dot * r * r * r / 4);
+        want_dw[i] = float(dyv[i] * xv[i] * r);
+    }
+    expect(close(host_f32(y), want_y, 1e-5f), "rmsnorm_forward");
+    expect(close(host_f32(dx), want_dx, 1e-5f), "rmsnorm_backward dx");
+    expect(close(host_f32(dw), want_dw, 1e-5f), "rmsnorm_backward dgamma");
+    expect(throws<std::invalid_argument>([&] { rmsnorm_backward(dx, dw, dy, x, w, 0.0f); }),
+           "rmsnorm epsilon 0 -> invalid_argument");
+
+    Tensor gate = device_f32({2, 2}, {0.5f, -1, 2, 0}), up = device_f32({2, 2}, {1, 2, -3, 4});
+    Tensor packed = device_f32({2, 4}, {0.5f, -1, 1, 2, 2, 0, -3, 4});
+    Tensor out = Tensor::zeros({2, 2}), out_packed = Tensor::zeros({2, 2});
+    swiglu_forward(out, gate, up);
+    swiglu_forward(out_packed, packed);
+    std::vector<float> want(4);
+    const float g[4] = {0.5f, -1, 2, 0}, u[4] = {1, 2, -3, 4};
+    for (int i = 0; i < 4; ++i) want[i] = g[i] / (1.0f + std::exp(-g[i])) * u[i];
+    expect(close(host_f32(out), want, 1e-6f), "swiglu_forward");
+    expect(close(host_f32(out_packed), want, 1e-6f), "swiglu_forward concatenated input");
+    Tensor go = device_f32({2, 2}, {1, -1, 0.5f, 2});
+    Tensor gg = Tensor::zeros({2, 2}), gu = Tensor::zeros({2, 2}), gp = Tensor::zeros({2, 4});
+    swiglu_backward(gg, gu, go, gate, up);
+    swiglu_backward(gp, go, packed);
+    const std::vector<float> a = host_f32(gg), b = host_f32(gu), p = host_f32(gp);
+    expect(close({p[0], p[1], p[4], p[5]}, a, 1e-6f) && close({p[2], p[3], p[6], p[7]}, b, 1e-6f),
+           "swiglu_backward concatenated = separate");
+}
+
+// Attention: options-driven call, LSE and no-LSE backward agree, bad options throw
+// (tests/flash_attention_test.cu:365-388 uses 4:2 heads of 32 with offset 2).
+void attention_interface() {
+    FlashAttentionOptions options;
+    options.num_query_heads = 4;
+    options.num_kv_heads = 2;
+    options.head_dim = 32;
+    options.attention_scale = 0.23f;
+    options.query_position_offset = 2;
+    const std::size_t B = 2, QS = 3, KS = 5;
+    auto pattern = [](std::size_t count, float phase) {
+        std::vector<float> v(count);
+        for (std::size_t i = 0; i < count; ++i) v[i] = 0.45f * std::sin(phase + i * 0.31f) + 0.1f * std::cos(i * 0.17f);
+        return v;
+    };
+    auto half_tensor = [&](std::vector<std::size_t> shape, const std::vector<float>& values) {
+        std::vector<std::uint16_t> bits(values.size());
+        for (std::size_t i = 0; i < values.size(); ++i) {  // float -> bf16, round to nearest even
+            std::uint32_t word;
+            std::memcpy(&word, &values[i], 4);
+            bits[i] = static_cast<std::uint16_t>((word + 0x7FFFu + ((word >> 16) & 1u)) >> 16);
+        }
+        Tensor t(std::move(shape), DeviceType::GPU, Dtype::BF16);
+        t.copy_raw_from_host({reinterpret_cast<const std::uint8_t*>(bits.data()), bits.size() * 2});
+        return t;
+    };
+    Tensor q = half_tensor({B, QS, 4, 32}, pattern(B * QS * 4 * 32, 0.2f));
+    Tensor k = half_tensor({B, KS, 2, 32}, pattern(B * KS * 2 * 32, 0.7f));
+    Tensor v = half_tensor({B, KS, 2, 32}, pattern(B * KS * 2 * 32, 1.4f));
+    Tensor dout = half_tensor({B, QS, 4, 32}, pattern(B * QS * 4 * 32, 2.1f));
+    Tensor out({B, QS, 4, 32}, DeviceType::GPU, Dtype::BF16), lse({B, QS, 4}, DeviceType::GPU, Dtype::F32);
+    flash_gqa_attention_forward_with_lse(out, lse, q, k, v, nullptr, options);
+    Tensor dq1({B, QS, 4, 32}, DeviceType::GPU, Dtype::BF16), dk1({B, KS, 2, 32}, DeviceType::GPU, Dtype::BF16),
+        dv1({B, KS, 2, 32}, DeviceType::GPU, Dtype::BF16);
+    Tensor dq2({B, QS, 4, 32}, DeviceType::GPU, Dtype::BF16), dk2({B, KS, 2, 32}, DeviceType::GPU, Dtype::BF16),
+        dv2({B, KS, 2, 32}, DeviceType::GPU, Dtype::BF16);
+    flash_gqa_attention_backward_with_lse(dq1, dk1, dv1, dout, out, lse, q, k, v, nullptr, options);
+    flash_gqa_attention_backward(dq2, dk2, dv2, dout, q, k, v, nullptr, options);
+    if (hipDeviceSynchronize() != hipSuccess) throw std::runtime_error("synchronize failed");
+    auto raw = [](const Tensor& t) {
+        std::vector<std::uint8_t> bytes(t.nbytes());
+        t.copy_raw_to_host(bytes);
+        return bytes;
+    };
+    // The no-LSE form recomputes the very same output and LSE, so the two agree bit for bit.
+    expect(raw(dq1) == raw(dq2) && raw(dk1) == raw(dk2) && raw(dv1) == raw(dv2), "attention backward with and without LSE agree");
+    const std::vector<float> lse_host = host_f32(lse);
+    bool finite = true;
+    for (float value : lse_host) finite = finite && std::isfinite(value);
+    expect(finite, "attention log-sum-exp is finite");
+    FlashAttentionOptions wrong = options;
+    wrong.num_kv_heads = 3;
+    expect(throws<std::invalid_argument>([&] { flash_gqa_attention_forward(out, q, k, v, nullptr, wrong); }),
+           "attention heads mismatch -> invalid_argument");
+}
+
+}  // namespace
+
+int main() {
+    int devices = 0;
+    if (hipGetDeviceCount(&devices) != hipSuccess || devices == 0) {
+        std::printf("no GPU visible\n");
+        return 2;
+    }
+    const std::pair<const char*, void (*)()> cases[] = {
+        {"linear", linear_backward_known_answers}, {"cross_entropy", cross_entropy_known_answers},
+        {"rope", rope_known_answers},              {"embedding", embedding_known_answers},
+        {"adamw", adamw_known_answers},            {"cut_cross_entropy", cut_cross_entropy_matches_dense},
+        {"rmsnorm_swiglu", rmsnorm_and_swiglu},    {"attention", attention_interface},
+    };
+    for (const auto& [name, run] : cases) {
+        const int before = failures;
+        try {
+            run();
+        } catch (const std::exception& error) {
+            ++failures;
+            std::printf("FAIL %s: unexpected exception: %s\n", name, error.what());
+        }
+        std::printf("%s %s\n", failures == before ? "ok  " : "FAIL", name);
+        std::fflush(stdout);
+    }
+    std::printf("%d failure(s)\n", failures);
+    return failures == 0 ? 0 : 1;
+}
