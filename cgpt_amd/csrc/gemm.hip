@@ -192,12 +192,13 @@ struct KTile {
                   (((lane % kChunksPerRow) ^ swizzle(wave * kRowsPerLoad + row)) * 16);
         group_bytes = static_cast<unsigned int>(kRowsPerLoad * ld * sizeof(T));
     }
-    __device__ __forceinline__ void issue(T* tile, int k0, int wave) const {
+    // past_end: 0, or an offset that pushes every lane out of the buffer's range.
+    __device__ __forceinline__ void issue(T* tile, int k0, int wave, unsigned int past_end) const {
 #pragma unroll
         for (int i = 0; i < kLoads; ++i) {
             const int group = i * kWaves + wave;
             load_to_lds(rsrc, lds_address_of(tile + group * kRowsPerLoad * kBK), voffset,
-                        group * group_bytes + k0 * static_cast<unsigned int>(sizeof(T)));
+                        (group * group_bytes + k0 * static_cast<unsigned int>(sizeof(T))) | past_end);
         }
     }
     // Element offset of the lane's fragment within a 32-row block, K sub-step kk: row lane%32,
@@ -240,12 +241,13 @@ struct NTile {
         voffset = static_cast<int>(row * ld * sizeof(T)) + chunk * 16;
         group_bytes = static_cast<unsigned int>(kRowsPerLoad * ld * sizeof(T));
     }
-    __device__ __forceinline__ void issue(T* tile, int k0, int wave) const {
+    // past_end: 0, or an offset that pushes every lane out of the buffer's range.
+    __device__ __forceinline__ void issue(T* tile, int k0, int wave, unsigned int past_end) const {
 #pragma unroll
         for (int i = 0; i < kLoads; ++i) {
             const int group = i * kWaves + wave;
             load_to_lds(rsrc, lds_address_of(tile + group * kRowsPerLoad * COLS), voffset,
-                        (group + k0 / kRowsPerLoad) * group_bytes);
+                        ((group + k0 / kRowsPerLoad) * group_bytes) | past_end);
         }
     }
     // Lane i of a 16-lane group addresses k row i/4, columns 4*(i%4) .. +3 of the group's 4 x 16
@@ -357,18 +359,21 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
     }
     if constexpr (B_K) b_src.init(static_cast<const T*>(p.b) + static_cast<long>(n0) * p.ldb, p.ldb, p.n - n0, p.k, wave);
     else b_src.init(static_cast<const T*>(p.b) + n0, p.ldb, p.n - n0, p.k, wave);
-    // K tiles past the end of the slice reload the last one (never multiplied): the loop stays free
-    // of data-dependent branches and every wavefront always has the same number of loads in flight.
+    // K tiles past the end of the slice are still "loaded" (the loop stays free of data-dependent
+    // branches and every wavefront always has the same number of loads in flight), but from an
+    // offset beyond the buffer: the range check answers those at once with zeros, no memory traffic.
     auto issue = [&](int t, int stage) {
+        const bool beyond = kt_begin + t >= kt_end;
+        const unsigned int past_end = beyond ? 0x80000000u : 0u;
         const int k0 = min(kt_begin + t, kt_end - 1) * kBK;
         if constexpr (A_K) {
-            if (k0 < a_end0) a_src.issue(smem + stage * kStage, k0, wave);
-            else if (k0 < a_end1) a_src1.issue(smem + stage * kStage, k0 - a_end0, wave);
-            else a_src2.issue(smem + stage * kStage, k0 - a_end1, wave);
+            if (k0 < a_end0) a_src.issue(smem + stage * kStage, k0, wave, past_end);
+            else if (k0 < a_end1) a_src1.issue(smem + stage * kStage, k0 - a_end0, wave, past_end);
+            else a_src2.issue(smem + stage * kStage, k0 - a_end1, wave, past_end);
         } else {
-            a_src.issue(smem + stage * kStage, k0, wave);
+            a_src.issue(smem + stage * kStage, k0, wave, past_end);
         }
-        b_src.issue(smem + stage * kStage + kATile, k0, wave);
+        b_src.issue(smem + stage * kStage + kATile, k0, wave, past_end);
     };
     constexpr int kTileLoads = ATile::kLoads + BTile::kLoads;  // per wavefront and K tile
 
