@@ -173,6 +173,17 @@ __device__ __forceinline__ typename Mma<T>::frag acc_frag(const acc_t& acc, int 
 // Streamed index of accumulator register i: 8*(i/4) + 4*(lane/32) + i%4.
 __device__ __forceinline__ int acc_row(int i) { return 8 * (i >> 2) + 4 * ((threadIdx.x & 63) >> 5) + (i & 3); }
 
+// Query block of a workgroup. Workgroups are dealt to the 8 XCDs round-robin by linear id, and under
+// a causal mask a query block's work grows with its position; with the plain mapping and a grid
+// whose x extent is a multiple of 8, one XCD would receive all the longest blocks. Rotating the
+// index by the (head, batch) coordinate gives every XCD every length; the longest come first.
+__device__ __forceinline__ int balanced_query_block() {
+    const unsigned int count = gridDim.x;
+    const unsigned int rotation = blockIdx.y + gridDim.y * blockIdx.z;
+    const unsigned int index = (blockIdx.x + rotation) % count;
+    return static_cast<int>(count - 1 - index) * kBlockRows;
+}
+
 // ------------------------------------------------------------------- forward
 template <typename T, int DP>
 __global__ __launch_bounds__(kThreads) void attention_forward_kernel(Params p) {
@@ -181,7 +192,7 @@ __global__ __launch_bounds__(kThreads) void attention_forward_kernel(Params p) {
     __shared__ __align__(16) T v_lds[kStream * lds_stride<DP>()];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int b = blockIdx.z, h = blockIdx.y, kvh = h / (p.hq / p.hkv);
-    const int q_block = blockIdx.x * kBlockRows;
+    const int q_block = balanced_query_block();
     const int q_row = q_block + wave * 32 + (lane & 31);
     const bool q_live = q_row < p.qs;
     const long q_stride = static_cast<long>(p.hq) * p.d, kv_stride = static_cast<long>(p.hkv) * p.d;
@@ -325,7 +336,7 @@ __global__ __launch_bounds__(kThreads) void attention_dq_kernel(Params p) {
     __shared__ __align__(16) T v_lds[kStream * lds_stride<DP>()];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int b = blockIdx.z, h = blockIdx.y, kvh = h / (p.hq / p.hkv);
-    const int q_block = blockIdx.x * kBlockRows;
+    const int q_block = balanced_query_block();
     const int q_row = q_block + wave * 32 + (lane & 31);
     const bool q_live = q_row < p.qs;
     const long q_stride = static_cast<long>(p.hq) * p.d, kv_stride = static_cast<long>(p.hkv) * p.d;
@@ -661,6 +672,15 @@ __device__ __forceinline__ typename Mma<T>::frag wide_transposed_frag(const T* b
     return __builtin_bit_cast(typename Mma<T>::frag, both);
 }
 
+// max(a, b, c) in one instruction; the operands are never NaN here.
+__device__ __forceinline__ float max3(float a, float b, float c) {
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+
+constexpr float kRescaleThreshold = 8.0f;  // log2 of the factor by which probabilities may exceed 1
+
 // Exchange between lane l and lane l^32.
 __device__ __forceinline__ float other_half(float v) {
     const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
@@ -675,7 +695,7 @@ __global__ __launch_bounds__(kThreads, 2) void attention_forward_wide_kernel(Par
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int b = blockIdx.z, h = blockIdx.y, kvh = h / (p.hq / p.hkv);
-    const int q_block = (gridDim.x - 1 - blockIdx.x) * kBlockRows;  // blocks with the most key tiles start first
+    const int q_block = balanced_query_block();
     const int q_row = q_block + wave * 32 + (lane & 31);
     const bool q_live = q_row < p.qs;
     const long q_stride = static_cast<long>(p.hq) * p.d, kv_stride = static_cast<long>(p.hkv) * p.d;
@@ -709,7 +729,7 @@ __global__ __launch_bounds__(kThreads, 2) void attention_forward_wide_kernel(Par
     for (int t = 0; t < DT; ++t) o[t] = acc_t(0.0f);
     // The running maximum m is kept on the raw scores (the scale is positive, so it commutes with
     // max); probabilities are exp2(s*scale2 - m*scale2), one FMA and one v_exp_f32 per score.
-    float m = -INFINITY, l = 0.0f;
+    float m = -INFINITY, mb = 0.0f, l = 0.0f;  // mb = m * scale2 (0 while m is -inf)
     const float scale2 = p.scale * kLog2e;
     const int wave_first_q = q_block + wave * 32;
     const int wave_last_q = min(wave_first_q + 31, p.qs - 1);
@@ -759,13 +779,25 @@ __global__ __launch_bounds__(kThreads, 2) void attention_forward_wide_kernel(Par
                 for (int i = 0; i < 16; ++i)
                     st[sub][i] = (sub * 32 + 8 * (i >> 2) + (i & 3) <= bound) ? st[sub][i] : -INFINITY;
         }
-        float tile_max = fmaxf(st[0][0], st[1][0]);
+        float tile_max = max3(st[0][0], st[1][0], st[0][1]);
+        tile_max = max3(tile_max, st[1][1], st[0][2]);
 #pragma unroll
-        for (int i = 1; i < 16; ++i) tile_max = fmaxf(tile_max, fmaxf(st[0][i], st[1][i]));
+        for (int i = 2; i < 16; ++i) tile_max = max3(tile_max, st[1][i], i + 1 < 16 ? st[0][i + 1] : st[1][i]);
         tile_max = fmaxf(tile_max, other_half(tile_max));
-        const float m_new = fmaxf(m, tile_max);
-        const float mb = m_new == -INFINITY ? 0.0f : m_new * scale2;
-        const float alpha = __builtin_amdgcn_exp2f(m * scale2 - mb);
+        // The reference point m of the exponentials only follows the running maximum when it has
+        // moved by more than 2^8 in probability terms for some query of the wavefront: until then
+        // probabilities are merely scaled by up to 2^8 (harmless in fp32 sums and bf16/f16 factors,
+        // and cancelled by the final division), and the accumulator rescaling is skipped.
+        if (__any(tile_max > m && (tile_max - m) * scale2 > kRescaleThreshold)) {
+            const float m_new = fmaxf(m, tile_max);
+            const float mb_new = m_new == -INFINITY ? 0.0f : m_new * scale2;
+            const float alpha = __builtin_amdgcn_exp2f(m == -INFINITY ? -INFINITY : m * scale2 - mb_new);
+            l *= alpha;
+#pragma unroll
+            for (int t = 0; t < DT; ++t) o[t] *= alpha;
+            m = m_new;
+            mb = mb_new;
+        }
         float tile_sum = 0.0f;
 #pragma unroll
         for (int sub = 0; sub < 2; ++sub)
@@ -775,12 +807,7 @@ __global__ __launch_bounds__(kThreads, 2) void attention_forward_wide_kernel(Par
                 st[sub][i] = e;
                 tile_sum += e;
             }
-        l = l * alpha + tile_sum;
-        m = m_new;
-        if (__any(alpha != 1.0f)) {  // the maximum moved for some query of the wavefront
-#pragma unroll
-            for (int t = 0; t < DT; ++t) o[t] *= alpha;
-        }
+        l += tile_sum;
         __builtin_amdgcn_sched_barrier(0);
 
         {
@@ -821,7 +848,7 @@ __global__ __launch_bounds__(kThreads, 2) void attention_forward_wide_kernel(Par
         }
     }
     if (p.lse_out != nullptr && lane < 32)
-        p.lse_out[(static_cast<long>(b) * p.qs + q_row) * p.hq + h] = (m * scale2 + log2f(l)) * kLn2;
+        p.lse_out[(static_cast<long>(b) * p.qs + q_row) * p.hq + h] = (mb + log2f(l)) * kLn2;
 }
 
 // dQ for head dimensions 65..128: the forward kernel's streaming scheme; per 32-key half tile
@@ -835,7 +862,7 @@ __global__ __launch_bounds__(kThreads, 2) void attention_dq_wide_kernel(Params p
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int b = blockIdx.z, h = blockIdx.y, kvh = h / (p.hq / p.hkv);
-    const int q_block = (gridDim.x - 1 - blockIdx.x) * kBlockRows;
+    const int q_block = balanced_query_block();
     const int q_row = q_block + wave * 32 + (lane & 31);
     const bool q_live = q_row < p.qs;
     const long q_stride = static_cast<long>(p.hq) * p.d, kv_stride = static_cast<long>(p.hkv) * p.d;
