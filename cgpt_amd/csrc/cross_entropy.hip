@@ -117,15 +117,24 @@ __global__ __launch_bounds__(kThreads) void cross_entropy_row_kernel(float* __re
 }  // namespace
 
 // Shared with the cut-cross-entropy path: loss[0] = (Σ row_loss) / rows, fixed order.
-__global__ __launch_bounds__(256) void mean_reduce_kernel(float* __restrict__ loss,
-                                                         const float* __restrict__ row_loss, unsigned int rows,
-                                                         float inv_rows) {
-    __shared__ double stage[256];
-    double sum = 0.0;
-    for (unsigned int i = threadIdx.x; i < rows; i += 256) sum += static_cast<double>(row_loss[i]);
-    stage[threadIdx.x] = sum;
+__global__ __launch_bounds__(1024) void mean_reduce_kernel(float* __restrict__ loss,
+                                                          const float* __restrict__ row_loss, unsigned int rows,
+                                                          float inv_rows) {
+    __shared__ double stage[1024];
+    // Four independent partial sums per thread keep four loads in flight; the order of additions is
+    // fixed by (rows, thread count), so the result is reproducible.
+    double s0 = 0.0, s1 = 0.0, s2 = 0.0, s3 = 0.0;
+    unsigned int i = threadIdx.x;
+    for (; i + 3 * 1024 < rows; i += 4 * 1024) {
+        s0 += static_cast<double>(row_loss[i]);
+        s1 += static_cast<double>(row_loss[i + 1024]);
+        s2 += static_cast<double>(row_loss[i + 2 * 1024]);
+        s3 += static_cast<double>(row_loss[i + 3 * 1024]);
+    }
+    for (; i < rows; i += 1024) s0 += static_cast<double>(row_loss[i]);
+    stage[threadIdx.x] = (s0 + s1) + (s2 + s3);
     __syncthreads();
-    for (int stride = 128; stride > 0; stride >>= 1) {
+    for (int stride = 512; stride > 0; stride >>= 1) {
         if (threadIdx.x < static_cast<unsigned int>(stride)) stage[threadIdx.x] += stage[threadIdx.x + stride];
         __syncthreads();
     }
@@ -153,7 +162,7 @@ int cross_entropy_rows(float* row_loss, void* gradient, const void* logits, cons
 }
 
 int mean_reduce(float* loss, const float* row_loss, std::size_t rows, hipStream_t stream) {
-    hipLaunchKernelGGL(mean_reduce_kernel, dim3(1), dim3(256), 0, stream, loss, row_loss,
+    hipLaunchKernelGGL(mean_reduce_kernel, dim3(1), dim3(1024), 0, stream, loss, row_loss,
                        static_cast<unsigned int>(rows), 1.0f / static_cast<float>(rows));
     CGPTX_LAUNCH_CHECK();
     return CGPTX_OK;

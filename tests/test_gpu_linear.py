@@ -56,6 +56,8 @@ def check_against_float64(got, want64, dtype, what, terms):
 SHAPES = [  # rows, in, out
     (5, 7, 3), (33, 20, 17), (64, 64, 64), (128, 128, 256), (256, 192, 128), (136, 64, 72), (200, 256, 264),
     (384, 1024, 256), (1024, 320, 1024),
+    # every reduction length (in for Y, out for dX, rows for dW) is an odd multiple of 32
+    (288, 96, 160), (1056, 160, 352),
 ]
 
 
