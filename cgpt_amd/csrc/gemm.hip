@@ -44,6 +44,7 @@
 
 #include <algorithm>
 #include <type_traits>
+#include <utility>
 #include <cstdlib>
 #include <limits>
 
@@ -53,10 +54,9 @@ namespace {
 constexpr int kThreads = 256;
 constexpr int kWaves = kThreads / kWave;
 constexpr int kBK = 32;          // K step per LDS stage
-// LDS stages of a BM x BN block: one being multiplied, one being refilled, the rest in flight.
-// 256x256 blocks own a CU (5 x 32 KiB); 128x256 blocks run two per CU, so that one block's
-// epilogue (LDS staging, stores draining to HBM) overlaps the other block's MFMAs (3 x 24 KiB each).
-constexpr int stages_for(int bm, int bn) { return bm + bn == 384 ? 3 : 5; }
+// LDS stages of a block: one being multiplied, one being refilled, the rest in flight. 256x256
+// blocks own a CU (5 x 32 KiB), 128x128 blocks run two per CU (5 x 16 KiB each).
+constexpr int stages_for(int /*bm*/, int /*bn*/) { return 5; }
 constexpr int kXcds = 8;
 constexpr int kGroupRows = 8;    // tile-rows per L2 locality group
 
@@ -103,6 +103,26 @@ struct KernelArgs {
     KernelSegments a_seg, c_seg;  // column segments of A (as stored) and of C; count 0 = one buffer
 };
 
+// The column segment (of up to three) that holds column `col`, picked with selects: indexing the
+// kernel-argument arrays by a run-time value would move them to private memory.
+struct SegmentPick {
+    const void* ptr;
+    long ld;
+    int first;  // first column of the segment
+    int cols;
+};
+__device__ __forceinline__ SegmentPick pick_segment(const KernelSegments& seg, int col) {
+    const int end0 = seg.cols[0], end1 = end0 + seg.cols[1];
+    const bool in1 = seg.count > 1 && col >= end0;
+    const bool in2 = seg.count > 2 && col >= end1;
+    SegmentPick pick;
+    pick.ptr = in2 ? seg.ptr[2] : in1 ? seg.ptr[1] : seg.ptr[0];
+    pick.ld = in2 ? seg.ld[2] : in1 ? seg.ld[1] : seg.ld[0];
+    pick.first = in2 ? end1 : in1 ? end0 : 0;
+    pick.cols = in2 ? seg.cols[2] : in1 ? seg.cols[1] : seg.cols[0];
+    return pick;
+}
+
 // Instruction classes of __builtin_amdgcn_sched_group_barrier.
 constexpr int kSchedMfma = 0x008, kSchedDsRead = 0x100;
 
@@ -139,14 +159,43 @@ __device__ __forceinline__ u32x4 make_rsrc(const void* base, long bytes) {
 }
 
 // One wavefront-wide 16-byte-per-lane load from a buffer straight into LDS: lane l's bytes land at
-// lds_address + 16 l. Written as assembly on purpose: the compiler would order every later LDS
-// read after *all* outstanding loads of this kind (vmcnt(0)), which defeats keeping several K tiles
-// in flight; the kernel counts its loads itself (vmcnt_immediate). M0 is used by nothing else here.
-__device__ __forceinline__ void load_to_lds(const u32x4& rsrc, unsigned int lds_address, int voffset,
-                                            unsigned int soffset) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-                 :
-                 : "s"(lds_address), "v"(voffset), "s"(rsrc), "s"(soffset));
+// lds_base + LDS_OFFSET + 16 l. Returns soffset + step, the scalar offset of the operand's next load
+// (that addition sits between the write of M0 and the load, which need one instruction between them
+// anyway). Written as assembly on purpose: the compiler would order every later LDS read after *all*
+// outstanding loads of this kind (vmcnt(0)), which defeats keeping several K tiles in flight; the
+// kernel counts its loads itself (vmcnt_immediate). M0 is used by nothing else here.
+template <int LDS_OFFSET>
+__device__ __forceinline__ unsigned int load_to_lds(const u32x4& rsrc, unsigned int lds_base, int voffset,
+                                                    unsigned int soffset, unsigned int step) {
+    unsigned int next;
+    asm volatile("s_add_u32 m0, %1, %2\n\ts_add_u32 %0, %3, %4\n\tbuffer_load_dwordx4 %5, %6, %3 offen lds"
+                 : "=&s"(next)
+                 : "s"(lds_base), "n"(LDS_OFFSET), "s"(soffset), "s"(step), "v"(voffset), "s"(rsrc)
+                 : "scc");
+    return next;
+}
+
+// Workgroup barrier without the fence __syncthreads() carries: LDS reads still in flight may
+// cross it (their registers are waited for where they are used).
+__device__ __forceinline__ void barrier_only() { asm volatile("s_barrier" ::: "memory"); }
+
+// Where a wavefront's loads of one operand's K tile come from: load i reads at scalar offset
+// soffset + i * step.
+struct TileCursor {
+    u32x4 rsrc;
+    int voffset;
+    unsigned int soffset;
+    unsigned int step;
+};
+
+template <int BEGIN, int... I, typename F>
+__device__ __forceinline__ void static_for_impl(std::integer_sequence<int, I...>, F&& f) {
+    (f(std::integral_constant<int, BEGIN + I>{}), ...);
+}
+// f(integral_constant<int, i>) for i = BEGIN .. END-1, unrolled at compile time.
+template <int BEGIN, int END, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+    static_for_impl<BEGIN>(std::make_integer_sequence<int, (END > BEGIN ? END - BEGIN : 0)>{}, f);
 }
 
 template <typename T>
@@ -192,14 +241,9 @@ struct KTile {
                   (((lane % kChunksPerRow) ^ swizzle(wave * kRowsPerLoad + row)) * 16);
         group_bytes = static_cast<unsigned int>(kRowsPerLoad * ld * sizeof(T));
     }
-    // past_end: 0, or an offset that pushes every lane out of the buffer's range.
-    __device__ __forceinline__ void issue(T* tile, int k0, int wave, unsigned int past_end) const {
-#pragma unroll
-        for (int i = 0; i < kLoads; ++i) {
-            const int group = i * kWaves + wave;
-            load_to_lds(rsrc, lds_address_of(tile + group * kRowsPerLoad * kBK), voffset,
-                        (group * group_bytes + k0 * static_cast<unsigned int>(sizeof(T))) | past_end);
-        }
+    // Scalar offset of wavefront `wave`'s first load of the tile that starts at column k0.
+    __device__ __forceinline__ unsigned int first_offset(int k0, int wave) const {
+        return wave * group_bytes + k0 * static_cast<unsigned int>(sizeof(T));
     }
     // Element offset of the lane's fragment within a 32-row block, K sub-step kk: row lane%32,
     // k = 16 kk + 8 (lane/32) .. +7.
@@ -241,14 +285,9 @@ struct NTile {
         voffset = static_cast<int>(row * ld * sizeof(T)) + chunk * 16;
         group_bytes = static_cast<unsigned int>(kRowsPerLoad * ld * sizeof(T));
     }
-    // past_end: 0, or an offset that pushes every lane out of the buffer's range.
-    __device__ __forceinline__ void issue(T* tile, int k0, int wave, unsigned int past_end) const {
-#pragma unroll
-        for (int i = 0; i < kLoads; ++i) {
-            const int group = i * kWaves + wave;
-            load_to_lds(rsrc, lds_address_of(tile + group * kRowsPerLoad * COLS), voffset,
-                        ((group + k0 / kRowsPerLoad) * group_bytes) | past_end);
-        }
+    // Scalar offset of wavefront `wave`'s first load of the tile that starts at row k0.
+    __device__ __forceinline__ unsigned int first_offset(int k0, int wave) const {
+        return (wave + k0 / kRowsPerLoad) * group_bytes;
     }
     // Lane i of a 16-lane group addresses k row i/4, columns 4*(i%4) .. +3 of the group's 4 x 16
     // block; groups 0/1 take columns 0-15/16-31 of the fragment, lanes 32-63 the k values 8-15.
@@ -349,11 +388,11 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
         long ld = p.lda;
         int first = 0, width = p.m;
         if (p.a_seg.count > 0) {
-            int s = 0;
-            while (s + 1 < p.a_seg.count && m0 >= first + p.a_seg.cols[s]) first += p.a_seg.cols[s++];
-            base = static_cast<const T*>(p.a_seg.ptr[s]);
-            ld = p.a_seg.ld[s];
-            width = p.a_seg.cols[s];
+            const SegmentPick pick = pick_segment(p.a_seg, m0);
+            base = static_cast<const T*>(pick.ptr);
+            ld = pick.ld;
+            first = pick.first;
+            width = pick.cols;
         }
         a_src.init(base + (m0 - first), ld, width - (m0 - first), p.k, wave);
     }
@@ -362,18 +401,44 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
     // K tiles past the end of the slice are still "loaded" (the loop stays free of data-dependent
     // branches and every wavefront always has the same number of loads in flight), but from an
     // offset beyond the buffer: the range check answers those at once with zeros, no memory traffic.
-    auto issue = [&](int t, int stage) {
-        const bool beyond = kt_begin + t >= kt_end;
-        const unsigned int past_end = beyond ? 0x80000000u : 0u;
+    // The source of a tile is picked with scalar selects, not branches, so that the loads can be
+    // issued one by one between MFMAs.
+    auto cursors = [&](int t, TileCursor& ca, TileCursor& cb) {
+        const unsigned int past_end = kt_begin + t >= kt_end ? 0x80000000u : 0u;
         const int k0 = min(kt_begin + t, kt_end - 1) * kBK;
         if constexpr (A_K) {
-            if (k0 < a_end0) a_src.issue(smem + stage * kStage, k0, wave, past_end);
-            else if (k0 < a_end1) a_src1.issue(smem + stage * kStage, k0 - a_end0, wave, past_end);
-            else a_src2.issue(smem + stage * kStage, k0 - a_end1, wave, past_end);
+            const bool in1 = k0 >= a_end0, in2 = k0 >= a_end1;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) ca.rsrc[e] = in2 ? a_src2.rsrc[e] : in1 ? a_src1.rsrc[e] : a_src.rsrc[e];
+            ca.voffset = in2 ? a_src2.voffset : in1 ? a_src1.voffset : a_src.voffset;
+            const unsigned int group_bytes = in2 ? a_src2.group_bytes : in1 ? a_src1.group_bytes : a_src.group_bytes;
+            const int start = in2 ? a_end1 : in1 ? a_end0 : 0;
+            ca.soffset = (wave * group_bytes + (k0 - start) * static_cast<unsigned int>(sizeof(T))) | past_end;
+            ca.step = kWaves * group_bytes;
         } else {
-            a_src.issue(smem + stage * kStage, k0, wave, past_end);
+            ca.rsrc = a_src.rsrc;
+            ca.voffset = a_src.voffset;
+            ca.soffset = a_src.first_offset(k0, wave) | past_end;
+            ca.step = kWaves * a_src.group_bytes;
         }
-        b_src.issue(smem + stage * kStage + kATile, k0, wave, past_end);
+        cb.rsrc = b_src.rsrc;
+        cb.voffset = b_src.voffset;
+        cb.soffset = b_src.first_offset(k0, wave) | past_end;
+        cb.step = kWaves * b_src.group_bytes;
+    };
+    // Load l of a K tile (A's loads first, then B's) into the stage whose LDS address, advanced to
+    // this wavefront's first 1 KiB slot, is stage_lds. One load fills 1 KiB; the wavefronts' slots
+    // interleave, so a wavefront's consecutive loads are kWaves KiB apart.
+    constexpr int kLoadBytes = 64 * 16;
+    constexpr int kATileBytes = kATile * static_cast<int>(sizeof(T));
+    auto issue_one = [&](auto index, unsigned int stage_lds, TileCursor& ca, TileCursor& cb) {
+        constexpr int l = decltype(index)::value;
+        if constexpr (l < ATile::kLoads) {
+            ca.soffset = load_to_lds<l * kWaves * kLoadBytes>(ca.rsrc, stage_lds, ca.voffset, ca.soffset, ca.step);
+        } else {
+            cb.soffset = load_to_lds<kATileBytes + (l - ATile::kLoads) * kWaves * kLoadBytes>(
+                cb.rsrc, stage_lds, cb.voffset, cb.soffset, cb.step);
+        }
     };
     constexpr int kTileLoads = ATile::kLoads + BTile::kLoads;  // per wavefront and K tile
 
@@ -417,14 +482,24 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
     //   wait        this wavefront's loads of tile t+1 have landed; barrier: everybody's have, and
     //               nobody reads stage (t-1) % kStages any more
     //   last sub-step  MFMAs ‖ loads of tile t+kStages-1 into that stage ‖ fragments of tile t+1, sub-step 0
-    // so LDS latency and kStages-2 K tiles of global latency sit in the shadow of MFMAs.
+    // so LDS latency and kStages-2 K tiles of global latency sit in the shadow of MFMAs. With one
+    // wavefront per SIMD nothing else hides an instruction that is not next to an MFMA, so in the
+    // last sub-step every MFMA is followed by its share of the loads and fragment reads and a
+    // scheduling fence keeps them there.
     constexpr int kMfmas = TM * TN;
+    constexpr int kFrags = TM + TN;
     constexpr int kFragReads = TM * ATile::kFragReads + TN * BTile::kFragReads;
     constexpr int kSubSteps = kBK / 16;
+    constexpr unsigned int kStageBytes = kStage * sizeof(T);
     static_assert(kSubSteps % 2 == 0, "fragment sets alternate per sub-step and must line up across tiles");
     if (count > 0) {
+        const unsigned int lds_wave = lds_address_of(smem) + wave * kLoadBytes;
+        TileCursor ca, cb;
 #pragma unroll
-        for (int t = 0; t < kStages - 1; ++t) issue(t, t);
+        for (int t = 0; t < kStages - 1; ++t) {
+            cursors(t, ca, cb);
+            static_for<0, kTileLoads>([&](auto l) { issue_one(l, lds_wave + t * kStageBytes, ca, cb); });
+        }
         __builtin_amdgcn_s_waitcnt(vmcnt_immediate((kStages - 2) * kTileLoads));
         __syncthreads();
         read_frags(0, 0, 0);
@@ -432,6 +507,8 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
         int free_stage = kStages - 1;  // of tile t-1, refilled with tile t+kStages-1
         for (int t = 0; t < count; ++t) {
             const int next_stage = stage + 1 == kStages ? 0 : stage + 1;
+            cursors(t + kStages - 1, ca, cb);
+            const unsigned int free_lds = lds_wave + free_stage * kStageBytes;
 #pragma unroll
             for (int kk = 0; kk + 1 < kSubSteps; ++kk) {
                 read_frags((kk + 1) & 1, stage, kk + 1);
@@ -440,12 +517,27 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
                 __builtin_amdgcn_sched_barrier(0);
             }
             __builtin_amdgcn_s_waitcnt(vmcnt_immediate((kStages - 3) * kTileLoads));
-            __syncthreads();
-            issue(t + kStages - 1, free_stage);
-            read_frags(0, next_stage, 0);
-            multiply(1);
-            sched_interleave<kMfmas, kSchedDsRead, kFragReads, 0, 0>();
-            __builtin_amdgcn_sched_barrier(0);
+            barrier_only();
+            const T* next_a = smem + next_stage * kStage;
+            const T* next_b = next_a + kATile;
+            static_for<0, kMfmas>([&](auto index) {
+                constexpr int m = decltype(index)::value;
+                constexpr int i = m / TN, j = m % TN;
+                acc[i][j] = Mfma<T>::run(bf[1][j], af[1][i], acc[i][j]);
+                static_for<(m * kFrags) / kMfmas, ((m + 1) * kFrags) / kMfmas>([&](auto which) {
+                    constexpr int f = decltype(which)::value;
+                    if constexpr (f < TM) {
+                        if constexpr (A_K) af[0][f] = ATile::frag(next_a, wm * WM + f * 32, a_off[0]);
+                        else af[0][f] = ATile::frag(next_a, 0, a_off[f]);
+                    } else {
+                        if constexpr (B_K) bf[0][f - TM] = BTile::frag(next_b, wn * WN + (f - TM) * 32, b_off[0]);
+                        else bf[0][f - TM] = BTile::frag(next_b, 0, b_off[f - TM]);
+                    }
+                });
+                static_for<(m * kTileLoads) / kMfmas, ((m + 1) * kTileLoads) / kMfmas>(
+                    [&](auto l) { issue_one(l, free_lds, ca, cb); });
+                __builtin_amdgcn_sched_barrier(0);
+            });
             free_stage = stage;
             stage = next_stage;
         }
@@ -453,141 +545,139 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
     __builtin_amdgcn_s_waitcnt(vmcnt_immediate(0));  // the staging below reuses LDS that loads may still target
     __syncthreads();
 
-    // Epilogue. acc[i][j][4g+e] holds C[m, n] with m = lane%32, n = 8g + 4*(lane/32) + e. The tile
-    // goes through LDS and leaves it row by row, so that a wavefront stores whole contiguous row
-    // segments of C per instruction instead of 32 separate 16-byte pieces. When bias, residual or
-    // the old C are added (or the output is fp32 / a split-K partial), the staging is fp32 (row
-    // stride BN+4: the 16 lanes of a ds_write_b128 pass hit 16 different bank groups) and rounding
-    // to the storage dtype still happens once, after the additions.
-    constexpr int kStageStride = BN + 4;
-    constexpr int kSmemBytes = Layout::kSmemBytes;
-    constexpr int kPassRows = (BM * kStageStride * 4 <= kSmemBytes) ? BM : BM / 2;
-    constexpr int kPasses = BM / kPassRows;
-    static_assert(kPassRows * kStageStride * 4 <= kSmemBytes, "epilogue staging does not fit in LDS");
-    static_assert(kPasses == 1 || kPassRows == WM, "a pass must be one row of wavefronts");
+    // Epilogue. acc[i][j][4g+e] holds C[m, n] with m = lane%32, n = 8g + 4*(lane/32) + e, relative
+    // to block (i, j) of the wavefront's WM x WN part of the tile. Each wavefront passes its part
+    // through a private quarter of the last LDS stage, 32 rows at a time, and stores it row by row:
+    // whole contiguous row segments of C per instruction instead of 32 separate 8-byte pieces, and
+    // no workgroup barrier. When bias, residual or the old C are added (or the output is fp32 / a
+    // split-K partial) the staging is fp32, half the columns per pass, and rounding to the storage
+    // dtype still happens once, after the additions; otherwise the values are rounded in registers
+    // and staged in the storage dtype. A staged row is kRowBytes long; its 16-byte chunk c sits at
+    // chunk position c ^ sw(row), which spreads both the column-wise writes and the row-wise reads
+    // over all banks.
+    constexpr int kRowBytes = WN * static_cast<int>(sizeof(T));
+    constexpr int kRowChunks = kRowBytes / 16;
+    static_assert(32 * kRowBytes * kWaves == static_cast<int>(kStageBytes), "staging is a quarter stage per wavefront");
+    unsigned char* region = smem_raw + (kStages - 1) * kStageBytes + wave * (kStageBytes / kWaves);
+    auto sw = [](int row) { return (row / (256 / kRowBytes)) % kRowChunks; };
     // C may be given as column segments too: this tile's columns then belong to one of them.
     void* c_base = p.c;
     long c_ld = p.ldc;
     int c_col0 = n0, c_cols = p.n;
     if (p.c_seg.count > 0) {
-        int s = 0, first = 0;
-        while (s + 1 < p.c_seg.count && n0 >= first + p.c_seg.cols[s]) first += p.c_seg.cols[s++];
-        c_base = const_cast<void*>(p.c_seg.ptr[s]);
-        c_ld = p.c_seg.ld[s];
-        c_col0 = n0 - first;
-        c_cols = p.c_seg.cols[s];
+        const SegmentPick pick = pick_segment(p.c_seg, n0);
+        c_base = const_cast<void*>(pick.ptr);
+        c_ld = pick.ld;
+        c_col0 = n0 - pick.first;
+        c_cols = pick.cols;
     }
-    const int m_lane = lane & 31, n_lane = (lane >> 5) * 4;
+    const int m_lane = lane & 31, h_lane = lane >> 5;
+    unsigned char* write_row = region + m_lane * kRowBytes;
+    const int write_sw = sw(m_lane);
+    // Stages blocks (i, j0 .. j0+JP-1) as element type S and hands each lane 8 consecutive staged
+    // elements at a time: consume(row, col, pointer to the 8 elements' first chunk, to the second
+    // chunk when S is float), row/col relative to the wavefront's part.
+    auto pass = [&]<typename S, int JP>(int i, int j0, auto&& consume) {
+        static_assert(JP * 32 * sizeof(S) == kRowBytes, "a pass fills whole staged rows");
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int jj = 0; jj < JP; ++jj) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                vec_t<float, 4> v;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = acc[i][j0 + jj][4 * g + e];
+                const int byte = (jj * 32 + g * 8 + h_lane * 4) * static_cast<int>(sizeof(S));
+                unsigned char* slot = write_row + (((byte / 16) ^ write_sw) * 16) + byte % 16;
+                if constexpr (std::is_same_v<S, float>) *reinterpret_cast<vec_t<float, 4>*>(slot) = v;
+                else store_vec<T, 4>(reinterpret_cast<T*>(slot), vec_from_f32<T, 4>(v));
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+        constexpr int kLanesPerRow = kRowBytes / (8 * static_cast<int>(sizeof(S)));
+        constexpr int kChunksPerLane = 8 * static_cast<int>(sizeof(S)) / 16;
+        constexpr int kRounds = 32 * kLanesPerRow / kWave;
+#pragma unroll
+        for (int u = 0; u < kRounds; ++u) {
+            const int q = u * kWave + lane;
+            const int row = q / kLanesPerRow, part = q % kLanesPerRow;
+            const unsigned char* base = region + row * kRowBytes;
+            const int first = part * kChunksPerLane;
+            consume(i * 32 + row, j0 * 32 + part * 8, base + ((first ^ sw(row)) * 16),
+                    base + (((first + kChunksPerLane - 1) ^ sw(row)) * 16));
+        }
+    };
+    const int row0 = m0 + wm * WM, col0 = wn * WN;  // of the wavefront's part; columns relative to n0
     if constexpr (!SPLIT) {
         if (p.bias == nullptr && p.residual == nullptr && !p.accumulate && !p.c_f32) {
-            // Nothing is added to the product: round in registers, stage the whole tile in the
-            // storage dtype (one pass, half the LDS traffic) and store 16 bytes per lane, eight
-            // chunks in flight per thread.
-            constexpr int kTileStride = BN + 8;
-            static_assert(BM * kTileStride * static_cast<int>(sizeof(T)) <= kSmemBytes, "tile staging does not fit in LDS");
-            T* tile = smem;
+            T* out = static_cast<T*>(c_base);
 #pragma unroll
             for (int i = 0; i < TM; ++i) {
-#pragma unroll
-                for (int j = 0; j < TN; ++j) {
-#pragma unroll
-                    for (int g = 0; g < 4; ++g) {
-                        vec_t<float, 4> v;
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) v[e] = acc[i][j][4 * g + e];
-                        store_vec<T, 4>(tile + (wm * WM + i * 32 + m_lane) * kTileStride + wn * WN + j * 32 + g * 8 + n_lane,
-                                        vec_from_f32<T, 4>(v));
-                    }
-                }
-            }
-            __syncthreads();
-            constexpr int kChunksPerRow = BN / 8;
-            constexpr int kPerThread = BM * kChunksPerRow / kThreads;
-            constexpr int kUnroll = 8;
-            static_assert(kPerThread % kUnroll == 0, "copy-out unrolling");
-            T* out = static_cast<T*>(c_base);
-            for (int base = 0; base < kPerThread; base += kUnroll) {
-                u32x4 data[kUnroll];
-#pragma unroll
-                for (int u = 0; u < kUnroll; ++u) {
-                    const int c = (base + u) * kThreads + threadIdx.x;
-                    const int r = c / kChunksPerRow, col = (c % kChunksPerRow) * 8;
-                    data[u] = *reinterpret_cast<const u32x4*>(tile + r * kTileStride + col);
-                }
-#pragma unroll
-                for (int u = 0; u < kUnroll; ++u) {
-                    const int c = (base + u) * kThreads + threadIdx.x;
-                    const int r = c / kChunksPerRow, col = (c % kChunksPerRow) * 8;
-                    const int m = m0 + r, c_col = c_col0 + col;
-                    if (m < p.m && c_col < c_cols)
-                        *reinterpret_cast<u32x4*>(out + static_cast<long>(m) * c_ld + c_col) = data[u];
-                }
+                pass.template operator()<T, TN>(i, 0, [&](int row, int col, const unsigned char* lo, const unsigned char*) {
+                    const int m = row0 + row, c_col = c_col0 + col0 + col;
+                    const u32x4 data = *reinterpret_cast<const u32x4*>(lo);
+                    if (m < p.m && c_col < c_cols) *reinterpret_cast<u32x4*>(out + static_cast<long>(m) * c_ld + c_col) = data;
+                });
             }
             return;
         }
     }
-    float* stage = reinterpret_cast<float*>(smem_raw);
 #pragma unroll
-    for (int pass = 0; pass < kPasses; ++pass) {
-        if (kPasses == 1 || wm == pass) {
-            const int row_base = kPasses == 1 ? wm * WM : 0;
+    for (int i = 0; i < TM; ++i) {
 #pragma unroll
-            for (int i = 0; i < TM; ++i) {
-#pragma unroll
-                for (int j = 0; j < TN; ++j) {
-#pragma unroll
-                    for (int g = 0; g < 4; ++g) {
-                        vec_t<float, 4> v;
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) v[e] = acc[i][j][4 * g + e];
-                        const int row = row_base + i * 32 + m_lane;
-                        const int col = wn * WN + j * 32 + g * 8 + n_lane;
-                        *reinterpret_cast<vec_t<float, 4>*>(stage + row * kStageStride + col) = v;
-                    }
-                }
-            }
-        }
-        __syncthreads();
-        constexpr int kChunksPerRow = BN / 4;
-        constexpr int kChunks = kPassRows * kChunksPerRow;
-        constexpr int kBatch = 4;  // LDS reads in flight per thread before the dependent global accesses
-        static_assert(kChunks % (kThreads * kBatch) == 0, "copy-out batching");
-        for (int first = threadIdx.x; first < kChunks; first += kThreads * kBatch) {
-            vec_t<float, 4> staged[kBatch];
-#pragma unroll
-            for (int u = 0; u < kBatch; ++u) {
-                const int c = first + u * kThreads;
-                staged[u] = *reinterpret_cast<const vec_t<float, 4>*>(stage + (c / kChunksPerRow) * kStageStride +
-                                                                      (c % kChunksPerRow) * 4);
-            }
-#pragma unroll
-            for (int u = 0; u < kBatch; ++u) {
-                const int c = first + u * kThreads;
-                const int r = c / kChunksPerRow, col = (c % kChunksPerRow) * 4;
-                const int m = m0 + pass * kPassRows + r, n = n0 + col, c_col = c_col0 + col;
-                if (m >= p.m || c_col >= c_cols) continue;
-                vec_t<float, 4> v = staged[u];
+        for (int half = 0; half < 2; ++half) {
+            pass.template operator()<float, TN / 2>(i, half * (TN / 2), [&](int row, int col, const unsigned char* lo,
+                                                                           const unsigned char* hi) {
+                const int m = row0 + row, n = n0 + col0 + col, c_col = c_col0 + col0 + col;
+                vec_t<float, 4> v0 = *reinterpret_cast<const vec_t<float, 4>*>(lo);
+                vec_t<float, 4> v1 = *reinterpret_cast<const vec_t<float, 4>*>(hi);
+                if (m >= p.m || c_col >= c_cols) return;
                 if constexpr (SPLIT) {
                     float* out = static_cast<float*>(p.c) +
                                  (static_cast<long>(blockIdx.y) * p.m + m) * static_cast<long>(p.n) + n;
-                    *reinterpret_cast<vec_t<float, 4>*>(out) = v;
+                    *reinterpret_cast<vec_t<float, 4>*>(out) = v0;
+                    *reinterpret_cast<vec_t<float, 4>*>(out + 4) = v1;
                 } else {
-                    if (p.bias != nullptr) v += vec_to_f32<T, 4>(load_vec<T, 4>(static_cast<const T*>(p.bias) + n));
-                    if (p.residual != nullptr)
-                        v += vec_to_f32<T, 4>(load_vec<T, 4>(static_cast<const T*>(p.residual) + static_cast<long>(m) * p.ldr + n));
+                    if (p.bias != nullptr) {
+                        const T* bias = static_cast<const T*>(p.bias) + n;
+                        v0 += vec_to_f32<T, 4>(load_vec<T, 4>(bias));
+                        v1 += vec_to_f32<T, 4>(load_vec<T, 4>(bias + 4));
+                    }
+                    if (p.residual != nullptr) {
+                        const T* residual = static_cast<const T*>(p.residual) + static_cast<long>(m) * p.ldr + n;
+                        v0 += vec_to_f32<T, 4>(load_vec<T, 4>(residual));
+                        v1 += vec_to_f32<T, 4>(load_vec<T, 4>(residual + 4));
+                    }
                     if (p.c_f32) {
                         float* out = static_cast<float*>(c_base) + static_cast<long>(m) * c_ld + c_col;
-                        if (p.accumulate) v += *reinterpret_cast<const vec_t<float, 4>*>(out);
-                        *reinterpret_cast<vec_t<float, 4>*>(out) = v;
+                        if (p.accumulate) {
+                            v0 += *reinterpret_cast<const vec_t<float, 4>*>(out);
+                            v1 += *reinterpret_cast<const vec_t<float, 4>*>(out + 4);
+                        }
+                        *reinterpret_cast<vec_t<float, 4>*>(out) = v0;
+                        *reinterpret_cast<vec_t<float, 4>*>(out + 4) = v1;
                     } else {
                         T* out = static_cast<T*>(c_base) + static_cast<long>(m) * c_ld + c_col;
-                        if (p.accumulate) v += vec_to_f32<T, 4>(load_vec<T, 4>(out));
-                        store_vec<T, 4>(out, vec_from_f32<T, 4>(v));
+                        if (p.accumulate) {
+                            const vec_t<T, 8> old = load_vec<T, 8>(out);
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) {
+                                v0[e] += to_f32(old[e]);
+                                v1[e] += to_f32(old[4 + e]);
+                            }
+                        }
+                        vec_t<T, 8> packed;
+                        const vec_t<T, 4> r0 = vec_from_f32<T, 4>(v0), r1 = vec_from_f32<T, 4>(v1);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            packed[e] = r0[e];
+                            packed[4 + e] = r1[e];
+                        }
+                        store_vec<T, 8>(out, packed);
                     }
                 }
-            }
+            });
         }
-        if (pass + 1 < kPasses) __syncthreads();
     }
 }
 
@@ -702,13 +792,13 @@ int launch_layout(const KernelArgs& p, bool a_k, bool b_k, int slices, hipStream
     return fail(CGPTX_RUNTIME, "gemm: unsupported operand layout");
 }
 
-// CGPTX_GEMM_TILE=128|256|384 pins the tile size (384 = 128x256; for experiments); anything else = automatic.
+// CGPTX_GEMM_TILE=128|256 pins the tile size (for experiments); anything else = automatic.
 int forced_tile() {
     static const int value = [] {
         const char* text = std::getenv("CGPTX_GEMM_TILE");
         if (text == nullptr) return 0;
         const int v = std::atoi(text);
-        return (v == 128 || v == 256 || v == 384) ? v : 0;
+        return (v == 128 || v == 256) ? v : 0;
     }();
     return value;
 }
@@ -768,7 +858,8 @@ int copy_segments(const GemmSegments& in, std::size_t total, std::size_t granule
 // The streamed loads address an operand relative to the block's tile origin with 32-bit byte
 // offsets: a tile's rows (k-contiguous operand) or the whole K extent (n-contiguous operand).
 bool offsets_fit_32bit(const GemmArgs& g, std::size_t elem) {
-    constexpr std::size_t limit = (std::size_t{1} << 32) - (std::size_t{1} << 20);
+    // Below 2 GiB: bit 31 of a scalar offset is what pushes the loads of K tiles past the end out of range.
+    constexpr std::size_t limit = (std::size_t{1} << 31) - (std::size_t{1} << 20);
     const std::size_t a_span = g.a_k_contiguous ? (256 * g.lda + g.k) * elem : (g.k * g.lda + 256) * elem;
     const std::size_t b_span = g.b_k_contiguous ? (256 * g.ldb + g.k) * elem : (g.k * g.ldb + 256) * elem;
     return a_span < limit && b_span < limit;
@@ -841,7 +932,6 @@ int run_typed(const GemmArgs& g, hipStream_t stream) {
         const bool splits = !g.no_split && g.residual == nullptr && g.c_segments.count == 0 && big_tiles >= 8 &&
                             g.k / kBK >= static_cast<std::size_t>(32 * ((units + big_tiles - 1) / big_tiles));
         const bool big = forced == 256 || (forced == 0 && (fills || splits));
-        if (forced == 384) return run_config<T, 128, 256>(g, p, stream);
         if (big) return run_config<T, 256, 256>(g, p, stream);
         return run_config<T, 128, 128>(g, p, stream);
     }
