@@ -97,7 +97,8 @@ struct KernelArgs {
     int m, n, k;
     long lda, ldb, ldc, ldr;
     int tiles_m, tiles_n;
-    int k_tiles_per_slice;  // K tiles (of 64) handled by one blockIdx.y
+    int k_tiles_per_slice;  // K tiles handled by one work item
+    int slices;             // K slices per output tile
     int accumulate;
     int c_f32;
     KernelSegments a_seg, c_seg;  // column segments of A (as stored) and of C; count 0 = one buffer
@@ -146,14 +147,18 @@ __device__ __forceinline__ void sched_interleave() {
 // (and for nothing else).
 constexpr int vmcnt_immediate(int count) { return (count & 15) | ((count >> 4) << 14) | 0x0F70; }
 
-// Buffer descriptor (raw buffer, range-checked) over `bytes` bytes starting at base.
+// Buffer descriptor (raw buffer, range-checked) over `bytes` bytes starting at base (both the same
+// for all lanes). The words are pinned to scalar registers: 64-bit comparisons have no scalar form,
+// and one of them on the way would drag the descriptor, and every address derived with it, into
+// vector registers.
 __device__ __forceinline__ u32x4 make_rsrc(const void* base, long bytes) {
     const unsigned long address = reinterpret_cast<unsigned long>(base);
-    const long limit = 0xFFFFFFFFl;
+    const unsigned int size_low = static_cast<unsigned int>(bytes);
+    const unsigned int size_high = static_cast<unsigned int>(static_cast<unsigned long>(bytes) >> 32);
     u32x4 words;
-    words[0] = static_cast<unsigned int>(address);
-    words[1] = static_cast<unsigned int>(address >> 32) & 0xFFFFu;  // stride 0
-    words[2] = static_cast<unsigned int>(bytes < limit ? bytes : limit);
+    words[0] = __builtin_amdgcn_readfirstlane(static_cast<unsigned int>(address));
+    words[1] = __builtin_amdgcn_readfirstlane(static_cast<unsigned int>(address >> 32) & 0xFFFFu);  // stride 0
+    words[2] = __builtin_amdgcn_readfirstlane(size_high != 0 ? 0xFFFFFFFFu : size_low);
     words[3] = 0x00020000u;
     return words;
 }
@@ -239,7 +244,7 @@ struct KTile {
         // The tile row of this lane's slot is (i*4 + wave) * kRowsPerLoad + row; its swizzle does not depend on i.
         voffset = static_cast<int>(row * ld * sizeof(T)) +
                   (((lane % kChunksPerRow) ^ swizzle(wave * kRowsPerLoad + row)) * 16);
-        group_bytes = static_cast<unsigned int>(kRowsPerLoad * ld * sizeof(T));
+        group_bytes = __builtin_amdgcn_readfirstlane(static_cast<unsigned int>(kRowsPerLoad * ld * sizeof(T)));
     }
     // Scalar offset of wavefront `wave`'s first load of the tile that starts at column k0.
     __device__ __forceinline__ unsigned int first_offset(int k0, int wave) const {
@@ -283,7 +288,7 @@ struct NTile {
         const int k_row = (wave * kRowsPerLoad + row) & 3;     // low bits of the tile row (groups step by 4*kRowsPerLoad)
         const int chunk = min((lane % kChunksPerRow) ^ (k_row << 2), cols_left / 8 - 1);
         voffset = static_cast<int>(row * ld * sizeof(T)) + chunk * 16;
-        group_bytes = static_cast<unsigned int>(kRowsPerLoad * ld * sizeof(T));
+        group_bytes = __builtin_amdgcn_readfirstlane(static_cast<unsigned int>(kRowsPerLoad * ld * sizeof(T)));
     }
     // Scalar offset of wavefront `wave`'s first load of the tile that starts at row k0.
     __device__ __forceinline__ unsigned int first_offset(int k0, int wave) const {
@@ -322,12 +327,16 @@ struct TileLayout {
     static constexpr int kSmemBytes = kStages * kStage * static_cast<int>(sizeof(T));
 };
 
+// One workgroup per CU slot walks its share of the work items (output tile x K slice) one after
+// the other: the first K tiles of the next item are requested before the epilogue of the current
+// one, whose stores then drain under the next item's MFMAs.
 template <typename T, int BM, int BN, bool A_K, bool B_K, bool SPLIT>
 __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
     using frag_t = typename Mfma<T>::frag;
     using Layout = TileLayout<T, BM, BN, A_K, B_K>;
     using ATile = typename Layout::ATile;
     using BTile = typename Layout::BTile;
+    static_assert(BM == BN, "the epilogue staging assumes square tiles");
     constexpr int WM = BM / 2, WN = BN / 2;
     constexpr int TM = WM / 32, TN = WN / 32;
     extern __shared__ __align__(1024) unsigned char smem_raw[];
@@ -336,83 +345,114 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
     constexpr int kStage = Layout::kStage;
     constexpr int kStages = Layout::kStages;
     constexpr int kATile = ATile::kElems;
-
-    // XCD-contiguous, grouped tile order.
-    const int total = p.tiles_m * p.tiles_n;
-    const int per_xcd = (total + kXcds - 1) / kXcds;
-    const int logical = (blockIdx.x % kXcds) * per_xcd + blockIdx.x / kXcds;
-    if (logical >= total) return;
-    const int group_size = kGroupRows * p.tiles_n;
-    const int group = logical / group_size;
-    const int first_m = group * kGroupRows;
-    const int rows_in_group = min(p.tiles_m - first_m, kGroupRows);
-    const int in_group = logical - group * group_size;
-    const int tile_m = first_m + in_group % rows_in_group;
-    const int tile_n = in_group / rows_in_group;
-    const int m0 = tile_m * BM, n0 = tile_n * BN;
-
-    const int k_tiles_total = p.k / kBK;
-    const int kt_begin = blockIdx.y * p.k_tiles_per_slice;
-    const int kt_end = min(k_tiles_total, kt_begin + p.k_tiles_per_slice);
-    const int count = kt_end - kt_begin;
+    constexpr unsigned int kStageBytes = kStage * sizeof(T);
 
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const int wm = wave >> 1, wn = wave & 1;
 
-    // A may be given as up to three column segments in separate buffers. Stored [M, K]: the K range
-    // is segmented and the source changes along the K loop (boundaries a_end0 / a_end1). Stored
-    // [K, M]: the M range is segmented and this block's rows pick their buffer once.
+    // Work items are numbered slice-major (all tiles of K slice 0, then of slice 1, ...), tiles in
+    // groups of kGroupRows tile-rows, down the rows first. Blocks are dealt round-robin to the 8
+    // XCDs, so XCD x takes the x-th eighth of the items and its blocks walk it side by side: the
+    // items in flight on one XCD are neighbours and share A and B panels in that XCD's L2.
+    const int tiles = p.tiles_m * p.tiles_n;
+    const int items = tiles * p.slices;
+    const int per_xcd = (items + kXcds - 1) / kXcds;
+    const int item_stride = gridDim.x / kXcds;
+    const int item_end = min(items, static_cast<int>(blockIdx.x % kXcds + 1) * per_xcd);
+    int item = static_cast<int>(blockIdx.x % kXcds) * per_xcd + static_cast<int>(blockIdx.x / kXcds);
+    if (item >= item_end) return;
+
+    struct Item {
+        int m0, n0, slice, kt_begin, kt_end;
+    };
+    auto locate = [&](int index) __attribute__((always_inline)) {
+        Item w;
+        w.slice = index / tiles;
+        const int logical = index - w.slice * tiles;
+        const int group_size = kGroupRows * p.tiles_n;
+        const int group = logical / group_size;
+        const int first_m = group * kGroupRows;
+        const int rows_in_group = min(p.tiles_m - first_m, kGroupRows);
+        const int in_group = logical - group * group_size;
+        w.m0 = (first_m + in_group % rows_in_group) * BM;
+        w.n0 = (in_group / rows_in_group) * BN;
+        w.kt_begin = w.slice * p.k_tiles_per_slice;
+        w.kt_end = min(p.k / kBK, w.kt_begin + p.k_tiles_per_slice);
+        return w;
+    };
+
+    // The operand sources of the item whose K tiles are being requested. A may be given as up to
+    // three column segments in separate buffers. Stored [M, K]: the K range is segmented and the
+    // source changes along the K loop (boundaries a_end0 / a_end1). Stored [K, M]: the M range is
+    // segmented and the item's rows pick their buffer once.
     ATile a_src, a_src1, a_src2;
     BTile b_src;
     int a_end0 = std::numeric_limits<int>::max(), a_end1 = std::numeric_limits<int>::max();
-    if constexpr (A_K) {
-        if (p.a_seg.count == 0) {
-            a_src.init(static_cast<const T*>(p.a) + static_cast<long>(m0) * p.lda, p.lda, p.m - m0, p.k, wave);
+    int src_begin = 0, src_end = 0;  // K tiles of that item
+    auto open = [&](const Item& w) __attribute__((always_inline)) {
+        const int m0 = w.m0, n0 = w.n0;
+        src_begin = w.kt_begin;
+        src_end = w.kt_end;
+        if constexpr (A_K) {
+            // All three sources are set up unconditionally (absent segments repeat the first and
+            // are never selected): conditional set-up would be merged into one piece of code that
+            // writes through a pointer, which keeps the sources in memory.
+            const int segments = p.a_seg.count;
+            const void* ptr0 = segments == 0 ? p.a : p.a_seg.ptr[0];
+            const long ld0 = segments == 0 ? p.lda : p.a_seg.ld[0];
+            const int cols0 = segments == 0 ? p.k : p.a_seg.cols[0];
+            const void* ptr1 = segments > 1 ? p.a_seg.ptr[1] : ptr0;
+            const long ld1 = segments > 1 ? p.a_seg.ld[1] : ld0;
+            const int cols1 = segments > 1 ? p.a_seg.cols[1] : cols0;
+            const void* ptr2 = segments > 2 ? p.a_seg.ptr[2] : ptr0;
+            const long ld2 = segments > 2 ? p.a_seg.ld[2] : ld0;
+            const int cols2 = segments > 2 ? p.a_seg.cols[2] : cols0;
+            a_src.init(static_cast<const T*>(ptr0) + static_cast<long>(m0) * ld0, ld0, p.m - m0, cols0, wave);
+            a_src1.init(static_cast<const T*>(ptr1) + static_cast<long>(m0) * ld1, ld1, p.m - m0, cols1, wave);
+            a_src2.init(static_cast<const T*>(ptr2) + static_cast<long>(m0) * ld2, ld2, p.m - m0, cols2, wave);
+            a_end0 = segments > 1 ? cols0 : std::numeric_limits<int>::max();
+            a_end1 = segments > 2 ? cols0 + cols1 : std::numeric_limits<int>::max();
         } else {
-            a_src.init(static_cast<const T*>(p.a_seg.ptr[0]) + static_cast<long>(m0) * p.a_seg.ld[0], p.a_seg.ld[0],
-                       p.m - m0, p.a_seg.cols[0], wave);
-            if (p.a_seg.count > 1) {
-                a_end0 = p.a_seg.cols[0];
-                a_src1.init(static_cast<const T*>(p.a_seg.ptr[1]) + static_cast<long>(m0) * p.a_seg.ld[1],
-                            p.a_seg.ld[1], p.m - m0, p.a_seg.cols[1], wave);
+            const T* base = static_cast<const T*>(p.a);
+            long ld = p.lda;
+            int first = 0, width = p.m;
+            if (p.a_seg.count > 0) {
+                const SegmentPick pick = pick_segment(p.a_seg, m0);
+                base = static_cast<const T*>(pick.ptr);
+                ld = pick.ld;
+                first = pick.first;
+                width = pick.cols;
             }
-            if (p.a_seg.count > 2) {
-                a_end1 = a_end0 + p.a_seg.cols[1];
-                a_src2.init(static_cast<const T*>(p.a_seg.ptr[2]) + static_cast<long>(m0) * p.a_seg.ld[2],
-                            p.a_seg.ld[2], p.m - m0, p.a_seg.cols[2], wave);
-            }
+            a_src.init(base + (m0 - first), ld, width - (m0 - first), p.k, wave);
         }
-    } else {
-        const T* base = static_cast<const T*>(p.a);
-        long ld = p.lda;
-        int first = 0, width = p.m;
-        if (p.a_seg.count > 0) {
-            const SegmentPick pick = pick_segment(p.a_seg, m0);
-            base = static_cast<const T*>(pick.ptr);
-            ld = pick.ld;
-            first = pick.first;
-            width = pick.cols;
-        }
-        a_src.init(base + (m0 - first), ld, width - (m0 - first), p.k, wave);
-    }
-    if constexpr (B_K) b_src.init(static_cast<const T*>(p.b) + static_cast<long>(n0) * p.ldb, p.ldb, p.n - n0, p.k, wave);
-    else b_src.init(static_cast<const T*>(p.b) + n0, p.ldb, p.n - n0, p.k, wave);
+        if constexpr (B_K) b_src.init(static_cast<const T*>(p.b) + static_cast<long>(n0) * p.ldb, p.ldb, p.n - n0, p.k, wave);
+        else b_src.init(static_cast<const T*>(p.b) + n0, p.ldb, p.n - n0, p.k, wave);
+    };
     // K tiles past the end of the slice are still "loaded" (the loop stays free of data-dependent
     // branches and every wavefront always has the same number of loads in flight), but from an
     // offset beyond the buffer: the range check answers those at once with zeros, no memory traffic.
     // The source of a tile is picked with scalar selects, not branches, so that the loads can be
     // issued one by one between MFMAs.
-    auto cursors = [&](int t, TileCursor& ca, TileCursor& cb) {
-        const unsigned int past_end = kt_begin + t >= kt_end ? 0x80000000u : 0u;
-        const int k0 = min(kt_begin + t, kt_end - 1) * kBK;
+    auto cursors = [&](int t, TileCursor& ca, TileCursor& cb) __attribute__((always_inline)) {
+        const unsigned int past_end = src_begin + t >= src_end ? 0x80000000u : 0u;
+        const int k0 = min(src_begin + t, src_end - 1) * kBK;
         if constexpr (A_K) {
+            // Values first, then selects: a conditional between the objects' members would select
+            // an address and keep all three sources in memory.
             const bool in1 = k0 >= a_end0, in2 = k0 >= a_end1;
+            const u32x4 rsrc0 = a_src.rsrc, rsrc1 = a_src1.rsrc, rsrc2 = a_src2.rsrc;
+            const int voffset0 = a_src.voffset, voffset1 = a_src1.voffset, voffset2 = a_src2.voffset;
+            const unsigned int bytes0 = a_src.group_bytes, bytes1 = a_src1.group_bytes, bytes2 = a_src2.group_bytes;
+            const int end0 = a_end0, end1 = a_end1;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) ca.rsrc[e] = in2 ? a_src2.rsrc[e] : in1 ? a_src1.rsrc[e] : a_src.rsrc[e];
-            ca.voffset = in2 ? a_src2.voffset : in1 ? a_src1.voffset : a_src.voffset;
-            const unsigned int group_bytes = in2 ? a_src2.group_bytes : in1 ? a_src1.group_bytes : a_src.group_bytes;
-            const int start = in2 ? a_end1 : in1 ? a_end0 : 0;
+            for (int e = 0; e < 4; ++e) {
+                const unsigned int w0 = rsrc0[e], w1 = rsrc1[e], w2 = rsrc2[e];
+                ca.rsrc[e] = in2 ? w2 : in1 ? w1 : w0;
+            }
+            ca.voffset = in2 ? voffset2 : in1 ? voffset1 : voffset0;
+            const unsigned int group_bytes = in2 ? bytes2 : in1 ? bytes1 : bytes0;
+            const int start = in2 ? end1 : in1 ? end0 : 0;
             ca.soffset = (wave * group_bytes + (k0 - start) * static_cast<unsigned int>(sizeof(T))) | past_end;
             ca.step = kWaves * group_bytes;
         } else {
@@ -431,7 +471,7 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
     // interleave, so a wavefront's consecutive loads are kWaves KiB apart.
     constexpr int kLoadBytes = 64 * 16;
     constexpr int kATileBytes = kATile * static_cast<int>(sizeof(T));
-    auto issue_one = [&](auto index, unsigned int stage_lds, TileCursor& ca, TileCursor& cb) {
+    auto issue_one = [&](auto index, unsigned int stage_lds, TileCursor& ca, TileCursor& cb) __attribute__((always_inline)) {
         constexpr int l = decltype(index)::value;
         if constexpr (l < ATile::kLoads) {
             ca.soffset = load_to_lds<l * kWaves * kLoadBytes>(ca.rsrc, stage_lds, ca.voffset, ca.soffset, ca.step);
@@ -441,6 +481,16 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
         }
     };
     constexpr int kTileLoads = ATile::kLoads + BTile::kLoads;  // per wavefront and K tile
+    const unsigned int lds_wave = lds_address_of(smem) + wave * kLoadBytes;
+    TileCursor ca, cb;
+    // Requests K tiles FIRST .. LAST-1 of the opened item into the stages of the same numbers.
+    auto request_tiles = [&]<int FIRST, int LAST>() __attribute__((always_inline)) {
+        static_for<FIRST, LAST>([&](auto index) {
+            constexpr int t = decltype(index)::value;
+            cursors(t, ca, cb);
+            static_for<0, kTileLoads>([&](auto l) { issue_one(l, lds_wave + t * kStageBytes, ca, cb); });
+        });
+    };
 
     int a_off[ATile::kOffsets], b_off[BTile::kOffsets];
 #pragma unroll
@@ -449,13 +499,8 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
     for (int j = 0; j < BTile::kOffsets; ++j) b_off[j] = BTile::lane_offset(lane, wn * WN + j * 32, j);
 
     acc_t acc[TM][TN];
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j) acc[i][j] = acc_t(0.0f);
-
     frag_t af[2][TM], bf[2][TN];
-    auto read_frags = [&](int set, int stage, int kk) {
+    auto read_frags = [&](int set, int stage, int kk) __attribute__((always_inline)) {
         const T* as = smem + stage * kStage;
         const T* bs = as + kATile;
 #pragma unroll
@@ -469,15 +514,164 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
             else bf[set][j] = BTile::frag(bs, kk, b_off[j]);
         }
     };
-    auto multiply = [&](int set) {
+    auto multiply = [&](int set) __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
             for (int j = 0; j < TN; ++j) acc[i][j] = Mfma<T>::run(bf[set][j], af[set][i], acc[i][j]);
     };
 
-    // Software pipeline over K tiles t = 0 .. count-1 (tile t lives in LDS stage t % kStages; tiles
-    // t+1 .. t+kStages-2 are in flight or landed), kBK/16 K sub-steps of 16 per tile:
+    // Epilogue staging. acc[i][j][4g+e] holds C[m, n] with m = lane%32, n = 8g + 4*(lane/32) + e,
+    // relative to block (i, j) of the wavefront's WM x WN part of the tile. Each wavefront passes
+    // its part through a private quarter of the last LDS stage (the only one the first K tiles of
+    // the next item do not fill), 32 rows at a time, and stores it row by row: whole contiguous
+    // row segments of C per instruction instead of 32 separate 8-byte pieces, and no workgroup
+    // barrier. When bias, residual or the old C are added (or the output is fp32 / a split-K
+    // partial) the staging is fp32, half the columns per pass, and rounding to the storage dtype
+    // still happens once, after the additions; otherwise the values are rounded in registers and
+    // staged in the storage dtype. A staged row is kRowBytes long; its 16-byte chunk c sits at
+    // chunk position c ^ sw(row), which spreads both the column-wise writes and the row-wise reads
+    // over all banks.
+    constexpr int kRowBytes = WN * static_cast<int>(sizeof(T));
+    constexpr int kRowChunks = kRowBytes / 16;
+    static_assert(32 * kRowBytes * kWaves == static_cast<int>(kStageBytes), "staging is a quarter stage per wavefront");
+    unsigned char* region = smem_raw + (kStages - 1) * kStageBytes + wave * (kStageBytes / kWaves);
+    auto sw = [](int row) { return (row / (256 / kRowBytes)) % kRowChunks; };
+    const int m_lane = lane & 31, h_lane = lane >> 5;
+    unsigned char* write_row = region + m_lane * kRowBytes;
+    const int write_sw = sw(m_lane);
+    // Stages blocks (i, j0 .. j0+JP-1) as element type S and hands each lane 8 consecutive staged
+    // elements at a time: consume(row, col, pointer to the 8 elements' first chunk, to the second
+    // chunk when S is float), row/col relative to the wavefront's part.
+    auto pass = [&]<typename S, int JP>(int i, int j0, auto&& consume) __attribute__((always_inline)) {
+        static_assert(JP * 32 * sizeof(S) == kRowBytes, "a pass fills whole staged rows");
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int jj = 0; jj < JP; ++jj) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                vec_t<float, 4> v;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = acc[i][j0 + jj][4 * g + e];
+                const int byte = (jj * 32 + g * 8 + h_lane * 4) * static_cast<int>(sizeof(S));
+                unsigned char* slot = write_row + (((byte / 16) ^ write_sw) * 16) + byte % 16;
+                if constexpr (std::is_same_v<S, float>) *reinterpret_cast<vec_t<float, 4>*>(slot) = v;
+                else store_vec<T, 4>(reinterpret_cast<T*>(slot), vec_from_f32<T, 4>(v));
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+        constexpr int kLanesPerRow = kRowBytes / (8 * static_cast<int>(sizeof(S)));
+        constexpr int kChunksPerLane = 8 * static_cast<int>(sizeof(S)) / 16;
+        constexpr int kRounds = 32 * kLanesPerRow / kWave;
+#pragma unroll
+        for (int u = 0; u < kRounds; ++u) {
+            const int q = u * kWave + lane;
+            const int row = q / kLanesPerRow, part = q % kLanesPerRow;
+            const unsigned char* base = region + row * kRowBytes;
+            const int first = part * kChunksPerLane;
+            consume(i * 32 + row, j0 * 32 + part * 8, base + ((first ^ sw(row)) * 16),
+                    base + (((first + kChunksPerLane - 1) ^ sw(row)) * 16));
+        }
+    };
+    auto request_share = [&](int i) __attribute__((always_inline)) {
+        static_for<0, TM>([&](auto index) {
+            constexpr int block = decltype(index)::value;
+            if (i == block) request_tiles.template operator()<block * (kStages - 1) / TM, (block + 1) * (kStages - 1) / TM>();
+        });
+    };
+    // Before row block i of the tile is staged and stored, K tiles i*(kStages-1)/TM .. of the next item
+    // are requested (if there is one): a burst of requests would hold the wavefront up for as long as
+    // the memory system takes to accept them, between the stores it costs nothing.
+    auto store_tile = [&](const Item& w, bool request) __attribute__((always_inline)) {
+        // C may be given as column segments too: this tile's columns then belong to one of them.
+        void* c_base = p.c;
+        long c_ld = p.ldc;
+        int c_col0 = w.n0, c_cols = p.n;
+        if (p.c_seg.count > 0) {
+            const SegmentPick pick = pick_segment(p.c_seg, w.n0);
+            c_base = const_cast<void*>(pick.ptr);
+            c_ld = pick.ld;
+            c_col0 = w.n0 - pick.first;
+            c_cols = pick.cols;
+        }
+        const int row0 = w.m0 + wm * WM, col0 = wn * WN;  // of the wavefront's part; columns relative to n0
+        bool plain = false;
+        if constexpr (!SPLIT) plain = p.bias == nullptr && p.residual == nullptr && !p.accumulate && !p.c_f32;
+        if (plain) {
+            T* out = static_cast<T*>(c_base);
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+                if (request) request_share(i);
+                pass.template operator()<T, TN>(i, 0, [&](int row, int col, const unsigned char* lo, const unsigned char*) {
+                    const int m = row0 + row, c_col = c_col0 + col0 + col;
+                    const u32x4 data = *reinterpret_cast<const u32x4*>(lo);
+                    if (m < p.m && c_col < c_cols) *reinterpret_cast<u32x4*>(out + static_cast<long>(m) * c_ld + c_col) = data;
+                });
+            }
+            return;
+        }
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            if (request) request_share(i);
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+                pass.template operator()<float, TN / 2>(i, half * (TN / 2), [&](int row, int col, const unsigned char* lo,
+                                                                               const unsigned char* hi) {
+                    const int m = row0 + row, n = w.n0 + col0 + col, c_col = c_col0 + col0 + col;
+                    vec_t<float, 4> v0 = *reinterpret_cast<const vec_t<float, 4>*>(lo);
+                    vec_t<float, 4> v1 = *reinterpret_cast<const vec_t<float, 4>*>(hi);
+                    if (m >= p.m || c_col >= c_cols) return;
+                    if constexpr (SPLIT) {
+                        float* out = static_cast<float*>(p.c) +
+                                     (static_cast<long>(w.slice) * p.m + m) * static_cast<long>(p.n) + n;
+                        *reinterpret_cast<vec_t<float, 4>*>(out) = v0;
+                        *reinterpret_cast<vec_t<float, 4>*>(out + 4) = v1;
+                    } else {
+                        if (p.bias != nullptr) {
+                            const T* bias = static_cast<const T*>(p.bias) + n;
+                            v0 += vec_to_f32<T, 4>(load_vec<T, 4>(bias));
+                            v1 += vec_to_f32<T, 4>(load_vec<T, 4>(bias + 4));
+                        }
+                        if (p.residual != nullptr) {
+                            const T* residual = static_cast<const T*>(p.residual) + static_cast<long>(m) * p.ldr + n;
+                            v0 += vec_to_f32<T, 4>(load_vec<T, 4>(residual));
+                            v1 += vec_to_f32<T, 4>(load_vec<T, 4>(residual + 4));
+                        }
+                        if (p.c_f32) {
+                            float* out = static_cast<float*>(c_base) + static_cast<long>(m) * c_ld + c_col;
+                            if (p.accumulate) {
+                                v0 += *reinterpret_cast<const vec_t<float, 4>*>(out);
+                                v1 += *reinterpret_cast<const vec_t<float, 4>*>(out + 4);
+                            }
+                            *reinterpret_cast<vec_t<float, 4>*>(out) = v0;
+                            *reinterpret_cast<vec_t<float, 4>*>(out + 4) = v1;
+                        } else {
+                            T* out = static_cast<T*>(c_base) + static_cast<long>(m) * c_ld + c_col;
+                            if (p.accumulate) {
+                                const vec_t<T, 8> old = load_vec<T, 8>(out);
+#pragma unroll
+                                for (int e = 0; e < 4; ++e) {
+                                    v0[e] += to_f32(old[e]);
+                                    v1[e] += to_f32(old[4 + e]);
+                                }
+                            }
+                            vec_t<T, 8> packed;
+                            const vec_t<T, 4> r0 = vec_from_f32<T, 4>(v0), r1 = vec_from_f32<T, 4>(v1);
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) {
+                                packed[e] = r0[e];
+                                packed[4 + e] = r1[e];
+                            }
+                            store_vec<T, 8>(out, packed);
+                        }
+                    }
+                });
+            }
+        }
+    };
+
+    // Software pipeline over the K tiles t = 0 .. count-1 of an item (tile t lives in LDS stage
+    // t % kStages; tiles t+1 .. t+kStages-2 are in flight or landed), kBK/16 K sub-steps of 16 per tile:
     //   all but the last sub-step  MFMAs ‖ LDS reads of the next sub-step's fragments
     //   wait        this wavefront's loads of tile t+1 have landed; barrier: everybody's have, and
     //               nobody reads stage (t-1) % kStages any more
@@ -490,20 +684,27 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
     constexpr int kFrags = TM + TN;
     constexpr int kFragReads = TM * ATile::kFragReads + TN * BTile::kFragReads;
     constexpr int kSubSteps = kBK / 16;
-    constexpr unsigned int kStageBytes = kStage * sizeof(T);
     static_assert(kSubSteps % 2 == 0, "fragment sets alternate per sub-step and must line up across tiles");
-    if (count > 0) {
-        const unsigned int lds_wave = lds_address_of(smem) + wave * kLoadBytes;
-        TileCursor ca, cb;
+
+    // Per round: multiply an item, request the first K tiles of the next one, store the finished
+    // tile (its stores drain under the MFMAs that follow). The sources are opened every round, also
+    // when no item is left (then for the last one again, unused): values that are set on every path
+    // stay in scalar registers.
+    Item current = locate(item);
+    open(current);
+    request_tiles.template operator()<0, kStages - 1>();
+    while (true) {
 #pragma unroll
-        for (int t = 0; t < kStages - 1; ++t) {
-            cursors(t, ca, cb);
-            static_for<0, kTileLoads>([&](auto l) { issue_one(l, lds_wave + t * kStageBytes, ca, cb); });
-        }
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) acc[i][j] = acc_t(0.0f);
+        const int count = current.kt_end - current.kt_begin;
+        // Loads and stores retire in the order they were issued: at most the loads of K tiles
+        // 1 .. kStages-2 (and no older store of the previous epilogue) may still be outstanding.
         __builtin_amdgcn_s_waitcnt(vmcnt_immediate((kStages - 2) * kTileLoads));
-        __syncthreads();
+        barrier_only();
         read_frags(0, 0, 0);
-        int stage = 0;       // of tile t
+        int stage = 0;                 // of tile t
         int free_stage = kStages - 1;  // of tile t-1, refilled with tile t+kStages-1
         for (int t = 0; t < count; ++t) {
             const int next_stage = stage + 1 == kStages ? 0 : stage + 1;
@@ -541,143 +742,17 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
             free_stage = stage;
             stage = next_stage;
         }
-    }
-    __builtin_amdgcn_s_waitcnt(vmcnt_immediate(0));  // the staging below reuses LDS that loads may still target
-    __syncthreads();
-
-    // Epilogue. acc[i][j][4g+e] holds C[m, n] with m = lane%32, n = 8g + 4*(lane/32) + e, relative
-    // to block (i, j) of the wavefront's WM x WN part of the tile. Each wavefront passes its part
-    // through a private quarter of the last LDS stage, 32 rows at a time, and stores it row by row:
-    // whole contiguous row segments of C per instruction instead of 32 separate 8-byte pieces, and
-    // no workgroup barrier. When bias, residual or the old C are added (or the output is fp32 / a
-    // split-K partial) the staging is fp32, half the columns per pass, and rounding to the storage
-    // dtype still happens once, after the additions; otherwise the values are rounded in registers
-    // and staged in the storage dtype. A staged row is kRowBytes long; its 16-byte chunk c sits at
-    // chunk position c ^ sw(row), which spreads both the column-wise writes and the row-wise reads
-    // over all banks.
-    constexpr int kRowBytes = WN * static_cast<int>(sizeof(T));
-    constexpr int kRowChunks = kRowBytes / 16;
-    static_assert(32 * kRowBytes * kWaves == static_cast<int>(kStageBytes), "staging is a quarter stage per wavefront");
-    unsigned char* region = smem_raw + (kStages - 1) * kStageBytes + wave * (kStageBytes / kWaves);
-    auto sw = [](int row) { return (row / (256 / kRowBytes)) % kRowChunks; };
-    // C may be given as column segments too: this tile's columns then belong to one of them.
-    void* c_base = p.c;
-    long c_ld = p.ldc;
-    int c_col0 = n0, c_cols = p.n;
-    if (p.c_seg.count > 0) {
-        const SegmentPick pick = pick_segment(p.c_seg, n0);
-        c_base = const_cast<void*>(pick.ptr);
-        c_ld = pick.ld;
-        c_col0 = n0 - pick.first;
-        c_cols = pick.cols;
-    }
-    const int m_lane = lane & 31, h_lane = lane >> 5;
-    unsigned char* write_row = region + m_lane * kRowBytes;
-    const int write_sw = sw(m_lane);
-    // Stages blocks (i, j0 .. j0+JP-1) as element type S and hands each lane 8 consecutive staged
-    // elements at a time: consume(row, col, pointer to the 8 elements' first chunk, to the second
-    // chunk when S is float), row/col relative to the wavefront's part.
-    auto pass = [&]<typename S, int JP>(int i, int j0, auto&& consume) {
-        static_assert(JP * 32 * sizeof(S) == kRowBytes, "a pass fills whole staged rows");
-        __builtin_amdgcn_wave_barrier();
-#pragma unroll
-        for (int jj = 0; jj < JP; ++jj) {
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                vec_t<float, 4> v;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) v[e] = acc[i][j0 + jj][4 * g + e];
-                const int byte = (jj * 32 + g * 8 + h_lane * 4) * static_cast<int>(sizeof(S));
-                unsigned char* slot = write_row + (((byte / 16) ^ write_sw) * 16) + byte % 16;
-                if constexpr (std::is_same_v<S, float>) *reinterpret_cast<vec_t<float, 4>*>(slot) = v;
-                else store_vec<T, 4>(reinterpret_cast<T*>(slot), vec_from_f32<T, 4>(v));
-            }
-        }
-        __builtin_amdgcn_wave_barrier();
-        constexpr int kLanesPerRow = kRowBytes / (8 * static_cast<int>(sizeof(S)));
-        constexpr int kChunksPerLane = 8 * static_cast<int>(sizeof(S)) / 16;
-        constexpr int kRounds = 32 * kLanesPerRow / kWave;
-#pragma unroll
-        for (int u = 0; u < kRounds; ++u) {
-            const int q = u * kWave + lane;
-            const int row = q / kLanesPerRow, part = q % kLanesPerRow;
-            const unsigned char* base = region + row * kRowBytes;
-            const int first = part * kChunksPerLane;
-            consume(i * 32 + row, j0 * 32 + part * 8, base + ((first ^ sw(row)) * 16),
-                    base + (((first + kChunksPerLane - 1) ^ sw(row)) * 16));
-        }
-    };
-    const int row0 = m0 + wm * WM, col0 = wn * WN;  // of the wavefront's part; columns relative to n0
-    if constexpr (!SPLIT) {
-        if (p.bias == nullptr && p.residual == nullptr && !p.accumulate && !p.c_f32) {
-            T* out = static_cast<T*>(c_base);
-#pragma unroll
-            for (int i = 0; i < TM; ++i) {
-                pass.template operator()<T, TN>(i, 0, [&](int row, int col, const unsigned char* lo, const unsigned char*) {
-                    const int m = row0 + row, c_col = c_col0 + col0 + col;
-                    const u32x4 data = *reinterpret_cast<const u32x4*>(lo);
-                    if (m < p.m && c_col < c_cols) *reinterpret_cast<u32x4*>(out + static_cast<long>(m) * c_ld + c_col) = data;
-                });
-            }
-            return;
-        }
-    }
-#pragma unroll
-    for (int i = 0; i < TM; ++i) {
-#pragma unroll
-        for (int half = 0; half < 2; ++half) {
-            pass.template operator()<float, TN / 2>(i, half * (TN / 2), [&](int row, int col, const unsigned char* lo,
-                                                                           const unsigned char* hi) {
-                const int m = row0 + row, n = n0 + col0 + col, c_col = c_col0 + col0 + col;
-                vec_t<float, 4> v0 = *reinterpret_cast<const vec_t<float, 4>*>(lo);
-                vec_t<float, 4> v1 = *reinterpret_cast<const vec_t<float, 4>*>(hi);
-                if (m >= p.m || c_col >= c_cols) return;
-                if constexpr (SPLIT) {
-                    float* out = static_cast<float*>(p.c) +
-                                 (static_cast<long>(blockIdx.y) * p.m + m) * static_cast<long>(p.n) + n;
-                    *reinterpret_cast<vec_t<float, 4>*>(out) = v0;
-                    *reinterpret_cast<vec_t<float, 4>*>(out + 4) = v1;
-                } else {
-                    if (p.bias != nullptr) {
-                        const T* bias = static_cast<const T*>(p.bias) + n;
-                        v0 += vec_to_f32<T, 4>(load_vec<T, 4>(bias));
-                        v1 += vec_to_f32<T, 4>(load_vec<T, 4>(bias + 4));
-                    }
-                    if (p.residual != nullptr) {
-                        const T* residual = static_cast<const T*>(p.residual) + static_cast<long>(m) * p.ldr + n;
-                        v0 += vec_to_f32<T, 4>(load_vec<T, 4>(residual));
-                        v1 += vec_to_f32<T, 4>(load_vec<T, 4>(residual + 4));
-                    }
-                    if (p.c_f32) {
-                        float* out = static_cast<float*>(c_base) + static_cast<long>(m) * c_ld + c_col;
-                        if (p.accumulate) {
-                            v0 += *reinterpret_cast<const vec_t<float, 4>*>(out);
-                            v1 += *reinterpret_cast<const vec_t<float, 4>*>(out + 4);
-                        }
-                        *reinterpret_cast<vec_t<float, 4>*>(out) = v0;
-                        *reinterpret_cast<vec_t<float, 4>*>(out + 4) = v1;
-                    } else {
-                        T* out = static_cast<T*>(c_base) + static_cast<long>(m) * c_ld + c_col;
-                        if (p.accumulate) {
-                            const vec_t<T, 8> old = load_vec<T, 8>(out);
-#pragma unroll
-                            for (int e = 0; e < 4; ++e) {
-                                v0[e] += to_f32(old[e]);
-                                v1[e] += to_f32(old[4 + e]);
-                            }
-                        }
-                        vec_t<T, 8> packed;
-                        const vec_t<T, 4> r0 = vec_from_f32<T, 4>(v0), r1 = vec_from_f32<T, 4>(v1);
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            packed[e] = r0[e];
-                            packed[4 + e] = r1[e];
-                        }
-                        store_vec<T, 8>(out, packed);
-                    }
-                }
-            });
-        }
+        // The loads still outstanding are of K tiles past the end (zeros, but they do write LDS):
+        // once they have landed and every wavefront has read its last fragments, all stages are free.
+        __builtin_amdgcn_s_waitcnt(vmcnt_immediate(0));
+        barrier_only();
+        item += item_stride;
+        const bool more = item < item_end;
+        const Item next = locate(more ? item : item_end - 1);
+        open(next);
+        store_tile(current, more);
+        if (!more) break;
+        current = next;
     }
 }
 
@@ -777,9 +852,14 @@ int launch_mfma(const KernelArgs& p, int slices, hipStream_t stream) {
                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem)));
         configured = true;
     }
-    const int total = p.tiles_m * p.tiles_n;
-    const int per_xcd = (total + kXcds - 1) / kXcds;
-    hipLaunchKernelGGL(kernel, dim3(per_xcd * kXcds, slices), dim3(kThreads), smem, stream, p);
+    // One block per CU slot (256x256 tiles: one per CU; 128x128: two), a multiple of the XCD count
+    // so that every XCD gets the same number of blocks; fewer when there are fewer work items.
+    KernelArgs args = p;
+    args.slices = slices;
+    const long items = static_cast<long>(p.tiles_m) * p.tiles_n * slices;
+    const long slots = static_cast<long>(compute_units()) * (BM == 256 ? 1 : 2) / kXcds * kXcds;
+    const long blocks = std::min<long>((items + kXcds - 1) / kXcds * kXcds, std::max<long>(slots, kXcds));
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned int>(blocks)), dim3(kThreads), smem, stream, args);
     CGPTX_LAUNCH_CHECK();
     return CGPTX_OK;
 }
