@@ -131,15 +131,17 @@ template <int MASK, int COUNT>
 __device__ __forceinline__ void sched_group() {
     if constexpr (COUNT > 0) __builtin_amdgcn_sched_group_barrier(MASK, COUNT, 0);
 }
-// Asks the scheduler for MFMAS matrix instructions with EXTRA0 instructions of class CLASS0 and EXTRA1 of
-// class CLASS1 spread evenly between them, so that their issue slots fall in the shadow of an MFMA.
-template <int MFMAS, int CLASS0, int EXTRA0, int CLASS1, int EXTRA1, int I = 0>
+// Asks the scheduler for MFMAS matrix instructions with EXTRA0 instructions of class CLASS0 spread
+// evenly between the first SPAN of them (and EXTRA1 of CLASS1 likewise), so that their issue slots
+// fall in the shadow of an MFMA and their results have the remaining MFMAs' time to arrive.
+template <int MFMAS, int SPAN, int CLASS0, int EXTRA0, int CLASS1, int EXTRA1, int I = 0>
 __device__ __forceinline__ void sched_interleave() {
     if constexpr (I < MFMAS) {
+        constexpr int before = I < SPAN ? I : SPAN, after = I + 1 < SPAN ? I + 1 : SPAN;
         sched_group<kSchedMfma, 1>();
-        sched_group<CLASS0, ((I + 1) * EXTRA0) / MFMAS - (I * EXTRA0) / MFMAS>();
-        sched_group<CLASS1, ((I + 1) * EXTRA1) / MFMAS - (I * EXTRA1) / MFMAS>();
-        sched_interleave<MFMAS, CLASS0, EXTRA0, CLASS1, EXTRA1, I + 1>();
+        sched_group<CLASS0, (after * EXTRA0) / SPAN - (before * EXTRA0) / SPAN>();
+        sched_group<CLASS1, (after * EXTRA1) / SPAN - (before * EXTRA1) / SPAN>();
+        sched_interleave<MFMAS, SPAN, CLASS0, EXTRA0, CLASS1, EXTRA1, I + 1>();
     }
 }
 
@@ -330,8 +332,10 @@ struct TileLayout {
 // One workgroup per CU slot walks its share of the work items (output tile x K slice) one after
 // the other: the first K tiles of the next item are requested before the epilogue of the current
 // one, whose stores then drain under the next item's MFMAs.
-template <typename T, int BM, int BN, bool A_K, bool B_K, bool SPLIT>
+// SEGMENTED: A is stored [M, K] in up to three column segments (separate buffers along K).
+template <typename T, int BM, int BN, bool A_K, bool B_K, bool SPLIT, bool SEGMENTED>
 __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
+    static_assert(!SEGMENTED || (A_K && !SPLIT), "segments along K are read by the unsplit kernels only");
     using frag_t = typename Mfma<T>::frag;
     using Layout = TileLayout<T, BM, BN, A_K, B_K>;
     using ATile = typename Layout::ATile;
@@ -394,7 +398,9 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
         const int m0 = w.m0, n0 = w.n0;
         src_begin = w.kt_begin;
         src_end = w.kt_end;
-        if constexpr (A_K) {
+        if constexpr (A_K && !SEGMENTED) {
+            a_src.init(static_cast<const T*>(p.a) + static_cast<long>(m0) * p.lda, p.lda, p.m - m0, p.k, wave);
+        } else if constexpr (A_K) {
             // All three sources are set up unconditionally (absent segments repeat the first and
             // are never selected): conditional set-up would be merged into one piece of code that
             // writes through a pointer, which keeps the sources in memory.
@@ -437,7 +443,7 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
     auto cursors = [&](int t, TileCursor& ca, TileCursor& cb) __attribute__((always_inline)) {
         const unsigned int past_end = src_begin + t >= src_end ? 0x80000000u : 0u;
         const int k0 = min(src_begin + t, src_end - 1) * kBK;
-        if constexpr (A_K) {
+        if constexpr (SEGMENTED) {
             // Values first, then selects: a conditional between the objects' members would select
             // an address and keep all three sources in memory.
             const bool in1 = k0 >= a_end0, in2 = k0 >= a_end1;
@@ -714,7 +720,7 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
             for (int kk = 0; kk + 1 < kSubSteps; ++kk) {
                 read_frags((kk + 1) & 1, stage, kk + 1);
                 multiply(kk & 1);
-                sched_interleave<kMfmas, kSchedDsRead, kFragReads, 0, 0>();
+                sched_interleave<kMfmas, (3 * kMfmas + 3) / 4, kSchedDsRead, kFragReads, 0, 0>();
                 __builtin_amdgcn_sched_barrier(0);
             }
             __builtin_amdgcn_s_waitcnt(vmcnt_immediate((kStages - 3) * kTileLoads));
@@ -842,10 +848,10 @@ __global__ __launch_bounds__(kGenericTile* kGenericTile / 4) void gemm_generic_k
 }
 
 // ------------------------------------------------------------------- host side
-template <typename T, int BM, int BN, bool A_K, bool B_K, bool SPLIT>
+template <typename T, int BM, int BN, bool A_K, bool B_K, bool SPLIT, bool SEGMENTED>
 int launch_mfma(const KernelArgs& p, int slices, hipStream_t stream) {
     constexpr std::size_t smem = TileLayout<T, BM, BN, A_K, B_K>::kSmemBytes;
-    auto kernel = gemm_mfma_kernel<T, BM, BN, A_K, B_K, SPLIT>;
+    auto kernel = gemm_mfma_kernel<T, BM, BN, A_K, B_K, SPLIT, SEGMENTED>;
     static bool configured = false;
     if (!configured) {
         CGPTX_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -866,9 +872,17 @@ int launch_mfma(const KernelArgs& p, int slices, hipStream_t stream) {
 
 template <typename T, int BM, int BN, bool SPLIT>
 int launch_layout(const KernelArgs& p, bool a_k, bool b_k, int slices, hipStream_t stream) {
-    if (a_k && b_k) return launch_mfma<T, BM, BN, true, true, SPLIT>(p, slices, stream);
-    if (a_k && !b_k) return launch_mfma<T, BM, BN, true, false, SPLIT>(p, slices, stream);
-    if (!a_k && !b_k) return launch_mfma<T, BM, BN, false, false, SPLIT>(p, slices, stream);
+    // A given in segments along K has kernels of its own (the source of a K tile is then picked
+    // per tile), and only unsplit ones.
+    const bool segmented = a_k && p.a_seg.count > 0;
+    if constexpr (!SPLIT) {
+        if (segmented && b_k) return launch_mfma<T, BM, BN, true, true, false, true>(p, slices, stream);
+        if (segmented && !b_k) return launch_mfma<T, BM, BN, true, false, false, true>(p, slices, stream);
+    }
+    if (segmented) return fail(CGPTX_RUNTIME, "gemm: a segmented operand cannot be split along K");
+    if (a_k && b_k) return launch_mfma<T, BM, BN, true, true, SPLIT, false>(p, slices, stream);
+    if (a_k && !b_k) return launch_mfma<T, BM, BN, true, false, SPLIT, false>(p, slices, stream);
+    if (!a_k && !b_k) return launch_mfma<T, BM, BN, false, false, SPLIT, false>(p, slices, stream);
     return fail(CGPTX_RUNTIME, "gemm: unsupported operand layout");
 }
 
@@ -891,7 +905,8 @@ int run_config(const GemmArgs& g, KernelArgs p, hipStream_t stream) {
     const long tiles = static_cast<long>(p.tiles_m) * p.tiles_n;
     const long want_blocks = static_cast<long>(compute_units()) * (BM == 256 ? 1 : 2);
     int slices = 1;
-    if (!g.no_split && g.residual == nullptr && g.c_segments.count == 0 && tiles < want_blocks && k_tiles >= 32) {
+    const bool k_segments = g.a_k_contiguous && g.a_segments.count > 0;
+    if (!g.no_split && g.residual == nullptr && g.c_segments.count == 0 && !k_segments && tiles < want_blocks && k_tiles >= 32) {
         slices = static_cast<int>(std::min<long>((want_blocks + tiles - 1) / tiles, k_tiles / 16));
         if (slices < 1) slices = 1;
     }
