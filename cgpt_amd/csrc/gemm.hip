@@ -60,22 +60,29 @@ constexpr int stages_for(int /*bm*/, int /*bn*/) { return 5; }
 constexpr int kXcds = 8;
 constexpr int kGroupRows = 8;    // tile-rows per L2 locality group
 
-using acc_t = vec_t<float, 16>;
+using acc_t = vec_t<float, 4>;
 
+// c += a x b with v_mfma_f32_16x16x32 (a: 16 rows x 32 k, b: 32 k x 16 columns; lane l holds row or
+// column l%16, k = 8*(l/16) .. +7; c: lane l holds rows 4*(l/16) .. +3 of column l%16). Written as
+// assembly so that the accumulator is updated in place: the four-register form of the instruction
+// does not tie its result to its addend, and with all 256 accumulator registers in use the register
+// allocator would otherwise shuffle accumulators around every MFMA. The kernel keeps the distances
+// the hardware asks for by construction: an accumulator is touched once per K tile (64 or 16 MFMAs
+// apart), zeroed long before its first MFMA and read by the epilogue only after a barrier.
 template <typename T>
 struct Mfma;
 template <>
 struct Mfma<bf16_t> {
     using frag = vec_t<bf16_t, 8>;
-    __device__ static __forceinline__ acc_t run(frag a, frag b, acc_t c) {
-        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+    __device__ static __forceinline__ void run(acc_t& c, const frag& a, const frag& b) {
+        asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
     }
 };
 template <>
 struct Mfma<f16_t> {
     using frag = vec_t<f16_t, 8>;
-    __device__ static __forceinline__ acc_t run(frag a, frag b, acc_t c) {
-        return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+    __device__ static __forceinline__ void run(acc_t& c, const frag& a, const frag& b) {
+        asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
     }
 };
 
@@ -229,7 +236,6 @@ struct KTile {
     static constexpr int kElems = ROWS * kBK;
     static constexpr int kLoads = ROWS / kRowsPerLoad / kWaves;  // load instructions per wavefront and tile
     static constexpr int kFragReads = 1;                        // LDS instructions per fragment
-    static constexpr int kOffsets = kBK / 16;                   // per-lane fragment offsets: one per K sub-step
 
     u32x4 rsrc = {0u, 0u, 0u, 0u};
     int voffset = 0;
@@ -252,10 +258,10 @@ struct KTile {
     __device__ __forceinline__ unsigned int first_offset(int k0, int wave) const {
         return wave * group_bytes + k0 * static_cast<unsigned int>(sizeof(T));
     }
-    // Element offset of the lane's fragment within a 32-row block, K sub-step kk: row lane%32,
-    // k = 16 kk + 8 (lane/32) .. +7.
-    __device__ __forceinline__ static int lane_offset(int lane, int /*block0*/, int kk) {
-        return (lane & 31) * kBK + (((kk * 2 + (lane >> 5)) ^ swizzle(lane & 31)) * 8);
+    // Element offset of the lane's fragment within a 16-row block (the whole K tile is one MFMA
+    // step): row lane%16, k = 8 (lane/16) .. +7. The swizzle of a row does not depend on the block.
+    __device__ __forceinline__ static int lane_offset(int lane) {
+        return (lane & 15) * kBK + (((lane >> 4) ^ swizzle(lane & 15)) * 8);
     }
     __device__ __forceinline__ static frag_t frag(const T* tile, int block0, int offset) {
         return *reinterpret_cast<const frag_t*>(tile + block0 * kBK + offset);
@@ -275,7 +281,6 @@ struct NTile {
     static constexpr int kElems = kBK * COLS;
     static constexpr int kLoads = kBK / kRowsPerLoad / kWaves;
     static constexpr int kFragReads = 2;
-    static constexpr int kOffsets = COLS / 64;  // per-lane fragment offsets: one per 32-column block of a wavefront
 
     u32x4 rsrc = {0u, 0u, 0u, 0u};
     int voffset = 0;
@@ -297,17 +302,18 @@ struct NTile {
         return (wave + k0 / kRowsPerLoad) * group_bytes;
     }
     // Lane i of a 16-lane group addresses k row i/4, columns 4*(i%4) .. +3 of the group's 4 x 16
-    // block; groups 0/1 take columns 0-15/16-31 of the fragment, lanes 32-63 the k values 8-15.
-    // The offset is for K sub-step 0 and the first of the two reads; block0 is a multiple of 32.
-    __device__ __forceinline__ static int lane_offset(int lane, int block0, int /*kk*/) {
-        const int k_row = (lane >> 5) * 8 + ((lane & 15) >> 2);
-        const int chunk = ((block0 / 8) ^ ((k_row & 3) << 2)) + ((lane >> 4) & 1) * 2 + ((lane & 3) >> 1);
+    // block; group g (lanes 16g .. 16g+15) takes the k values 8g .. 8g+7 of the fragment's 16
+    // columns in two reads (k rows +0..3, +4..7). The offset is for the first read; block0 is a
+    // multiple of 16.
+    __device__ __forceinline__ static int lane_offset(int lane, int block0) {
+        const int k_row = (lane >> 4) * 8 + ((lane & 15) >> 2);
+        const int chunk = ((block0 / 8) ^ ((k_row & 3) << 2)) + ((lane & 3) >> 1);
         return k_row * COLS + chunk * 8 + (lane & 1) * 4;
     }
-    __device__ __forceinline__ static frag_t frag(const T* tile, int kk, int offset) {
+    __device__ __forceinline__ static frag_t frag(const T* tile, int offset) {
         using s16x4 = vec_t<short, 4>;
         using lds_ptr = __attribute__((address_space(3))) s16x4*;
-        const T* q = tile + kk * 16 * COLS + offset;
+        const T* q = tile + offset;
         const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(q));
         const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(q + 4 * COLS));
         vec_t<short, 8> both;
@@ -342,7 +348,7 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
     using BTile = typename Layout::BTile;
     static_assert(BM == BN, "the epilogue staging assumes square tiles");
     constexpr int WM = BM / 2, WN = BN / 2;
-    constexpr int TM = WM / 32, TN = WN / 32;
+    constexpr int TM = WM / 16, TN = WN / 16;  // 16 x 16 MFMA blocks of a wavefront's part
     extern __shared__ __align__(1024) unsigned char smem_raw[];
     T* smem = reinterpret_cast<T*>(smem_raw);
     // Stage s holds [A tile | B tile] at smem + s * kStage.
@@ -498,37 +504,39 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
         });
     };
 
-    int a_off[ATile::kOffsets], b_off[BTile::kOffsets];
+    // Per-lane LDS offsets of the fragments: one for a k-contiguous operand (the block is a
+    // scalar offset), one per 16-column block for an n-contiguous one (the swizzle depends on it).
+    constexpr int kAOffsets = A_K ? 1 : TM, kBOffsets = B_K ? 1 : TN;
+    int a_off[kAOffsets], b_off[kBOffsets];
+    if constexpr (A_K) {
+        a_off[0] = ATile::lane_offset(lane);
+    } else {
 #pragma unroll
-    for (int i = 0; i < ATile::kOffsets; ++i) a_off[i] = ATile::lane_offset(lane, wm * WM + i * 32, i);
+        for (int i = 0; i < TM; ++i) a_off[i] = ATile::lane_offset(lane, wm * WM + i * 16);
+    }
+    if constexpr (B_K) {
+        b_off[0] = BTile::lane_offset(lane);
+    } else {
 #pragma unroll
-    for (int j = 0; j < BTile::kOffsets; ++j) b_off[j] = BTile::lane_offset(lane, wn * WN + j * 32, j);
+        for (int j = 0; j < TN; ++j) b_off[j] = BTile::lane_offset(lane, wn * WN + j * 16);
+    }
 
     acc_t acc[TM][TN];
-    frag_t af[2][TM], bf[2][TN];
-    auto read_frags = [&](int set, int stage, int kk) __attribute__((always_inline)) {
-        const T* as = smem + stage * kStage;
-        const T* bs = as + kATile;
-#pragma unroll
-        for (int i = 0; i < TM; ++i) {
-            if constexpr (A_K) af[set][i] = ATile::frag(as, wm * WM + i * 32, a_off[kk]);
-            else af[set][i] = ATile::frag(as, kk, a_off[i]);
+    frag_t af[TM], bf[TN];
+    // Fragment F (A's TM blocks first, then B's TN) of the K tile in `stage_tile`.
+    auto read_frag = [&]<int F>(const T* stage_tile) __attribute__((always_inline)) {
+        if constexpr (F < TM) {
+            if constexpr (A_K) af[F] = ATile::frag(stage_tile, wm * WM + F * 16, a_off[0]);
+            else af[F] = ATile::frag(stage_tile, a_off[F]);
+        } else {
+            constexpr int j = F - TM;
+            if constexpr (B_K) bf[j] = BTile::frag(stage_tile + kATile, wn * WN + j * 16, b_off[0]);
+            else bf[j] = BTile::frag(stage_tile + kATile, b_off[j]);
         }
-#pragma unroll
-        for (int j = 0; j < TN; ++j) {
-            if constexpr (B_K) bf[set][j] = BTile::frag(bs, wn * WN + j * 32, b_off[kk]);
-            else bf[set][j] = BTile::frag(bs, kk, b_off[j]);
-        }
-    };
-    auto multiply = [&](int set) __attribute__((always_inline)) {
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-            for (int j = 0; j < TN; ++j) acc[i][j] = Mfma<T>::run(bf[set][j], af[set][i], acc[i][j]);
     };
 
-    // Epilogue staging. acc[i][j][4g+e] holds C[m, n] with m = lane%32, n = 8g + 4*(lane/32) + e,
-    // relative to block (i, j) of the wavefront's WM x WN part of the tile. Each wavefront passes
+    // Epilogue staging. acc[i][j][e] holds C[m, n] with m = lane%16, n = 4*(lane/16) + e, relative
+    // to the 16 x 16 block (i, j) of the wavefront's WM x WN part of the tile. Each wavefront passes
     // its part through a private quarter of the last LDS stage (the only one the first K tiles of
     // the next item do not fill), 32 rows at a time, and stores it row by row: whole contiguous
     // row segments of C per instruction instead of 32 separate 8-byte pieces, and no workgroup
@@ -543,24 +551,22 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
     static_assert(32 * kRowBytes * kWaves == static_cast<int>(kStageBytes), "staging is a quarter stage per wavefront");
     unsigned char* region = smem_raw + (kStages - 1) * kStageBytes + wave * (kStageBytes / kWaves);
     auto sw = [](int row) { return (row / (256 / kRowBytes)) % kRowChunks; };
-    const int m_lane = lane & 31, h_lane = lane >> 5;
-    unsigned char* write_row = region + m_lane * kRowBytes;
-    const int write_sw = sw(m_lane);
-    // Stages blocks (i, j0 .. j0+JP-1) as element type S and hands each lane 8 consecutive staged
+    const int m_lane = lane & 15, q_lane = lane >> 4;
+    // Stages blocks (2r, j0 .. j0+JP-1) and (2r+1, ...), 32 rows, as element type S and hands each lane 8 consecutive staged
     // elements at a time: consume(row, col, pointer to the 8 elements' first chunk, to the second
     // chunk when S is float), row/col relative to the wavefront's part.
-    auto pass = [&]<typename S, int JP>(int i, int j0, auto&& consume) __attribute__((always_inline)) {
-        static_assert(JP * 32 * sizeof(S) == kRowBytes, "a pass fills whole staged rows");
+    auto pass = [&]<typename S, int JP>(int r, int j0, auto&& consume) __attribute__((always_inline)) {
+        static_assert(JP * 16 * sizeof(S) == kRowBytes, "a pass fills whole staged rows");
         __builtin_amdgcn_wave_barrier();
 #pragma unroll
-        for (int jj = 0; jj < JP; ++jj) {
+        for (int ii = 0; ii < 2; ++ii) {
+            const int row = ii * 16 + m_lane;
+            unsigned char* write_row = region + row * kRowBytes;
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                vec_t<float, 4> v;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) v[e] = acc[i][j0 + jj][4 * g + e];
-                const int byte = (jj * 32 + g * 8 + h_lane * 4) * static_cast<int>(sizeof(S));
-                unsigned char* slot = write_row + (((byte / 16) ^ write_sw) * 16) + byte % 16;
+            for (int jj = 0; jj < JP; ++jj) {
+                const acc_t v = acc[2 * r + ii][j0 + jj];
+                const int byte = (jj * 16 + q_lane * 4) * static_cast<int>(sizeof(S));
+                unsigned char* slot = write_row + (((byte / 16) ^ sw(row)) * 16) + byte % 16;
                 if constexpr (std::is_same_v<S, float>) *reinterpret_cast<vec_t<float, 4>*>(slot) = v;
                 else store_vec<T, 4>(reinterpret_cast<T*>(slot), vec_from_f32<T, 4>(v));
             }
@@ -575,17 +581,19 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
             const int row = q / kLanesPerRow, part = q % kLanesPerRow;
             const unsigned char* base = region + row * kRowBytes;
             const int first = part * kChunksPerLane;
-            consume(i * 32 + row, j0 * 32 + part * 8, base + ((first ^ sw(row)) * 16),
+            consume(r * 32 + row, j0 * 16 + part * 8, base + ((first ^ sw(row)) * 16),
                     base + (((first + kChunksPerLane - 1) ^ sw(row)) * 16));
         }
     };
-    auto request_share = [&](int i) __attribute__((always_inline)) {
-        static_for<0, TM>([&](auto index) {
+    constexpr int kRowBlocks = WM / 32;  // 32-row blocks of a wavefront's part
+    auto request_share = [&](int r) __attribute__((always_inline)) {
+        static_for<0, kRowBlocks>([&](auto index) {
             constexpr int block = decltype(index)::value;
-            if (i == block) request_tiles.template operator()<block * (kStages - 1) / TM, (block + 1) * (kStages - 1) / TM>();
+            if (r == block)
+                request_tiles.template operator()<block * (kStages - 1) / kRowBlocks, (block + 1) * (kStages - 1) / kRowBlocks>();
         });
     };
-    // Before row block i of the tile is staged and stored, K tiles i*(kStages-1)/TM .. of the next item
+    // Before 32-row block r of the tile is staged and stored, its share of the first K tiles of the next item
     // are requested (if there is one): a burst of requests would hold the wavefront up for as long as
     // the memory system takes to accept them, between the stores it costs nothing.
     auto store_tile = [&](const Item& w, bool request) __attribute__((always_inline)) {
@@ -606,9 +614,9 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
         if (plain) {
             T* out = static_cast<T*>(c_base);
 #pragma unroll
-            for (int i = 0; i < TM; ++i) {
-                if (request) request_share(i);
-                pass.template operator()<T, TN>(i, 0, [&](int row, int col, const unsigned char* lo, const unsigned char*) {
+            for (int r = 0; r < kRowBlocks; ++r) {
+                if (request) request_share(r);
+                pass.template operator()<T, TN>(r, 0, [&](int row, int col, const unsigned char* lo, const unsigned char*) {
                     const int m = row0 + row, c_col = c_col0 + col0 + col;
                     const u32x4 data = *reinterpret_cast<const u32x4*>(lo);
                     if (m < p.m && c_col < c_cols) *reinterpret_cast<u32x4*>(out + static_cast<long>(m) * c_ld + c_col) = data;
@@ -617,11 +625,11 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
             return;
         }
 #pragma unroll
-        for (int i = 0; i < TM; ++i) {
-            if (request) request_share(i);
+        for (int r = 0; r < kRowBlocks; ++r) {
+            if (request) request_share(r);
 #pragma unroll
             for (int half = 0; half < 2; ++half) {
-                pass.template operator()<float, TN / 2>(i, half * (TN / 2), [&](int row, int col, const unsigned char* lo,
+                pass.template operator()<float, TN / 2>(r, half * (TN / 2), [&](int row, int col, const unsigned char* lo,
                                                                                const unsigned char* hi) {
                     const int m = row0 + row, n = w.n0 + col0 + col, c_col = c_col0 + col0 + col;
                     vec_t<float, 4> v0 = *reinterpret_cast<const vec_t<float, 4>*>(lo);
@@ -677,20 +685,43 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
     };
 
     // Software pipeline over the K tiles t = 0 .. count-1 of an item (tile t lives in LDS stage
-    // t % kStages; tiles t+1 .. t+kStages-2 are in flight or landed), kBK/16 K sub-steps of 16 per tile:
-    //   all but the last sub-step  MFMAs ‖ LDS reads of the next sub-step's fragments
-    //   wait        this wavefront's loads of tile t+1 have landed; barrier: everybody's have, and
-    //               nobody reads stage (t-1) % kStages any more
-    //   last sub-step  MFMAs ‖ loads of tile t+kStages-1 into that stage ‖ fragments of tile t+1, sub-step 0
+    // t % kStages; tiles t+1 .. t+kStages-2 are in flight or landed). A K tile is one MFMA step
+    // (k = 32) of TM x TN MFMAs, taken as two column halves (all rows x the left TN/2 blocks, then
+    // all rows x the right ones) so that one set of fragment registers suffices: a fragment is read
+    // for the next tile as soon as its last MFMA of this tile has been issued.
+    //   left half    MFMAs ‖ LDS reads of this tile's right-half B fragments
+    //   wait         this wavefront's loads of tile t+1 have landed; barrier: everybody's have, and
+    //                nobody reads stage (t-1) % kStages any more
+    //   right half   MFMAs ‖ loads of tile t+kStages-1 into that stage ‖ tile t+1's left-half B
+    //                fragments (first thing) and its A fragment i after row i
     // so LDS latency and kStages-2 K tiles of global latency sit in the shadow of MFMAs. With one
-    // wavefront per SIMD nothing else hides an instruction that is not next to an MFMA, so in the
-    // last sub-step every MFMA is followed by its share of the loads and fragment reads and a
-    // scheduling fence keeps them there.
+    // wavefront per SIMD nothing else hides an instruction that is not next to an MFMA, so every
+    // MFMA is followed by its share of the loads and fragment reads and a scheduling fence keeps
+    // them there.
     constexpr int kMfmas = TM * TN;
     constexpr int kFrags = TM + TN;
-    constexpr int kFragReads = TM * ATile::kFragReads + TN * BTile::kFragReads;
-    constexpr int kSubSteps = kBK / 16;
-    static_assert(kSubSteps % 2 == 0, "fragment sets alternate per sub-step and must line up across tiles");
+    constexpr int kHalf = TN / 2;
+    static_assert(TN % 2 == 0 && kHalf <= TM, "the left-half B fragments are read one per row");
+    // HALF 0: this_tile = tile t (its right-half B fragments are read); HALF 1: next_tile = tile t+1.
+    auto multiply_half = [&]<int HALF>(const T* tile, unsigned int free_lds) __attribute__((always_inline)) {
+        static_for<0, kMfmas / 2>([&](auto index) {
+            constexpr int m = decltype(index)::value;
+            constexpr int i = m / kHalf, jj = m % kHalf, j = HALF * kHalf + jj;
+            Mfma<T>::run(acc[i][j], bf[j], af[i]);
+            if constexpr (HALF == 0) {
+                // Right-half B fragment i of this tile after the first MFMA of row i (rows 0 .. kHalf-1).
+                if constexpr (jj == 0 && i < kHalf) read_frag.template operator()<TM + kHalf + i>(tile);
+            } else {
+                // Left-half B fragment i of the next tile after the first MFMA of row i (its last use
+                // was in the left half), A fragment i after the last MFMA of row i.
+                if constexpr (jj == 0 && i < kHalf) read_frag.template operator()<TM + i>(tile);
+                if constexpr (jj == kHalf - 1) read_frag.template operator()<i>(tile);
+                static_for<(m * kTileLoads) / (kMfmas / 2), ((m + 1) * kTileLoads) / (kMfmas / 2)>(
+                    [&](auto l) { issue_one(l, free_lds, ca, cb); });
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        });
+    };
 
     // Per round: multiply an item, request the first K tiles of the next one, store the finished
     // tile (its stores drain under the MFMAs that follow). The sources are opened every round, also
@@ -709,42 +740,16 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
         // 1 .. kStages-2 (and no older store of the previous epilogue) may still be outstanding.
         __builtin_amdgcn_s_waitcnt(vmcnt_immediate((kStages - 2) * kTileLoads));
         barrier_only();
-        read_frags(0, 0, 0);
+        static_for<0, TM + kHalf>([&](auto f) { read_frag.template operator()<decltype(f)::value>(smem); });
         int stage = 0;                 // of tile t
         int free_stage = kStages - 1;  // of tile t-1, refilled with tile t+kStages-1
         for (int t = 0; t < count; ++t) {
             const int next_stage = stage + 1 == kStages ? 0 : stage + 1;
             cursors(t + kStages - 1, ca, cb);
-            const unsigned int free_lds = lds_wave + free_stage * kStageBytes;
-#pragma unroll
-            for (int kk = 0; kk + 1 < kSubSteps; ++kk) {
-                read_frags((kk + 1) & 1, stage, kk + 1);
-                multiply(kk & 1);
-                sched_interleave<kMfmas, (3 * kMfmas + 3) / 4, kSchedDsRead, kFragReads, 0, 0>();
-                __builtin_amdgcn_sched_barrier(0);
-            }
+            multiply_half.template operator()<0>(smem + stage * kStage, 0u);
             __builtin_amdgcn_s_waitcnt(vmcnt_immediate((kStages - 3) * kTileLoads));
             barrier_only();
-            const T* next_a = smem + next_stage * kStage;
-            const T* next_b = next_a + kATile;
-            static_for<0, kMfmas>([&](auto index) {
-                constexpr int m = decltype(index)::value;
-                constexpr int i = m / TN, j = m % TN;
-                acc[i][j] = Mfma<T>::run(bf[1][j], af[1][i], acc[i][j]);
-                static_for<(m * kFrags) / kMfmas, ((m + 1) * kFrags) / kMfmas>([&](auto which) {
-                    constexpr int f = decltype(which)::value;
-                    if constexpr (f < TM) {
-                        if constexpr (A_K) af[0][f] = ATile::frag(next_a, wm * WM + f * 32, a_off[0]);
-                        else af[0][f] = ATile::frag(next_a, 0, a_off[f]);
-                    } else {
-                        if constexpr (B_K) bf[0][f - TM] = BTile::frag(next_b, wn * WN + (f - TM) * 32, b_off[0]);
-                        else bf[0][f - TM] = BTile::frag(next_b, 0, b_off[f - TM]);
-                    }
-                });
-                static_for<(m * kTileLoads) / kMfmas, ((m + 1) * kTileLoads) / kMfmas>(
-                    [&](auto l) { issue_one(l, free_lds, ca, cb); });
-                __builtin_amdgcn_sched_barrier(0);
-            });
+            multiply_half.template operator()<1>(smem + next_stage * kStage, lds_wave + free_stage * kStageBytes);
             free_stage = stage;
             stage = next_stage;
         }
