@@ -11,8 +11,12 @@
 // Design
 //   * 256 threads = 4 wavefronts in a 2x2 grid; a block owns a BM x BN tile of C
 //     and walks K in steps of 32. Each wavefront owns (BM/2) x (BN/2) and issues
-//     v_mfma_f32_32x32x16 (bf16 or f16), so every LDS fragment read feeds
-//     (BM/64)·(BN/64) MFMAs.
+//     v_mfma_f32_16x16x32 (bf16 or f16): per flop that form moves half the accumulator
+//     data of the 32x32x16 one, which counts on a chip whose clock is power-limited.
+//   * The kernel is persistent: one block per CU slot walks its share of the work items
+//     (output tile x K slice). The 8 XCDs (blocks are dealt round-robin to them) each take
+//     a contiguous eighth of the items, ordered in groups of 8 tile-rows, so that the
+//     tiles in flight on one XCD share A and B panels in that XCD's L2.
 //   * Operand tiles go global -> LDS with buffer_load ... lds (no staging registers, no
 //     LDS stores, one loop-invariant per-lane offset) into a ring of five LDS stages:
 //     one being multiplied, up to three K tiles in flight, one being refilled. LDS rows
@@ -20,20 +24,17 @@
 //   * Operands that are not k-contiguous in memory (dX's weight, both dW operands) sit
 //     in LDS as they are in memory and are transposed by the LDS read itself
 //     (ds_read_b64_tr_b16): no transpose pass over HBM, no VALU shuffles.
-//   * The K loop is a software pipeline with one barrier per K step whose issue order is
-//     pinned with sched_group_barrier: fragment reads are spread between the MFMAs they
-//     overlap with, the wait for the next K tile sits in the middle of the step, and the
-//     loop has no data-dependent branch (edges are clamped or zero-filled by the
-//     buffer range check, never predicated).
+//   * The K loop is a software pipeline with one barrier per K tile whose issue order is
+//     pinned in the source: every MFMA is followed by its share of the fragment reads and
+//     of the loads, the wait for the next K tile sits in the middle of the tile, and the
+//     loop has no data-dependent branch (edges are clamped or zero-filled by the buffer
+//     range check, never predicated).
 //   * MFMA is issued as (B-fragment, A-fragment), so a lane ends up holding four
-//     consecutive n for one m per accumulator group; the finished tile is staged in
-//     LDS as fp32 and written out row by row (512 contiguous bytes per wavefront
-//     store), with bias / accumulate added in fp32 and one rounding to the dtype.
-//   * Block ids are remapped so that the 8 XCDs (blocks are dealt round-robin to
-//     them) each walk a contiguous range of tiles, and tiles are ordered in groups
-//     of 8 tile-rows so that the tiles resident on one XCD share A and B panels in
-//     that XCD's L2.
-//   * dW has few output tiles and K = rows (32768): K is split across blockIdx.y,
+//     consecutive n for one m per accumulator; each wavefront stages its part of the
+//     finished tile in a private piece of LDS and writes it out row by row (256
+//     contiguous bytes per row), with bias / residual / old C added in fp32 and one
+//     rounding to the dtype. The next item's first K tiles are requested meanwhile.
+//   * dW has few output tiles and K = rows (32768): K is split into slices (work items),
 //     fp32 partial tiles go to scratch and a second kernel adds them in slice order
 //     (deterministic), applying accumulate and the dtype conversion.
 //
