@@ -913,7 +913,9 @@ int run_config(const GemmArgs& g, KernelArgs p, hipStream_t stream) {
     int slices = 1;
     const bool k_segments = g.a_k_contiguous && g.a_segments.count > 0;
     if (!g.no_split && g.residual == nullptr && g.c_segments.count == 0 && !k_segments && tiles < want_blocks && k_tiles >= 32) {
-        slices = static_cast<int>(std::min<long>((want_blocks + tiles - 1) / tiles, k_tiles / 16));
+        // As many slices as fit the CU slots in one go: one item more than that would cost a
+        // second round of the persistent blocks.
+        slices = static_cast<int>(std::min<long>(want_blocks / tiles, k_tiles / 16));
         if (slices < 1) slices = 1;
     }
     p.k_tiles_per_slice = (k_tiles + slices - 1) / slices;
