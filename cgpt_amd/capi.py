@@ -85,6 +85,18 @@ PROTOTYPES = {
     "cgptx_model_parameter": [_vp, _sz, ctypes.POINTER(ctypes.c_char_p), ctypes.POINTER(_vp), ctypes.POINTER(_vp),
                               ctypes.POINTER(_sz)],
     "cgptx_model_activation": [_vp, ctypes.c_char_p, ctypes.POINTER(_vp), ctypes.POINTER(_sz)],
+    "cgptx_model_describe": [_vp, ctypes.POINTER(ModelConfig), ctypes.POINTER(_sz), ctypes.POINTER(_sz)],
+    "cgptx_model_optimizer_state": [_vp, _sz, ctypes.POINTER(_vp), ctypes.POINTER(_vp), ctypes.POINTER(_vp)],
+    "cgptx_model_set_optimizer_step": [_vp, _u64],
+    "cgptx_model_save_checkpoint": [_vp, ctypes.c_char_p, _sz],
+    "cgptx_model_load_checkpoint": [_vp, ctypes.c_char_p],
+    "cgptx_model_save_optimizer": [_vp, ctypes.c_char_p, _u64],
+    "cgptx_model_load_optimizer": [_vp, ctypes.c_char_p, ctypes.POINTER(_u64)],
+    "cgptx_token_upload_create": [ctypes.POINTER(_vp), _sz, _sz],
+    "cgptx_token_upload_destroy": [_vp],
+    "cgptx_token_upload_acquire": [_vp, ctypes.POINTER(_vp), ctypes.POINTER(_vp)],
+    "cgptx_token_upload_submit": [_vp, _vp, _vp, _vp],
+    "cgptx_model_upload_tokens": [_vp, _vp, _vp],
     "cgptx_model_profile": [_vp, _f, _i, _vp],
     "cgptx_model_profile_entry": [_vp, _sz, ctypes.POINTER(ctypes.c_char_p), ctypes.POINTER(_f)],
 }

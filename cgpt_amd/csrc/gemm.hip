@@ -132,27 +132,6 @@ __device__ __forceinline__ SegmentPick pick_segment(const KernelSegments& seg, i
     return pick;
 }
 
-// Instruction classes of __builtin_amdgcn_sched_group_barrier.
-constexpr int kSchedMfma = 0x008, kSchedDsRead = 0x100;
-
-template <int MASK, int COUNT>
-__device__ __forceinline__ void sched_group() {
-    if constexpr (COUNT > 0) __builtin_amdgcn_sched_group_barrier(MASK, COUNT, 0);
-}
-// Asks the scheduler for MFMAS matrix instructions with EXTRA0 instructions of class CLASS0 spread
-// evenly between the first SPAN of them (and EXTRA1 of CLASS1 likewise), so that their issue slots
-// fall in the shadow of an MFMA and their results have the remaining MFMAs' time to arrive.
-template <int MFMAS, int SPAN, int CLASS0, int EXTRA0, int CLASS1, int EXTRA1, int I = 0>
-__device__ __forceinline__ void sched_interleave() {
-    if constexpr (I < MFMAS) {
-        constexpr int before = I < SPAN ? I : SPAN, after = I + 1 < SPAN ? I + 1 : SPAN;
-        sched_group<kSchedMfma, 1>();
-        sched_group<CLASS0, (after * EXTRA0) / SPAN - (before * EXTRA0) / SPAN>();
-        sched_group<CLASS1, (after * EXTRA1) / SPAN - (before * EXTRA1) / SPAN>();
-        sched_interleave<MFMAS, SPAN, CLASS0, EXTRA0, CLASS1, EXTRA1, I + 1>();
-    }
-}
-
 // s_waitcnt immediate that waits until at most `count` vector-memory operations are outstanding
 // (and for nothing else).
 constexpr int vmcnt_immediate(int count) { return (count & 15) | ((count >> 4) << 14) | 0x0F70; }
@@ -236,7 +215,6 @@ struct KTile {
     static constexpr int kRowsPerLoad = 64 / kChunksPerRow;
     static constexpr int kElems = ROWS * kBK;
     static constexpr int kLoads = ROWS / kRowsPerLoad / kWaves;  // load instructions per wavefront and tile
-    static constexpr int kFragReads = 1;                        // LDS instructions per fragment
 
     u32x4 rsrc = {0u, 0u, 0u, 0u};
     int voffset = 0;
@@ -281,7 +259,6 @@ struct NTile {
     static constexpr int kRowsPerLoad = 64 / kChunksPerRow;  // k rows one load instruction covers (2 or 4)
     static constexpr int kElems = kBK * COLS;
     static constexpr int kLoads = kBK / kRowsPerLoad / kWaves;
-    static constexpr int kFragReads = 2;
 
     u32x4 rsrc = {0u, 0u, 0u, 0u};
     int voffset = 0;
@@ -700,7 +677,6 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
     // MFMA is followed by its share of the loads and fragment reads and a scheduling fence keeps
     // them there.
     constexpr int kMfmas = TM * TN;
-    constexpr int kFrags = TM + TN;
     constexpr int kHalf = TN / 2;
     static_assert(TN % 2 == 0 && kHalf <= TM, "the left-half B fragments are read one per row");
     // HALF 0: this_tile = tile t (its right-half B fragments are read); HALF 1: next_tile = tile t+1.

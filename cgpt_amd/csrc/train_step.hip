@@ -107,6 +107,7 @@ struct cgptx_model {
          *d_norm_in = nullptr, *d_attn_out = nullptr, *d_q = nullptr,
          *d_k = nullptr, *d_v = nullptr, *d_q_pre = nullptr, *d_k_pre = nullptr;
     cgptx_adamw_workspace* optimizer = nullptr;
+    std::uint64_t initial_step = 0;  // step count the optimizer workspace starts from when it is first used
     std::vector<cgptx_adamw_entry> entries;
     // captured graph
     hipGraphExec_t graph_exec = nullptr;
@@ -575,6 +576,102 @@ extern "C" int cgptx_model_set_tokens(cgptx_model* m, const uint32_t* inputs, co
     return CGPTX_OK;
 }
 
+// ---- token upload: two pinned host slots, one event each ------------------------------------------
+struct cgptx_token_upload {
+    std::size_t count = 0;                         // tokens per batch
+    std::uint32_t* inputs[2] = {nullptr, nullptr};  // pinned
+    std::uint32_t* targets[2] = {nullptr, nullptr};
+    hipEvent_t copied[2] = {nullptr, nullptr};      // recorded after the copies out of a slot
+    bool in_flight[2] = {false, false};
+    int slot = 0;                                   // the one handed out by acquire
+    bool acquired = false;
+};
+
+extern "C" int cgptx_token_upload_create(cgptx_token_upload** out, size_t batch, size_t sequence) {
+    using namespace cgptx;
+    clear_error();
+    if (out == nullptr) return fail(CGPTX_INVALID_ARGUMENT, "token_upload_create: null argument");
+    if (batch != 0 && sequence > static_cast<std::size_t>(-1) / sizeof(std::uint32_t) / batch)
+        return fail(CGPTX_OVERFLOW, "token_upload_create: batch size overflows");
+    auto* u = new cgptx_token_upload();
+    u->count = batch * sequence;
+    const std::size_t bytes = std::max<std::size_t>(u->count, 1) * sizeof(std::uint32_t);
+    int status = CGPTX_OK;
+    for (int s = 0; s < 2 && status == CGPTX_OK; ++s) {
+        // Allocated pinned (registering existing memory is not an option everywhere).
+        status = check_hip(hipHostMalloc(reinterpret_cast<void**>(&u->inputs[s]), bytes, hipHostMallocDefault), "hipHostMalloc");
+        if (status == CGPTX_OK)
+            status = check_hip(hipHostMalloc(reinterpret_cast<void**>(&u->targets[s]), bytes, hipHostMallocDefault), "hipHostMalloc");
+        if (status == CGPTX_OK) status = check_hip(hipEventCreateWithFlags(&u->copied[s], hipEventDisableTiming), "hipEventCreate");
+    }
+    if (status != CGPTX_OK) {
+        cgptx_token_upload_destroy(u);
+        return status;
+    }
+    *out = u;
+    return CGPTX_OK;
+}
+
+extern "C" int cgptx_token_upload_destroy(cgptx_token_upload* u) {
+    if (u == nullptr) return CGPTX_OK;
+    for (int s = 0; s < 2; ++s) {
+        if (u->copied[s] != nullptr) {
+            if (u->in_flight[s]) (void)hipEventSynchronize(u->copied[s]);
+            (void)hipEventDestroy(u->copied[s]);
+        }
+        if (u->inputs[s] != nullptr) (void)hipHostFree(u->inputs[s]);
+        if (u->targets[s] != nullptr) (void)hipHostFree(u->targets[s]);
+    }
+    delete u;
+    return CGPTX_OK;
+}
+
+extern "C" int cgptx_token_upload_acquire(cgptx_token_upload* u, uint32_t** inputs, uint32_t** targets) {
+    using namespace cgptx;
+    clear_error();
+    if (u == nullptr || inputs == nullptr || targets == nullptr)
+        return fail(CGPTX_INVALID_ARGUMENT, "token_upload_acquire: null argument");
+    // Batch::wait_until_reusable: the copies out of this slot, enqueued two submits ago, must be done
+    // before the host writes it again.
+    if (u->in_flight[u->slot]) {
+        CGPTX_HIP(hipEventSynchronize(u->copied[u->slot]));
+        u->in_flight[u->slot] = false;
+    }
+    *inputs = u->inputs[u->slot];
+    *targets = u->targets[u->slot];
+    u->acquired = true;
+    return CGPTX_OK;
+}
+
+extern "C" int cgptx_token_upload_submit(cgptx_token_upload* u, uint32_t* device_inputs, uint32_t* device_targets,
+                                         cgptx_stream stream_) {
+    using namespace cgptx;
+    clear_error();
+    if (u == nullptr || device_inputs == nullptr || device_targets == nullptr)
+        return fail(CGPTX_INVALID_ARGUMENT, "token_upload_submit: null argument");
+    if (!u->acquired) return fail(CGPTX_INVALID_ARGUMENT, "token_upload_submit: no slot was acquired");
+    auto stream = static_cast<hipStream_t>(stream_);
+    const std::size_t bytes = u->count * sizeof(std::uint32_t);
+    if (bytes != 0) {
+        CGPTX_HIP(hipMemcpyAsync(device_inputs, u->inputs[u->slot], bytes, hipMemcpyHostToDevice, stream));
+        CGPTX_HIP(hipMemcpyAsync(device_targets, u->targets[u->slot], bytes, hipMemcpyHostToDevice, stream));
+    }
+    CGPTX_HIP(hipEventRecord(u->copied[u->slot], stream));  // Batch::mark_upload_complete
+    u->in_flight[u->slot] = true;
+    u->acquired = false;
+    u->slot ^= 1;
+    return CGPTX_OK;
+}
+
+extern "C" int cgptx_model_upload_tokens(cgptx_model* m, cgptx_token_upload* u, cgptx_stream stream) {
+    using namespace cgptx;
+    clear_error();
+    if (m == nullptr || u == nullptr) return fail(CGPTX_INVALID_ARGUMENT, "model_upload_tokens: null argument");
+    if (u->count != m->rows)
+        return fail(CGPTX_INVALID_ARGUMENT, "model_upload_tokens: batch buffers do not match the model's step shape");
+    return cgptx_token_upload_submit(u, m->tokens, m->targets, stream);
+}
+
 extern "C" int cgptx_model_forward_backward(cgptx_model* m, float loss_scale, int loss_mode, int use_graph,
                                             cgptx_stream stream_) {
     using namespace cgptx;
@@ -627,7 +724,8 @@ extern "C" int cgptx_model_forward_backward(cgptx_model* m, float loss_scale, in
 extern "C" int cgptx_model_optimizer_step(cgptx_model* m, const cgptx_adamw_options* options, cgptx_stream stream) {
     using namespace cgptx;
     if (m == nullptr) return fail(CGPTX_INVALID_ARGUMENT, "model_optimizer_step: null model");
-    return cgptx_adamw_step_many_async(m->optimizer, m->entries.data(), m->entries.size(), options, 0, stream);
+    return cgptx_adamw_step_many_async(m->optimizer, m->entries.data(), m->entries.size(), options, m->initial_step,
+                                       stream);
 }
 
 extern "C" int cgptx_model_train_step(cgptx_model* m, const cgptx_adamw_options* options, int loss_mode,
@@ -703,6 +801,38 @@ extern "C" int cgptx_model_parameter(const cgptx_model* m, size_t index, const c
     if (parameter != nullptr) *parameter = all[index]->value;
     if (gradient != nullptr) *gradient = all[index]->gradient;
     if (count != nullptr) *count = all[index]->count;
+    return CGPTX_OK;
+}
+
+extern "C" int cgptx_model_describe(const cgptx_model* m, cgptx_model_config* config, size_t* batch, size_t* sequence) {
+    using namespace cgptx;
+    if (m == nullptr) return fail(CGPTX_INVALID_ARGUMENT, "model_describe: null model");
+    if (config != nullptr) *config = m->config;
+    if (batch != nullptr) *batch = m->batch;
+    if (sequence != nullptr) *sequence = m->sequence;
+    return CGPTX_OK;
+}
+
+extern "C" int cgptx_model_optimizer_state(const cgptx_model* m, size_t index, float** master, float** first_moment,
+                                           float** second_moment) {
+    using namespace cgptx;
+    if (m == nullptr || index >= m->entries.size())
+        return fail(CGPTX_INVALID_ARGUMENT, "model_optimizer_state: index out of range");
+    if (master != nullptr) *master = m->entries[index].master_parameter;
+    if (first_moment != nullptr) *first_moment = m->entries[index].first_moment;
+    if (second_moment != nullptr) *second_moment = m->entries[index].second_moment;
+    return CGPTX_OK;
+}
+
+extern "C" int cgptx_model_set_optimizer_step(cgptx_model* m, uint64_t step) {
+    using namespace cgptx;
+    if (m == nullptr) return fail(CGPTX_INVALID_ARGUMENT, "model_set_optimizer_step: null model");
+    CGPTX_HIP(hipDeviceSynchronize());
+    // The workspace reads its starting step when it is first used: a fresh one picks the new value up.
+    if (int s = cgptx_adamw_workspace_destroy(m->optimizer)) return s;
+    m->optimizer = nullptr;
+    if (int s = cgptx_adamw_workspace_create(&m->optimizer)) return s;
+    m->initial_step = step;
     return CGPTX_OK;
 }
 

@@ -85,6 +85,33 @@ class Model:
         capi.call("cgptx_model_set_tokens", self._handle, a.ctypes.data_as(ctypes.c_void_p),
                   b.ctypes.data_as(ctypes.c_void_p))
 
+    def upload_tokens(self, upload: "TokenUpload", stream=None) -> None:
+        """Enqueues the asynchronous copy of the upload's acquired slot into the model's token buffers."""
+        capi.call("cgptx_model_upload_tokens", self._handle, upload._handle, _stream(stream))
+
+    def save_checkpoint(self, directory, max_position_embeddings=None) -> None:
+        """config.json + model.safetensors with the reference exporter's names (directory must exist)."""
+        capi.call("cgptx_model_save_checkpoint", self._handle, str(directory).encode(),
+                  self.sequence if max_position_embeddings is None else max_position_embeddings)
+
+    def load_checkpoint(self, directory) -> None:
+        capi.call("cgptx_model_load_checkpoint", self._handle, str(directory).encode())
+
+    def save_optimizer(self, path, step: int) -> None:
+        capi.call("cgptx_model_save_optimizer", self._handle, str(path).encode(), step)
+
+    def load_optimizer(self, path) -> int:
+        step = ctypes.c_uint64(0)
+        capi.call("cgptx_model_load_optimizer", self._handle, str(path).encode(), ctypes.byref(step))
+        return step.value
+
+    def optimizer_state(self, index: int):
+        """(master, first moment, second moment) of parameter `index` as flat fp32 views."""
+        count = self.parameters()[index][1].numel()
+        m, a, b = ctypes.c_void_p(), ctypes.c_void_p(), ctypes.c_void_p()
+        capi.call("cgptx_model_optimizer_state", self._handle, index, ctypes.byref(m), ctypes.byref(a), ctypes.byref(b))
+        return tuple(_as_tensor(x.value, count, torch.float32, self.device) for x in (m, a, b))
+
     def forward_backward(self, loss_scale=1.0, loss_mode=LOSS_CUT, use_graph=False, stream=None) -> None:
         capi.call("cgptx_model_forward_backward", self._handle, loss_scale, loss_mode, int(use_graph),
                   _stream(stream))
@@ -131,3 +158,38 @@ class Model:
             capi.call("cgptx_model_profile_entry", self._handle, i, ctypes.byref(label), ctypes.byref(ms))
             out[label.value.decode()] = ms.value
         return out
+
+
+class TokenUpload:
+    """Two page-locked host slots for [batch, sequence] input and target ids and their asynchronous
+    upload (the reference's pair of data::Batch with data::upload_batch, train/train.cpp:463-465,
+    570-574). `acquire()` returns numpy views of the slot to fill next (waiting until its previous
+    upload has finished); `Model.upload_tokens` or `submit` enqueues the copies and switches slots."""
+
+    def __init__(self, batch: int, sequence: int):
+        self.batch, self.sequence = batch, sequence
+        handle = ctypes.c_void_p()
+        capi.call("cgptx_token_upload_create", ctypes.byref(handle), batch, sequence)
+        self._handle = handle
+
+    def close(self):
+        if getattr(self, "_handle", None):
+            capi.call("cgptx_token_upload_destroy", self._handle)
+            self._handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def acquire(self):
+        a, b = ctypes.c_void_p(), ctypes.c_void_p()
+        capi.call("cgptx_token_upload_acquire", self._handle, ctypes.byref(a), ctypes.byref(b))
+        n = self.batch * self.sequence
+        as_array = lambda p: np.ctypeslib.as_array(ctypes.cast(p, ctypes.POINTER(ctypes.c_uint32)), shape=(n,))
+        return as_array(a), as_array(b)
+
+    def submit(self, device_inputs: torch.Tensor, device_targets: torch.Tensor, stream=None) -> None:
+        capi.call("cgptx_token_upload_submit", self._handle, ctypes.c_void_p(device_inputs.data_ptr()),
+                  ctypes.c_void_p(device_targets.data_ptr()), _stream(stream))

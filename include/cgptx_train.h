@@ -50,6 +50,24 @@ int cgptx_model_destroy(cgptx_model* model);
  * device buffers (data::upload_batch, src/data/dataset_loader.cpp:145-166). Synchronous. */
 int cgptx_model_set_tokens(cgptx_model* model, const uint32_t* inputs, const uint32_t* targets);
 
+/* data::Batch x 2 + data::upload_batch (include/data/dataset_loader.h:111-170 →
+ * src/data/dataset_loader.cpp:120-166; train/train.cpp:463-465, 570-574): two page-locked host
+ * slots for [batch, sequence] input and target ids, each with the event that says when the copies
+ * out of it have finished. acquire hands out the slot to fill next and first waits until its last
+ * upload has completed (Batch::wait_until_reusable); submit enqueues the two asynchronous copies
+ * to the device buffers on `stream`, records the slot's event (Batch::mark_upload_complete) and
+ * switches to the other slot. Nothing but acquire ever blocks the host. */
+typedef struct cgptx_token_upload cgptx_token_upload;
+int cgptx_token_upload_create(cgptx_token_upload** upload, size_t batch, size_t sequence);
+int cgptx_token_upload_destroy(cgptx_token_upload* upload);
+int cgptx_token_upload_acquire(cgptx_token_upload* upload, uint32_t** inputs, uint32_t** targets);
+int cgptx_token_upload_submit(cgptx_token_upload* upload, uint32_t* device_inputs, uint32_t* device_targets,
+                              cgptx_stream stream);
+/* submit into the model's own token buffers, whose addresses a captured step keeps reading
+ * (train/train.cpp:551-553 checks exactly that they never change). INVALID_ARGUMENT when the
+ * upload's shape is not the model's ("Batch buffers do not match its declared shape"). */
+int cgptx_model_upload_tokens(cgptx_model* model, cgptx_token_upload* upload, cgptx_stream stream);
+
 /* Enqueues forward + loss + backward on `stream` (gradient of loss·loss_scale). With use_graph
  * the sequence is captured on first use (after one eager run) and replayed afterwards. */
 int cgptx_model_forward_backward(cgptx_model* model, float loss_scale, int loss_mode, int use_graph,
@@ -80,6 +98,32 @@ int cgptx_model_parameter(const cgptx_model* model, size_t index, const char** n
                           void** gradient, size_t* count);
 /* Total number of parameters (tied embedding counted once). */
 size_t cgptx_model_num_parameters(const cgptx_model* model);
+
+/* The configuration and step shape the model was created with. */
+int cgptx_model_describe(const cgptx_model* model, cgptx_model_config* config, size_t* batch, size_t* sequence);
+/* Device pointers to the AdamW state of parameter `index`: fp32 master copy, first and second moment
+ * (AdamWState, include/optim/adamw.h:45-58). */
+int cgptx_model_optimizer_state(const cgptx_model* model, size_t index, float** master, float** first_moment,
+                                float** second_moment);
+/* Makes the optimizer continue from `step` completed steps (bias correction uses step + 1 next).
+ * Synchronises the device. */
+int cgptx_model_set_optimizer_step(cgptx_model* model, uint64_t step);
+
+/* export_huggingface_model without the tokenizer files (include/core/huggingface_export.h →
+ * src/core/huggingface_export.cpp:135-158, 180-225, 345-380): writes `config.json` (same keys) and
+ * `model.safetensors` (same tensor names, order and layout; the tied classifier is written as
+ * `lm_head.weight` too) into an existing directory. Synchronises the device. */
+int cgptx_model_save_checkpoint(const cgptx_model* model, const char* directory, size_t max_position_embeddings);
+/* load_huggingface_model (src/core/huggingface_export.cpp:400-430): reads `model.safetensors` from
+ * `directory` into the model's weights; every tensor of the list must be present with the model's
+ * dtype, shape and byte size (RUNTIME status otherwise, nothing is loaded partially into a tensor).
+ * The fp32 master copies restart from the loaded values; moments and step are left alone. */
+int cgptx_model_load_checkpoint(cgptx_model* model, const char* directory);
+/* Optimizer state, which the reference does not save: `<name>.master`, `.exp_avg`, `.exp_avg_sq`
+ * (fp32) and the step counter `step` (U64) in one safetensors file. `step` is the count
+ * cgptx_model_status last reported. Loading also restores the step counter. */
+int cgptx_model_save_optimizer(const cgptx_model* model, const char* path, uint64_t step);
+int cgptx_model_load_optimizer(cgptx_model* model, const char* path, uint64_t* step);
 
 /* Device pointer to a named saved activation of the last forward ("hidden.<l>", "logits" ...);
  * used by tests. Returns INVALID_ARGUMENT for unknown names. */
