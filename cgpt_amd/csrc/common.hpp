@@ -106,6 +106,21 @@ int rmsnorm_backward_residual(void* grad_input, void* grad_weight, const void* g
                               const void* weight, const void* residual, std::size_t rows, std::size_t hidden,
                               float epsilon, int dtype, hipStream_t stream);
 
+// Per-head RMSNorm and rotary embedding in one pass over [rows = tokens x heads, head_dim]:
+//   forward   output = rope(rmsnorm(input));   backward   the gradient of that, with the weight gradient.
+// Bit for bit what the separate operators give (their intermediate roundings are kept). Positions are
+// position_offset + token % sequence, token = row / heads. `rmsnorm_rope_fusable` says whether the shape,
+// dtype and alignment are served; callers run the separate operators otherwise.
+bool rmsnorm_rope_fusable(const void* a, const void* b, const void* c, const void* weight, const void* cos_cache,
+                          const void* sin_cache, std::size_t head_dim, std::size_t rotary_dim, int dtype);
+int rmsnorm_rope_forward(void* output, const void* input, const void* weight, const void* cos_cache, const void* sin_cache,
+                         std::size_t rows, std::size_t head_dim, std::size_t heads, std::size_t sequence,
+                         std::size_t rotary_dim, std::size_t position_offset, float epsilon, int dtype, hipStream_t stream);
+int rmsnorm_rope_backward(void* grad_input, void* grad_weight, const void* grad_output, const void* input,
+                          const void* weight, const void* cos_cache, const void* sin_cache, std::size_t rows,
+                          std::size_t head_dim, std::size_t heads, std::size_t sequence, std::size_t rotary_dim,
+                          std::size_t position_offset, float epsilon, int dtype, hipStream_t stream);
+
 // ---- scratch arena ----------------------------------------------------------
 // Returns `bytes` of device scratch bound to (current device, stream), 256-byte
 // aligned. Grows by reallocation on eager calls; refuses to grow during capture.

@@ -26,14 +26,65 @@ namespace {
 constexpr int kThreads = 256;
 constexpr int kWavesPerBlock = kThreads / kWave;
 
+// Rotary embedding applied to the rows on the way (rows are heads of head_dim = hidden elements):
+// forward  y = rope(round(rmsnorm(x)));  backward  the incoming gradient is rotated back (and
+// rounded) first. The roundings are those of the separate operators' stores, so the fused pass gives
+// bit for bit what rmsnorm and rope give one after the other.
+struct RopeArgs {
+    const void* cos_cache;  // [positions, rotary_dim/2], element type of the rows
+    const void* sin_cache;
+    int heads;      // rows per token
+    int sequence;   // tokens per sequence: position = offset + token % sequence
+    int rotary_dim;
+    int position_offset;
+};
+
+// Rotation of the pair (x, y) by +angle (forward) or -angle (backward); the arithmetic of the
+// separate rotary kernels.
+template <bool Inverse>
+__device__ __forceinline__ void rotate_pair(float x, float y, float c, float s, float& ox, float& oy) {
+    if constexpr (Inverse) {
+        ox = fmaf(y, s, x * c);
+        oy = fmaf(-x, s, y * c);
+    } else {
+        ox = fmaf(-y, s, x * c);
+        oy = fmaf(x, s, y * c);
+    }
+}
+
+template <typename T, bool Inverse>
+__device__ __forceinline__ vec_t<float, kVec128<T>> rope_vector(vec_t<float, kVec128<T>> v, const RopeArgs& rope, int row,
+                                                                int col) {
+    constexpr int VEC = kVec128<T>;
+    constexpr int HALF = VEC / 2;
+    // What the separate operator would have read back from memory.
+    v = vec_to_f32<T, VEC>(vec_from_f32<T, VEC>(v));
+    if (col >= rope.rotary_dim) return v;
+    const int token = row / rope.heads;
+    const int pos = rope.position_offset + token % rope.sequence;
+    const std::size_t index = static_cast<std::size_t>(pos) * (rope.rotary_dim / 2) + col / 2;
+    const vec_t<float, HALF> c = vec_to_f32<T, HALF>(load_vec<T, HALF>(static_cast<const T*>(rope.cos_cache) + index));
+    const vec_t<float, HALF> s = vec_to_f32<T, HALF>(load_vec<T, HALF>(static_cast<const T*>(rope.sin_cache) + index));
+    vec_t<float, VEC> r;
+#pragma unroll
+    for (int p = 0; p < HALF; ++p) {
+        float a, b;
+        rotate_pair<Inverse>(v[2 * p], v[2 * p + 1], c[p], s[p], a, b);
+        r[2 * p] = a;
+        r[2 * p + 1] = b;
+    }
+    return r;
+}
+
 // ------------------------------------------------------------------ fast path
-template <typename T, int LPR, int K, bool Backward>
+template <typename T, int LPR, int K, bool Backward, bool Rope = false>
 __global__ __launch_bounds__(kThreads) void rmsnorm_rows_kernel(
     T* out,                         // dx (backward) or y (forward)
     float* __restrict__ partial,    // [gridDim.x, H] dgamma partials (backward)
-    const T* __restrict__ dy,       // backward only
+    const T* dy,                    // backward only; may be out itself
     const T* residual,              // backward only, optional: added to dx (may be out itself)
-    const T* __restrict__ x, const T* __restrict__ w, int rows, int hidden, float inv_hidden, float eps) {
+    const T* __restrict__ x, const T* __restrict__ w, int rows, int hidden, float inv_hidden, float eps,
+    RopeArgs rope = RopeArgs{}) {
     constexpr int VEC = kVec128<T>;
     constexpr int RPW = kWave / LPR;  // rows per wavefront iteration
     using F = vec_t<float, VEC>;
@@ -67,7 +118,10 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_rows_kernel(
             const int col = (c * LPR + sub) * VEC;
             if (row_live && live[c]) {
                 xv[c] = vec_to_f32<T, VEC>(load_vec<T, VEC>(x + base + col));
-                if constexpr (Backward) gv[c] = vec_to_f32<T, VEC>(load_vec<T, VEC>(dy + base + col));
+                if constexpr (Backward) {
+                    gv[c] = vec_to_f32<T, VEC>(load_vec<T, VEC>(dy + base + col));
+                    if constexpr (Rope) gv[c] = vec_to_f32<T, VEC>(vec_from_f32<T, VEC>(rope_vector<T, true>(gv[c], rope, row, col)));
+                }
             } else {
                 xv[c] = F(0.0f);
                 if constexpr (Backward) gv[c] = F(0.0f);
@@ -108,7 +162,10 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_rows_kernel(
 #pragma unroll
                 for (int e = 0; e < VEC; ++e) r[e] = xv[c][e] * inv * wv[c][e];
                 const int col = (c * LPR + sub) * VEC;
-                if (row_live && live[c]) store_vec<T, VEC>(out + base + col, vec_from_f32<T, VEC>(r));
+                if (row_live && live[c]) {
+                    if constexpr (Rope) r = rope_vector<T, false>(r, rope, row, col);
+                    store_vec<T, VEC>(out + base + col, vec_from_f32<T, VEC>(r));
+                }
             }
         }
     }
@@ -232,8 +289,14 @@ FastShape pick_fast_shape(int hidden) {
 
 template <typename T, bool Backward>
 int launch_fast(const FastShape shape, T* out, float* partial, const T* dy, const T* residual, const T* x, const T* w,
-                int rows, int hidden, float eps, int blocks, hipStream_t stream) {
+                int rows, int hidden, float eps, int blocks, hipStream_t stream, const RopeArgs* rope = nullptr) {
     const float inv_hidden = 1.0f / static_cast<float>(hidden);
+    if (rope != nullptr) {
+        if (shape.lpr != 16 || shape.k != 1) return fail(CGPTX_RUNTIME, "rmsnorm: no rotary kernel for shape");
+        hipLaunchKernelGGL((rmsnorm_rows_kernel<T, 16, 1, Backward, true>), dim3(blocks), dim3(kThreads), 0, stream, out,
+                           partial, dy, residual, x, w, rows, hidden, inv_hidden, eps, *rope);
+        return CGPTX_OK;
+    }
 #define CGPTX_RMS_CASE(L, KK)                                                                             \
     if (shape.lpr == L && shape.k == KK) {                                                                \
         hipLaunchKernelGGL((rmsnorm_rows_kernel<T, L, KK, Backward>), dim3(blocks), dim3(kThreads), 0,   \
@@ -272,6 +335,91 @@ int validate(const void* a, const void* b, const void* c, std::size_t rows, std:
 }
 
 }  // namespace
+
+bool rmsnorm_rope_fusable(const void* a, const void* b, const void* c, const void* weight, const void* cos_cache,
+                          const void* sin_cache, std::size_t head_dim, std::size_t rotary_dim, int dtype) {
+    if (!valid_dtype(dtype) || head_dim == 0 || head_dim > 4096) return false;
+    const std::size_t elem = dtype_size(dtype), vec = 16 / elem;
+    bool shape_ok = false;
+    dispatch_dtype(dtype, [&]<typename T>() -> int {
+        const FastShape shape = pick_fast_shape<T>(static_cast<int>(head_dim));
+        shape_ok = shape.lpr == 16 && shape.k == 1;
+        return CGPTX_OK;
+    });
+    const auto half_aligned = [&](const void* p) { return (reinterpret_cast<std::uintptr_t>(p) % (vec / 2 * elem)) == 0; };
+    return shape_ok && rotary_dim % vec == 0 && rotary_dim <= head_dim && is_aligned16(a) && is_aligned16(b) &&
+           (c == nullptr || is_aligned16(c)) && is_aligned16(weight) && half_aligned(cos_cache) && half_aligned(sin_cache);
+}
+
+namespace {
+RopeArgs make_rope(const void* cos_cache, const void* sin_cache, std::size_t heads, std::size_t sequence,
+                   std::size_t rotary_dim, std::size_t position_offset) {
+    return RopeArgs{cos_cache, sin_cache, static_cast<int>(heads), static_cast<int>(sequence), static_cast<int>(rotary_dim),
+                    static_cast<int>(position_offset)};
+}
+}  // namespace
+
+int rmsnorm_rope_forward(void* output, const void* input, const void* weight, const void* cos_cache, const void* sin_cache,
+                         std::size_t rows, std::size_t head_dim, std::size_t heads, std::size_t sequence,
+                         std::size_t rotary_dim, std::size_t position_offset, float epsilon, int dtype, hipStream_t stream) {
+    if (int s = validate(output, input, weight, rows, head_dim, epsilon, dtype, "rmsnorm_rope_forward")) return s;
+    if (cos_cache == nullptr || sin_cache == nullptr || heads == 0 || sequence == 0 ||
+        !rmsnorm_rope_fusable(output, input, nullptr, weight, cos_cache, sin_cache, head_dim, rotary_dim, dtype))
+        return fail(CGPTX_INVALID_ARGUMENT, "rmsnorm_rope_forward: shape or alignment not served by the fused pass");
+    const int r = static_cast<int>(rows), h = static_cast<int>(head_dim);
+    const RopeArgs rope = make_rope(cos_cache, sin_cache, heads, sequence, rotary_dim, position_offset);
+    return dispatch_dtype(dtype, [&]<typename T>() -> int {
+        const FastShape shape = pick_fast_shape<T>(h);
+        if (int s = launch_fast<T, false>(shape, static_cast<T*>(output), nullptr, nullptr, nullptr,
+                                          static_cast<const T*>(input), static_cast<const T*>(weight), r, h, epsilon,
+                                          fast_blocks(shape, r), stream, &rope))
+            return s;
+        CGPTX_LAUNCH_CHECK();
+        return CGPTX_OK;
+    });
+}
+
+int rmsnorm_rope_backward(void* grad_input, void* grad_weight, const void* grad_output, const void* input,
+                          const void* weight, const void* cos_cache, const void* sin_cache, std::size_t rows,
+                          std::size_t head_dim, std::size_t heads, std::size_t sequence, std::size_t rotary_dim,
+                          std::size_t position_offset, float epsilon, int dtype, hipStream_t stream) {
+    if (int s = validate(grad_input, grad_output, input, rows, head_dim, epsilon, dtype, "rmsnorm_rope_backward")) return s;
+    if (grad_weight == nullptr || weight == nullptr || cos_cache == nullptr || sin_cache == nullptr || heads == 0 ||
+        sequence == 0 ||
+        !rmsnorm_rope_fusable(grad_input, grad_output, input, weight, cos_cache, sin_cache, head_dim, rotary_dim, dtype))
+        return fail(CGPTX_INVALID_ARGUMENT, "rmsnorm_rope_backward: shape or alignment not served by the fused pass");
+    const int r = static_cast<int>(rows), h = static_cast<int>(head_dim);
+    const RopeArgs rope = make_rope(cos_cache, sin_cache, heads, sequence, rotary_dim, position_offset);
+    return dispatch_dtype(dtype, [&]<typename T>() -> int {
+        const FastShape shape = pick_fast_shape<T>(h);
+        const int blocks = fast_blocks(shape, r);
+        const int reduce_blocks = (h + kWave - 1) / kWave;
+        const int slices = wide_reduce_slices(blocks, h, compute_units());
+        void* mem = nullptr;
+        const std::size_t partial_bytes = static_cast<std::size_t>(blocks) * head_dim * sizeof(float);
+        if (int s = scratch(stream, partial_bytes + static_cast<std::size_t>(slices) * head_dim * sizeof(float), &mem)) return s;
+        auto* partial = static_cast<float*>(mem);
+        if (int s = launch_fast<T, true>(shape, static_cast<T*>(grad_input), partial, static_cast<const T*>(grad_output),
+                                         nullptr, static_cast<const T*>(input), static_cast<const T*>(weight), r, h, epsilon,
+                                         blocks, stream, &rope))
+            return s;
+        CGPTX_LAUNCH_CHECK();
+        auto* dw = static_cast<T*>(grad_weight);
+        if (slices > 1) {
+            auto* second = reinterpret_cast<float*>(static_cast<char*>(mem) + partial_bytes);
+            hipLaunchKernelGGL(column_partial_fold_kernel, dim3(reduce_blocks, slices), dim3(kThreads), 0, stream, second,
+                               partial, blocks, h);
+            CGPTX_LAUNCH_CHECK();
+            hipLaunchKernelGGL((column_partial_reduce_kernel<T>), dim3(reduce_blocks), dim3(kThreads), 0, stream, dw, second,
+                               slices, h, 0);
+        } else {
+            hipLaunchKernelGGL((column_partial_reduce_kernel<T>), dim3(reduce_blocks), dim3(kThreads), 0, stream, dw, partial,
+                               blocks, h, 0);
+        }
+        CGPTX_LAUNCH_CHECK();
+        return CGPTX_OK;
+    });
+}
 
 int rmsnorm_backward_residual(void* grad_input, void* grad_weight, const void* grad_output, const void* input,
                               const void* weight, const void* residual, std::size_t rows, std::size_t hidden,

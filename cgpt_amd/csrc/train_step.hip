@@ -18,6 +18,7 @@
 #include "gemm.hpp"
 
 #include <cmath>
+#include <cstdlib>
 #include <cstring>
 #include <string>
 #include <vector>
@@ -321,6 +322,15 @@ int qkv_backward_weight(void* qkv_gradient, const void* dq, const void* dk, cons
     return gemm(g, stream);
 }
 
+// Whether the per-head norm and the rotary embedding of q or k run as one pass (CGPTX_FUSE_QK=0 keeps
+// the separate operators, for comparisons).
+bool fused_qk_norm_rope(const cgptx_model* m, const void* a, const void* b, const void* c, const void* weight) {
+    const char* text = std::getenv("CGPTX_FUSE_QK");  // read per enqueue: a captured graph keeps what it was captured with
+    const bool enabled = text == nullptr || text[0] != '0';
+    return enabled && rmsnorm_rope_fusable(a, b, c, weight, m->cos_cache, m->sin_cache, m->config.head_dim,
+                                           m->config.rotary_dim, m->config.dtype);
+}
+
 int enqueue_forward_backward(cgptx_model* m, float loss_scale, int loss_mode, hipStream_t stream) {
     const auto& c = m->config;
     const int dt = c.dtype;
@@ -347,10 +357,17 @@ int enqueue_forward_backward(cgptx_model* m, float loss_scale, int loss_mode, hi
             CGPTX_OP("gemm_fwd", cgptx_linear_forward(a.k_pre, a.norm_a, w.k.value, nullptr, N, H, KW, dt, s));
             CGPTX_OP("gemm_fwd", cgptx_linear_forward(a.v, a.norm_a, w.v.value, nullptr, N, H, KW, dt, s));
         }
-        CGPTX_OP("rmsnorm_fwd", cgptx_rmsnorm_forward(a.q, a.q_pre, w.q_norm.value, N * HQ, D, eps, dt, s));
-        CGPTX_OP("rmsnorm_fwd", cgptx_rmsnorm_forward(a.k, a.k_pre, w.k_norm.value, N * HKV, D, eps, dt, s));
-        CGPTX_OP("rope_fwd", cgptx_rope_forward(a.q, a.k, m->cos_cache, m->sin_cache, m->batch, m->sequence, HQ, HKV, D,
-                                     c.rotary_dim, 0, m->sequence, dt, s));
+        if (fused_qk_norm_rope(m, a.q, a.q_pre, nullptr, w.q_norm.value) && fused_qk_norm_rope(m, a.k, a.k_pre, nullptr, w.k_norm.value)) {
+            CGPTX_OP("rmsnorm_fwd", rmsnorm_rope_forward(a.q, a.q_pre, w.q_norm.value, m->cos_cache, m->sin_cache, N * HQ, D, HQ,
+                                                         m->sequence, c.rotary_dim, 0, eps, dt, stream));
+            CGPTX_OP("rmsnorm_fwd", rmsnorm_rope_forward(a.k, a.k_pre, w.k_norm.value, m->cos_cache, m->sin_cache, N * HKV, D, HKV,
+                                                         m->sequence, c.rotary_dim, 0, eps, dt, stream));
+        } else {
+            CGPTX_OP("rmsnorm_fwd", cgptx_rmsnorm_forward(a.q, a.q_pre, w.q_norm.value, N * HQ, D, eps, dt, s));
+            CGPTX_OP("rmsnorm_fwd", cgptx_rmsnorm_forward(a.k, a.k_pre, w.k_norm.value, N * HKV, D, eps, dt, s));
+            CGPTX_OP("rope_fwd", cgptx_rope_forward(a.q, a.k, m->cos_cache, m->sin_cache, m->batch, m->sequence, HQ, HKV, D,
+                                         c.rotary_dim, 0, m->sequence, dt, s));
+        }
         CGPTX_OP("attn_fwd", cgptx_flash_gqa_attention_forward(a.attn_out, a.lse, a.q, a.k, a.v, m->batch, m->sequence,
                                                     m->sequence, HQ, HKV, D, 0.0f, 1, 0, dt, s));
         // out = x + attention_projection, then out += ffn_output (src/core/transformer_block.cu:594-595)
@@ -396,12 +413,21 @@ int enqueue_forward_backward(cgptx_model* m, float loss_scale, int loss_mode, hi
         CGPTX_OP("attn_bwd", cgptx_flash_gqa_attention_backward_with_lse(m->d_q, m->d_k, m->d_v, m->d_attn_out, a.attn_out,
                                                               a.lse, a.q, a.k, a.v, m->batch, m->sequence,
                                                               m->sequence, HQ, HKV, D, 0.0f, 1, 0, 0, dt, s));
-        CGPTX_OP("rope_bwd", cgptx_rope_backward(m->d_q_pre, m->d_k_pre, m->d_q, m->d_k, m->cos_cache, m->sin_cache, m->batch,
-                                      m->sequence, HQ, HKV, D, c.rotary_dim, 0, m->sequence, dt, s));
-        CGPTX_OP("rmsnorm_bwd", cgptx_rmsnorm_backward(m->d_q, w.q_norm.gradient, m->d_q_pre, a.q_pre, w.q_norm.value, N * HQ, D,
-                                         eps, dt, s));
-        CGPTX_OP("rmsnorm_bwd", cgptx_rmsnorm_backward(m->d_k, w.k_norm.gradient, m->d_k_pre, a.k_pre, w.k_norm.value, N * HKV, D,
-                                         eps, dt, s));
+        // In place over the attention gradients (a lane reads and writes the same elements).
+        if (fused_qk_norm_rope(m, m->d_q, m->d_q, a.q_pre, w.q_norm.value) &&
+            fused_qk_norm_rope(m, m->d_k, m->d_k, a.k_pre, w.k_norm.value)) {
+            CGPTX_OP("rmsnorm_bwd", rmsnorm_rope_backward(m->d_q, w.q_norm.gradient, m->d_q, a.q_pre, w.q_norm.value, m->cos_cache,
+                                                          m->sin_cache, N * HQ, D, HQ, m->sequence, c.rotary_dim, 0, eps, dt, stream));
+            CGPTX_OP("rmsnorm_bwd", rmsnorm_rope_backward(m->d_k, w.k_norm.gradient, m->d_k, a.k_pre, w.k_norm.value, m->cos_cache,
+                                                          m->sin_cache, N * HKV, D, HKV, m->sequence, c.rotary_dim, 0, eps, dt, stream));
+        } else {
+            CGPTX_OP("rope_bwd", cgptx_rope_backward(m->d_q_pre, m->d_k_pre, m->d_q, m->d_k, m->cos_cache, m->sin_cache, m->batch,
+                                          m->sequence, HQ, HKV, D, c.rotary_dim, 0, m->sequence, dt, s));
+            CGPTX_OP("rmsnorm_bwd", cgptx_rmsnorm_backward(m->d_q, w.q_norm.gradient, m->d_q_pre, a.q_pre, w.q_norm.value, N * HQ, D,
+                                             eps, dt, s));
+            CGPTX_OP("rmsnorm_bwd", cgptx_rmsnorm_backward(m->d_k, w.k_norm.gradient, m->d_k_pre, a.k_pre, w.k_norm.value, N * HKV, D,
+                                             eps, dt, s));
+        }
         if (fused_qkv) {
             CGPTX_OP("gemm_dx", qkv_backward_input(m->d_norm_in, m->d_q, m->d_k, m->d_v, w.q.value, N, H, QW, KW, dt, stream));
             CGPTX_OP("gemm_dw", qkv_backward_weight(w.q.gradient, m->d_q, m->d_k, m->d_v, a.norm_a, N, H, QW, KW, dt, stream));

@@ -247,3 +247,28 @@ def test_cpu_float32_step_matches_float64_composition():
     want_loss, want, _ = model64.forward_backward(params, tokens.numpy(), targets.numpy(), cfg, 8.0)
     assert abs(loss - want_loss) <= 1e-5 * want_loss
     compare_gradients(grads, want, 1e-4, 8.0)
+
+
+@pytest.mark.gpu
+def test_fused_qk_norm_rope_is_bit_identical_to_the_separate_operators(device, monkeypatch):
+    """Per-head RMSNorm + rotary embedding run as one pass (forward and backward) when head_dim is
+    served by the row kernel; the pass keeps the separate operators' intermediate roundings, so a whole
+    step gives the same bits either way. CGPTX_FUSE_QK=0 selects the separate operators."""
+    from cgpt_amd.model import LOSS_DENSE, Model, ModelConfig
+    config = ModelConfig(vocabulary_size=128, num_layers=2, hidden_size=256, intermediate_size=256, num_query_heads=4,
+                         num_kv_heads=2, head_dim=64, rotary_dim=32, dtype=torch.bfloat16)
+    rng = np.random.default_rng(3)
+    inputs = rng.integers(0, 128, size=2 * 48).astype(np.uint32)
+    targets = rng.integers(0, 128, size=2 * 48).astype(np.uint32)
+    results = []
+    for fuse in ("1", "0"):
+        monkeypatch.setenv("CGPTX_FUSE_QK", fuse)
+        model = Model(config, 2, 48, seed=4, device=device)
+        model.set_tokens(inputs, targets)
+        model.forward_backward(loss_scale=4.0, loss_mode=LOSS_DENSE)
+        loss = model.status()[0]
+        results.append((loss, [g.clone() for _, _, g in model.parameters()], model.activation("hidden.2").clone()))
+    assert results[0][0] == results[1][0]
+    assert torch.equal(results[0][2], results[1][2])
+    for a, b in zip(results[0][1], results[1][1]):
+        assert torch.equal(a, b)
