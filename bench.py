@@ -105,12 +105,18 @@ def measured_traffic():
 
 
 def cpu_baseline(seed):
-    """Times the CPU port on B=1, T=128 of the same 104m model (forward + loss + backward + AdamW)."""
+    """Times the CPU port on one step of the same 104m model (forward + loss + backward + AdamW) at B=1
+    and the longest sequence that keeps the sample near 10-30 s on this host: T doubles from 16 while the
+    last step took under 8 s and four times as long (the port's attention backward grows faster than
+    linearly in T) would still stay under 40 s. The last timing is the sample."""
     from oracle import cpu_model, cpu_ops
 
     cfg = dict(vocab=32000, layers=8, hidden=1024, inter=2048, hq=8, hkv=2, d=128, eps=1e-5)
-    batch, seq = 1, 128  # sized for 10-30 s on the 16 host cores of the GPU box
+    batch, seq = 1, 16
     seconds, loss = cpu_model.timed_train_step(cfg, batch, seq, seed)
+    while seconds < 8.0 and 4.0 * seconds < 40.0 and seq < 128:
+        seq *= 2
+        seconds, loss = cpu_model.timed_train_step(cfg, batch, seq, seed)
     return {"value": batch * seq / seconds, "unit": "tokens/s", "cores": cpu_ops.max_threads(), "kind": "port",
             "sample": f"one full 104m train step (fwd+loss+bwd+AdamW, fp32) at B={batch}, T={seq}: "
                       f"{seconds:.1f} s, loss {loss:.3f}; the fixed AdamW pass over 104M parameters is part of "
