@@ -121,6 +121,20 @@ int rmsnorm_rope_backward(void* grad_input, void* grad_weight, const void* grad_
                           std::size_t head_dim, std::size_t heads, std::size_t sequence, std::size_t rotary_dim,
                           std::size_t position_offset, float epsilon, int dtype, hipStream_t stream);
 
+// Two RMSNorms of the same rows with different weights in one pass (x is read once):
+//   forward   output_a = rmsnorm(input; weight_a), output_f = rmsnorm(input; weight_f)
+//   backward  grad_input = d(norm_a) + d(norm_f) + residual (residual may be null or alias grad_input),
+//             and both weight gradients. `rmsnorm_dual_fusable` says whether shape, dtype and the
+//             alignment of the five tensors are served.
+bool rmsnorm_dual_fusable(const void* a, const void* b, const void* c, const void* d, const void* e, std::size_t hidden,
+                          int dtype);
+int rmsnorm_forward_dual(void* output_a, void* output_f, const void* input, const void* weight_a, const void* weight_f,
+                         std::size_t rows, std::size_t hidden, float epsilon, int dtype, hipStream_t stream);
+int rmsnorm_backward_dual(void* grad_input, void* grad_weight_a, void* grad_weight_f, const void* grad_output_a,
+                          const void* grad_output_f, const void* input, const void* weight_a, const void* weight_f,
+                          const void* residual, std::size_t rows, std::size_t hidden, float epsilon, int dtype,
+                          hipStream_t stream);
+
 // ---- scratch arena ----------------------------------------------------------
 // Returns `bytes` of device scratch bound to (current device, stream), 256-byte
 // aligned. Grows by reallocation on eager calls; refuses to grow during capture.

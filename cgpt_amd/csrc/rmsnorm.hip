@@ -193,6 +193,134 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_rows_kernel(
     }
 }
 
+// Two RMSNorms of the same rows with different weights (the block's attention and feed-forward norms
+// both read the block input): one pass reads x once.
+//   forward   y_a = x r w_a,  y_f = x r w_f
+//   backward  dx = g r - x (sum_j g_j x_j) r^3 / H + residual  with g = dy_a w_a + dy_f w_f  (the two
+//             gradients add up before the row reduction: the norm is the same for both),
+//             dgamma_a = sum_rows dy_a x r,  dgamma_f = sum_rows dy_f x r
+template <typename T, int LPR, int K, bool Backward>
+__global__ __launch_bounds__(kThreads) void rmsnorm_dual_rows_kernel(
+    T* out_a,                       // y_a (forward) or dx (backward)
+    T* out_f,                       // y_f (forward)
+    float* __restrict__ partial_a,  // [gridDim.x, H] dgamma partials (backward)
+    float* __restrict__ partial_f,
+    const T* __restrict__ dy_a, const T* __restrict__ dy_f,  // backward only
+    const T* residual,              // backward only, optional: added to dx (may be out_a itself)
+    const T* __restrict__ x, const T* __restrict__ w_a, const T* __restrict__ w_f, int rows, int hidden,
+    float inv_hidden, float eps) {
+    constexpr int VEC = kVec128<T>;
+    constexpr int RPW = kWave / LPR;
+    using F = vec_t<float, VEC>;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    const int sub = lane % LPR;
+    const int rsel = lane / LPR;
+
+    F wa[K], wf[K], acc_a[K], acc_f[K];
+    bool live[K];
+#pragma unroll
+    for (int c = 0; c < K; ++c) {
+        const int col = (c * LPR + sub) * VEC;
+        live[c] = col < hidden;
+        wa[c] = live[c] ? vec_to_f32<T, VEC>(load_vec<T, VEC>(w_a + col)) : F(0.0f);
+        wf[c] = live[c] ? vec_to_f32<T, VEC>(load_vec<T, VEC>(w_f + col)) : F(0.0f);
+        acc_a[c] = F(0.0f);
+        acc_f[c] = F(0.0f);
+    }
+    const int groups = (rows + RPW - 1) / RPW;
+    const int wave_global = blockIdx.x * kWavesPerBlock + wave;
+    const int wave_count = gridDim.x * kWavesPerBlock;
+    for (int g = wave_global; g < groups; g += wave_count) {
+        const int row = g * RPW + rsel;
+        const bool row_live = row < rows;
+        const std::size_t base = static_cast<std::size_t>(row) * hidden;
+        F xv[K], ga[K], gf[K];
+#pragma unroll
+        for (int c = 0; c < K; ++c) {
+            const int col = (c * LPR + sub) * VEC;
+            const bool on = row_live && live[c];
+            xv[c] = on ? vec_to_f32<T, VEC>(load_vec<T, VEC>(x + base + col)) : F(0.0f);
+            if constexpr (Backward) {
+                ga[c] = on ? vec_to_f32<T, VEC>(load_vec<T, VEC>(dy_a + base + col)) : F(0.0f);
+                gf[c] = on ? vec_to_f32<T, VEC>(load_vec<T, VEC>(dy_f + base + col)) : F(0.0f);
+            }
+        }
+        float ss = 0.0f, dd = 0.0f;
+#pragma unroll
+        for (int c = 0; c < K; ++c) {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                ss = fmaf(xv[c][e], xv[c][e], ss);
+                if constexpr (Backward) dd = fmaf(fmaf(ga[c][e], wa[c][e], gf[c][e] * wf[c][e]), xv[c][e], dd);
+            }
+        }
+        ss = wave_sum<LPR>(ss);
+        const float inv = 1.0f / sqrtf(ss * inv_hidden + eps);
+        if constexpr (Backward) {
+            dd = wave_sum<LPR>(dd);
+            const float corr = dd * inv * inv * inv * inv_hidden;
+#pragma unroll
+            for (int c = 0; c < K; ++c) {
+                F r;
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    const float scaled = xv[c][e] * inv;
+                    r[e] = fmaf(ga[c][e], wa[c][e], gf[c][e] * wf[c][e]) * inv - xv[c][e] * corr;
+                    acc_a[c][e] = fmaf(ga[c][e], scaled, acc_a[c][e]);
+                    acc_f[c][e] = fmaf(gf[c][e], scaled, acc_f[c][e]);
+                }
+                const int col = (c * LPR + sub) * VEC;
+                if (row_live && live[c]) {
+                    if (residual != nullptr) r += vec_to_f32<T, VEC>(load_vec<T, VEC>(residual + base + col));
+                    store_vec<T, VEC>(out_a + base + col, vec_from_f32<T, VEC>(r));
+                }
+            }
+        } else {
+#pragma unroll
+            for (int c = 0; c < K; ++c) {
+                F ra, rf;
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    ra[e] = xv[c][e] * inv * wa[c][e];
+                    rf[e] = xv[c][e] * inv * wf[c][e];
+                }
+                const int col = (c * LPR + sub) * VEC;
+                if (row_live && live[c]) {
+                    store_vec<T, VEC>(out_a + base + col, vec_from_f32<T, VEC>(ra));
+                    store_vec<T, VEC>(out_f + base + col, vec_from_f32<T, VEC>(rf));
+                }
+            }
+        }
+    }
+    if constexpr (Backward) {
+        // Fold the RPW row slots of the wavefront, then the block's wavefronts; first one weight, then the other.
+        __shared__ float stage[kWavesPerBlock][LPR * K * VEC];
+#pragma unroll
+        for (int which = 0; which < 2; ++which) {
+#pragma unroll
+            for (int c = 0; c < K; ++c) {
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    float v = which == 0 ? acc_a[c][e] : acc_f[c][e];
+#pragma unroll
+                    for (int offset = LPR; offset < kWave; offset <<= 1) v += __shfl_xor(v, offset, kWave);
+                    if (rsel == 0) stage[wave][(c * LPR + sub) * VEC + e] = v;
+                }
+            }
+            __syncthreads();
+            float* partial = which == 0 ? partial_a : partial_f;
+            for (int col = threadIdx.x; col < hidden; col += kThreads) {
+                float v = 0.0f;
+#pragma unroll
+                for (int s = 0; s < kWavesPerBlock; ++s) v += stage[s][col];
+                partial[static_cast<std::size_t>(blockIdx.x) * hidden + col] = v;
+            }
+            __syncthreads();
+        }
+    }
+}
+
 // --------------------------------------------------------------- generic path
 template <typename T, bool Backward>
 __global__ __launch_bounds__(kThreads) void rmsnorm_row_generic_kernel(
@@ -417,6 +545,109 @@ int rmsnorm_rope_backward(void* grad_input, void* grad_weight, const void* grad_
                                blocks, h, 0);
         }
         CGPTX_LAUNCH_CHECK();
+        return CGPTX_OK;
+    });
+}
+
+bool rmsnorm_dual_fusable(const void* a, const void* b, const void* c, const void* d, const void* e, std::size_t hidden,
+                          int dtype) {
+    if (!valid_dtype(dtype) || hidden == 0 || hidden > (1u << 20)) return false;
+    bool shape_ok = false;
+    dispatch_dtype(dtype, [&]<typename T>() -> int {
+        shape_ok = pick_fast_shape<T>(static_cast<int>(hidden)).lpr != 0;
+        return CGPTX_OK;
+    });
+    return shape_ok && is_aligned16(a) && is_aligned16(b) && is_aligned16(c) && is_aligned16(d) && is_aligned16(e);
+}
+
+namespace {
+template <typename T, bool Backward>
+int launch_dual(const FastShape shape, T* out_a, T* out_f, float* partial_a, float* partial_f, const T* dy_a, const T* dy_f,
+                const T* residual, const T* x, const T* w_a, const T* w_f, int rows, int hidden, float eps, int blocks,
+                hipStream_t stream) {
+    const float inv_hidden = 1.0f / static_cast<float>(hidden);
+#define CGPTX_RMS_CASE(L, KK)                                                                                         \
+    if (shape.lpr == L && shape.k == KK) {                                                                            \
+        hipLaunchKernelGGL((rmsnorm_dual_rows_kernel<T, L, KK, Backward>), dim3(blocks), dim3(kThreads), 0, stream,   \
+                           out_a, out_f, partial_a, partial_f, dy_a, dy_f, residual, x, w_a, w_f, rows, hidden,      \
+                           inv_hidden, eps);                                                                          \
+        return CGPTX_OK;                                                                                              \
+    }
+    CGPTX_RMS_CASE(16, 1)
+    CGPTX_RMS_CASE(32, 1)
+    CGPTX_RMS_CASE(64, 1)
+    CGPTX_RMS_CASE(64, 2)
+    CGPTX_RMS_CASE(64, 4)
+#undef CGPTX_RMS_CASE
+    return fail(CGPTX_RUNTIME, "rmsnorm: no kernel for shape");
+}
+}  // namespace
+
+int rmsnorm_forward_dual(void* output_a, void* output_f, const void* input, const void* weight_a, const void* weight_f,
+                         std::size_t rows, std::size_t hidden, float epsilon, int dtype, hipStream_t stream) {
+    if (int s = validate(output_a, output_f, input, rows, hidden, epsilon, dtype, "rmsnorm_forward_dual")) return s;
+    if (weight_a == nullptr || weight_f == nullptr ||
+        !rmsnorm_dual_fusable(output_a, output_f, input, weight_a, weight_f, hidden, dtype))
+        return fail(CGPTX_INVALID_ARGUMENT, "rmsnorm_forward_dual: shape or alignment not served by the fused pass");
+    const int r = static_cast<int>(rows), h = static_cast<int>(hidden);
+    return dispatch_dtype(dtype, [&]<typename T>() -> int {
+        const FastShape shape = pick_fast_shape<T>(h);
+        if (int s = launch_dual<T, false>(shape, static_cast<T*>(output_a), static_cast<T*>(output_f), nullptr, nullptr, nullptr,
+                                          nullptr, nullptr, static_cast<const T*>(input), static_cast<const T*>(weight_a),
+                                          static_cast<const T*>(weight_f), r, h, epsilon, fast_blocks(shape, r), stream))
+            return s;
+        CGPTX_LAUNCH_CHECK();
+        return CGPTX_OK;
+    });
+}
+
+int rmsnorm_backward_dual(void* grad_input, void* grad_weight_a, void* grad_weight_f, const void* grad_output_a,
+                          const void* grad_output_f, const void* input, const void* weight_a, const void* weight_f,
+                          const void* residual, std::size_t rows, std::size_t hidden, float epsilon, int dtype,
+                          hipStream_t stream) {
+    if (int s = validate(grad_input, grad_output_a, input, rows, hidden, epsilon, dtype, "rmsnorm_backward_dual")) return s;
+    if (grad_weight_a == nullptr || grad_weight_f == nullptr || weight_a == nullptr || weight_f == nullptr ||
+        grad_output_f == nullptr ||
+        !rmsnorm_dual_fusable(grad_input, grad_output_a, grad_output_f, input, residual, hidden, dtype) ||
+        !is_aligned16(weight_a) || !is_aligned16(weight_f))
+        return fail(CGPTX_INVALID_ARGUMENT, "rmsnorm_backward_dual: shape or alignment not served by the fused pass");
+    const int r = static_cast<int>(rows), h = static_cast<int>(hidden);
+    return dispatch_dtype(dtype, [&]<typename T>() -> int {
+        const FastShape shape = pick_fast_shape<T>(h);
+        const int blocks = fast_blocks(shape, r);
+        const int reduce_blocks = (h + kWave - 1) / kWave;
+        const int slices = wide_reduce_slices(blocks, h, compute_units());
+        void* mem = nullptr;
+        const std::size_t partial_bytes = static_cast<std::size_t>(blocks) * hidden * sizeof(float);
+        const std::size_t second_bytes = static_cast<std::size_t>(slices) * hidden * sizeof(float);
+        if (int s = scratch(stream, 2 * partial_bytes + second_bytes, &mem)) return s;
+        auto* partial_a = static_cast<float*>(mem);
+        auto* partial_f = reinterpret_cast<float*>(static_cast<char*>(mem) + partial_bytes);
+        auto* second = reinterpret_cast<float*>(static_cast<char*>(mem) + 2 * partial_bytes);
+        if (int s = launch_dual<T, true>(shape, static_cast<T*>(grad_input), nullptr, partial_a, partial_f,
+                                         static_cast<const T*>(grad_output_a), static_cast<const T*>(grad_output_f),
+                                         static_cast<const T*>(residual), static_cast<const T*>(input),
+                                         static_cast<const T*>(weight_a), static_cast<const T*>(weight_f), r, h, epsilon, blocks,
+                                         stream))
+            return s;
+        CGPTX_LAUNCH_CHECK();
+        // The two weight gradients are reduced one after the other through the same second-stage buffer
+        // (launches on one stream run in order).
+        for (int which = 0; which < 2; ++which) {
+            float* partial = which == 0 ? partial_a : partial_f;
+            auto* dw = static_cast<T*>(which == 0 ? grad_weight_a : grad_weight_f);
+            if (slices > 1) {
+                hipLaunchKernelGGL(column_partial_fold_kernel, dim3(reduce_blocks, slices), dim3(kThreads), 0, stream, second,
+                                   partial, blocks, h);
+                CGPTX_LAUNCH_CHECK();
+                hipLaunchKernelGGL((column_partial_reduce_kernel<T>), dim3(reduce_blocks), dim3(kThreads), 0, stream, dw, second,
+                                   slices, h, 0);
+            } else {
+                hipLaunchKernelGGL((column_partial_reduce_kernel<T>), dim3(reduce_blocks), dim3(kThreads), 0, stream, dw, partial,
+                                   blocks, h, 0);
+            }
+            CGPTX_LAUNCH_CHECK();
+        }
         return CGPTX_OK;
     });
 }

@@ -105,7 +105,7 @@ struct cgptx_model {
     float* loss = nullptr;
     // backward workspace
     void *d_normalized = nullptr, *grad_a = nullptr, *grad_b = nullptr, *d_act = nullptr, *d_gate_up = nullptr,
-         *d_norm_in = nullptr, *d_attn_out = nullptr, *d_q = nullptr,
+         *d_norm_in = nullptr, *d_norm_in_f = nullptr, *d_attn_out = nullptr, *d_q = nullptr,
          *d_k = nullptr, *d_v = nullptr, *d_q_pre = nullptr, *d_k_pre = nullptr;
     cgptx_adamw_workspace* optimizer = nullptr;
     std::uint64_t initial_step = 0;  // step count the optimizer workspace starts from when it is first used
@@ -322,6 +322,13 @@ int qkv_backward_weight(void* qkv_gradient, const void* dq, const void* dk, cons
     return gemm(g, stream);
 }
 
+// Whether the block's two norms run as one pass over the block input (CGPTX_FUSE_NORMS=0 keeps them
+// separate, for comparisons).
+bool fused_block_norms(const cgptx_model* m, const void* a, const void* b, const void* c, const void* d, const void* e) {
+    const char* text = std::getenv("CGPTX_FUSE_NORMS");  // read per enqueue
+    return (text == nullptr || text[0] != '0') && rmsnorm_dual_fusable(a, b, c, d, e, m->config.hidden_size, m->config.dtype);
+}
+
 // Whether the per-head norm and the rotary embedding of q or k run as one pass (CGPTX_FUSE_QK=0 keeps
 // the separate operators, for comparisons).
 bool fused_qk_norm_rope(const cgptx_model* m, const void* a, const void* b, const void* c, const void* weight) {
@@ -349,7 +356,14 @@ int enqueue_forward_backward(cgptx_model* m, float loss_scale, int loss_mode, hi
         const auto& a = m->acts[l];
         void* x = m->hidden[l];
         void* out = m->hidden[l + 1];
-        CGPTX_OP("rmsnorm_fwd", cgptx_rmsnorm_forward(a.norm_a, x, w.attention_norm.value, N, H, eps, dt, s));
+        // Both norms of the block read its input: one pass when the shape allows.
+        const bool dual_norms = fused_block_norms(m, a.norm_a, a.norm_f, x, w.attention_norm.value, w.ffn_norm.value);
+        if (dual_norms) {
+            CGPTX_OP("rmsnorm_fwd", rmsnorm_forward_dual(a.norm_a, a.norm_f, x, w.attention_norm.value, w.ffn_norm.value, N, H, eps,
+                                                         dt, stream));
+        } else {
+            CGPTX_OP("rmsnorm_fwd", cgptx_rmsnorm_forward(a.norm_a, x, w.attention_norm.value, N, H, eps, dt, s));
+        }
         if (fused_qkv) {
             CGPTX_OP("gemm_fwd", qkv_forward(a.q_pre, a.k_pre, a.v, a.norm_a, w.q.value, N, H, QW, KW, dt, stream));
         } else {
@@ -372,7 +386,7 @@ int enqueue_forward_backward(cgptx_model* m, float loss_scale, int loss_mode, hi
                                                     m->sequence, HQ, HKV, D, 0.0f, 1, 0, dt, s));
         // out = x + attention_projection, then out += ffn_output (src/core/transformer_block.cu:594-595)
         CGPTX_OP("gemm_fwd", linear_forward_residual(out, a.attn_out, w.o.value, x, false, N, QW, H, dt, stream));
-        CGPTX_OP("rmsnorm_fwd", cgptx_rmsnorm_forward(a.norm_f, x, w.ffn_norm.value, N, H, eps, dt, s));
+        if (!dual_norms) CGPTX_OP("rmsnorm_fwd", cgptx_rmsnorm_forward(a.norm_f, x, w.ffn_norm.value, N, H, eps, dt, s));
         CGPTX_OP("gemm_fwd", cgptx_linear_forward(a.gate_up, a.norm_f, w.gate.value, nullptr, N, H, 2 * I, dt, s));
         CGPTX_OP("swiglu_fwd", cgptx_swiglu_forward_packed(a.act, a.gate_up, N, I, dt, s));
         CGPTX_OP("gemm_fwd", linear_forward_residual(out, a.act, w.down.value, nullptr, true, N, I, H, dt, stream));
@@ -404,11 +418,17 @@ int enqueue_forward_backward(cgptx_model* m, float loss_scale, int loss_mode, hi
         void* x = m->hidden[reverse];
         CGPTX_TRY(linear_backward_split(m, m->d_act, w.down.gradient, current, a.act, w.down.value, N, I, H, 0, dt, stream));
         CGPTX_OP("swiglu_bwd", cgptx_swiglu_backward_packed(m->d_gate_up, m->d_act, a.gate_up, N, I, 0, dt, s));
-        CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.gate.gradient, m->d_gate_up, a.norm_f, w.gate.value, N, H, 2 * I, 0, dt, stream));
-        // The gradient of the residual stream collects the two norm branches as they are produced:
-        // previous = current + d(ffn branch), later previous += d(attention branch).
-        CGPTX_OP("rmsnorm_bwd", rmsnorm_backward_residual(previous, w.ffn_norm.gradient, m->d_norm_in, x, w.ffn_norm.value,
-                                                          current, N, H, eps, dt, stream));
+        // The gradient of the residual stream collects the two norm branches: in one pass at the end of
+        // the block when the shape allows (previous = current + d(ffn norm) + d(attention norm)), else as
+        // they are produced (previous = current + d(ffn branch), later previous += d(attention branch)).
+        const bool dual_norms = fused_block_norms(m, previous, m->d_norm_in, m->d_norm_in_f, x, current) &&
+                                is_aligned16(w.attention_norm.value) && is_aligned16(w.ffn_norm.value);
+        void* d_norm_f = dual_norms ? m->d_norm_in_f : m->d_norm_in;
+        CGPTX_TRY(linear_backward_split(m, d_norm_f, w.gate.gradient, m->d_gate_up, a.norm_f, w.gate.value, N, H, 2 * I, 0, dt, stream));
+        if (!dual_norms) {
+            CGPTX_OP("rmsnorm_bwd", rmsnorm_backward_residual(previous, w.ffn_norm.gradient, m->d_norm_in, x, w.ffn_norm.value,
+                                                              current, N, H, eps, dt, stream));
+        }
         CGPTX_TRY(linear_backward_split(m, m->d_attn_out, w.o.gradient, current, a.attn_out, w.o.value, N, QW, H, 0, dt, stream));
         CGPTX_OP("attn_bwd", cgptx_flash_gqa_attention_backward_with_lse(m->d_q, m->d_k, m->d_v, m->d_attn_out, a.attn_out,
                                                               a.lse, a.q, a.k, a.v, m->batch, m->sequence,
@@ -436,8 +456,14 @@ int enqueue_forward_backward(cgptx_model* m, float loss_scale, int loss_mode, hi
             CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.k.gradient, m->d_k, a.norm_a, w.k.value, N, H, KW, 1, dt, stream));
             CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.v.gradient, m->d_v, a.norm_a, w.v.value, N, H, KW, 1, dt, stream));
         }
-        CGPTX_OP("rmsnorm_bwd", rmsnorm_backward_residual(previous, w.attention_norm.gradient, m->d_norm_in, x,
-                                                          w.attention_norm.value, previous, N, H, eps, dt, stream));
+        if (dual_norms) {
+            CGPTX_OP("rmsnorm_bwd", rmsnorm_backward_dual(previous, w.attention_norm.gradient, w.ffn_norm.gradient, m->d_norm_in,
+                                                          m->d_norm_in_f, x, w.attention_norm.value, w.ffn_norm.value, current, N, H,
+                                                          eps, dt, stream));
+        } else {
+            CGPTX_OP("rmsnorm_bwd", rmsnorm_backward_residual(previous, w.attention_norm.gradient, m->d_norm_in, x,
+                                                              w.attention_norm.value, previous, N, H, eps, dt, stream));
+        }
         std::swap(current, previous);
     }
     // Tied embedding: the classifier gradient is already in place; add the lookup's gradient
@@ -551,7 +577,7 @@ extern "C" int cgptx_model_create(cgptx_model** out, const cgptx_model_config* c
         CGPTX_HIP(hipMemset(m->targets, 0, N * sizeof(std::uint32_t)));
         CGPTX_TRY(allocate_typed(m, &m->loss, 256));
         CGPTX_HIP(hipMemset(m->loss, 0, 256));
-        for (void** p : {&m->d_normalized, &m->grad_a, &m->grad_b, &m->d_norm_in})
+        for (void** p : {&m->d_normalized, &m->grad_a, &m->grad_b, &m->d_norm_in, &m->d_norm_in_f})
             CGPTX_TRY(allocate(m, p, N * H * elem));
         CGPTX_TRY(allocate(m, &m->d_act, N * I * elem));
         CGPTX_TRY(allocate(m, &m->d_gate_up, N * 2 * I * elem));
