@@ -173,15 +173,25 @@ __device__ __forceinline__ typename Mma<T>::frag acc_frag(const acc_t& acc, int 
 // Streamed index of accumulator register i: 8*(i/4) + 4*(lane/32) + i%4.
 __device__ __forceinline__ int acc_row(int i) { return 8 * (i >> 2) + 4 * ((threadIdx.x & 63) >> 5) + (i & 3); }
 
-// Query block of a workgroup. Workgroups are dealt to the 8 XCDs round-robin by linear id, and under
-// a causal mask a query block's work grows with its position; with the plain mapping and a grid
-// whose x extent is a multiple of 8, one XCD would receive all the longest blocks. Rotating the
-// index by the (head, batch) coordinate gives every XCD every length; the longest come first.
-__device__ __forceinline__ int balanced_query_block() {
-    const unsigned int count = gridDim.x;
-    const unsigned int rotation = blockIdx.y + gridDim.y * blockIdx.z;
-    const unsigned int index = (blockIdx.x + rotation) % count;
-    return static_cast<int>(count - 1 - index) * kBlockRows;
+// Query block, head and batch entry of a workgroup of the forward and dQ kernels (grid: query blocks
+// x heads x batch). Workgroups start in the order of their linear id, as slots become free, and go
+// to the 8 XCDs round-robin. Under a causal mask a query block's work grows with its position, so
+// the linear id is read position-major with the last (longest) query blocks first: the work that
+// is handed out last is the shortest, which keeps the tail of the launch short, and every XCD
+// receives the same mix of lengths (heads x batch workgroups of each).
+struct BlockCoordinates {
+    int q_block;  // first query row
+    int h, b;
+};
+__device__ __forceinline__ BlockCoordinates block_coordinates() {
+    const unsigned int linear = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+    const unsigned int per_position = gridDim.y * gridDim.z;
+    const unsigned int position = linear / per_position, rest = linear - position * per_position;
+    BlockCoordinates c;
+    c.q_block = static_cast<int>(gridDim.x - 1 - position) * kBlockRows;
+    c.h = static_cast<int>(rest % gridDim.y);
+    c.b = static_cast<int>(rest / gridDim.y);
+    return c;
 }
 
 // ------------------------------------------------------------------- forward
@@ -191,8 +201,9 @@ __global__ __launch_bounds__(kThreads) void attention_forward_kernel(Params p) {
     __shared__ __align__(16) T k_lds[kStream * lds_stride<DP>()];
     __shared__ __align__(16) T v_lds[kStream * lds_stride<DP>()];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int b = blockIdx.z, h = blockIdx.y, kvh = h / (p.hq / p.hkv);
-    const int q_block = balanced_query_block();
+    const BlockCoordinates where = block_coordinates();
+    const int b = where.b, h = where.h, kvh = h / (p.hq / p.hkv);
+    const int q_block = where.q_block;
     const int q_row = q_block + wave * 32 + (lane & 31);
     const bool q_live = q_row < p.qs;
     const long q_stride = static_cast<long>(p.hq) * p.d, kv_stride = static_cast<long>(p.hkv) * p.d;
@@ -335,8 +346,9 @@ __global__ __launch_bounds__(kThreads) void attention_dq_kernel(Params p) {
     __shared__ __align__(16) T k_lds[kStream * lds_stride<DP>()];
     __shared__ __align__(16) T v_lds[kStream * lds_stride<DP>()];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int b = blockIdx.z, h = blockIdx.y, kvh = h / (p.hq / p.hkv);
-    const int q_block = balanced_query_block();
+    const BlockCoordinates where = block_coordinates();
+    const int b = where.b, h = where.h, kvh = h / (p.hq / p.hkv);
+    const int q_block = where.q_block;
     const int q_row = q_block + wave * 32 + (lane & 31);
     const bool q_live = q_row < p.qs;
     const long q_stride = static_cast<long>(p.hq) * p.d, kv_stride = static_cast<long>(p.hkv) * p.d;
@@ -694,8 +706,9 @@ __global__ __launch_bounds__(kThreads, 2) void attention_forward_wide_kernel(Par
     __shared__ __align__(1024) T lds[4 * kWideTile];  // [stage][K | V]
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int b = blockIdx.z, h = blockIdx.y, kvh = h / (p.hq / p.hkv);
-    const int q_block = balanced_query_block();
+    const BlockCoordinates where = block_coordinates();
+    const int b = where.b, h = where.h, kvh = h / (p.hq / p.hkv);
+    const int q_block = where.q_block;
     const int q_row = q_block + wave * 32 + (lane & 31);
     const bool q_live = q_row < p.qs;
     const long q_stride = static_cast<long>(p.hq) * p.d, kv_stride = static_cast<long>(p.hkv) * p.d;
@@ -861,8 +874,9 @@ __global__ __launch_bounds__(kThreads, 2) void attention_dq_wide_kernel(Params p
     __shared__ __align__(1024) T lds[4 * kWideTile];  // [stage][K | V]
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int b = blockIdx.z, h = blockIdx.y, kvh = h / (p.hq / p.hkv);
-    const int q_block = balanced_query_block();
+    const BlockCoordinates where = block_coordinates();
+    const int b = where.b, h = where.h, kvh = h / (p.hq / p.hkv);
+    const int q_block = where.q_block;
     const int q_row = q_block + wave * 32 + (lane & 31);
     const bool q_live = q_row < p.qs;
     const long q_stride = static_cast<long>(p.hq) * p.d, kv_stride = static_cast<long>(p.hkv) * p.d;
