@@ -190,6 +190,10 @@ def main() -> int:
     probe = kernel_probe(torch, cfg, args.batch, args.seq, stream, 20, args.seed)
     breakdown = model.profile(options.loss_scale, loss_mode, stream)
     work = op_work(cfg, args.batch, args.seq, args.loss)
+    # When the per-head norms carry the rotary embedding (one pass), its algorithmic bytes count with theirs.
+    for rope, norm in (("rope_fwd", "rmsnorm_fwd"), ("rope_bwd", "rmsnorm_bwd")):
+        if rope not in breakdown:
+            work[norm] = (work[norm][0], work[norm][1] + work[rope][1])
     achieved = probe["flops"] / probe["seconds"] / 1e12
     per_kind = {}
     for kind, ms in sorted(breakdown.items(), key=lambda kv: -kv[1]):
