@@ -58,6 +58,8 @@ SHAPES = [  # rows, in, out
     (384, 1024, 256), (1024, 320, 1024),
     # every reduction length (in for Y, out for dX, rows for dW) is an odd multiple of 32
     (288, 96, 160), (1056, 160, 352),
+    # a single K tile; partial tiles in both directions with more work items than persistent blocks
+    (64, 32, 64), (1000, 96, 520), (4104, 64, 2056),
 ]
 
 
