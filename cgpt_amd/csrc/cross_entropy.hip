@@ -5,11 +5,11 @@
 //   loss = mean_r [ y_r < V ] (log Σ_j e^{z_rj} − z_{r,y_r}),
 //   grad_rj = (softmax(z_r)_j − [j = y_r]) · scale / rows   (stored in the logits dtype).
 //
-// One block per row. Pass 1 streams the row once with 128-bit loads keeping an
-// online (max, Σexp) pair per thread; pass 2 re-reads the row (64 KB at V=32000
-// in 16-bit, still resident in L2) and writes the gradient. HBM traffic is one
-// read and one write of the logits. Per-row losses go to scratch and one block
-// adds them in a fixed order, where the reference uses a float atomicAdd
+// One block per row. Rows of up to 8192 128-bit vectors (65536 16-bit logits) are loaded once
+// into registers, reduced to (max, Σexp) and turned into the gradient from the registers: one
+// read and one write of the logits. Longer or unaligned rows stream: pass 1 keeps an online
+// (max, Σexp) pair per thread, pass 2 re-reads the row through the caches. Per-row losses go to
+// scratch and one block adds them in a fixed order, where the reference uses a float atomicAdd
 // (src/ops/cross_entropy.cu:134-245).
 #include "cross_entropy.hpp"
 
@@ -32,6 +32,7 @@ __device__ __forceinline__ MaxSum combine(MaxSum a, MaxSum b) {
     return {m, a.s * __expf(a.m - m) + b.s * __expf(b.m - m)};
 }
 
+template <int WAVES = kWaves>
 __device__ __forceinline__ MaxSum block_combine(MaxSum v, MaxSum* stage) {
 #pragma unroll
     for (int offset = kWave / 2; offset > 0; offset >>= 1) {
@@ -43,7 +44,7 @@ __device__ __forceinline__ MaxSum block_combine(MaxSum v, MaxSum* stage) {
     __syncthreads();
     MaxSum total = stage[0];
 #pragma unroll
-    for (int w = 1; w < kWaves; ++w) total = combine(total, stage[w]);
+    for (int w = 1; w < WAVES; ++w) total = combine(total, stage[w]);
     return total;
 }
 
@@ -114,6 +115,88 @@ __global__ __launch_bounds__(kThreads) void cross_entropy_row_kernel(float* __re
     }
 }
 
+// Rows of up to kResidentThreads * SLOTS 128-bit vectors stay in registers between the two passes:
+// every load of the row is in flight at once, and the memory system sees exactly one read and one
+// write of the row (the streaming kernel's second pass finds the row in L2 only while the rows in
+// flight on an XCD fit there, which 8 rows of 64 KB per CU do not).
+constexpr int kResidentThreads = 512;
+template <typename T, int SLOTS, bool WithGradient>
+__global__ __launch_bounds__(kResidentThreads) void cross_entropy_row_resident_kernel(
+    float* __restrict__ row_loss, T* gradient /* may alias logits */, const T* logits,
+    const std::uint32_t* __restrict__ targets, unsigned int vocab, float factor) {
+    constexpr int VEC = kVec128<T>;
+    constexpr int WAVES = kResidentThreads / kWave;
+    __shared__ MaxSum stage[WAVES];
+    const std::size_t base = static_cast<std::size_t>(blockIdx.x) * vocab;
+    const T* row = logits + base;
+    const unsigned int vectors = vocab / VEC;
+    const std::uint32_t target = targets[blockIdx.x];
+    // Read before the barrier in block_combine: in-place use overwrites the row after it.
+    const float target_logit = (threadIdx.x == 0 && target < vocab) ? to_f32(row[target]) : 0.0f;
+
+    vec_t<T, VEC> held[SLOTS];
+#pragma unroll
+    for (int s = 0; s < SLOTS; ++s) {
+        const unsigned int v = s * kResidentThreads + threadIdx.x;
+        if (v < vectors) held[s] = load_vec<T, VEC>(row + v * VEC);
+    }
+    MaxSum acc{-INFINITY, 0.0f};
+#pragma unroll
+    for (int s = 0; s < SLOTS; ++s) {
+        if (s * kResidentThreads + threadIdx.x < vectors) {
+            const vec_t<float, VEC> x = vec_to_f32<T, VEC>(held[s]);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) acc.m = fmaxf(acc.m, x[e]);
+        }
+    }
+    if (acc.m != -INFINITY) {
+#pragma unroll
+        for (int s = 0; s < SLOTS; ++s) {
+            if (s * kResidentThreads + threadIdx.x < vectors) {
+                const vec_t<float, VEC> x = vec_to_f32<T, VEC>(held[s]);
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) acc.s += __expf(x[e] - acc.m);
+            }
+        }
+    }
+    const MaxSum total = block_combine<WAVES>(acc, stage);
+    if (threadIdx.x == 0) {
+        float loss = 0.0f;
+        if (target < vocab) loss = __logf(total.s) + total.m - target_logit;
+        row_loss[blockIdx.x] = loss;
+    }
+    if constexpr (WithGradient) {
+        const float inv = 1.0f / total.s;
+        T* out = gradient + base;
+#pragma unroll
+        for (int s = 0; s < SLOTS; ++s) {
+            const unsigned int v = s * kResidentThreads + threadIdx.x;
+            if (v < vectors) {
+                const vec_t<float, VEC> x = vec_to_f32<T, VEC>(held[s]);
+                vec_t<float, VEC> g;
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    float value = __expf(x[e] - total.m) * inv;
+                    if (v * VEC + e == target) value -= 1.0f;
+                    g[e] = value * factor;
+                }
+                store_vec<T, VEC>(out + v * VEC, vec_from_f32<T, VEC>(g));
+            }
+        }
+    }
+}
+
+template <typename T, int SLOTS>
+void launch_resident(float* row_loss, T* gradient, const T* logits, const std::uint32_t* targets, unsigned int rows,
+                     unsigned int vocab, float factor, hipStream_t stream) {
+    if (gradient != nullptr)
+        hipLaunchKernelGGL((cross_entropy_row_resident_kernel<T, SLOTS, true>), dim3(rows), dim3(kResidentThreads), 0,
+                           stream, row_loss, gradient, logits, targets, vocab, factor);
+    else
+        hipLaunchKernelGGL((cross_entropy_row_resident_kernel<T, SLOTS, false>), dim3(rows), dim3(kResidentThreads), 0,
+                           stream, row_loss, gradient, logits, targets, vocab, factor);
+}
+
 }  // namespace
 
 // Shared with the cut-cross-entropy path: loss[0] = (Σ row_loss) / rows, fixed order.
@@ -149,7 +232,14 @@ int cross_entropy_rows(float* row_loss, void* gradient, const void* logits, cons
     return dispatch_dtype(dtype, [&]<typename T>() -> int {
         const bool vector_ok = vocab % kVec128<T> == 0 && is_aligned16(logits) &&
                                (!with_gradient || is_aligned16(gradient));
-        if (with_gradient) {
+        const unsigned int vectors = v / kVec128<T>;
+        if (vector_ok && vectors <= 16u * kResidentThreads) {
+            auto* g = static_cast<T*>(gradient);
+            auto* z = static_cast<const T*>(logits);
+            if (vectors <= 2u * kResidentThreads) launch_resident<T, 2>(row_loss, g, z, targets, r, v, factor, stream);
+            else if (vectors <= 8u * kResidentThreads) launch_resident<T, 8>(row_loss, g, z, targets, r, v, factor, stream);
+            else launch_resident<T, 16>(row_loss, g, z, targets, r, v, factor, stream);
+        } else if (with_gradient) {
             hipLaunchKernelGGL((cross_entropy_row_kernel<T, true>), dim3(r), dim3(kThreads), 0, stream, row_loss,
                                static_cast<T*>(gradient), static_cast<const T*>(logits), targets, v, factor, vector_ok);
         } else {

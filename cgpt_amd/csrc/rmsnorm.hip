@@ -113,12 +113,14 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_rows_kernel(
         const bool row_live = row < rows;
         const std::size_t base = static_cast<std::size_t>(row) * hidden;
         F xv[K], gv[K];
+        vec_t<T, VEC> rv[K];  // residual, requested with the other operands: one memory round trip per row
 #pragma unroll
         for (int c = 0; c < K; ++c) {
             const int col = (c * LPR + sub) * VEC;
             if (row_live && live[c]) {
                 xv[c] = vec_to_f32<T, VEC>(load_vec<T, VEC>(x + base + col));
                 if constexpr (Backward) {
+                    if (residual != nullptr) rv[c] = load_vec<T, VEC>(residual + base + col);
                     gv[c] = vec_to_f32<T, VEC>(load_vec<T, VEC>(dy + base + col));
                     if constexpr (Rope) gv[c] = vec_to_f32<T, VEC>(vec_from_f32<T, VEC>(rope_vector<T, true>(gv[c], rope, row, col)));
                 }
@@ -151,7 +153,7 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_rows_kernel(
                 }
                 const int col = (c * LPR + sub) * VEC;
                 if (row_live && live[c]) {
-                    if (residual != nullptr) r += vec_to_f32<T, VEC>(load_vec<T, VEC>(residual + base + col));
+                    if (residual != nullptr) r += vec_to_f32<T, VEC>(rv[c]);
                     store_vec<T, VEC>(out + base + col, vec_from_f32<T, VEC>(r));
                 }
             }
@@ -236,6 +238,7 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_dual_rows_kernel(
         const bool row_live = row < rows;
         const std::size_t base = static_cast<std::size_t>(row) * hidden;
         F xv[K], ga[K], gf[K];
+        vec_t<T, VEC> rv[K];  // residual, requested with the other operands: one memory round trip per row
 #pragma unroll
         for (int c = 0; c < K; ++c) {
             const int col = (c * LPR + sub) * VEC;
@@ -244,6 +247,7 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_dual_rows_kernel(
             if constexpr (Backward) {
                 ga[c] = on ? vec_to_f32<T, VEC>(load_vec<T, VEC>(dy_a + base + col)) : F(0.0f);
                 gf[c] = on ? vec_to_f32<T, VEC>(load_vec<T, VEC>(dy_f + base + col)) : F(0.0f);
+                if (on && residual != nullptr) rv[c] = load_vec<T, VEC>(residual + base + col);
             }
         }
         float ss = 0.0f, dd = 0.0f;
@@ -272,7 +276,7 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_dual_rows_kernel(
                 }
                 const int col = (c * LPR + sub) * VEC;
                 if (row_live && live[c]) {
-                    if (residual != nullptr) r += vec_to_f32<T, VEC>(load_vec<T, VEC>(residual + base + col));
+                    if (residual != nullptr) r += vec_to_f32<T, VEC>(rv[c]);
                     store_vec<T, VEC>(out_a + base + col, vec_from_f32<T, VEC>(r));
                 }
             }
