@@ -19,6 +19,8 @@
 
 #include <cmath>
 #include <limits>
+#include <mutex>
+#include <unordered_map>
 
 namespace cgptx {
 namespace {
@@ -444,11 +446,47 @@ int launch_fast(const FastShape shape, T* out, float* partial, const T* dy, cons
     return fail(CGPTX_RUNTIME, "rmsnorm: no kernel for shape");
 }
 
-int fast_blocks(const FastShape shape, int rows) {
+// The kernel launch_fast would launch (null when there is none).
+template <typename T, bool Backward>
+const void* fast_kernel(const FastShape shape, bool rope) {
+    if (rope)
+        return shape.lpr == 16 && shape.k == 1 ? reinterpret_cast<const void*>(&rmsnorm_rows_kernel<T, 16, 1, Backward, true>)
+                                               : nullptr;
+#define CGPTX_RMS_CASE(L, KK) \
+    if (shape.lpr == L && shape.k == KK) return reinterpret_cast<const void*>(&rmsnorm_rows_kernel<T, L, KK, Backward>);
+    CGPTX_RMS_CASE(16, 1)
+    CGPTX_RMS_CASE(32, 1)
+    CGPTX_RMS_CASE(64, 1)
+    CGPTX_RMS_CASE(64, 2)
+    CGPTX_RMS_CASE(64, 4)
+#undef CGPTX_RMS_CASE
+    return nullptr;
+}
+
+// Blocks of `kernel` the device holds at once. The row kernels are grid-stride loops with equal
+// shares: launched with more blocks than fit, the surplus would run as a second, mostly idle round.
+int resident_blocks(const void* kernel) {
+    static std::mutex guard;
+    static std::unordered_map<const void*, int> known;
+    std::lock_guard<std::mutex> lock(guard);
+    auto found = known.find(kernel);
+    if (found == known.end()) {
+        int per_cu = 0;
+        if (kernel == nullptr || hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, kThreads, 0) != hipSuccess ||
+            per_cu < 1) {
+            (void)hipGetLastError();
+            per_cu = 1;
+        }
+        found = known.emplace(kernel, per_cu).first;
+    }
+    return found->second * compute_units();
+}
+
+int fast_blocks(const FastShape shape, int rows, const void* kernel) {
     const int rpw = kWave / shape.lpr;
     const long groups = (static_cast<long>(rows) + rpw - 1) / rpw;
     const long wanted = (groups + kWavesPerBlock - 1) / kWavesPerBlock;
-    const long cap = static_cast<long>(compute_units()) * 4;
+    const long cap = resident_blocks(kernel);
     return static_cast<int>(wanted < cap ? wanted : cap);
 }
 
@@ -504,7 +542,7 @@ int rmsnorm_rope_forward(void* output, const void* input, const void* weight, co
         const FastShape shape = pick_fast_shape<T>(h);
         if (int s = launch_fast<T, false>(shape, static_cast<T*>(output), nullptr, nullptr, nullptr,
                                           static_cast<const T*>(input), static_cast<const T*>(weight), r, h, epsilon,
-                                          fast_blocks(shape, r), stream, &rope))
+                                          fast_blocks(shape, r, fast_kernel<T, false>(shape, true)), stream, &rope))
             return s;
         CGPTX_LAUNCH_CHECK();
         return CGPTX_OK;
@@ -524,7 +562,7 @@ int rmsnorm_rope_backward(void* grad_input, void* grad_weight, const void* grad_
     const RopeArgs rope = make_rope(cos_cache, sin_cache, heads, sequence, rotary_dim, position_offset);
     return dispatch_dtype(dtype, [&]<typename T>() -> int {
         const FastShape shape = pick_fast_shape<T>(h);
-        const int blocks = fast_blocks(shape, r);
+        const int blocks = fast_blocks(shape, r, fast_kernel<T, true>(shape, true));
         const int reduce_blocks = (h + kWave - 1) / kWave;
         const int slices = wide_reduce_slices(blocks, h, compute_units());
         void* mem = nullptr;
@@ -587,6 +625,21 @@ int launch_dual(const FastShape shape, T* out_a, T* out_f, float* partial_a, flo
 }
 }  // namespace
 
+namespace {
+template <typename T, bool Backward>
+const void* dual_kernel(const FastShape shape) {
+#define CGPTX_RMS_CASE(L, KK) \
+    if (shape.lpr == L && shape.k == KK) return reinterpret_cast<const void*>(&rmsnorm_dual_rows_kernel<T, L, KK, Backward>);
+    CGPTX_RMS_CASE(16, 1)
+    CGPTX_RMS_CASE(32, 1)
+    CGPTX_RMS_CASE(64, 1)
+    CGPTX_RMS_CASE(64, 2)
+    CGPTX_RMS_CASE(64, 4)
+#undef CGPTX_RMS_CASE
+    return nullptr;
+}
+}  // namespace
+
 int rmsnorm_forward_dual(void* output_a, void* output_f, const void* input, const void* weight_a, const void* weight_f,
                          std::size_t rows, std::size_t hidden, float epsilon, int dtype, hipStream_t stream) {
     if (int s = validate(output_a, output_f, input, rows, hidden, epsilon, dtype, "rmsnorm_forward_dual")) return s;
@@ -598,7 +651,8 @@ int rmsnorm_forward_dual(void* output_a, void* output_f, const void* input, cons
         const FastShape shape = pick_fast_shape<T>(h);
         if (int s = launch_dual<T, false>(shape, static_cast<T*>(output_a), static_cast<T*>(output_f), nullptr, nullptr, nullptr,
                                           nullptr, nullptr, static_cast<const T*>(input), static_cast<const T*>(weight_a),
-                                          static_cast<const T*>(weight_f), r, h, epsilon, fast_blocks(shape, r), stream))
+                                          static_cast<const T*>(weight_f), r, h, epsilon,
+                                          fast_blocks(shape, r, dual_kernel<T, false>(shape)), stream))
             return s;
         CGPTX_LAUNCH_CHECK();
         return CGPTX_OK;
@@ -618,7 +672,7 @@ int rmsnorm_backward_dual(void* grad_input, void* grad_weight_a, void* grad_weig
     const int r = static_cast<int>(rows), h = static_cast<int>(hidden);
     return dispatch_dtype(dtype, [&]<typename T>() -> int {
         const FastShape shape = pick_fast_shape<T>(h);
-        const int blocks = fast_blocks(shape, r);
+        const int blocks = fast_blocks(shape, r, dual_kernel<T, true>(shape));
         const int reduce_blocks = (h + kWave - 1) / kWave;
         const int slices = wide_reduce_slices(blocks, h, compute_units());
         void* mem = nullptr;
@@ -674,7 +728,7 @@ int rmsnorm_backward_residual(void* grad_input, void* grad_weight, const void* g
         const bool aligned = is_aligned16(dx) && is_aligned16(dy) && is_aligned16(x) && is_aligned16(w) && is_aligned16(res);
         const int reduce_blocks = (h + kWave - 1) / kWave;
         if (shape.lpr != 0 && aligned) {
-            const int blocks = fast_blocks(shape, r);
+            const int blocks = fast_blocks(shape, r, fast_kernel<T, true>(shape, false));
             const int slices = wide_reduce_slices(blocks, h, compute_units());
             void* mem = nullptr;
             const std::size_t partial_bytes = static_cast<std::size_t>(blocks) * hidden * sizeof(float);
@@ -741,7 +795,7 @@ extern "C" int cgptx_rmsnorm_forward(void* output, const void* input, const void
         auto* w = static_cast<const T*>(weight);
         const FastShape shape = pick_fast_shape<T>(h);
         if (shape.lpr != 0 && is_aligned16(y) && is_aligned16(x) && is_aligned16(w)) {
-            const int blocks = fast_blocks(shape, r);
+            const int blocks = fast_blocks(shape, r, fast_kernel<T, false>(shape, false));
             if (int s = launch_fast<T, false>(shape, y, nullptr, nullptr, nullptr, x, w, r, h, epsilon, blocks, stream)) return s;
             CGPTX_LAUNCH_CHECK();
             return CGPTX_OK;
