@@ -63,10 +63,13 @@ extern "C" int cgptx_cut_cross_entropy_forward_backward(float* loss, void* input
     auto stream = static_cast<hipStream_t>(stream_);
     const std::size_t elem = dtype_size(dtype);
     // Chunk so that the logits scratch stays near 1 GiB whatever the number of rows, while each
-    // chunk still gives the three contractions enough 256x256 tiles to fill the chip (16384 rows at
-    // V=32000: the input-gradient contraction then has 64 x 4 tiles, one per CU).
-    std::size_t chunk = (std::size_t{1} << 30) / (vocab * elem);
-    chunk = std::max<std::size_t>(256, chunk / 256 * 256);
+    // chunk still gives the three contractions enough 256x256 tiles to fill the chip. The rows are
+    // split evenly over the chunks (32768 rows at V=32000: 2 x 16384, so that the input-gradient
+    // contraction has 64 x 4 tiles, one per CU; 16640 + 16128 would cost it a second round for 4 tiles).
+    std::size_t limit = (std::size_t{1} << 30) / (vocab * elem);
+    limit = std::max<std::size_t>(256, limit / 256 * 256);
+    const std::size_t pieces = (rows + limit - 1) / limit;
+    std::size_t chunk = ((rows + pieces - 1) / pieces + 255) / 256 * 256;
     chunk = std::min(chunk, rows);
     const std::size_t loss_bytes = (rows * sizeof(float) + 255) & ~std::size_t{255};
     const std::size_t acc_bytes = (vocab * hidden * sizeof(float) + 255) & ~std::size_t{255};

@@ -530,10 +530,8 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
     unsigned char* region = smem_raw + (kStages - 1) * kStageBytes + wave * (kStageBytes / kWaves);
     auto sw = [](int row) { return (row / (256 / kRowBytes)) % kRowChunks; };
     const int m_lane = lane & 15, q_lane = lane >> 4;
-    // Stages blocks (2r, j0 .. j0+JP-1) and (2r+1, ...), 32 rows, as element type S and hands each lane 8 consecutive staged
-    // elements at a time: consume(row, col, pointer to the 8 elements' first chunk, to the second
-    // chunk when S is float), row/col relative to the wavefront's part.
-    auto pass = [&]<typename S, int JP>(int r, int j0, auto&& consume) __attribute__((always_inline)) {
+    // Writes blocks (2r, j0 .. j0+JP-1) and (2r+1, ...) into the wavefront's staging region as element type S.
+    auto stage = [&]<typename S, int JP>(int r, int j0) __attribute__((always_inline)) {
         static_assert(JP * 16 * sizeof(S) == kRowBytes, "a pass fills whole staged rows");
         __builtin_amdgcn_wave_barrier();
 #pragma unroll
@@ -550,6 +548,13 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
             }
         }
         __builtin_amdgcn_wave_barrier();
+    };
+    // Stages those blocks, 32 rows, and hands each lane 8 consecutive staged elements at a time:
+    // consume(round, row, col, pointer to the 8 elements' first chunk, to the second chunk when S is
+    // float), row/col relative to the wavefront's part; in round u the lane gets element
+    // q = 64 u + lane of the 32 x (8-element groups per row) grid, row-major.
+    auto pass = [&]<typename S, int JP>(int r, int j0, auto&& consume) __attribute__((always_inline)) {
+        stage.template operator()<S, JP>(r, j0);
         constexpr int kLanesPerRow = kRowBytes / (8 * static_cast<int>(sizeof(S)));
         constexpr int kChunksPerLane = 8 * static_cast<int>(sizeof(S)) / 16;
         constexpr int kRounds = 32 * kLanesPerRow / kWave;
@@ -559,7 +564,7 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
             const int row = q / kLanesPerRow, part = q % kLanesPerRow;
             const unsigned char* base = region + row * kRowBytes;
             const int first = part * kChunksPerLane;
-            consume(r * 32 + row, j0 * 16 + part * 8, base + ((first ^ sw(row)) * 16),
+            consume(u, r * 32 + row, j0 * 16 + part * 8, base + ((first ^ sw(row)) * 16),
                     base + (((first + kChunksPerLane - 1) ^ sw(row)) * 16));
         }
     };
@@ -590,25 +595,49 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
         bool plain = false;
         if constexpr (!SPLIT) plain = p.bias == nullptr && p.residual == nullptr && !p.accumulate && !p.c_f32;
         if (plain) {
-            T* out = static_cast<T*>(c_base);
+            // Straight-line code, no per-lane predicates or address arithmetic (with one wavefront per
+            // SIMD every branch and every dependent wait is exposed): the stores go through a buffer
+            // descriptor over the wavefront's part of C, whose range ends with the last valid row, so
+            // rows past the matrix are dropped by the range check; a lane whose columns lie past the
+            // matrix gets an offset beyond every range. Lane l of round u holds 16 bytes of row
+            // 4u + l/16 (256-byte rows): the row advance is a scalar offset.
+            T* part = static_cast<T*>(c_base) + static_cast<long>(row0) * c_ld + (c_col0 + col0);
+            const int rows_left = min(WM, p.m - row0), cols_left = min(WN, c_cols - (c_col0 + col0));
+            const long extent = rows_left > 0 && cols_left > 0
+                                    ? (static_cast<long>(rows_left - 1) * c_ld + cols_left) * static_cast<long>(sizeof(T))
+                                    : 0;
+            const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(part, 0, static_cast<int>(extent), 0x00020000);
+            constexpr int kLanesPerRow = kRowBytes / 16, kRowsPerRound = kWave / kLanesPerRow, kRounds = 32 / kRowsPerRound;
+            const int lane_row = lane / kLanesPerRow, lane_chunk = lane % kLanesPerRow;
+            const int row_bytes = static_cast<int>(c_ld * static_cast<long>(sizeof(T)));
+            const int voffset = lane_chunk * 8 < cols_left ? lane_row * row_bytes + lane_chunk * 16 : std::numeric_limits<int>::min();
 #pragma unroll
             for (int r = 0; r < kRowBlocks; ++r) {
+                // Accumulators leave their registers block by block: read ahead of their block they
+                // would not fit the vector registers.
+                __builtin_amdgcn_sched_barrier(0);
                 if (request) request_share(r);
-                pass.template operator()<T, TN>(r, 0, [&](int row, int col, const unsigned char* lo, const unsigned char*) {
-                    const int m = row0 + row, c_col = c_col0 + col0 + col;
-                    const u32x4 data = *reinterpret_cast<const u32x4*>(lo);
-                    if (m < p.m && c_col < c_cols) *reinterpret_cast<u32x4*>(out + static_cast<long>(m) * c_ld + c_col) = data;
-                });
+                stage.template operator()<T, TN>(r, 0);
+                u32x4 data[kRounds];
+#pragma unroll
+                for (int u = 0; u < kRounds; ++u) {
+                    const int row = u * kRowsPerRound + lane_row;
+                    data[u] = *reinterpret_cast<const u32x4*>(region + row * kRowBytes + ((lane_chunk ^ sw(row)) * 16));
+                }
+#pragma unroll
+                for (int u = 0; u < kRounds; ++u)
+                    __builtin_amdgcn_raw_buffer_store_b128(data[u], rsrc, voffset, (r * 32 + u * kRowsPerRound) * row_bytes, 0);
             }
             return;
         }
 #pragma unroll
         for (int r = 0; r < kRowBlocks; ++r) {
+            __builtin_amdgcn_sched_barrier(0);
             if (request) request_share(r);
 #pragma unroll
             for (int half = 0; half < 2; ++half) {
-                pass.template operator()<float, TN / 2>(r, half * (TN / 2), [&](int row, int col, const unsigned char* lo,
-                                                                               const unsigned char* hi) {
+                pass.template operator()<float, TN / 2>(r, half * (TN / 2), [&](int, int row, int col, const unsigned char* lo,
+                                                                              const unsigned char* hi) {
                     const int m = row0 + row, n = w.n0 + col0 + col, c_col = c_col0 + col0 + col;
                     vec_t<float, 4> v0 = *reinterpret_cast<const vec_t<float, 4>*>(lo);
                     vec_t<float, 4> v1 = *reinterpret_cast<const vec_t<float, 4>*>(hi);
