@@ -317,9 +317,13 @@ struct TileLayout {
 // the other: the first K tiles of the next item are requested before the epilogue of the current
 // one, whose stores then drain under the next item's MFMAs.
 // SEGMENTED: A is stored [M, K] in up to three column segments (separate buffers along K).
-template <typename T, int BM, int BN, bool A_K, bool B_K, bool SPLIT, bool SEGMENTED>
+// RESIDUAL: the epilogue adds a residual to a 16-bit result and nothing else (the output
+// projections of a transformer block); a kernel of its own, so that each kernel carries one
+// straight-line epilogue besides the general one.
+template <typename T, int BM, int BN, bool A_K, bool B_K, bool SPLIT, bool SEGMENTED, bool RESIDUAL = false>
 __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
     static_assert(!SEGMENTED || (A_K && !SPLIT), "segments along K are read by the unsplit kernels only");
+    static_assert(!RESIDUAL || (!SPLIT && !SEGMENTED), "the residual epilogue belongs to plain unsplit kernels");
     using frag_t = typename Mfma<T>::frag;
     using Layout = TileLayout<T, BM, BN, A_K, B_K>;
     using ATile = typename Layout::ATile;
@@ -592,6 +596,77 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
             c_cols = pick.cols;
         }
         const int row0 = w.m0 + wm * WM, col0 = wn * WN;  // of the wavefront's part; columns relative to n0
+        // The two fp32-staged cases of the training step get straight-line code as well: split-K
+        // partial tiles (nothing added, fp32 out) and a residual added to a 16-bit result. Half the
+        // columns are staged per pass; lane l of round u holds 8 consecutive columns (group l%8) of
+        // row 8u + l/8.
+        constexpr int kGroups = WN / 2 / 8, kRowsF = kWave / kGroups, kRoundsF = 32 / kRowsF;
+        const int f_row = lane / kGroups, f_col = (lane % kGroups) * 8;  // f_col within the staged half
+        auto read_staged = [&](int u, vec_t<float, 4>& v0, vec_t<float, 4>& v1) __attribute__((always_inline)) {
+            const int row = u * kRowsF + f_row;
+            const unsigned char* base = region + row * kRowBytes;
+            v0 = *reinterpret_cast<const vec_t<float, 4>*>(base + (((f_col / 4) ^ sw(row)) * 16));
+            v1 = *reinterpret_cast<const vec_t<float, 4>*>(base + (((f_col / 4 + 1) ^ sw(row)) * 16));
+        };
+        // Descriptor over a wavefront's part of a row-major matrix (see the 16-bit case above).
+        auto part_rsrc = [&](const void* origin, long ld, int elem, int rows_left, int cols_left) __attribute__((always_inline)) {
+            const long extent = rows_left > 0 && cols_left > 0 ? (static_cast<long>(rows_left - 1) * ld + cols_left) * elem : 0;
+            return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(origin), 0, static_cast<int>(extent), 0x00020000);
+        };
+        const int rows_left = min(WM, p.m - row0);
+        if constexpr (RESIDUAL) {
+            const int cols_left = min(WN, c_cols - (c_col0 + col0));
+            const T* out_origin = static_cast<const T*>(c_base) + static_cast<long>(row0) * c_ld + (c_col0 + col0);
+            const T* res_origin = static_cast<const T*>(p.residual) + static_cast<long>(row0) * p.ldr + (w.n0 + col0);
+            const __amdgpu_buffer_rsrc_t out_rsrc = part_rsrc(out_origin, c_ld, sizeof(T), rows_left, cols_left);
+            const __amdgpu_buffer_rsrc_t res_rsrc = part_rsrc(res_origin, p.ldr, sizeof(T), rows_left, cols_left);
+            const int out_row_bytes = static_cast<int>(c_ld * static_cast<long>(sizeof(T)));
+            const int res_row_bytes = static_cast<int>(p.ldr * static_cast<long>(sizeof(T)));
+            // The residual of a 32-row block is requested one block ahead (the first one before
+            // anything is staged): its memory round trip passes under the previous block's work.
+            u32x4 ahead[2][2][kRoundsF];
+            auto request_residual = [&](int r, u32x4 (&into)[2][kRoundsF]) __attribute__((always_inline)) {
+#pragma unroll
+                for (int half = 0; half < 2; ++half) {
+                    const int col = half * (WN / 2) + f_col;
+                    const int voffset = col < cols_left ? f_row * res_row_bytes + col * static_cast<int>(sizeof(T))
+                                                        : std::numeric_limits<int>::min();
+#pragma unroll
+                    for (int u = 0; u < kRoundsF; ++u)
+                        into[half][u] = __builtin_amdgcn_raw_buffer_load_b128(res_rsrc, voffset, (r * 32 + u * kRowsF) * res_row_bytes, 0);
+                }
+            };
+            request_residual(0, ahead[0]);
+#pragma unroll
+            for (int r = 0; r < kRowBlocks; ++r) {
+                __builtin_amdgcn_sched_barrier(0);
+                if (request) request_share(r);
+                if (r + 1 < kRowBlocks) request_residual(r + 1, ahead[(r + 1) & 1]);
+#pragma unroll
+                for (int half = 0; half < 2; ++half) {
+                    stage.template operator()<float, TN / 2>(r, half * (TN / 2));
+                    const int col = half * (WN / 2) + f_col;
+                    const int voffset = col < cols_left ? f_row * out_row_bytes + col * static_cast<int>(sizeof(T))
+                                                        : std::numeric_limits<int>::min();
+                    vec_t<float, 4> v0[kRoundsF], v1[kRoundsF];
+#pragma unroll
+                    for (int u = 0; u < kRoundsF; ++u) read_staged(u, v0[u], v1[u]);
+#pragma unroll
+                    for (int u = 0; u < kRoundsF; ++u) {
+                        const vec_t<float, 8> add = vec_to_f32<T, 8>(__builtin_bit_cast(vec_t<T, 8>, ahead[r & 1][half][u]));
+                        vec_t<float, 8> sum;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            sum[e] = v0[u][e] + add[e];
+                            sum[4 + e] = v1[u][e] + add[4 + e];
+                        }
+                        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, vec_from_f32<T, 8>(sum)), out_rsrc, voffset,
+                                                               (r * 32 + u * kRowsF) * out_row_bytes, 0);
+                    }
+                }
+            }
+            return;
+        }
         bool plain = false;
         if constexpr (!SPLIT) plain = p.bias == nullptr && p.residual == nullptr && !p.accumulate && !p.c_f32;
         if (plain) {
@@ -630,6 +705,34 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
             }
             return;
         }
+        if constexpr (SPLIT) {
+            const float* origin = static_cast<const float*>(p.c) +
+                                  (static_cast<long>(w.slice) * p.m + row0) * static_cast<long>(p.n) + (w.n0 + col0);
+            const int cols_left = min(WN, p.n - (w.n0 + col0));
+            const __amdgpu_buffer_rsrc_t rsrc = part_rsrc(origin, p.n, 4, rows_left, cols_left);
+            const int row_bytes = p.n * 4;
+#pragma unroll
+            for (int r = 0; r < kRowBlocks; ++r) {
+                __builtin_amdgcn_sched_barrier(0);
+                if (request) request_share(r);
+#pragma unroll
+                for (int half = 0; half < 2; ++half) {
+                    stage.template operator()<float, TN / 2>(r, half * (TN / 2));
+                    const int col = half * (WN / 2) + f_col;
+                    const int voffset = col < cols_left ? f_row * row_bytes + col * 4 : std::numeric_limits<int>::min();
+                    vec_t<float, 4> v0[kRoundsF], v1[kRoundsF];
+#pragma unroll
+                    for (int u = 0; u < kRoundsF; ++u) read_staged(u, v0[u], v1[u]);
+#pragma unroll
+                    for (int u = 0; u < kRoundsF; ++u) {
+                        const int soffset = (r * 32 + u * kRowsF) * row_bytes;
+                        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v0[u]), rsrc, voffset, soffset, 0);
+                        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v1[u]), rsrc, voffset + 16, soffset, 0);
+                    }
+                }
+            }
+            return;
+        }
 #pragma unroll
         for (int r = 0; r < kRowBlocks; ++r) {
             __builtin_amdgcn_sched_barrier(0);
@@ -642,12 +745,7 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
                     vec_t<float, 4> v0 = *reinterpret_cast<const vec_t<float, 4>*>(lo);
                     vec_t<float, 4> v1 = *reinterpret_cast<const vec_t<float, 4>*>(hi);
                     if (m >= p.m || c_col >= c_cols) return;
-                    if constexpr (SPLIT) {
-                        float* out = static_cast<float*>(p.c) +
-                                     (static_cast<long>(w.slice) * p.m + m) * static_cast<long>(p.n) + n;
-                        *reinterpret_cast<vec_t<float, 4>*>(out) = v0;
-                        *reinterpret_cast<vec_t<float, 4>*>(out + 4) = v1;
-                    } else {
+                    {
                         if (p.bias != nullptr) {
                             const T* bias = static_cast<const T*>(p.bias) + n;
                             v0 += vec_to_f32<T, 4>(load_vec<T, 4>(bias));
@@ -861,10 +959,10 @@ __global__ __launch_bounds__(kGenericTile* kGenericTile / 4) void gemm_generic_k
 }
 
 // ------------------------------------------------------------------- host side
-template <typename T, int BM, int BN, bool A_K, bool B_K, bool SPLIT, bool SEGMENTED>
+template <typename T, int BM, int BN, bool A_K, bool B_K, bool SPLIT, bool SEGMENTED, bool RESIDUAL = false>
 int launch_mfma(const KernelArgs& p, int slices, hipStream_t stream) {
     constexpr std::size_t smem = TileLayout<T, BM, BN, A_K, B_K>::kSmemBytes;
-    auto kernel = gemm_mfma_kernel<T, BM, BN, A_K, B_K, SPLIT, SEGMENTED>;
+    auto kernel = gemm_mfma_kernel<T, BM, BN, A_K, B_K, SPLIT, SEGMENTED, RESIDUAL>;
     static bool configured = false;
     if (!configured) {
         CGPTX_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -893,6 +991,20 @@ int launch_layout(const KernelArgs& p, bool a_k, bool b_k, int slices, hipStream
         if (segmented && !b_k) return launch_mfma<T, BM, BN, true, false, false, true>(p, slices, stream);
     }
     if (segmented) return fail(CGPTX_RUNTIME, "gemm: a segmented operand cannot be split along K");
+    if constexpr (!SPLIT) {
+        if (a_k && b_k && p.bias == nullptr && !p.c_f32) {
+            if (p.residual != nullptr && !p.accumulate) return launch_mfma<T, BM, BN, true, true, false, false, true>(p, slices, stream);
+            if (p.residual == nullptr && p.accumulate && p.c_seg.count == 0) {
+                // C += A·B in the storage dtype is the same epilogue with C as its own residual
+                // (every lane reads the elements it later writes, and reads them first).
+                KernelArgs self = p;
+                self.residual = p.c;
+                self.ldr = p.ldc;
+                self.accumulate = 0;
+                return launch_mfma<T, BM, BN, true, true, false, false, true>(self, slices, stream);
+            }
+        }
+    }
     if (a_k && b_k) return launch_mfma<T, BM, BN, true, true, SPLIT, false>(p, slices, stream);
     if (a_k && !b_k) return launch_mfma<T, BM, BN, true, false, SPLIT, false>(p, slices, stream);
     if (!a_k && !b_k) return launch_mfma<T, BM, BN, false, false, SPLIT, false>(p, slices, stream);
