@@ -387,7 +387,8 @@ int enqueue_forward_backward(cgptx_model* m, float loss_scale, int loss_mode, hi
         // out = x + attention_projection, then out += ffn_output (src/core/transformer_block.cu:594-595)
         CGPTX_OP("gemm_fwd", linear_forward_residual(out, a.attn_out, w.o.value, x, false, N, QW, H, dt, stream));
         if (!dual_norms) CGPTX_OP("rmsnorm_fwd", cgptx_rmsnorm_forward(a.norm_f, x, w.ffn_norm.value, N, H, eps, dt, s));
-        CGPTX_OP("gemm_fwd", cgptx_linear_forward(a.gate_up, a.norm_f, w.gate.value, nullptr, N, H, 2 * I, dt, s));
+        // Labelled on its own ("kind.part"): the launch the kernel roofline of the benchmark is quoted on.
+        CGPTX_OP("gemm_fwd.gate_up", cgptx_linear_forward(a.gate_up, a.norm_f, w.gate.value, nullptr, N, H, 2 * I, dt, s));
         CGPTX_OP("swiglu_fwd", cgptx_swiglu_forward_packed(a.act, a.gate_up, N, I, dt, s));
         CGPTX_OP("gemm_fwd", linear_forward_residual(out, a.act, w.down.value, nullptr, true, N, I, H, dt, stream));
     }
