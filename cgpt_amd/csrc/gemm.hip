@@ -1084,7 +1084,13 @@ bool offsets_fit_32bit(const GemmArgs& g, std::size_t elem) {
     constexpr std::size_t limit = (std::size_t{1} << 31) - (std::size_t{1} << 20);
     const std::size_t a_span = g.a_k_contiguous ? (256 * g.lda + g.k) * elem : (g.k * g.lda + 256) * elem;
     const std::size_t b_span = g.b_k_contiguous ? (256 * g.ldb + g.k) * elem : (g.k * g.ldb + 256) * elem;
-    return a_span < limit && b_span < limit;
+    // The epilogues address a wavefront's part of C (of the residual, of a split-K partial tile)
+    // through a range-checked descriptor with 32-bit offsets as well: up to 256 rows.
+    std::size_t c_ld = std::max(g.ldc, g.n);
+    for (int s = 0; s < g.c_segments.count; ++s) c_ld = std::max(c_ld, g.c_segments.ld[s]);
+    const std::size_t c_span = 256 * c_ld * 4;
+    const std::size_t r_span = g.residual != nullptr ? 256 * g.ldr * elem : 0;
+    return a_span < limit && b_span < limit && c_span < limit && r_span < limit;
 }
 
 template <typename T>
