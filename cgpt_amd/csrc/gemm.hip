@@ -110,6 +110,9 @@ struct KernelArgs {
     int accumulate;
     int c_f32;
     KernelSegments a_seg, c_seg;  // column segments of A (as stored) and of C; count 0 = one buffer
+    void* act;      // SWIGLU kernels: [M, inter] = silu(gate) * up, T*
+    long ld_act;
+    int inter;      // SWIGLU kernels: columns of gate (= of up); n = 2 * inter
 };
 
 // The column segment (of up to three) that holds column `col`, picked with selects: indexing the
@@ -180,6 +183,7 @@ struct TileCursor {
     int voffset;
     unsigned int soffset;
     unsigned int step;
+    unsigned int step2;  // advance after the operand's odd-numbered loads (differs from step only for SWIGLU's B)
 };
 
 template <int BEGIN, int... I, typename F>
@@ -320,10 +324,20 @@ struct TileLayout {
 // RESIDUAL: the epilogue adds a residual to a 16-bit result and nothing else (the output
 // projections of a transformer block); a kernel of its own, so that each kernel carries one
 // straight-line epilogue besides the general one.
-template <typename T, int BM, int BN, bool A_K, bool B_K, bool SPLIT, bool SEGMENTED, bool RESIDUAL = false>
+// SWIGLU: B is the concatenated [gate; up] weight ([2·inter, K]) and C the concatenated [gate | up]
+// activation; the kernel also writes silu(gate)·up. A tile's 256 columns are 128 gate columns and
+// the 128 up columns of the same indices, interleaved in units of 64 so that each wavefront holds
+// gate and up of its 64 indices in the same lanes: the B rows of an LDS tile are
+// [gate 0-63 | up 0-63 | gate 64-127 | up 64-127] (one unit per load instruction of a wavefront,
+// so only the scalar offsets of the loads change), and the epilogue computes the product from the
+// rounded gate and up values, as the separate operator would from memory.
+template <typename T, int BM, int BN, bool A_K, bool B_K, bool SPLIT, bool SEGMENTED, bool RESIDUAL = false,
+          bool SWIGLU = false>
 __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
     static_assert(!SEGMENTED || (A_K && !SPLIT), "segments along K are read by the unsplit kernels only");
     static_assert(!RESIDUAL || (!SPLIT && !SEGMENTED), "the residual epilogue belongs to plain unsplit kernels");
+    static_assert(!SWIGLU || (A_K && B_K && !SPLIT && !SEGMENTED && !RESIDUAL && BN == 256),
+                  "the SwiGLU epilogue belongs to the plain forward kernel with 256-wide tiles");
     using frag_t = typename Mfma<T>::frag;
     using Layout = TileLayout<T, BM, BN, A_K, B_K>;
     using ATile = typename Layout::ATile;
@@ -420,7 +434,8 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
             }
             a_src.init(base + (m0 - first), ld, width - (m0 - first), p.k, wave);
         }
-        if constexpr (B_K) b_src.init(static_cast<const T*>(p.b) + static_cast<long>(n0) * p.ldb, p.ldb, p.n - n0, p.k, wave);
+        if constexpr (SWIGLU) b_src.init(static_cast<const T*>(p.b) + static_cast<long>(n0 / 2) * p.ldb, p.ldb, p.n - n0 / 2, p.k, wave);
+        else if constexpr (B_K) b_src.init(static_cast<const T*>(p.b) + static_cast<long>(n0) * p.ldb, p.ldb, p.n - n0, p.k, wave);
         else b_src.init(static_cast<const T*>(p.b) + n0, p.ldb, p.n - n0, p.k, wave);
     };
     // K tiles past the end of the slice are still "loaded" (the loop stays free of data-dependent
@@ -449,16 +464,26 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
             const int start = in2 ? end1 : in1 ? end0 : 0;
             ca.soffset = (wave * group_bytes + (k0 - start) * static_cast<unsigned int>(sizeof(T))) | past_end;
             ca.step = kWaves * group_bytes;
+            ca.step2 = ca.step;
         } else {
             ca.rsrc = a_src.rsrc;
             ca.voffset = a_src.voffset;
             ca.soffset = a_src.first_offset(k0, wave) | past_end;
             ca.step = kWaves * a_src.group_bytes;
+            ca.step2 = ca.step;
         }
         cb.rsrc = b_src.rsrc;
         cb.voffset = b_src.voffset;
         cb.soffset = b_src.first_offset(k0, wave) | past_end;
         cb.step = kWaves * b_src.group_bytes;
+        cb.step2 = cb.step;
+        if constexpr (SWIGLU) {
+            // gate unit -> up unit of the same rows (inter rows further), then back and 64 rows on.
+            const unsigned int up = __builtin_amdgcn_readfirstlane(
+                static_cast<unsigned int>(static_cast<long>(p.inter) * p.ldb * static_cast<long>(sizeof(T))));
+            cb.step2 = cb.step - up;
+            cb.step = up;
+        }
     };
     // Load l of a K tile (A's loads first, then B's) into the stage whose LDS address, advanced to
     // this wavefront's first 1 KiB slot, is stage_lds. One load fills 1 KiB; the wavefronts' slots
@@ -470,8 +495,9 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
         if constexpr (l < ATile::kLoads) {
             ca.soffset = load_to_lds<l * kWaves * kLoadBytes>(ca.rsrc, stage_lds, ca.voffset, ca.soffset, ca.step);
         } else {
-            cb.soffset = load_to_lds<kATileBytes + (l - ATile::kLoads) * kWaves * kLoadBytes>(
-                cb.rsrc, stage_lds, cb.voffset, cb.soffset, cb.step);
+            constexpr int lb = l - ATile::kLoads;
+            cb.soffset = load_to_lds<kATileBytes + lb * kWaves * kLoadBytes>(cb.rsrc, stage_lds, cb.voffset, cb.soffset,
+                                                                            (lb & 1) ? cb.step2 : cb.step);
         }
     };
     constexpr int kTileLoads = ATile::kLoads + BTile::kLoads;  // per wavefront and K tile
@@ -544,7 +570,16 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
             unsigned char* write_row = region + row * kRowBytes;
 #pragma unroll
             for (int jj = 0; jj < JP; ++jj) {
-                const acc_t v = acc[2 * r + ii][j0 + jj];
+                // Read out of the accumulator registers here and now: left to the register allocator,
+                // some kernels copy all 256 accumulators to vector registers right after the K loop
+                // and spill what does not fit.
+                acc_t v;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    float x;
+                    asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(x) : "a"(acc[2 * r + ii][j0 + jj][e]));
+                    v[e] = x;
+                }
                 const int byte = (jj * 16 + q_lane * 4) * static_cast<int>(sizeof(S));
                 unsigned char* slot = write_row + (((byte / 16) ^ sw(row)) * 16) + byte % 16;
                 if constexpr (std::is_same_v<S, float>) *reinterpret_cast<vec_t<float, 4>*>(slot) = v;
@@ -614,6 +649,51 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
             return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(origin), 0, static_cast<int>(extent), 0x00020000);
         };
         const int rows_left = min(WM, p.m - row0);
+        if constexpr (SWIGLU) {
+            // The wavefront's 128 staged columns are gate g0 .. g0+63 and up g0 .. g0+63. Lane l of
+            // round u takes 8 gate and the 8 matching up values of row 8u + l/8 from the staging
+            // region, stores both where the concatenated layout wants them, and the product beside.
+            const int g0 = w.n0 / 2 + wn * (WN / 2);
+            const int cols_left = min(WN / 2, p.inter - g0);
+            const T* c_origin = static_cast<const T*>(p.c) + static_cast<long>(row0) * p.ldc + g0;
+            const __amdgpu_buffer_rsrc_t gate_rsrc = part_rsrc(c_origin, p.ldc, sizeof(T), rows_left, cols_left);
+            const __amdgpu_buffer_rsrc_t up_rsrc = part_rsrc(c_origin + p.inter, p.ldc, sizeof(T), rows_left, cols_left);
+            const __amdgpu_buffer_rsrc_t act_rsrc = part_rsrc(static_cast<const T*>(p.act) + static_cast<long>(row0) * p.ld_act + g0,
+                                                              p.ld_act, sizeof(T), rows_left, cols_left);
+            const int c_row_bytes = static_cast<int>(p.ldc * static_cast<long>(sizeof(T)));
+            const int act_row_bytes = static_cast<int>(p.ld_act * static_cast<long>(sizeof(T)));
+            const bool live = f_col < cols_left;
+            const int c_voffset = live ? f_row * c_row_bytes + f_col * static_cast<int>(sizeof(T)) : std::numeric_limits<int>::min();
+            const int act_voffset = live ? f_row * act_row_bytes + f_col * static_cast<int>(sizeof(T)) : std::numeric_limits<int>::min();
+#pragma unroll
+            for (int r = 0; r < kRowBlocks; ++r) {
+                __builtin_amdgcn_sched_barrier(0);
+                if (request) request_share(r);
+                stage.template operator()<T, TN>(r, 0);
+                u32x4 gate[kRoundsF], up[kRoundsF];
+#pragma unroll
+                for (int u = 0; u < kRoundsF; ++u) {
+                    const int row = u * kRowsF + f_row;
+                    const unsigned char* base = region + row * kRowBytes;
+                    gate[u] = *reinterpret_cast<const u32x4*>(base + (((f_col / 8) ^ sw(row)) * 16));
+                    up[u] = *reinterpret_cast<const u32x4*>(base + (((kGroups + f_col / 8) ^ sw(row)) * 16));
+                }
+#pragma unroll
+                for (int u = 0; u < kRoundsF; ++u) {
+                    const int row = r * 32 + u * kRowsF;
+                    __builtin_amdgcn_raw_buffer_store_b128(gate[u], gate_rsrc, c_voffset, row * c_row_bytes, 0);
+                    __builtin_amdgcn_raw_buffer_store_b128(up[u], up_rsrc, c_voffset, row * c_row_bytes, 0);
+                    const vec_t<float, 8> g = vec_to_f32<T, 8>(__builtin_bit_cast(vec_t<T, 8>, gate[u]));
+                    const vec_t<float, 8> v = vec_to_f32<T, 8>(__builtin_bit_cast(vec_t<T, 8>, up[u]));
+                    vec_t<float, 8> product;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) product[e] = g[e] * (1.0f / (1.0f + __expf(-g[e]))) * v[e];
+                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, vec_from_f32<T, 8>(product)), act_rsrc,
+                                                           act_voffset, row * act_row_bytes, 0);
+                }
+            }
+            return;
+        }
         if constexpr (RESIDUAL) {
             const int cols_left = min(WN, c_cols - (c_col0 + col0));
             const T* out_origin = static_cast<const T*>(c_base) + static_cast<long>(row0) * c_ld + (c_col0 + col0);
@@ -959,10 +1039,11 @@ __global__ __launch_bounds__(kGenericTile* kGenericTile / 4) void gemm_generic_k
 }
 
 // ------------------------------------------------------------------- host side
-template <typename T, int BM, int BN, bool A_K, bool B_K, bool SPLIT, bool SEGMENTED, bool RESIDUAL = false>
+template <typename T, int BM, int BN, bool A_K, bool B_K, bool SPLIT, bool SEGMENTED, bool RESIDUAL = false,
+          bool SWIGLU = false>
 int launch_mfma(const KernelArgs& p, int slices, hipStream_t stream) {
     constexpr std::size_t smem = TileLayout<T, BM, BN, A_K, B_K>::kSmemBytes;
-    auto kernel = gemm_mfma_kernel<T, BM, BN, A_K, B_K, SPLIT, SEGMENTED, RESIDUAL>;
+    auto kernel = gemm_mfma_kernel<T, BM, BN, A_K, B_K, SPLIT, SEGMENTED, RESIDUAL, SWIGLU>;
     static bool configured = false;
     if (!configured) {
         CGPTX_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -991,6 +1072,10 @@ int launch_layout(const KernelArgs& p, bool a_k, bool b_k, int slices, hipStream
         if (segmented && !b_k) return launch_mfma<T, BM, BN, true, false, false, true>(p, slices, stream);
     }
     if (segmented) return fail(CGPTX_RUNTIME, "gemm: a segmented operand cannot be split along K");
+    if constexpr (!SPLIT && BN == 256) {
+        if (p.act != nullptr) return launch_mfma<T, BM, BN, true, true, false, false, false, true>(p, slices, stream);
+    }
+    if (p.act != nullptr) return fail(CGPTX_RUNTIME, "gemm: the SwiGLU epilogue needs 256-wide unsplit tiles");
     if constexpr (!SPLIT) {
         if (a_k && b_k && p.bias == nullptr && !p.c_f32) {
             if (p.residual != nullptr && !p.accumulate) return launch_mfma<T, BM, BN, true, true, false, false, true>(p, slices, stream);
@@ -1031,7 +1116,8 @@ int run_config(const GemmArgs& g, KernelArgs p, hipStream_t stream) {
     const long want_blocks = static_cast<long>(compute_units()) * (BM == 256 ? 1 : 2);
     int slices = 1;
     const bool k_segments = g.a_k_contiguous && g.a_segments.count > 0;
-    if (!g.no_split && g.residual == nullptr && g.c_segments.count == 0 && !k_segments && tiles < want_blocks && k_tiles >= 32) {
+    if (!g.no_split && g.residual == nullptr && g.swiglu_out == nullptr && g.c_segments.count == 0 && !k_segments &&
+        tiles < want_blocks && k_tiles >= 32) {
         // As many slices as fit the CU slots in one go: one item more than that would cost a
         // second round of the persistent blocks.
         slices = static_cast<int>(std::min<long>(want_blocks / tiles, k_tiles / 16));
@@ -1110,6 +1196,12 @@ int run_typed(const GemmArgs& g, hipStream_t stream) {
     p.ldc = static_cast<long>(g.ldc);
     p.accumulate = g.accumulate ? 1 : 0;
     p.c_f32 = g.c_is_f32 ? 1 : 0;
+    if (g.swiglu_out != nullptr) {
+        if (!gemm_fuses_swiglu(g)) return fail(CGPTX_INVALID_ARGUMENT, "gemm: this call cannot carry the SwiGLU epilogue");
+        p.act = g.swiglu_out;
+        p.ld_act = static_cast<long>(g.ld_swiglu);
+        p.inter = static_cast<int>(g.n / 2);
+    }
     const bool segmented = g.a_segments.count > 0 || g.c_segments.count > 0;
     if (segmented) {
         if (int s = copy_segments(g.a_segments, g.a_k_contiguous ? g.k : g.m, g.a_k_contiguous ? kBK : 256, p.a_seg))
@@ -1159,7 +1251,7 @@ int run_typed(const GemmArgs& g, hipStream_t stream) {
         const bool fills = big_tiles * 5 >= units * 4;
         const bool splits = !g.no_split && g.residual == nullptr && g.c_segments.count == 0 && big_tiles >= 8 &&
                             g.k / kBK >= static_cast<std::size_t>(32 * ((units + big_tiles - 1) / big_tiles));
-        const bool big = forced == 256 || (forced == 0 && (fills || splits));
+        const bool big = g.swiglu_out != nullptr || forced == 256 || (forced == 0 && (fills || splits));
         if (big) return run_config<T, 256, 256>(g, p, stream);
         return run_config<T, 128, 128>(g, p, stream);
     }
@@ -1167,6 +1259,24 @@ int run_typed(const GemmArgs& g, hipStream_t stream) {
 }
 
 }  // namespace
+
+bool gemm_fuses_swiglu(const GemmArgs& g) {
+    if (g.swiglu_out == nullptr || g.dtype == CGPTX_F32 || !g.a_k_contiguous || !g.b_k_contiguous || g.bias != nullptr ||
+        g.residual != nullptr || g.accumulate || g.c_is_f32 || g.a_segments.count > 0 || g.c_segments.count > 0 ||
+        g.a == nullptr || g.b == nullptr || g.c == nullptr)
+        return false;
+    const std::size_t elem = 2, inter = g.n / 2;
+    // Whole 128-column units of gate and of up per tile, tiles that fill the chip (the 256x256
+    // configuration), 16-byte aligned rows everywhere, and the whole weight within 32-bit offsets.
+    if (g.n % 256 != 0 || g.m % 8 != 0 || g.k % kBK != 0 || g.lda % 8 != 0 || g.ldb % 8 != 0 || g.ldc % 8 != 0 ||
+        g.ld_swiglu % 8 != 0 || g.ld_swiglu < inter || !is_aligned16(g.a) || !is_aligned16(g.b) || !is_aligned16(g.c) ||
+        !is_aligned16(g.swiglu_out))
+        return false;
+    const long tiles = static_cast<long>((g.m + 255) / 256) * static_cast<long>(g.n / 256);
+    if (forced_tile() == 128 || tiles * 5 < static_cast<long>(compute_units()) * 4) return false;
+    constexpr std::size_t limit = (std::size_t{1} << 31) - (std::size_t{1} << 20);
+    return offsets_fit_32bit(g, elem) && (g.n * g.ldb + g.k) * elem < limit && 256 * g.ld_swiglu * elem < limit;
+}
 
 int gemm(const GemmArgs& g, hipStream_t stream) {
     if ((g.a == nullptr && g.a_segments.count == 0) || g.b == nullptr || (g.c == nullptr && g.c_segments.count == 0) ||

@@ -40,8 +40,16 @@ struct GemmArgs {
     // multiples of 256 (of 32 for a k-contiguous A) except the last; a and lda / c and ldc are
     // ignored for a segmented operand.
     GemmSegments a_segments, c_segments;
+    // Forward projection into the concatenated [gate | up] layout (n = 2·inter, b = [gate; up]
+    // weights) that also writes swiglu_out[m, inter] = silu(gate)·up, computed from the rounded
+    // gate and up values (the bits the separate operator would produce). Only for calls that
+    // gemm_fuses_swiglu() accepts.
+    void* swiglu_out = nullptr;
+    std::size_t ld_swiglu = 0;
 };
 
 int gemm(const GemmArgs& args, hipStream_t stream);
+// Whether gemm() serves args.swiglu_out for this call (shape, layout and alignment of the fused kernel).
+bool gemm_fuses_swiglu(const GemmArgs& args);
 
 }  // namespace cgptx

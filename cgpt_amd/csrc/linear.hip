@@ -46,6 +46,36 @@ extern "C" int cgptx_linear_forward(void* output, const void* input, const void*
     return gemm(g, static_cast<hipStream_t>(stream));
 }
 
+extern "C" int cgptx_linear_swiglu_forward(void* gate_up, void* activated, const void* input, const void* weight,
+                                           size_t rows, size_t in_features, size_t hidden, int dtype,
+                                           cgptx_stream stream_) {
+    using namespace cgptx;
+    if (hidden > std::numeric_limits<std::size_t>::max() / 2)
+        return fail(CGPTX_OVERFLOW, "linear_swiglu_forward: dimension exceeds int range");
+    if (int s = validate("linear_swiglu_forward", rows, in_features, 2 * hidden, dtype)) return s;
+    if (gate_up == nullptr || activated == nullptr || input == nullptr || weight == nullptr)
+        return fail(CGPTX_INVALID_ARGUMENT, "linear_swiglu_forward: null tensor");
+    auto stream = static_cast<hipStream_t>(stream_);
+    GemmArgs g;
+    g.a = input;
+    g.b = weight;
+    g.c = gate_up;
+    g.m = rows;
+    g.n = 2 * hidden;
+    g.k = in_features;
+    g.lda = in_features;
+    g.ldb = in_features;
+    g.ldc = 2 * hidden;
+    g.dtype = dtype;
+    g.swiglu_out = activated;
+    g.ld_swiglu = hidden;
+    if (gemm_fuses_swiglu(g)) return gemm(g, stream);
+    // Shapes the fused kernel does not take: the two operators one after the other (same bits).
+    g.swiglu_out = nullptr;
+    if (int s = gemm(g, stream)) return s;
+    return cgptx_swiglu_forward_packed(activated, gate_up, rows, hidden, dtype, stream_);
+}
+
 extern "C" int cgptx_linear_backward(void* grad_input, void* grad_weight, void* grad_bias, const void* grad_output,
                                      const void* input, const void* weight, size_t rows, size_t in_features,
                                      size_t out_features, int accumulate_input, int accumulate_weight,

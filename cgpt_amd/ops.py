@@ -525,6 +525,22 @@ def linear_forward(output, input, weight, gemm_context=None, stream=None, bias=N
               input.numel() // in_features, in_features, out_features, _code(input), _stream(stream))
 
 
+def linear_swiglu_forward(gate_up, activated, input, weight, gemm_context=None, stream=None):
+    """The feed-forward's gate and up projections and SwiGLU in one call (src/core/transformer_block.cu:586-590
+    with the concatenated layouts of include/ops/swiglu.h:33-37): weight = [gate_proj; up_proj] ([2*hidden, in]),
+    gate_up = [..., 2*hidden] = [gate | up], activated = [..., hidden] = silu(gate) * up."""
+    name = "linear_swiglu_forward"
+    _require_device(name, gate_up, activated, input, weight)
+    _same_dtype(name, input, gate_up, activated, weight)
+    if weight.dim() != 2 or weight.shape[0] % 2 != 0 or input.shape[-1] != weight.shape[1] or \
+            gate_up.shape[-1] != weight.shape[0] or activated.shape[-1] * 2 != weight.shape[0] or \
+            tuple(gate_up.shape[:-1]) != tuple(input.shape[:-1]) or tuple(activated.shape[:-1]) != tuple(input.shape[:-1]):
+        raise ValueError(f"{name}: incompatible tensors")
+    out_features, in_features = weight.shape
+    capi.call("cgptx_linear_swiglu_forward", _ptr(gate_up), _ptr(activated), _ptr(input), _ptr(weight),
+              input.numel() // in_features, in_features, out_features // 2, _code(input), _stream(stream))
+
+
 def embedding_forward(output, device_token_ids, token_count, weight, stream=None):
     """include/ops/embedding.h."""
     name = "embedding_forward"

@@ -246,6 +246,16 @@ int cgptx_linear_forward(void* output, const void* input, const void* weight,
                          const void* bias, size_t rows, size_t in_features,
                          size_t out_features, int dtype, cgptx_stream stream);
 
+/* The feed-forward's gate and up projections and its SwiGLU in one call — the sequence
+ * linear_forward(gate), linear_forward(up), swiglu_forward(activated, gate, up) of
+ * src/core/transformer_block.cu:586-590 with the concatenated layouts of include/ops/swiglu.h:33-37:
+ * weight = [gate_proj; up_proj] ([2*hidden, in]), gate_up = [rows, 2*hidden] = [gate | up] (kept for the
+ * backward pass), activated[rows, hidden] = silu(gate)·up from the rounded gate and up values. Large
+ * aligned shapes run as one contraction whose epilogue writes all three; the rest as the two operators. */
+int cgptx_linear_swiglu_forward(void* gate_up, void* activated, const void* input,
+                                const void* weight, size_t rows, size_t in_features,
+                                size_t hidden, int dtype, cgptx_stream stream);
+
 /* embedding_forward — include/ops/embedding.h. out[t,:] = W[id_t,:]; ids >= vocab give a zero row. */
 int cgptx_embedding_forward(void* output, const uint32_t* token_ids,
                             size_t token_count, const void* weight,

@@ -147,3 +147,30 @@ def test_linear_argument_errors(device):
         ops.linear_backward(gi, gw, gb, dy, x.half(), w)
     with pytest.raises(ValueError):
         ops.linear_backward(gi, torch.zeros(3, 7, device=device), gb, dy, x, w)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+@pytest.mark.parametrize("rows,fin,hidden", [(4096, 256, 1664), (4104, 64, 1664), (2056, 96, 3328), (64, 32, 64), (520, 96, 200)],
+                         ids=["fused", "fused-ragged-rows", "fused-wide", "small", "unaligned-columns"])
+def test_linear_swiglu_forward_equals_the_two_operators(device, rows, fin, hidden, dtype):
+    """Gate/up projection with the SwiGLU product from its epilogue (one contraction over interleaved
+    gate and up columns when the shape fills the chip) against linear_forward into the concatenated
+    layout followed by swiglu_forward: the same bits, and the float64 product within the 16-bit tolerance."""
+    g = torch.Generator().manual_seed(rows + hidden)
+    x = torch.randn(rows, fin, generator=g).to(dtype).to(device)
+    w = (torch.randn(2 * hidden, fin, generator=g) * 0.3).to(dtype).to(device)
+    want_gate_up = torch.empty(rows, 2 * hidden, dtype=dtype, device=device)
+    want_act = torch.empty(rows, hidden, dtype=dtype, device=device)
+    ops.linear_forward(want_gate_up, x, w)
+    ops.swiglu_forward(want_act, want_gate_up)
+    got_gate_up = torch.full_like(want_gate_up, float("nan"))
+    got_act = torch.full_like(want_act, float("nan"))
+    ops.linear_swiglu_forward(got_gate_up, got_act, x, w)
+    torch.cuda.synchronize()
+    assert torch.equal(got_gate_up, want_gate_up)
+    assert torch.equal(got_act, want_act)
+    exact = x.double().cpu() @ w.double().cpu().t()
+    gate, up = exact[:, :hidden], exact[:, hidden:]
+    reference = gate / (1 + torch.exp(-gate)) * up
+    err = (got_act.double().cpu() - reference).abs().max() / reference.abs().max()
+    assert err <= 2e-2
