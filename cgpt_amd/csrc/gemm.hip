@@ -78,12 +78,19 @@ struct Mfma<bf16_t> {
     __device__ static __forceinline__ void run(acc_t& c, const frag& a, const frag& b) {
         asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
     }
+    // c = a x b: the first K tile of an item starts the sums, so the accumulators are never cleared.
+    __device__ static __forceinline__ void start(acc_t& c, const frag& a, const frag& b) {
+        asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, 0" : "=a"(c) : "v"(a), "v"(b));
+    }
 };
 template <>
 struct Mfma<f16_t> {
     using frag = vec_t<f16_t, 8>;
     __device__ static __forceinline__ void run(acc_t& c, const frag& a, const frag& b) {
         asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+    }
+    __device__ static __forceinline__ void start(acc_t& c, const frag& a, const frag& b) {
+        asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, 0" : "=a"(c) : "v"(a), "v"(b));
     }
 };
 
@@ -887,13 +894,14 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
     constexpr int kHalf = TN / 2;
     static_assert(TN % 2 == 0 && kHalf <= TM, "the left-half B fragments are read one per row");
     // HALF 0: this_tile = tile t (its right-half B fragments are read); HALF 1: next_tile = tile t+1.
-    auto multiply_half = [&]<int HALF>(const T* tile, unsigned int free_lds) __attribute__((always_inline)) {
+    auto multiply_half = [&]<int HALF, bool FIRST>(const T* tile, unsigned int free_lds) __attribute__((always_inline)) {
         static_for<0, kMfmas / 2>([&](auto index) {
             constexpr int m = decltype(index)::value;
             // Rows one after the other, their columns left to right and right to left alternately:
             // consecutive MFMAs always share an operand (measurably less power on a power-limited chip).
             constexpr int i = m / kHalf, jj = m % kHalf, j = HALF * kHalf + ((i & 1) ? kHalf - 1 - jj : jj);
-            Mfma<T>::run(acc[i][j], bf[j], af[i]);
+            if constexpr (FIRST) Mfma<T>::start(acc[i][j], bf[j], af[i]);
+            else Mfma<T>::run(acc[i][j], bf[j], af[i]);
             if constexpr (HALF == 0) {
                 // Right-half B fragment i of this tile after the first MFMA of row i (rows 0 .. kHalf-1).
                 if constexpr (jj == 0 && i < kHalf) read_frag.template operator()<TM + kHalf + i>(tile);
@@ -917,10 +925,6 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
     open(current);
     request_tiles.template operator()<0, kStages - 1>();
     while (true) {
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-            for (int j = 0; j < TN; ++j) acc[i][j] = acc_t(0.0f);
         const int count = current.kt_end - current.kt_begin;
         // Loads and stores retire in the order they were issued: at most the loads of K tiles
         // 1 .. kStages-2 (and no older store of the previous epilogue) may still be outstanding.
@@ -929,16 +933,21 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
         static_for<0, TM + kHalf>([&](auto f) { read_frag.template operator()<decltype(f)::value>(smem); });
         int stage = 0;                 // of tile t
         int free_stage = kStages - 1;  // of tile t-1, refilled with tile t+kStages-1
-        for (int t = 0; t < count; ++t) {
+        auto multiply_tile = [&]<bool FIRST>(int t) __attribute__((always_inline)) {
             const int next_stage = stage + 1 == kStages ? 0 : stage + 1;
             cursors(t + kStages - 1, ca, cb);
-            multiply_half.template operator()<0>(smem + stage * kStage, 0u);
+            multiply_half.template operator()<0, FIRST>(smem + stage * kStage, 0u);
             __builtin_amdgcn_s_waitcnt(vmcnt_immediate((kStages - 3) * kTileLoads));
             barrier_only();
-            multiply_half.template operator()<1>(smem + next_stage * kStage, lds_wave + free_stage * kStageBytes);
+            multiply_half.template operator()<1, FIRST>(smem + next_stage * kStage, lds_wave + free_stage * kStageBytes);
             free_stage = stage;
             stage = next_stage;
-        }
+        };
+        // The first K tile starts the sums (MFMA with a zero addend): no pass over the 256
+        // accumulator registers to clear them. Every item has at least one K tile (the host makes
+        // K slices non-empty).
+        multiply_tile.template operator()<true>(0);
+        for (int t = 1; t < count; ++t) multiply_tile.template operator()<false>(t);
         // The loads still outstanding are of K tiles past the end (zeros, but they do write LDS):
         // once they have landed and every wavefront has read its last fragments, all stages are free.
         __builtin_amdgcn_s_waitcnt(vmcnt_immediate(0));
