@@ -7,7 +7,7 @@ and random-init weights.
 
 Prints ONE JSON line. Besides the contract fields it carries
   roofline     – the kernel that takes the most time in the step, on the launch it spends most
-                 of it in (the gate/up projection): algorithmic FLOPs of that launch / its average
+                 of it in (dX of the gate/up projection): algorithmic FLOPs of that launch / its average
                  duration inside the step (HIP events around every operator call of one eager
                  pass on the step's stream), against the 2.5 PFLOP/s dense bf16 MFMA peak; the
                  same launch timed 20 times back to back; the per-kind breakdown of the step;
@@ -60,12 +60,13 @@ def op_work(cfg, batch, seq, loss_mode):
     return work
 
 
-# The kernel that takes the largest share of a step is the 256x256-tile contraction with both
-# operands k-contiguous (every forward projection and the classifier logits). Its roofline entry is
-# measured on the launch it spends most time in: the fused gate/up projection, [N, H] x [2I, H]^T.
-PROBE_KERNEL = "gemm_mfma_kernel<bf16, 256, 256, A k-contiguous, B k-contiguous> (gate/up projection shape)"
+# The kernel that takes the largest share of a step is the 256x256-tile contraction with a k-contiguous
+# A and an n-contiguous B (dX = dY W: every input gradient of a projection and of the classifier). Its
+# roofline entry is measured on the launch it spends most time in: the input gradient of the fused
+# gate/up projection, [N, 2I] x [2I, H].
+PROBE_KERNEL = "gemm_mfma_kernel<bf16, 256, 256, A k-contiguous, B n-contiguous> (dX of the gate/up projection)"
 TRAFFIC_FILE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles",
-                            "gemm_nt_256x256_gate_projection_pmc.txt")
+                            "gemm_dx_256x256_gate_projection_pmc.txt")
 
 
 def kernel_probe(torch, cfg, batch, seq, stream, launches, seed):
@@ -74,23 +75,24 @@ def kernel_probe(torch, cfg, batch, seq, stream, launches, seed):
 
     rows, hidden, inter = batch * seq, cfg.hidden_size, 2 * cfg.intermediate_size  # [gate; up] as one weight
     generator = torch.Generator(device="cuda").manual_seed(seed)
-    x = torch.randn(rows, hidden, device="cuda", generator=generator).to(torch.bfloat16)
+    dy = torch.randn(rows, inter, device="cuda", generator=generator).to(torch.bfloat16)
+    x = torch.empty(rows, hidden, device="cuda", dtype=torch.bfloat16)  # shape only: no weight gradient is asked for
     w = (torch.randn(inter, hidden, device="cuda", generator=generator) * 0.02).to(torch.bfloat16)
-    y = torch.empty(rows, inter, device="cuda", dtype=torch.bfloat16)
+    dx = torch.empty(rows, hidden, device="cuda", dtype=torch.bfloat16)
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     with torch.cuda.stream(stream):
         for _ in range(3):
-            ops.linear_forward(y, x, w, None, stream)
+            ops.linear_backward(dx, None, None, dy, x, w, None, stream)
         start.record(stream)
         for _ in range(launches):
-            ops.linear_forward(y, x, w, None, stream)
+            ops.linear_backward(dx, None, None, dy, x, w, None, stream)
         stop.record(stream)
     stop.synchronize()
     seconds = start.elapsed_time(stop) * 1e-3 / launches
     flops = 2.0 * rows * hidden * inter
-    algorithmic_bytes = 2 * (rows * hidden + inter * hidden + rows * inter)
+    algorithmic_bytes = 2 * (rows * inter + inter * hidden + rows * hidden)
     return {"seconds": seconds, "flops": flops, "algorithmic_bytes": algorithmic_bytes, "launches": launches,
-            "shape": f"[{rows}, {hidden}] x [{inter}, {hidden}]^T"}
+            "shape": f"[{rows}, {inter}] x [{inter}, {hidden}]"}
 
 
 def measured_traffic():
@@ -196,7 +198,7 @@ def main() -> int:
         kind = label.split(".")[0]
         breakdown[kind] = breakdown.get(kind, 0.0) + ms
     # The probe's launch inside the step: one per layer in the event-timed eager pass.
-    in_step_seconds = labelled["gemm_fwd.gate_up"] * 1e-3 / cfg.num_layers
+    in_step_seconds = labelled["gemm_dx.gate_up"] * 1e-3 / cfg.num_layers
     work = op_work(cfg, args.batch, args.seq, args.loss)
     # When the per-head norms carry the rotary embedding (one pass), its algorithmic bytes count with theirs.
     for rope, norm in (("rope_fwd", "rmsnorm_fwd"), ("rope_bwd", "rmsnorm_bwd")):
@@ -212,7 +214,7 @@ def main() -> int:
                           "frac": round(rate / (PEAK_BF16_TFLOPS if b == "mfma" else PEAK_HBM_GBS), 4)}
 
     result = {
-        "metric": "train tokens/sec, 104m fwd+bwd+AdamW B=32 T=1024",
+        "metric": f"train tokens/sec, 104m fwd+bwd+AdamW B={args.batch} T={args.seq}",
         "value": tokens * args.steps / elapsed,
         "unit": "tokens/s",
         "n_gpus": 1,

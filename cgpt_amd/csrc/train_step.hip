@@ -227,9 +227,9 @@ void collect(cgptx_model* m, std::vector<Parameter*>& out) {
 // linear_backward as two single-kernel calls so that each can be timed on its own.
 int linear_backward_split(cgptx_model* m, void* dx, void* dw, const void* dy, const void* x, const void* w,
                           std::size_t rows, std::size_t in_features, std::size_t out_features, int accumulate_input,
-                          int dt, hipStream_t stream) {
+                          int dt, hipStream_t stream, const char* dx_label = "gemm_dx") {
     auto* s = static_cast<cgptx_stream>(stream);
-    CGPTX_OP("gemm_dx", cgptx_linear_backward(dx, nullptr, nullptr, dy, x, w, rows, in_features, out_features,
+    CGPTX_OP(dx_label, cgptx_linear_backward(dx, nullptr, nullptr, dy, x, w, rows, in_features, out_features,
                                               accumulate_input, 0, 0, dt, s));
     CGPTX_OP("gemm_dw", cgptx_linear_backward(nullptr, dw, nullptr, dy, x, w, rows, in_features, out_features, 0, 0,
                                               0, dt, s));
@@ -395,11 +395,10 @@ int enqueue_forward_backward(cgptx_model* m, float loss_scale, int loss_mode, hi
         // out = x + attention_projection, then out += ffn_output (src/core/transformer_block.cu:594-595)
         CGPTX_OP("gemm_fwd", linear_forward_residual(out, a.attn_out, w.o.value, x, false, N, QW, H, dt, stream));
         if (!dual_norms) CGPTX_OP("rmsnorm_fwd", cgptx_rmsnorm_forward(a.norm_f, x, w.ffn_norm.value, N, H, eps, dt, s));
-        // Labelled on its own ("kind.part"): the launch the kernel roofline of the benchmark is quoted on.
         if (fused_swiglu()) {
-            CGPTX_OP("gemm_fwd.gate_up", cgptx_linear_swiglu_forward(a.gate_up, a.act, a.norm_f, w.gate.value, N, H, I, dt, s));
+            CGPTX_OP("gemm_fwd", cgptx_linear_swiglu_forward(a.gate_up, a.act, a.norm_f, w.gate.value, N, H, I, dt, s));
         } else {
-            CGPTX_OP("gemm_fwd.gate_up", cgptx_linear_forward(a.gate_up, a.norm_f, w.gate.value, nullptr, N, H, 2 * I, dt, s));
+            CGPTX_OP("gemm_fwd", cgptx_linear_forward(a.gate_up, a.norm_f, w.gate.value, nullptr, N, H, 2 * I, dt, s));
             CGPTX_OP("swiglu_fwd", cgptx_swiglu_forward_packed(a.act, a.gate_up, N, I, dt, s));
         }
         CGPTX_OP("gemm_fwd", linear_forward_residual(out, a.act, w.down.value, nullptr, true, N, I, H, dt, stream));
@@ -437,7 +436,10 @@ int enqueue_forward_backward(cgptx_model* m, float loss_scale, int loss_mode, hi
         const bool dual_norms = fused_block_norms(m, previous, m->d_norm_in, m->d_norm_in_f, x, current) &&
                                 is_aligned16(w.attention_norm.value) && is_aligned16(w.ffn_norm.value);
         void* d_norm_f = dual_norms ? m->d_norm_in_f : m->d_norm_in;
-        CGPTX_TRY(linear_backward_split(m, d_norm_f, w.gate.gradient, m->d_gate_up, a.norm_f, w.gate.value, N, H, 2 * I, 0, dt, stream));
+        // The input gradient of the gate/up projection is labelled on its own ("kind.part"): the launch
+        // the kernel roofline of the benchmark is quoted on.
+        CGPTX_TRY(linear_backward_split(m, d_norm_f, w.gate.gradient, m->d_gate_up, a.norm_f, w.gate.value, N, H, 2 * I, 0, dt, stream,
+                                        "gemm_dx.gate_up"));
         if (!dual_norms) {
             CGPTX_OP("rmsnorm_bwd", rmsnorm_backward_residual(previous, w.ffn_norm.gradient, m->d_norm_in, x, w.ffn_norm.value,
                                                               current, N, H, eps, dt, stream));
