@@ -39,3 +39,20 @@ inline void linear_forward(Tensor& output, const Tensor& input, const Tensor& we
                            const GemmContext&, hipStream_t stream = nullptr, const LinearOptions& = {}) {
     cgptx_detail::linear_forward_impl(output, input, weight, &bias, stream);
 }
+
+// The feed-forward's gate and up projections and its SwiGLU as one call: the sequence
+// linear_forward(gate), linear_forward(up), swiglu_forward(activated, gate, up) of the reference's
+// src/core/transformer_block.cu:586-590 over the concatenated layouts of include/ops/swiglu.h:33-37
+// (weight = [gate_proj; up_proj], gate_up = [gate | up]); no single reference function corresponds.
+inline void linear_swiglu_forward(Tensor& gate_up, Tensor& activated, const Tensor& input, const Tensor& weight,
+                                  const GemmContext&, hipStream_t stream = nullptr) {
+    const char* op = "linear_swiglu_forward";
+    cgptx_detail::require_device(op, {&gate_up, &activated, &input, &weight});
+    cgptx_detail::require_same_dtype(op, input, {&gate_up, &activated, &weight});
+    if (weight.dim() != 2 || weight.size(0) % 2 != 0 || input.numel() == 0 || input.dim() == 0 || input.shape().back() != weight.size(1) ||
+        gate_up.numel() != input.numel() / weight.size(1) * weight.size(0) || activated.numel() * 2 != gate_up.numel())
+        throw std::invalid_argument("linear_swiglu_forward: incompatible tensors");
+    cgptx_detail::check(cgptx_linear_swiglu_forward(gate_up.raw_data(), activated.raw_data(), input.raw_data(), weight.raw_data(),
+                                                    input.numel() / weight.size(1), weight.size(1), weight.size(0) / 2,
+                                                    cgptx_detail::dtype_code(input.dtype()), stream));
+}

@@ -247,6 +247,17 @@ void rmsnorm_and_swiglu() {
     for (int i = 0; i < 4; ++i) want[i] = g[i] / (1.0f + std::exp(-g[i])) * u[i];
     expect(close(host_f32(out), want, 1e-6f), "swiglu_forward");
     expect(close(host_f32(out_packed), want, 1e-6f), "swiglu_forward concatenated input");
+    // Gate and up projections plus SwiGLU as one call: x [2, 2], weight [gate_proj; up_proj] chosen so
+    // that the projection reproduces `packed` above (x = identity).
+    GemmContext context;
+    Tensor eye = device_f32({2, 2}, {1, 0, 0, 1});
+    Tensor gate_up_proj = device_f32({4, 2}, {0.5f, 2, -1, 0, 1, -3, 2, 4});  // rows: gate 0, gate 1, up 0, up 1
+    Tensor gate_up = Tensor::zeros({2, 4}), activated = Tensor::zeros({2, 2});
+    linear_swiglu_forward(gate_up, activated, eye, gate_up_proj, context);
+    expect(close(host_f32(gate_up), {0.5f, -1, 1, 2, 2, 0, -3, 4}, 0), "linear_swiglu_forward gate_up");
+    expect(close(host_f32(activated), want, 1e-6f), "linear_swiglu_forward activated");
+    expect(throws<std::invalid_argument>([&] { linear_swiglu_forward(gate_up, out, eye, eye, context); }),
+           "linear_swiglu_forward mismatched tensors -> invalid_argument");
     Tensor go = device_f32({2, 2}, {1, -1, 0.5f, 2});
     Tensor gg = Tensor::zeros({2, 2}), gu = Tensor::zeros({2, 2}), gp = Tensor::zeros({2, 4});
     swiglu_backward(gg, gu, go, gate, up);
