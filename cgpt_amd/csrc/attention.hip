@@ -28,9 +28,13 @@
 //             accumulators: no atomics, results independent of scheduling.
 //             S = Q·Kᵀ, dP = dO·Vᵀ, dVᵀ += dOᵀ·P, dKᵀ += Qᵀ·dS.
 // Causal tiles above the diagonal are skipped; ragged sequence ends are masked.
+// Two families implement this scheme: the register-staged kernels (templated on the padded head
+// dimension 32 / 64 / 128) and, further down, the LDS-direct kernels (padded width 128), which
+// serve every call whose operands fit 32-bit offsets.
 #include "common.hpp"
 
 #include <cmath>
+#include <cstdlib>
 #include <limits>
 
 namespace cgptx {
@@ -583,7 +587,7 @@ __global__ __launch_bounds__(kThreads) void attention_dkv_kernel(Params p) {
 }
 
 // ============================================================================================
-// Head dimensions 65..128 (padded width 128): the streamed tiles go from global memory straight
+// Head dimensions up to 128 (padded width 128): the streamed tiles go from global memory straight
 // into LDS with buffer_load ... lds — no staging registers, no LDS stores, no address arithmetic in
 // the loop (one loop-invariant per-lane offset, the tile position is a scalar offset), rows past
 // the end of the sequence and columns past head_dim zero-filled by the buffer's range check. Two
@@ -864,7 +868,7 @@ __global__ __launch_bounds__(kThreads, 2) void attention_forward_wide_kernel(Par
         p.lse_out[(static_cast<long>(b) * p.qs + q_row) * p.hq + h] = (mb + log2f(l)) * kLn2;
 }
 
-// dQ for head dimensions 65..128: the forward kernel's streaming scheme; per 32-key half tile
+// dQ, LDS-direct family: the forward kernel's streaming scheme; per 32-key half tile
 // Sᵀ = K·Qᵀ and dPᵀ = V·dOᵀ (two independent MFMA chains), dS = P∘(dP − delta) in registers,
 // dQᵀ += Kᵀ·dSᵀ with K read back transposed. lse2 holds LSE·log2(e).
 template <typename T>
@@ -1000,7 +1004,7 @@ __global__ __launch_bounds__(kThreads, 2) void attention_dq_wide_kernel(Params p
     }
 }
 
-// dK/dV for head dimensions 65..128. A block owns 128 keys of one (batch, kv-head) — 32 per
+// dK/dV, LDS-direct family. A block owns 128 keys of one (batch, kv-head) — 32 per
 // wavefront, K and V fragments and the two accumulator tiles in registers — and streams the 64-query
 // Q/dO tiles (plus their LSE·log2 e and delta values) of every q-head of the group through two LDS
 // stages with LDS-direct loads. Registers allow one wavefront per SIMD here; the tile is handled
@@ -1257,14 +1261,20 @@ Params make_params(const Shape& s) {
     return p;
 }
 
-// The LDS-direct kernels cover head dimensions 65..128 and address K/V (and Q/dO) of one batch
-// element with 32-bit byte offsets.
+// The LDS-direct kernels take every supported head dimension (anything below 128 is padded with
+// zeros in LDS and registers: even at 32, with three quarters of their MFMA work on zeros, they
+// beat the register-staged kernels: forward 150 vs 163 us and backward 569 vs 665 us at B=32,
+// T=1024, 16:4 heads; at 64, 12:4 heads, 113 vs 162 and 420 vs 878 us). They address K/V (and Q/dO)
+// of one batch element with 32-bit byte offsets; what exceeds that, and CGPTX_ATTENTION_WIDE=0 (for
+// comparisons and tests), runs on the register-staged kernels.
 // Bytes reserved for one float per (batch, query, head), rounded so that blocks stay 256-byte aligned.
 std::size_t stat_block_bytes(std::size_t rows) { return (rows * sizeof(float) + 255) & ~std::size_t{255}; }
 
 bool wide_path(const Shape& s) {
     constexpr std::size_t limit = std::size_t{1} << 30;
-    return s.d > 64 && s.ks * s.hkv * s.d * 2 < limit && s.qs * s.hq * s.d * 2 < limit;
+    const char* text = std::getenv("CGPTX_ATTENTION_WIDE");  // read per call
+    const bool enabled = text == nullptr || text[0] != '0';
+    return enabled && s.ks * s.hkv * s.d * 2 < limit && s.qs * s.hq * s.d * 2 < limit;
 }
 
 template <typename Fn>

@@ -104,9 +104,20 @@ def make_inputs(c, dtype, seed):
     return q, k, v, do
 
 
+@pytest.fixture(params=["lds-direct", "register-staged"])
+def kernel_family(request, monkeypatch):
+    """Both kernel families take every case: the LDS-direct kernels are the default, the register-staged
+    ones serve inputs beyond 32-bit offsets and CGPTX_ATTENTION_WIDE=0 (read per call)."""
+    if request.param == "register-staged":
+        monkeypatch.setenv("CGPTX_ATTENTION_WIDE", "0")
+    else:
+        monkeypatch.delenv("CGPTX_ATTENTION_WIDE", raising=False)
+    return request.param
+
+
 @pytest.mark.parametrize("dtype", HALF, ids=HALF_IDS)
 @pytest.mark.parametrize("case", range(len(CASES)))
-def test_forward_parity(device, case, dtype):
+def test_forward_parity(device, case, dtype, kernel_family):
     c = CASES[case]
     q, k, v, _ = make_inputs(c, dtype, 10 * case)
     out, lse = run_forward(device, q, k, v, c)
@@ -122,7 +133,7 @@ def test_forward_parity(device, case, dtype):
 @pytest.mark.parametrize("dtype", HALF, ids=HALF_IDS)
 @pytest.mark.parametrize("case", range(len(CASES)))
 @pytest.mark.parametrize("with_lse", [True, False])
-def test_backward_parity(device, case, dtype, with_lse):
+def test_backward_parity(device, case, dtype, with_lse, kernel_family):
     c = CASES[case]
     q, k, v, do = make_inputs(c, dtype, 10 * case)
     want = oracle64.attention_backward(to_np(do), to_np(q), to_np(k), to_np(v), *oracle_args(c))
