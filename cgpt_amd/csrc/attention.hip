@@ -587,21 +587,24 @@ __global__ __launch_bounds__(kThreads) void attention_dkv_kernel(Params p) {
 }
 
 // ============================================================================================
-// Head dimensions up to 128 (padded width 128): the streamed tiles go from global memory straight
-// into LDS with buffer_load ... lds — no staging registers, no LDS stores, no address arithmetic in
-// the loop (one loop-invariant per-lane offset, the tile position is a scalar offset), rows past
-// the end of the sequence and columns past head_dim zero-filled by the buffer's range check. Two
-// LDS stages, one barrier per tile, two blocks per CU so that one block's softmax runs under the
-// other's MFMAs.
+// LDS-direct family (padded width W = 128, or 64 for head dimensions up to 64): the streamed tiles
+// go from global memory straight into LDS with buffer_load ... lds — no staging registers, no LDS
+// stores, no address arithmetic in the loop (one loop-invariant per-lane offset, the tile position
+// is a scalar offset), rows past the end of the sequence and columns past head_dim zero-filled by
+// the buffer's range check. Two LDS stages, one barrier per tile, at least two blocks per CU so
+// that one block's softmax runs under the other's MFMAs.
 //
-// A wavefront-wide LDS-direct load writes 64 x 16 B contiguously, so LDS rows are exactly 256 B
+// A wavefront-wide LDS-direct load writes 64 x 16 B contiguously, so LDS rows are exactly 2 W bytes
 // and cannot be padded. Instead the 16-byte chunk c of tile row r is kept at chunk position
-// c ^ swizzle(r), swizzle(r) = (r%4)*4 + (r/4)%4: the 16 rows a ds_read_b128 fragment read touches
-// hit 16 different chunk positions, and the 4 rows x 64 B a ds_read_b64_tr_b16 touches hit four
-// different 64-byte windows — both conflict-free. The lane that owns LDS slot (r, c') simply fetches
-// global chunk c' ^ swizzle(r).
-constexpr int kWideDim = 128;
-constexpr int kWideTile = kStream * kWideDim;  // elements of one 64 x 128 tile (16 KiB)
+// c ^ swizzle(r). W = 128 (256-byte rows, 16 chunks): swizzle(r) = (r%4)*4 + (r/4)%4 — the 16 rows a
+// ds_read_b128 fragment read touches hit 16 different chunk positions, and the 4 rows x 64 B a
+// ds_read_b64_tr_b16 touches hit four different 64-byte windows. W = 64 (128-byte rows, 8 chunks,
+// two rows per 256-byte bank period): swizzle(r) = ((r/2)%2)*4 + (r/4)%4 — rows of equal parity among
+// 16 consecutive ones get 8 different chunk positions, and of the 4 rows of a transposed read the
+// two of equal parity get different 64-byte halves. Both conflict-free. The lane that owns LDS slot
+// (r, c') simply fetches global chunk c' ^ swizzle(r).
+template <int W>
+constexpr int kWideTile = kStream * W;  // elements of one 64 x W tile
 
 constexpr int kSchedMfma = 0x008, kSchedDsRead = 0x100;
 template <int CLASS, int COUNT>
@@ -624,12 +627,18 @@ __device__ __forceinline__ void sched_reads_under_mfmas() {
     }
 }
 
-__device__ __forceinline__ int swizzle(int row) { return ((row & 3) << 2) | ((row >> 2) & 3); }
+template <int W>
+__device__ __forceinline__ int swizzle(int row) {
+    static_assert(W == 64 || W == 128, "padded widths of the LDS-direct kernels");
+    if constexpr (W == 128) return ((row & 3) << 2) | ((row >> 2) & 3);
+    else return (((row >> 1) & 1) << 2) | ((row >> 2) & 3);
+}
 
 using lds_void_ptr = __attribute__((address_space(3))) void*;
 
-// Where a lane's 16 bytes of a streamed tile come from: rows r0 + 16 i (i = 0..3) of the tile go
-// through the four loads of wavefront w, lane l owning LDS slot (row 4w + l/16, chunk l%16).
+// Where a lane's 16 bytes of a streamed tile come from. One load instruction fills 1 KiB = R rows
+// (R = 4 for W = 128, 8 for W = 64); load i of wavefront w covers tile rows 4 R i + R w .. + R - 1,
+// lane l owning LDS slot (row R w + l / chunks per row, chunk l % chunks per row).
 struct TileSource {
     __amdgpu_buffer_rsrc_t rsrc;
     int voffset;    // bytes, loop-invariant
@@ -638,41 +647,45 @@ struct TileSource {
 
 // last_row: elements of the last row that belong to the buffer (head_dim when base points at one
 // head, the whole row when the head is chosen by the scalar offset of each load).
-template <typename T>
+template <typename T, int W>
 __device__ __forceinline__ TileSource make_source(const T* base, long row_stride, int rows, int d, int wave,
                                                   long last_row) {
+    constexpr int kChunks = W / 8, kRowsPerLoad = 64 / kChunks;
     const int lane = threadIdx.x & 63;
     TileSource s;
     s.row_bytes = static_cast<int>(row_stride * sizeof(T));
     const int bytes = static_cast<int>(((rows - 1) * row_stride + last_row) * sizeof(T));
     s.rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(base), 0, bytes, 0x00020000);
-    const int r = wave * 4 + (lane >> 4);
-    const int chunk = (lane & 15) ^ swizzle(r);
+    const int r = wave * kRowsPerLoad + lane / kChunks;
+    const int chunk = (lane % kChunks) ^ swizzle<W>(r);
     // Chunks beyond head_dim get an offset past every valid byte: the load then returns zeros.
     s.voffset = chunk * 8 < d ? r * s.row_bytes + chunk * 16 : (1 << 30);
     return s;
 }
 
-template <typename T>
+template <typename T, int W>
 __device__ __forceinline__ void stream_tile(const TileSource& s, int row0, T* tile, int wave) {
+    constexpr int kRowsPerLoad = 64 / (W / 8), kLoads = kStream / (4 * kRowsPerLoad);
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(s.rsrc, (lds_void_ptr)(tile + (i * 16 + wave * 4) * kWideDim), 16,
-                                                 s.voffset, (row0 + i * 16) * s.row_bytes, 0, 0);
+    for (int i = 0; i < kLoads; ++i)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(s.rsrc, (lds_void_ptr)(tile + (i * 4 + wave) * kRowsPerLoad * W), 16,
+                                                 s.voffset, (row0 + i * 4 * kRowsPerLoad) * s.row_bytes, 0, 0);
 }
 
 // Element offset (within a 32-row block of a swizzled tile) of the lane's ds_read_b128 fragment:
 // row lane%32, head-dim elements 16*step + 8*(lane/32) .. +7.
+template <int W>
 __device__ __forceinline__ int wide_direct_offset(int lane, int step) {
     const int row = lane & 31;
-    return row * kWideDim + (((2 * step + (lane >> 5)) ^ swizzle(row)) * 8);
+    return row * W + (((2 * step + (lane >> 5)) ^ swizzle<W>(row)) * 8);
 }
 // Element offset (within a 16-row block) of the lane's ds_read_b64_tr_b16 address for head-dim
 // columns 32t .. 32t+31: rows {0-3 | 4-7} (+8 for the second read), see transposed_frag.
+template <int W>
 __device__ __forceinline__ int wide_transposed_offset(int lane, int t, int second) {
     const int row = (lane >> 5) * 4 + ((lane & 15) >> 2) + second * 8;
     const int chunk = t * 4 + ((lane >> 4) & 1) * 2 + ((lane & 3) >> 1);
-    return row * kWideDim + ((chunk ^ swizzle(row)) * 8) + (lane & 1) * 4;
+    return row * W + ((chunk ^ swizzle<W>(row)) * 8) + (lane & 1) * 4;
 }
 template <typename T>
 __device__ __forceinline__ typename Mma<T>::frag wide_transposed_frag(const T* block, int first, int second) {
@@ -703,11 +716,11 @@ __device__ __forceinline__ float other_half(float v) {
     return __uint_as_float((threadIdx.x & 32) ? r[0] : r[1]);
 }
 
-template <typename T>
+template <typename T, int W>
 __global__ __launch_bounds__(kThreads, 2) void attention_forward_wide_kernel(Params p) {
     using frag = typename Mma<T>::frag;
-    constexpr int STEPS = kWideDim / 16, DT = kWideDim / 32;
-    __shared__ __align__(1024) T lds[4 * kWideTile];  // [stage][K | V]
+    constexpr int STEPS = W / 16, DT = W / 32;
+    __shared__ __align__(1024) T lds[4 * kWideTile<W>];  // [stage][K | V]
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const BlockCoordinates where = block_coordinates();
@@ -718,15 +731,15 @@ __global__ __launch_bounds__(kThreads, 2) void attention_forward_wide_kernel(Par
     const long q_stride = static_cast<long>(p.hq) * p.d, kv_stride = static_cast<long>(p.hkv) * p.d;
     const T* q_ptr = static_cast<const T*>(p.q) + (static_cast<long>(b) * p.qs + q_row) * q_stride + h * p.d;
     const long kv_offset = static_cast<long>(b) * p.ks * kv_stride + kvh * p.d;
-    const TileSource k_src = make_source(static_cast<const T*>(p.k) + kv_offset, kv_stride, p.ks, p.d, wave, p.d);
-    const TileSource v_src = make_source(static_cast<const T*>(p.v) + kv_offset, kv_stride, p.ks, p.d, wave, p.d);
+    const TileSource k_src = make_source<T, W>(static_cast<const T*>(p.k) + kv_offset, kv_stride, p.ks, p.d, wave, p.d);
+    const TileSource v_src = make_source<T, W>(static_cast<const T*>(p.v) + kv_offset, kv_stride, p.ks, p.d, wave, p.d);
 
     const int last_q_block = min(q_block + kBlockRows, p.qs) - 1;
     const int k_end = p.causal ? min(p.ks, p.offset + last_q_block + 1) : p.ks;
     const int tiles = (k_end + kStream - 1) / kStream;
     if (tiles > 0) {
-        stream_tile(k_src, 0, lds, wave);
-        stream_tile(v_src, 0, lds + kWideTile, wave);
+        stream_tile<T, W>(k_src, 0, lds, wave);
+        stream_tile<T, W>(v_src, 0, lds + kWideTile<W>, wave);
     }
 
     frag qf[STEPS];
@@ -734,11 +747,11 @@ __global__ __launch_bounds__(kThreads, 2) void attention_forward_wide_kernel(Par
     for (int s = 0; s < STEPS; ++s) qf[s] = global_frag<T>(q_ptr, q_live, s, p.d);
     int k_off[STEPS], v_off[DT][2];
 #pragma unroll
-    for (int s = 0; s < STEPS; ++s) k_off[s] = wide_direct_offset(lane, s);
+    for (int s = 0; s < STEPS; ++s) k_off[s] = wide_direct_offset<W>(lane, s);
 #pragma unroll
     for (int t = 0; t < DT; ++t) {
-        v_off[t][0] = wide_transposed_offset(lane, t, 0);
-        v_off[t][1] = wide_transposed_offset(lane, t, 1);
+        v_off[t][0] = wide_transposed_offset<W>(lane, t, 0);
+        v_off[t][1] = wide_transposed_offset<W>(lane, t, 1);
     }
 
     acc_t o[DT];
@@ -757,14 +770,14 @@ __global__ __launch_bounds__(kThreads, 2) void attention_forward_wide_kernel(Par
 
     for (int j = 0; j < tiles; ++j) {
         const int k0 = j * kStream;
-        const T* k_tile = lds + (j & 1) * 2 * kWideTile;
-        const T* v_tile = k_tile + kWideTile;
+        const T* k_tile = lds + (j & 1) * 2 * kWideTile<W>;
+        const T* v_tile = k_tile + kWideTile<W>;
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wavefront's part of tile j is in LDS
         __syncthreads();                     // ... and everybody else's; stage (j+1)%2 is free
         if (j + 1 < tiles) {
-            T* next = lds + ((j + 1) & 1) * 2 * kWideTile;
-            stream_tile(k_src, k0 + kStream, next, wave);
-            stream_tile(v_src, k0 + kStream, next + kWideTile, wave);
+            T* next = lds + ((j + 1) & 1) * 2 * kWideTile<W>;
+            stream_tile<T, W>(k_src, k0 + kStream, next, wave);
+            stream_tile<T, W>(v_src, k0 + kStream, next + kWideTile<W>, wave);
         }
         if (!wave_live || (p.causal && k0 > p.offset + wave_last_q)) continue;
 
@@ -774,7 +787,7 @@ __global__ __launch_bounds__(kThreads, 2) void attention_forward_wide_kernel(Par
 #pragma unroll
             for (int s = 0; s < STEPS; ++s) {
                 ka[0][s] = *reinterpret_cast<const frag*>(k_tile + k_off[s]);
-                ka[1][s] = *reinterpret_cast<const frag*>(k_tile + 32 * kWideDim + k_off[s]);
+                ka[1][s] = *reinterpret_cast<const frag*>(k_tile + 32 * W + k_off[s]);
             }
 #pragma unroll
             for (int s = 0; s < STEPS; ++s) {
@@ -834,7 +847,7 @@ __global__ __launch_bounds__(kThreads, 2) void attention_forward_wide_kernel(Par
 #pragma unroll
                 for (int s = 0; s < 2; ++s) {
                     pf[sub][s] = acc_frag<T>(st[sub], s);
-                    const T* block = v_tile + (sub * 32 + s * 16) * kWideDim;
+                    const T* block = v_tile + (sub * 32 + s * 16) * W;
 #pragma unroll
                     for (int t = 0; t < DT; ++t) vt[sub][s][t] = wide_transposed_frag<T>(block, v_off[t][0], v_off[t][1]);
                 }
@@ -871,11 +884,11 @@ __global__ __launch_bounds__(kThreads, 2) void attention_forward_wide_kernel(Par
 // dQ, LDS-direct family: the forward kernel's streaming scheme; per 32-key half tile
 // Sᵀ = K·Qᵀ and dPᵀ = V·dOᵀ (two independent MFMA chains), dS = P∘(dP − delta) in registers,
 // dQᵀ += Kᵀ·dSᵀ with K read back transposed. lse2 holds LSE·log2(e).
-template <typename T>
+template <typename T, int W>
 __global__ __launch_bounds__(kThreads, 2) void attention_dq_wide_kernel(Params p) {
     using frag = typename Mma<T>::frag;
-    constexpr int STEPS = kWideDim / 16, DT = kWideDim / 32;
-    __shared__ __align__(1024) T lds[4 * kWideTile];  // [stage][K | V]
+    constexpr int STEPS = W / 16, DT = W / 32;
+    __shared__ __align__(1024) T lds[4 * kWideTile<W>];  // [stage][K | V]
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const BlockCoordinates where = block_coordinates();
@@ -886,15 +899,15 @@ __global__ __launch_bounds__(kThreads, 2) void attention_dq_wide_kernel(Params p
     const long q_stride = static_cast<long>(p.hq) * p.d, kv_stride = static_cast<long>(p.hkv) * p.d;
     const long q_offset = (static_cast<long>(b) * p.qs + q_row) * q_stride + h * p.d;
     const long kv_offset = static_cast<long>(b) * p.ks * kv_stride + kvh * p.d;
-    const TileSource k_src = make_source(static_cast<const T*>(p.k) + kv_offset, kv_stride, p.ks, p.d, wave, p.d);
-    const TileSource v_src = make_source(static_cast<const T*>(p.v) + kv_offset, kv_stride, p.ks, p.d, wave, p.d);
+    const TileSource k_src = make_source<T, W>(static_cast<const T*>(p.k) + kv_offset, kv_stride, p.ks, p.d, wave, p.d);
+    const TileSource v_src = make_source<T, W>(static_cast<const T*>(p.v) + kv_offset, kv_stride, p.ks, p.d, wave, p.d);
 
     const int last_q_block = min(q_block + kBlockRows, p.qs) - 1;
     const int k_end = p.causal ? min(p.ks, p.offset + last_q_block + 1) : p.ks;
     const int tiles = (k_end + kStream - 1) / kStream;
     if (tiles > 0) {
-        stream_tile(k_src, 0, lds, wave);
-        stream_tile(v_src, 0, lds + kWideTile, wave);
+        stream_tile<T, W>(k_src, 0, lds, wave);
+        stream_tile<T, W>(v_src, 0, lds + kWideTile<W>, wave);
     }
 
     frag qf[STEPS], dof[STEPS];
@@ -908,11 +921,11 @@ __global__ __launch_bounds__(kThreads, 2) void attention_dq_wide_kernel(Params p
     const float delta = q_live ? p.delta[stat_index] : 0.0f;
     int k_off[STEPS], kt_off[DT][2];
 #pragma unroll
-    for (int s = 0; s < STEPS; ++s) k_off[s] = wide_direct_offset(lane, s);
+    for (int s = 0; s < STEPS; ++s) k_off[s] = wide_direct_offset<W>(lane, s);
 #pragma unroll
     for (int t = 0; t < DT; ++t) {
-        kt_off[t][0] = wide_transposed_offset(lane, t, 0);
-        kt_off[t][1] = wide_transposed_offset(lane, t, 1);
+        kt_off[t][0] = wide_transposed_offset<W>(lane, t, 0);
+        kt_off[t][1] = wide_transposed_offset<W>(lane, t, 1);
     }
 
     acc_t dq[DT];
@@ -927,14 +940,14 @@ __global__ __launch_bounds__(kThreads, 2) void attention_dq_wide_kernel(Params p
 
     for (int j = 0; j < tiles; ++j) {
         const int k0 = j * kStream;
-        const T* k_tile = lds + (j & 1) * 2 * kWideTile;
-        const T* v_tile = k_tile + kWideTile;
+        const T* k_tile = lds + (j & 1) * 2 * kWideTile<W>;
+        const T* v_tile = k_tile + kWideTile<W>;
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
         __syncthreads();
         if (j + 1 < tiles) {
-            T* next = lds + ((j + 1) & 1) * 2 * kWideTile;
-            stream_tile(k_src, k0 + kStream, next, wave);
-            stream_tile(v_src, k0 + kStream, next + kWideTile, wave);
+            T* next = lds + ((j + 1) & 1) * 2 * kWideTile<W>;
+            stream_tile<T, W>(k_src, k0 + kStream, next, wave);
+            stream_tile<T, W>(v_src, k0 + kStream, next + kWideTile<W>, wave);
         }
         if (!wave_live || (p.causal && k0 > p.offset + wave_last_q)) continue;
         const bool masked = k0 + kStream - 1 > clear_limit;
@@ -946,8 +959,8 @@ __global__ __launch_bounds__(kThreads, 2) void attention_dq_wide_kernel(Params p
                 frag ka[STEPS], va[STEPS];
 #pragma unroll
                 for (int s = 0; s < STEPS; ++s) {
-                    ka[s] = *reinterpret_cast<const frag*>(k_tile + sub * 32 * kWideDim + k_off[s]);
-                    va[s] = *reinterpret_cast<const frag*>(v_tile + sub * 32 * kWideDim + k_off[s]);
+                    ka[s] = *reinterpret_cast<const frag*>(k_tile + sub * 32 * W + k_off[s]);
+                    va[s] = *reinterpret_cast<const frag*>(v_tile + sub * 32 * W + k_off[s]);
                 }
 #pragma unroll
                 for (int s = 0; s < STEPS; ++s) {
@@ -974,7 +987,7 @@ __global__ __launch_bounds__(kThreads, 2) void attention_dq_wide_kernel(Params p
 #pragma unroll
                 for (int s = 0; s < 2; ++s) {
                     dsf[s] = acc_frag<T>(st, s);
-                    const T* block = k_tile + (sub * 32 + s * 16) * kWideDim;
+                    const T* block = k_tile + (sub * 32 + s * 16) * W;
 #pragma unroll
                     for (int t = 0; t < DT; ++t) kt[s][t] = wide_transposed_frag<T>(block, kt_off[t][0], kt_off[t][1]);
                 }
@@ -1017,15 +1030,16 @@ __global__ __launch_bounds__(kThreads, 2) void attention_dq_wide_kernel(Params p
 // 256 CUs exactly at the training shape.
 // Queries past the end of the sequence need no masking: their dO rows and delta arrive as zeros
 // (buffer range check), so P·dO and P∘(dP−delta) vanish whatever P is.
-constexpr int kWideDkvSmem = 4 * kWideTile * 2 + 4 * kStream * static_cast<int>(sizeof(float));
+template <int W>
+constexpr int kWideDkvSmem = 4 * kWideTile<W> * 2 + 4 * kStream * static_cast<int>(sizeof(float));
 
-template <typename T>
+template <typename T, int W>
 __global__ __launch_bounds__(kThreads, 1) void attention_dkv_wide_kernel(Params p) {
     using frag = typename Mma<T>::frag;
-    constexpr int STEPS = kWideDim / 16, DT = kWideDim / 32;
+    constexpr int STEPS = W / 16, DT = W / 32;
     extern __shared__ __align__(1024) unsigned char wide_smem[];
     T* lds = reinterpret_cast<T*>(wide_smem);                             // [stage][Q | dO]
-    float* stats = reinterpret_cast<float*>(wide_smem + 4 * kWideTile * sizeof(T));  // [stage][lse2 | delta][64]
+    float* stats = reinterpret_cast<float*>(wide_smem + 4 * kWideTile<W> * sizeof(T));  // [stage][lse2 | delta][64]
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int b = blockIdx.z, kvh = blockIdx.y, group = p.hq / p.hkv;
@@ -1035,8 +1049,8 @@ __global__ __launch_bounds__(kThreads, 1) void attention_dkv_wide_kernel(Params 
     // Sources: Q and dO of this batch element (the head is part of the scalar offset), and the two
     // per-(query, head) statistics, one float per lane.
     const long q_batch = static_cast<long>(b) * p.qs * q_stride;
-    const TileSource q_src = make_source(static_cast<const T*>(p.q) + q_batch, q_stride, p.qs, p.d, wave, q_stride);
-    const TileSource do_src = make_source(static_cast<const T*>(p.dout) + q_batch, q_stride, p.qs, p.d, wave, q_stride);
+    const TileSource q_src = make_source<T, W>(static_cast<const T*>(p.q) + q_batch, q_stride, p.qs, p.d, wave, q_stride);
+    const TileSource do_src = make_source<T, W>(static_cast<const T*>(p.dout) + q_batch, q_stride, p.qs, p.d, wave, q_stride);
     const int stat_bytes = p.qs * p.hq * static_cast<int>(sizeof(float));
     const float* stat_base = (wave == 0 ? p.lse : p.delta) + static_cast<long>(b) * p.qs * p.hq;
     const __amdgpu_buffer_rsrc_t stat_rsrc =
@@ -1045,11 +1059,11 @@ __global__ __launch_bounds__(kThreads, 1) void attention_dkv_wide_kernel(Params 
 
     int q_off[STEPS], t_off[DT][2];
 #pragma unroll
-    for (int s = 0; s < STEPS; ++s) q_off[s] = wide_direct_offset(lane, s);
+    for (int s = 0; s < STEPS; ++s) q_off[s] = wide_direct_offset<W>(lane, s);
 #pragma unroll
     for (int t = 0; t < DT; ++t) {
-        t_off[t][0] = wide_transposed_offset(lane, t, 0);
-        t_off[t][1] = wide_transposed_offset(lane, t, 1);
+        t_off[t][0] = wide_transposed_offset<W>(lane, t, 0);
+        t_off[t][1] = wide_transposed_offset<W>(lane, t, 1);
     }
 
     const int key_blocks = (p.ks + kBlockRows - 1) / kBlockRows;
@@ -1083,16 +1097,16 @@ __global__ __launch_bounds__(kThreads, 1) void attention_dkv_wide_kernel(Params 
         auto issue = [&](int tile) {
             const int h = kvh * group + tile / tiles_per_head;
             const int q0 = q_begin + (tile % tiles_per_head) * kStream;
-            T* stage = lds + (tile & 1) * 2 * kWideTile;
+            T* stage = lds + (tile & 1) * 2 * kWideTile<W>;
             const int head_bytes = h * p.d * static_cast<int>(sizeof(T));
+            constexpr int kRowsPerLoad = 64 / (W / 8), kLoads = kStream / (4 * kRowsPerLoad);
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int soffset = (q0 + i * 16) * q_src.row_bytes + head_bytes;
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(q_src.rsrc, (lds_void_ptr)(stage + (i * 16 + wave * 4) * kWideDim),
-                                                         16, q_src.voffset, soffset, 0, 0);
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(
-                    do_src.rsrc, (lds_void_ptr)(stage + kWideTile + (i * 16 + wave * 4) * kWideDim), 16, do_src.voffset,
-                    soffset, 0, 0);
+            for (int i = 0; i < kLoads; ++i) {
+                const int soffset = (q0 + i * 4 * kRowsPerLoad) * q_src.row_bytes + head_bytes;
+                T* rows = stage + (i * 4 + wave) * kRowsPerLoad * W;
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(q_src.rsrc, (lds_void_ptr)(rows), 16, q_src.voffset, soffset, 0, 0);
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(do_src.rsrc, (lds_void_ptr)(rows + kWideTile<W>), 16, do_src.voffset,
+                                                         soffset, 0, 0);
             }
             if (wave < 2)
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(
@@ -1109,8 +1123,8 @@ __global__ __launch_bounds__(kThreads, 1) void attention_dkv_wide_kernel(Params 
                 frag qa[STEPS], da[STEPS];
 #pragma unroll
                 for (int s = 0; s < STEPS; ++s) {
-                    qa[s] = *reinterpret_cast<const frag*>(q_tile + sub * 32 * kWideDim + q_off[s]);
-                    da[s] = *reinterpret_cast<const frag*>(do_tile + sub * 32 * kWideDim + q_off[s]);
+                    qa[s] = *reinterpret_cast<const frag*>(q_tile + sub * 32 * W + q_off[s]);
+                    da[s] = *reinterpret_cast<const frag*>(do_tile + sub * 32 * W + q_off[s]);
                 }
 #pragma unroll
                 for (int s = 0; s < STEPS; ++s) {
@@ -1147,7 +1161,7 @@ __global__ __launch_bounds__(kThreads, 1) void attention_dkv_wide_kernel(Params 
                 frag dot[2][DT], qt[2][DT];
 #pragma unroll
                 for (int s = 0; s < 2; ++s) {
-                    const int block = (sub * 32 + s * 16) * kWideDim;
+                    const int block = (sub * 32 + s * 16) * W;
 #pragma unroll
                     for (int t = 0; t < DT; ++t) {
                         dot[s][t] = wide_transposed_frag<T>(do_tile + block, t_off[t][0], t_off[t][1]);
@@ -1178,7 +1192,7 @@ __global__ __launch_bounds__(kThreads, 1) void attention_dkv_wide_kernel(Params 
         if (total_tiles > 0) issue(0);
         for (int tile = 0; tile < total_tiles; ++tile) {
             const int q0 = q_begin + (tile % tiles_per_head) * kStream;
-            const T* q_tile = lds + (tile & 1) * 2 * kWideTile;
+            const T* q_tile = lds + (tile & 1) * 2 * kWideTile<W>;
             const float* stat = stats + (tile & 1) * 2 * kStream;
             __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wavefront's part of the tile is in LDS
             __syncthreads();                     // ... and everybody else's; the other stage is free
@@ -1190,7 +1204,7 @@ __global__ __launch_bounds__(kThreads, 1) void attention_dkv_wide_kernel(Params 
             const bool masked = (p.causal && wave_last_key > p.offset + q0) || wave_last_key >= p.ks;
             const int causal_first = p.causal ? k_row - p.offset - q0 - 4 * (lane >> 5) : -(1 << 30);
             const int first = k_live ? causal_first : (1 << 30);
-            tile_body(q_tile, q_tile + kWideTile, stat, masked, first);
+            tile_body(q_tile, q_tile + kWideTile<W>, stat, masked, first);
         }
         __syncthreads();  // the next key block's first loads overwrite stage 0
         if (k_live) {
@@ -1261,12 +1275,11 @@ Params make_params(const Shape& s) {
     return p;
 }
 
-// The LDS-direct kernels take every supported head dimension (anything below 128 is padded with
-// zeros in LDS and registers: even at 32, with three quarters of their MFMA work on zeros, they
-// beat the register-staged kernels: forward 150 vs 163 us and backward 569 vs 665 us at B=32,
-// T=1024, 16:4 heads; at 64, 12:4 heads, 113 vs 162 and 420 vs 878 us). They address K/V (and Q/dO)
-// of one batch element with 32-bit byte offsets; what exceeds that, and CGPTX_ATTENTION_WIDE=0 (for
-// comparisons and tests), runs on the register-staged kernels.
+// The LDS-direct kernels take every supported head dimension (padded to 64 or 128 with zeros in LDS
+// and registers; at B=32, T=1024: head_dim 64, 12:4 heads, forward 86 vs 162 us and backward 279 vs
+// 878 us against the register-staged kernels; head_dim 32, 16:4 heads, 103 vs 163 and 325 vs 665 us).
+// They address K/V (and Q/dO) of one batch element with 32-bit byte offsets; what exceeds that, and
+// CGPTX_ATTENTION_WIDE=0 (for comparisons and tests), runs on the register-staged kernels.
 // Bytes reserved for one float per (batch, query, head), rounded so that blocks stay 256-byte aligned.
 std::size_t stat_block_bytes(std::size_t rows) { return (rows * sizeof(float) + 255) & ~std::size_t{255}; }
 
@@ -1294,7 +1307,8 @@ int launch_forward(const Shape& s, Params p, hipStream_t stream) {
                     static_cast<unsigned int>(s.batch));
     return dispatch_16bit(s.dtype, [&]<typename T>() -> int {
         if (wide_path(s)) {
-            hipLaunchKernelGGL((attention_forward_wide_kernel<T>), grid, dim3(kThreads), 0, stream, p);
+            if (s.d <= 64) hipLaunchKernelGGL((attention_forward_wide_kernel<T, 64>), grid, dim3(kThreads), 0, stream, p);
+            else hipLaunchKernelGGL((attention_forward_wide_kernel<T, 128>), grid, dim3(kThreads), 0, stream, p);
             CGPTX_LAUNCH_CHECK();
             return CGPTX_OK;
         }
@@ -1342,7 +1356,8 @@ int launch_backward(const Shape& s, Params p, void* dq, void* dk, void* dv, cons
                               static_cast<unsigned int>(s.hq), static_cast<unsigned int>(s.batch));
             if (wide_path(s)) {
                 pq.lse = lse2;
-                hipLaunchKernelGGL((attention_dq_wide_kernel<T>), q_grid, dim3(kThreads), 0, stream, pq);
+                if (s.d <= 64) hipLaunchKernelGGL((attention_dq_wide_kernel<T, 64>), q_grid, dim3(kThreads), 0, stream, pq);
+                else hipLaunchKernelGGL((attention_dq_wide_kernel<T, 128>), q_grid, dim3(kThreads), 0, stream, pq);
             } else {
                 hipLaunchKernelGGL((attention_dq_kernel<T, DP>), q_grid, dim3(kThreads), 0, stream, pq);
             }
@@ -1353,16 +1368,20 @@ int launch_backward(const Shape& s, Params p, void* dq, void* dk, void* dv, cons
             const unsigned int key_blocks = static_cast<unsigned int>((s.ks + kBlockRows - 1) / kBlockRows);
             if (wide_path(s)) {
                 pk.lse = lse2;
-                auto kernel = attention_dkv_wide_kernel<T>;
-                static bool configured = false;
-                if (!configured) {
-                    CGPTX_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                                  hipFuncAttributeMaxDynamicSharedMemorySize, kWideDkvSmem));
-                    configured = true;
-                }
                 const dim3 pair_grid((key_blocks + 1) / 2, static_cast<unsigned int>(s.hkv),
                                      static_cast<unsigned int>(s.batch));
-                hipLaunchKernelGGL(kernel, pair_grid, dim3(kThreads), kWideDkvSmem, stream, pk);
+                auto launch = [&]<int W>() -> int {
+                    auto kernel = attention_dkv_wide_kernel<T, W>;
+                    static bool configured = false;
+                    if (!configured) {
+                        CGPTX_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                                      hipFuncAttributeMaxDynamicSharedMemorySize, kWideDkvSmem<W>));
+                        configured = true;
+                    }
+                    hipLaunchKernelGGL(kernel, pair_grid, dim3(kThreads), kWideDkvSmem<W>, stream, pk);
+                    return CGPTX_OK;
+                };
+                if (int st = s.d <= 64 ? launch.template operator()<64>() : launch.template operator()<128>()) return st;
             } else {
                 const dim3 k_grid(key_blocks, static_cast<unsigned int>(s.hkv), static_cast<unsigned int>(s.batch));
                 hipLaunchKernelGGL((attention_dkv_kernel<T, DP>), k_grid, dim3(kThreads), 0, stream, pk);
