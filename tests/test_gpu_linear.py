@@ -174,3 +174,20 @@ def test_linear_swiglu_forward_equals_the_two_operators(device, rows, fin, hidde
     reference = gate / (1 + torch.exp(-gate)) * up
     err = (got_act.double().cpu() - reference).abs().max() / reference.abs().max()
     assert err <= 2e-2
+
+
+def test_linear_swiglu_forward_argument_errors(device):
+    x = torch.zeros(8, 32, dtype=torch.bfloat16, device=device)
+    w = torch.zeros(64, 32, dtype=torch.bfloat16, device=device)
+    gate_up = torch.zeros(8, 64, dtype=torch.bfloat16, device=device)
+    act = torch.zeros(8, 32, dtype=torch.bfloat16, device=device)
+    ops.linear_swiglu_forward(gate_up, act, x, w)  # valid
+    with pytest.raises(ValueError):
+        ops.linear_swiglu_forward(gate_up, torch.zeros(8, 16, dtype=torch.bfloat16, device=device), x, w)
+    with pytest.raises(ValueError):
+        ops.linear_swiglu_forward(gate_up, act, x, torch.zeros(63, 32, dtype=torch.bfloat16, device=device))
+    with pytest.raises(ValueError):
+        ops.linear_swiglu_forward(gate_up, act.float(), x, w)
+    from cgpt_amd import capi
+    with pytest.raises(ValueError):  # the C entry point rejects null tensors itself
+        capi.call("cgptx_linear_swiglu_forward", None, act.data_ptr(), x.data_ptr(), w.data_ptr(), 8, 32, 32, 1, None)
