@@ -117,6 +117,9 @@ struct KernelArgs {
     int accumulate;
     int c_f32;
     KernelSegments a_seg, c_seg;  // column segments of A (as stored) and of C; count 0 = one buffer
+    // ceil(2^32 / (kGroupRows * tiles_n)) when multiplying by it divides every item index of the
+    // launch exactly, else 0 (the kernel then divides).
+    unsigned int group_reciprocal;
     void* act;      // SWIGLU kernels: [M, inter] = silu(gate) * up, T*
     long ld_act;
     int inter;      // SWIGLU kernels: columns of gate (= of up); n = 2 * inter
@@ -380,16 +383,23 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
         int m0, n0, slice, kt_begin, kt_end;
     };
     auto locate = [&](int index) __attribute__((always_inline)) {
+        // Integer divisions by run-time values cost some thirty scalar instructions each, with
+        // nothing to hide them between two items: unsplit launches skip the first, the second is a
+        // multiplication by a reciprocal the host prepared, the third a shift in all but the last,
+        // ragged group of tile rows.
         Item w;
-        w.slice = index / tiles;
+        w.slice = p.slices == 1 ? 0 : index / tiles;
         const int logical = index - w.slice * tiles;
         const int group_size = kGroupRows * p.tiles_n;
-        const int group = logical / group_size;
+        const int group = p.group_reciprocal != 0u
+                              ? static_cast<int>(__umulhi(static_cast<unsigned int>(logical), p.group_reciprocal))
+                              : logical / group_size;
         const int first_m = group * kGroupRows;
         const int rows_in_group = min(p.tiles_m - first_m, kGroupRows);
         const int in_group = logical - group * group_size;
-        w.m0 = (first_m + in_group % rows_in_group) * BM;
-        w.n0 = (in_group / rows_in_group) * BN;
+        const int column = rows_in_group == kGroupRows ? in_group / kGroupRows : in_group / rows_in_group;
+        w.m0 = (first_m + in_group - column * rows_in_group) * BM;
+        w.n0 = column * BN;
         w.kt_begin = w.slice * p.k_tiles_per_slice;
         w.kt_end = min(p.k / kBK, w.kt_begin + p.k_tiles_per_slice);
         return w;
@@ -1064,6 +1074,13 @@ int launch_mfma(const KernelArgs& p, int slices, hipStream_t stream) {
     KernelArgs args = p;
     args.slices = slices;
     const long items = static_cast<long>(p.tiles_m) * p.tiles_n * slices;
+    {
+        // x * ceil(2^32 / d) >> 32 == x / d for every x with x * d < 2^32.
+        const unsigned long divisor = static_cast<unsigned long>(kGroupRows) * static_cast<unsigned long>(p.tiles_n);
+        const unsigned long tiles = static_cast<unsigned long>(p.tiles_m) * static_cast<unsigned long>(p.tiles_n);
+        const bool exact = divisor > 1 && tiles * divisor < (1ul << 32);
+        args.group_reciprocal = exact ? static_cast<unsigned int>(((1ul << 32) + divisor - 1) / divisor) : 0u;
+    }
     const long slots = static_cast<long>(compute_units()) * (BM == 256 ? 1 : 2) / kXcds * kXcds;
     const long blocks = std::min<long>((items + kXcds - 1) / kXcds * kXcds, std::max<long>(slots, kXcds));
     hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned int>(blocks)), dim3(kThreads), smem, stream, args);
