@@ -122,6 +122,8 @@ struct KernelArgs {
     unsigned int group_reciprocal;
     void* act;      // SWIGLU kernels: [M, inter] = silu(gate) * up, T*
     long ld_act;
+    const void* saved;  // GRAD kernels: the forward's [M, 2 * inter] = [gate | up], T*
+    long ld_saved;
     int inter;      // SWIGLU kernels: columns of gate (= of up); n = 2 * inter
 };
 
@@ -342,8 +344,10 @@ struct TileLayout {
 // so only the scalar offsets of the loads change), and the epilogue computes the product from the
 // rounded gate and up values, as the separate operator would from memory.
 template <typename T, int BM, int BN, bool A_K, bool B_K, bool SPLIT, bool SEGMENTED, bool RESIDUAL = false,
-          bool SWIGLU = false>
+          bool SWIGLU = false, bool GRAD = false>
 __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
+    static_assert(!GRAD || (A_K && !B_K && !SPLIT && !SEGMENTED && !RESIDUAL && !SWIGLU && BN == 256),
+                  "the SwiGLU gradient epilogue belongs to the plain input-gradient kernel with 256-wide tiles");
     static_assert(!SEGMENTED || (A_K && !SPLIT), "segments along K are read by the unsplit kernels only");
     static_assert(!RESIDUAL || (!SPLIT && !SEGMENTED), "the residual epilogue belongs to plain unsplit kernels");
     static_assert(!SWIGLU || (A_K && B_K && !SPLIT && !SEGMENTED && !RESIDUAL && BN == 256),
@@ -711,6 +715,69 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
             }
             return;
         }
+        if constexpr (GRAD) {
+            // The contraction is the gradient of silu(gate)·up; what is written is the gradient of
+            // [gate | up]: dgate = d·up·s·(1 + gate·(1 - s)), dup = d·gate·s with s = sigmoid(gate),
+            // from d rounded to the storage dtype (the bits the separate operator reads) and the
+            // forward's saved gate and up. The tile is staged in the storage dtype; lane l of round u
+            // holds 8 consecutive columns (chunk l%16) of row 4u + l/16, loads the matching gate and up
+            // values one 32-row block ahead and stores both gradients.
+            const int g0 = w.n0 + col0;  // first gate column of the wavefront's part
+            const int cols_left = min(WN, p.inter - g0);
+            const T* out_origin = static_cast<const T*>(p.c) + static_cast<long>(row0) * p.ldc + g0;
+            const T* in_origin = static_cast<const T*>(p.saved) + static_cast<long>(row0) * p.ld_saved + g0;
+            const __amdgpu_buffer_rsrc_t dgate_rsrc = part_rsrc(out_origin, p.ldc, sizeof(T), rows_left, cols_left);
+            const __amdgpu_buffer_rsrc_t dup_rsrc = part_rsrc(out_origin + p.inter, p.ldc, sizeof(T), rows_left, cols_left);
+            const __amdgpu_buffer_rsrc_t gate_rsrc = part_rsrc(in_origin, p.ld_saved, sizeof(T), rows_left, cols_left);
+            const __amdgpu_buffer_rsrc_t up_rsrc = part_rsrc(in_origin + p.inter, p.ld_saved, sizeof(T), rows_left, cols_left);
+            constexpr int kLanesPerRow = kRowBytes / 16, kRowsPerRound = kWave / kLanesPerRow, kRounds = 32 / kRowsPerRound;
+            const int lane_row = lane / kLanesPerRow, lane_chunk = lane % kLanesPerRow;
+            const int out_row_bytes = static_cast<int>(p.ldc * static_cast<long>(sizeof(T)));
+            const int in_row_bytes = static_cast<int>(p.ld_saved * static_cast<long>(sizeof(T)));
+            const bool live = lane_chunk * 8 < cols_left;
+            const int out_voffset = live ? lane_row * out_row_bytes + lane_chunk * 16 : std::numeric_limits<int>::min();
+            const int in_voffset = live ? lane_row * in_row_bytes + lane_chunk * 16 : std::numeric_limits<int>::min();
+            u32x4 ahead[2][2][kRounds];
+            auto request_saved = [&](int r, u32x4 (&into)[2][kRounds]) __attribute__((always_inline)) {
+#pragma unroll
+                for (int u = 0; u < kRounds; ++u) {
+                    const int soffset = (r * 32 + u * kRowsPerRound) * in_row_bytes;
+                    into[0][u] = __builtin_amdgcn_raw_buffer_load_b128(gate_rsrc, in_voffset, soffset, 0);
+                    into[1][u] = __builtin_amdgcn_raw_buffer_load_b128(up_rsrc, in_voffset, soffset, 0);
+                }
+            };
+            request_saved(0, ahead[0]);
+#pragma unroll
+            for (int r = 0; r < kRowBlocks; ++r) {
+                __builtin_amdgcn_sched_barrier(0);
+                if (request) request_share(r);
+                if (r + 1 < kRowBlocks) request_saved(r + 1, ahead[(r + 1) & 1]);
+                stage.template operator()<T, TN>(r, 0);
+                u32x4 data[kRounds];
+#pragma unroll
+                for (int u = 0; u < kRounds; ++u) {
+                    const int row = u * kRowsPerRound + lane_row;
+                    data[u] = *reinterpret_cast<const u32x4*>(region + row * kRowBytes + ((lane_chunk ^ sw(row)) * 16));
+                }
+#pragma unroll
+                for (int u = 0; u < kRounds; ++u) {
+                    const vec_t<float, 8> d = vec_to_f32<T, 8>(__builtin_bit_cast(vec_t<T, 8>, data[u]));
+                    const vec_t<float, 8> g = vec_to_f32<T, 8>(__builtin_bit_cast(vec_t<T, 8>, ahead[r & 1][0][u]));
+                    const vec_t<float, 8> v = vec_to_f32<T, 8>(__builtin_bit_cast(vec_t<T, 8>, ahead[r & 1][1][u]));
+                    vec_t<float, 8> dg, du;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const float sg = 1.0f / (1.0f + __expf(-g[e]));
+                        dg[e] = d[e] * v[e] * (sg * (1.0f + g[e] * (1.0f - sg)));
+                        du[e] = d[e] * (g[e] * sg);
+                    }
+                    const int soffset = (r * 32 + u * kRowsPerRound) * out_row_bytes;
+                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, vec_from_f32<T, 8>(dg)), dgate_rsrc, out_voffset, soffset, 0);
+                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, vec_from_f32<T, 8>(du)), dup_rsrc, out_voffset, soffset, 0);
+                }
+            }
+            return;
+        }
         if constexpr (RESIDUAL) {
             const int cols_left = min(WN, c_cols - (c_col0 + col0));
             const T* out_origin = static_cast<const T*>(c_base) + static_cast<long>(row0) * c_ld + (c_col0 + col0);
@@ -1059,10 +1126,10 @@ __global__ __launch_bounds__(kGenericTile* kGenericTile / 4) void gemm_generic_k
 
 // ------------------------------------------------------------------- host side
 template <typename T, int BM, int BN, bool A_K, bool B_K, bool SPLIT, bool SEGMENTED, bool RESIDUAL = false,
-          bool SWIGLU = false>
+          bool SWIGLU = false, bool GRAD = false>
 int launch_mfma(const KernelArgs& p, int slices, hipStream_t stream) {
     constexpr std::size_t smem = TileLayout<T, BM, BN, A_K, B_K>::kSmemBytes;
-    auto kernel = gemm_mfma_kernel<T, BM, BN, A_K, B_K, SPLIT, SEGMENTED, RESIDUAL, SWIGLU>;
+    auto kernel = gemm_mfma_kernel<T, BM, BN, A_K, B_K, SPLIT, SEGMENTED, RESIDUAL, SWIGLU, GRAD>;
     static bool configured = false;
     if (!configured) {
         CGPTX_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -1102,6 +1169,10 @@ int launch_layout(const KernelArgs& p, bool a_k, bool b_k, int slices, hipStream
         if (p.act != nullptr) return launch_mfma<T, BM, BN, true, true, false, false, false, true>(p, slices, stream);
     }
     if (p.act != nullptr) return fail(CGPTX_RUNTIME, "gemm: the SwiGLU epilogue needs 256-wide unsplit tiles");
+    if constexpr (!SPLIT && BN == 256) {
+        if (p.saved != nullptr) return launch_mfma<T, BM, BN, true, false, false, false, false, false, true>(p, slices, stream);
+    }
+    if (p.saved != nullptr) return fail(CGPTX_RUNTIME, "gemm: the SwiGLU gradient epilogue needs 256-wide unsplit tiles");
     if constexpr (!SPLIT) {
         if (a_k && b_k && p.bias == nullptr && !p.c_f32) {
             if (p.residual != nullptr && !p.accumulate) return launch_mfma<T, BM, BN, true, true, false, false, true>(p, slices, stream);
@@ -1142,7 +1213,8 @@ int run_config(const GemmArgs& g, KernelArgs p, hipStream_t stream) {
     const long want_blocks = static_cast<long>(compute_units()) * (BM == 256 ? 1 : 2);
     int slices = 1;
     const bool k_segments = g.a_k_contiguous && g.a_segments.count > 0;
-    if (!g.no_split && g.residual == nullptr && g.swiglu_out == nullptr && g.c_segments.count == 0 && !k_segments &&
+    if (!g.no_split && g.residual == nullptr && g.swiglu_out == nullptr && g.swiglu_saved == nullptr &&
+        g.c_segments.count == 0 && !k_segments &&
         tiles < want_blocks && k_tiles >= 32) {
         // As many slices as fit the CU slots in one go: one item more than that would cost a
         // second round of the persistent blocks.
@@ -1228,6 +1300,12 @@ int run_typed(const GemmArgs& g, hipStream_t stream) {
         p.ld_act = static_cast<long>(g.ld_swiglu);
         p.inter = static_cast<int>(g.n / 2);
     }
+    if (g.swiglu_saved != nullptr) {
+        if (!gemm_fuses_swiglu_gradient(g)) return fail(CGPTX_INVALID_ARGUMENT, "gemm: this call cannot carry the SwiGLU gradient epilogue");
+        p.saved = g.swiglu_saved;
+        p.ld_saved = static_cast<long>(g.ld_swiglu);
+        p.inter = static_cast<int>(g.n);
+    }
     const bool segmented = g.a_segments.count > 0 || g.c_segments.count > 0;
     if (segmented) {
         if (int s = copy_segments(g.a_segments, g.a_k_contiguous ? g.k : g.m, g.a_k_contiguous ? kBK : 256, p.a_seg))
@@ -1277,7 +1355,7 @@ int run_typed(const GemmArgs& g, hipStream_t stream) {
         const bool fills = big_tiles * 5 >= units * 4;
         const bool splits = !g.no_split && g.residual == nullptr && g.c_segments.count == 0 && big_tiles >= 8 &&
                             g.k / kBK >= static_cast<std::size_t>(32 * ((units + big_tiles - 1) / big_tiles));
-        const bool big = g.swiglu_out != nullptr || forced == 256 || (forced == 0 && (fills || splits));
+        const bool big = g.swiglu_out != nullptr || g.swiglu_saved != nullptr || forced == 256 || (forced == 0 && (fills || splits));
         if (big) return run_config<T, 256, 256>(g, p, stream);
         return run_config<T, 128, 128>(g, p, stream);
     }
@@ -1302,6 +1380,24 @@ bool gemm_fuses_swiglu(const GemmArgs& g) {
     if (forced_tile() == 128 || tiles * 5 < static_cast<long>(compute_units()) * 4) return false;
     constexpr std::size_t limit = (std::size_t{1} << 31) - (std::size_t{1} << 20);
     return offsets_fit_32bit(g, elem) && (g.n * g.ldb + g.k) * elem < limit && 256 * g.ld_swiglu * elem < limit;
+}
+
+bool gemm_fuses_swiglu_gradient(const GemmArgs& g) {
+    if (g.swiglu_saved == nullptr || g.swiglu_out != nullptr || g.dtype == CGPTX_F32 || !g.a_k_contiguous || g.b_k_contiguous ||
+        g.bias != nullptr || g.residual != nullptr || g.accumulate || g.c_is_f32 || g.a_segments.count > 0 ||
+        g.c_segments.count > 0 || g.a == nullptr || g.b == nullptr || g.c == nullptr)
+        return false;
+    const std::size_t elem = 2;
+    // 16-byte chunks of whole rows everywhere, tiles that fill the chip (the 256x256 configuration),
+    // and a wavefront's 128 rows of the saved and of the written [gate | up] within 32-bit offsets.
+    if (g.n % 8 != 0 || g.m % 8 != 0 || g.k % kBK != 0 || g.lda % 8 != 0 || g.ldb % 8 != 0 || g.ldc % 8 != 0 ||
+        g.ld_swiglu % 8 != 0 || g.ldc < 2 * g.n || g.ld_swiglu < 2 * g.n || !is_aligned16(g.a) || !is_aligned16(g.b) ||
+        !is_aligned16(g.c) || !is_aligned16(g.swiglu_saved))
+        return false;
+    const long tiles = static_cast<long>((g.m + 255) / 256) * static_cast<long>((g.n + 255) / 256);
+    if (forced_tile() == 128 || tiles * 5 < static_cast<long>(compute_units()) * 4) return false;
+    constexpr std::size_t limit = (std::size_t{1} << 31) - (std::size_t{1} << 20);
+    return offsets_fit_32bit(g, elem) && 256 * g.ld_swiglu * elem < limit;
 }
 
 int gemm(const GemmArgs& g, hipStream_t stream) {

@@ -46,10 +46,18 @@ struct GemmArgs {
     // gemm_fuses_swiglu() accepts.
     void* swiglu_out = nullptr;
     std::size_t ld_swiglu = 0;
+    // Input gradient of the down projection (c = dY·W with n = inter) that writes the gradient of
+    // the forward's [gate | up] instead of the gradient of silu(gate)·up: c is [m, 2·inter] = [dgate |
+    // dup] (ldc >= 2·inter), swiglu_saved the forward's [m, 2·inter] = [gate | up] with row stride
+    // ld_swiglu. The contraction is rounded to the storage dtype before the SwiGLU gradient is
+    // applied (the bits of the two separate operators). Only for calls that
+    // gemm_fuses_swiglu_gradient() accepts.
+    const void* swiglu_saved = nullptr;
 };
 
 int gemm(const GemmArgs& args, hipStream_t stream);
 // Whether gemm() serves args.swiglu_out for this call (shape, layout and alignment of the fused kernel).
 bool gemm_fuses_swiglu(const GemmArgs& args);
+bool gemm_fuses_swiglu_gradient(const GemmArgs& args);
 
 }  // namespace cgptx

@@ -76,6 +76,39 @@ extern "C" int cgptx_linear_swiglu_forward(void* gate_up, void* activated, const
     return cgptx_swiglu_forward_packed(activated, gate_up, rows, hidden, dtype, stream_);
 }
 
+extern "C" int cgptx_linear_swiglu_backward(void* grad_gate_up, void* grad_activated, const void* grad_output,
+                                            const void* weight, const void* gate_up, size_t rows, size_t hidden,
+                                            size_t out_features, int dtype, cgptx_stream stream_) {
+    using namespace cgptx;
+    if (hidden > std::numeric_limits<std::size_t>::max() / 2)
+        return fail(CGPTX_OVERFLOW, "linear_swiglu_backward: dimension exceeds int range");
+    if (int s = validate("linear_swiglu_backward", rows, 2 * hidden, out_features, dtype)) return s;
+    if (grad_gate_up == nullptr || grad_activated == nullptr || grad_output == nullptr || weight == nullptr || gate_up == nullptr)
+        return fail(CGPTX_INVALID_ARGUMENT, "linear_swiglu_backward: null tensor");
+    auto stream = static_cast<hipStream_t>(stream_);
+    GemmArgs g;  // d(activated)[rows, hidden] = dY[rows, out] · W[out, hidden]
+    g.a = grad_output;
+    g.b = weight;
+    g.c = grad_gate_up;
+    g.m = rows;
+    g.n = hidden;
+    g.k = out_features;
+    g.lda = out_features;
+    g.ldb = hidden;
+    g.ldc = 2 * hidden;
+    g.b_k_contiguous = false;
+    g.dtype = dtype;
+    g.swiglu_saved = gate_up;
+    g.ld_swiglu = 2 * hidden;
+    if (gemm_fuses_swiglu_gradient(g)) return gemm(g, stream);
+    // Shapes the fused kernel does not take: the two operators one after the other (same bits).
+    g.swiglu_saved = nullptr;
+    g.c = grad_activated;
+    g.ldc = hidden;
+    if (int s = gemm(g, stream)) return s;
+    return cgptx_swiglu_backward_packed(grad_gate_up, grad_activated, gate_up, rows, hidden, 0, dtype, stream_);
+}
+
 extern "C" int cgptx_linear_backward(void* grad_input, void* grad_weight, void* grad_bias, const void* grad_output,
                                      const void* input, const void* weight, size_t rows, size_t in_features,
                                      size_t out_features, int accumulate_input, int accumulate_weight,

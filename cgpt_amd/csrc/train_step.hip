@@ -428,8 +428,14 @@ int enqueue_forward_backward(cgptx_model* m, float loss_scale, int loss_mode, hi
         const auto& w = m->layers[reverse];
         const auto& a = m->acts[reverse];
         void* x = m->hidden[reverse];
-        CGPTX_TRY(linear_backward_split(m, m->d_act, w.down.gradient, current, a.act, w.down.value, N, I, H, 0, dt, stream));
-        CGPTX_OP("swiglu_bwd", cgptx_swiglu_backward_packed(m->d_gate_up, m->d_act, a.gate_up, N, I, 0, dt, s));
+        if (fused_swiglu()) {
+            // The SwiGLU gradient rides in the epilogue of the down projection's input gradient.
+            CGPTX_OP("gemm_dx", cgptx_linear_swiglu_backward(m->d_gate_up, m->d_act, current, w.down.value, a.gate_up, N, I, H, dt, s));
+            CGPTX_OP("gemm_dw", cgptx_linear_backward(nullptr, w.down.gradient, nullptr, current, a.act, w.down.value, N, I, H, 0, 0, 0, dt, s));
+        } else {
+            CGPTX_TRY(linear_backward_split(m, m->d_act, w.down.gradient, current, a.act, w.down.value, N, I, H, 0, dt, stream));
+            CGPTX_OP("swiglu_bwd", cgptx_swiglu_backward_packed(m->d_gate_up, m->d_act, a.gate_up, N, I, 0, dt, s));
+        }
         // The gradient of the residual stream collects the two norm branches: in one pass at the end of
         // the block when the shape allows (previous = current + d(ffn norm) + d(attention norm)), else as
         // they are produced (previous = current + d(ffn branch), later previous += d(attention branch)).

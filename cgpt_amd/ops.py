@@ -541,6 +541,24 @@ def linear_swiglu_forward(gate_up, activated, input, weight, gemm_context=None, 
               input.numel() // in_features, in_features, out_features // 2, _code(input), _stream(stream))
 
 
+def linear_swiglu_backward(grad_gate_up, grad_activated, grad_output, weight, gate_up, gemm_context=None, stream=None):
+    """The input gradient of the down projection and the SwiGLU gradient in one call (src/core/transformer_block.cu:663-666
+    with the concatenated layouts of src/ops/backward/swiglu_backward.cu:830-883): weight = down_proj ([out, hidden]),
+    gate_up = the forward's [..., 2*hidden] = [gate | up], grad_gate_up = [..., 2*hidden] = [dgate | dup];
+    grad_activated ([..., hidden]) is working memory (written only when the two operators run one after the other)."""
+    name = "linear_swiglu_backward"
+    _require_device(name, grad_gate_up, grad_activated, grad_output, weight, gate_up)
+    _same_dtype(name, grad_output, grad_gate_up, grad_activated, weight, gate_up)
+    if weight.dim() != 2 or grad_output.shape[-1] != weight.shape[0] or grad_activated.shape[-1] != weight.shape[1] or \
+            gate_up.shape[-1] != 2 * weight.shape[1] or tuple(grad_gate_up.shape) != tuple(gate_up.shape) or \
+            tuple(gate_up.shape[:-1]) != tuple(grad_output.shape[:-1]) or \
+            tuple(grad_activated.shape[:-1]) != tuple(grad_output.shape[:-1]):
+        raise ValueError(f"{name}: incompatible tensors")
+    out_features, hidden = weight.shape
+    capi.call("cgptx_linear_swiglu_backward", _ptr(grad_gate_up), _ptr(grad_activated), _ptr(grad_output), _ptr(weight),
+              _ptr(gate_up), grad_output.numel() // out_features, hidden, out_features, _code(grad_output), _stream(stream))
+
+
 def embedding_forward(output, device_token_ids, token_count, weight, stream=None):
     """include/ops/embedding.h."""
     name = "embedding_forward"

@@ -256,6 +256,18 @@ int cgptx_linear_swiglu_forward(void* gate_up, void* activated, const void* inpu
                                 const void* weight, size_t rows, size_t in_features,
                                 size_t hidden, int dtype, cgptx_stream stream);
 
+/* The input gradient of the feed-forward's down projection and the SwiGLU gradient in one call — the
+ * sequence linear_backward(down) (input gradient only), swiglu_backward of
+ * src/core/transformer_block.cu:663-666 with the concatenated layouts of
+ * src/ops/backward/swiglu_backward.cu:830-883: weight = down_proj ([out, hidden]), gate_up = the forward's
+ * [rows, 2*hidden] = [gate | up], grad_gate_up = [rows, 2*hidden] = [dgate | dup], computed from
+ * grad_output·weight rounded to the storage dtype. grad_activated ([rows, hidden]) is working memory: the
+ * two-operator path writes the intermediate gradient there, the fused contraction (large aligned shapes)
+ * leaves it untouched. */
+int cgptx_linear_swiglu_backward(void* grad_gate_up, void* grad_activated, const void* grad_output,
+                                 const void* weight, const void* gate_up, size_t rows,
+                                 size_t hidden, size_t out_features, int dtype, cgptx_stream stream);
+
 /* embedding_forward — include/ops/embedding.h. out[t,:] = W[id_t,:]; ids >= vocab give a zero row. */
 int cgptx_embedding_forward(void* output, const uint32_t* token_ids,
                             size_t token_count, const void* weight,

@@ -56,3 +56,23 @@ inline void linear_swiglu_forward(Tensor& gate_up, Tensor& activated, const Tens
                                                     input.numel() / weight.size(1), weight.size(1), weight.size(0) / 2,
                                                     cgptx_detail::dtype_code(input.dtype()), stream));
 }
+
+// The input gradient of the down projection and the SwiGLU gradient as one call: the sequence
+// linear_backward(down) (input gradient), swiglu_backward of the reference's
+// src/core/transformer_block.cu:663-666 over the concatenated layouts of
+// src/ops/backward/swiglu_backward.cu:830-883 (gate_up = the forward's [gate | up], grad_gate_up =
+// [dgate | dup]); grad_activated is working memory. No single reference function corresponds.
+inline void linear_swiglu_backward(Tensor& grad_gate_up, Tensor& grad_activated, const Tensor& grad_output, const Tensor& weight,
+                                   const Tensor& gate_up, const GemmContext&, hipStream_t stream = nullptr) {
+    const char* op = "linear_swiglu_backward";
+    cgptx_detail::require_device(op, {&grad_gate_up, &grad_activated, &grad_output, &weight, &gate_up});
+    cgptx_detail::require_same_dtype(op, grad_output, {&grad_gate_up, &grad_activated, &weight, &gate_up});
+    if (weight.dim() != 2 || grad_output.numel() == 0 || grad_output.dim() == 0 || grad_output.shape().back() != weight.size(0) ||
+        grad_activated.numel() != grad_output.numel() / weight.size(0) * weight.size(1) ||
+        gate_up.numel() != 2 * grad_activated.numel() || grad_gate_up.numel() != gate_up.numel())
+        throw std::invalid_argument("linear_swiglu_backward: incompatible tensors");
+    cgptx_detail::check(cgptx_linear_swiglu_backward(grad_gate_up.raw_data(), grad_activated.raw_data(), grad_output.raw_data(),
+                                                     weight.raw_data(), gate_up.raw_data(), grad_output.numel() / weight.size(0),
+                                                     weight.size(1), weight.size(0), cgptx_detail::dtype_code(grad_output.dtype()),
+                                                     stream));
+}

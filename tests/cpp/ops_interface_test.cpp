@@ -265,6 +265,13 @@ void rmsnorm_and_swiglu() {
     const std::vector<float> a = host_f32(gg), b = host_f32(gu), p = host_f32(gp);
     expect(close({p[0], p[1], p[4], p[5]}, a, 1e-6f) && close({p[2], p[3], p[6], p[7]}, b, 1e-6f),
            "swiglu_backward concatenated = separate");
+    // Down projection's input gradient plus the SwiGLU gradient as one call: with an identity weight the
+    // contraction hands `go` through, so the result is swiglu_backward(go, packed).
+    Tensor fused = Tensor::zeros({2, 4}), work = Tensor::zeros({2, 2});
+    linear_swiglu_backward(fused, work, go, eye, packed, context);
+    expect(close(host_f32(fused), p, 0), "linear_swiglu_backward = linear_backward + swiglu_backward");
+    expect(throws<std::invalid_argument>([&] { linear_swiglu_backward(fused, work, go, gate_up_proj, packed, context); }),
+           "linear_swiglu_backward mismatched tensors -> invalid_argument");
 }
 
 // Attention: options-driven call, LSE and no-LSE backward agree, bad options throw

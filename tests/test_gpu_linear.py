@@ -176,6 +176,57 @@ def test_linear_swiglu_forward_equals_the_two_operators(device, rows, fin, hidde
     assert err <= 2e-2
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+@pytest.mark.parametrize("rows,out,hidden", [(4096, 256, 3328), (4104, 64, 3328), (4096, 96, 3336), (64, 32, 64), (520, 96, 200)],
+                         ids=["fused", "fused-ragged-rows", "fused-ragged-columns", "small", "unaligned-columns"])
+def test_linear_swiglu_backward_equals_the_two_operators(device, rows, out, hidden, dtype):
+    """Input gradient of the down projection with the SwiGLU gradient from its epilogue (when the shape
+    fills the chip) against linear_backward followed by the packed swiglu_backward: the same bits, rows and
+    columns past the matrix untouched, and the float64 gradient within the 16-bit tolerance."""
+    g = torch.Generator().manual_seed(rows + hidden + 1)
+    dy = torch.randn(rows, out, generator=g).to(dtype).to(device)
+    w = (torch.randn(out, hidden, generator=g) * 0.3).to(dtype).to(device)
+    gate_up = torch.randn(rows, 2 * hidden, generator=g).to(dtype).to(device)
+    act = torch.empty(rows, hidden, dtype=dtype, device=device)  # the projection's input: unused by its input gradient
+    d_act = torch.empty(rows, hidden, dtype=dtype, device=device)
+    want = torch.empty(rows, 2 * hidden, dtype=dtype, device=device)
+    ops.linear_backward(d_act, None, None, dy, act, w)
+    ops.swiglu_backward_packed(want, d_act, gate_up)
+    guarded = torch.full((rows + 8, 2 * hidden), 7.0, dtype=dtype, device=device)  # rows after the output
+    got = guarded[:rows]
+    work = torch.empty_like(d_act)
+    ops.linear_swiglu_backward(got, work, dy, w, gate_up)
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
+    assert bool((guarded[rows:] == 7.0).all())
+    exact = dy.double().cpu() @ w.double().cpu()
+    gate, up = gate_up.double().cpu()[:, :hidden], gate_up.double().cpu()[:, hidden:]
+    sig = 1 / (1 + torch.exp(-gate))
+    reference = torch.cat([exact * up * sig * (1 + gate * (1 - sig)), exact * gate * sig], dim=1)
+    err = (got.double().cpu() - reference).abs().max() / reference.abs().max()
+    assert err <= 2e-2
+
+
+def test_linear_swiglu_backward_argument_errors(device):
+    bf = torch.bfloat16
+    dy = torch.zeros(8, 16, dtype=bf, device=device)
+    w = torch.zeros(16, 32, dtype=bf, device=device)
+    gate_up = torch.zeros(8, 64, dtype=bf, device=device)
+    grad = torch.zeros(8, 64, dtype=bf, device=device)
+    work = torch.zeros(8, 32, dtype=bf, device=device)
+    ops.linear_swiglu_backward(grad, work, dy, w, gate_up)  # valid
+    with pytest.raises(ValueError):
+        ops.linear_swiglu_backward(grad, torch.zeros(8, 16, dtype=bf, device=device), dy, w, gate_up)
+    with pytest.raises(ValueError):
+        ops.linear_swiglu_backward(grad, work, dy, torch.zeros(15, 32, dtype=bf, device=device), gate_up)
+    with pytest.raises(ValueError):
+        ops.linear_swiglu_backward(grad.float(), work, dy, w, gate_up)
+    from cgpt_amd import capi
+    with pytest.raises(ValueError):  # the C entry point rejects null tensors itself
+        capi.call("cgptx_linear_swiglu_backward", grad.data_ptr(), None, dy.data_ptr(), w.data_ptr(), gate_up.data_ptr(),
+                  8, 32, 16, 1, None)
+
+
 def test_linear_swiglu_forward_argument_errors(device):
     x = torch.zeros(8, 32, dtype=torch.bfloat16, device=device)
     w = torch.zeros(64, 32, dtype=torch.bfloat16, device=device)

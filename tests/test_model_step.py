@@ -275,6 +275,32 @@ def test_fused_qk_norm_rope_is_bit_identical_to_the_separate_operators(device, m
 
 
 @pytest.mark.gpu
+def test_swiglu_in_the_projection_epilogues_is_bit_identical_to_the_separate_operators(device, monkeypatch):
+    """The SwiGLU product rides in the gate/up projection's epilogue and its gradient in the epilogue of the
+    down projection's input gradient when the shapes fill the chip (here 4096 rows x 3328 feed-forward
+    columns); both work from the rounded 16-bit values the separate operators would exchange, so a whole
+    step gives the same bits either way. CGPTX_FUSE_SWIGLU=0 selects the separate operators."""
+    from cgpt_amd.model import LOSS_DENSE, Model, ModelConfig
+    config = ModelConfig(vocabulary_size=128, num_layers=2, hidden_size=256, intermediate_size=3328, num_query_heads=4,
+                         num_kv_heads=2, head_dim=64, rotary_dim=64, dtype=torch.bfloat16)
+    rng = np.random.default_rng(5)
+    inputs = rng.integers(0, 128, size=4 * 1024).astype(np.uint32)
+    targets = rng.integers(0, 128, size=4 * 1024).astype(np.uint32)
+    results = []
+    for fuse in ("1", "0"):
+        monkeypatch.setenv("CGPTX_FUSE_SWIGLU", fuse)
+        model = Model(config, 4, 1024, seed=6, device=device)
+        model.set_tokens(inputs, targets)
+        model.forward_backward(loss_scale=4.0, loss_mode=LOSS_DENSE)
+        loss = model.status()[0]
+        results.append((loss, [g.clone() for _, _, g in model.parameters()], model.activation("hidden.2").clone()))
+    assert np.isfinite(results[0][0]) and results[0][0] == results[1][0]
+    assert torch.equal(results[0][2], results[1][2])
+    for a, b in zip(results[0][1], results[1][1]):
+        assert torch.equal(a, b)
+
+
+@pytest.mark.gpu
 def test_block_norms_in_one_pass_match_the_separate_operators(device, monkeypatch):
     """The attention and feed-forward norms of a block read the same input and run as one pass: forward
     bit-identical; backward adds the two branch gradients before the one rounding instead of rounding
