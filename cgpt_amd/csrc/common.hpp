@@ -140,6 +140,12 @@ int rmsnorm_backward_dual(void* grad_input, void* grad_weight_a, void* grad_weig
 // aligned. Grows by reallocation on eager calls; refuses to grow during capture.
 int scratch(hipStream_t stream, std::size_t bytes, void** out);
 
+// Identifies the block currently behind the (current device, stream) arena: it changes whenever that
+// arena is reallocated (a larger request) and reads 0 after cgptx_release_scratch. A captured graph
+// holds the block's address, so whoever replays one compares this value with the one at capture time
+// and captures again when they differ.
+std::uint64_t scratch_generation(hipStream_t stream);
+
 // Number of compute units of the current device (cached).
 int compute_units();
 

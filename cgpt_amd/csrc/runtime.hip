@@ -13,10 +13,12 @@ thread_local std::string g_last_error;
 struct Arena {
     void* data = nullptr;
     std::size_t bytes = 0;
+    std::uint64_t generation = 0;  // value of g_generation when this block was allocated
 };
 
 std::mutex g_arena_mutex;
 std::map<std::pair<int, hipStream_t>, Arena> g_arenas;
+std::uint64_t g_generation = 0;  // bumped by every allocation; a released arena reads as generation 0
 
 }  // namespace
 
@@ -54,9 +56,18 @@ int scratch(hipStream_t stream, std::size_t bytes, void** out) {
         }
         arena.data = fresh;
         arena.bytes = rounded;
+        arena.generation = ++g_generation;
     }
     *out = arena.data;
     return CGPTX_OK;
+}
+
+std::uint64_t scratch_generation(hipStream_t stream) {
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess) return 0;
+    std::lock_guard<std::mutex> lock(g_arena_mutex);
+    const auto it = g_arenas.find({device, stream});
+    return it == g_arenas.end() ? 0 : it->second.generation;
 }
 
 int compute_units() {

@@ -115,6 +115,7 @@ struct cgptx_model {
     float graph_loss_scale = 0.0f;
     int graph_loss_mode = -1;
     hipStream_t graph_stream = nullptr;
+    std::uint64_t graph_scratch_generation = 0;  // scratch arena block the recorded kernels point into
     // optional per-operator timing of one eager pass
     struct Timed {
         const char* label;
@@ -763,7 +764,10 @@ extern "C" int cgptx_model_forward_backward(cgptx_model* m, float loss_scale, in
     if (stream == nullptr)
         return fail(CGPTX_INVALID_ARGUMENT, "model_forward_backward: graph capture needs a non-default stream");
     const bool have_graph = m->graph_exec != nullptr && m->graph_loss_scale == loss_scale &&
-                            m->graph_loss_mode == loss_mode && m->graph_stream == stream;
+                            m->graph_loss_mode == loss_mode && m->graph_stream == stream &&
+                            // The recorded kernels hold addresses inside the stream's scratch arena: a graph
+                            // whose arena block has since been reallocated or released is recorded again.
+                            m->graph_scratch_generation == scratch_generation(stream);
     if (have_graph) {
         CGPTX_HIP(hipGraphLaunch(m->graph_exec, stream));
         return CGPTX_OK;
@@ -791,6 +795,7 @@ extern "C" int cgptx_model_forward_backward(cgptx_model* m, float loss_scale, in
     m->graph_loss_scale = loss_scale;
     m->graph_loss_mode = loss_mode;
     m->graph_stream = stream;
+    m->graph_scratch_generation = scratch_generation(stream);
     return CGPTX_OK;
 }
 

@@ -8,7 +8,7 @@ import torch
 
 from cgpt_amd import ops
 from oracle import oracle64
-from tests.util import DTYPES, DTYPE_IDS, TOL, assert_close, randint, randn, to_np
+from tests.util import DTYPES, DTYPE_IDS, TOL, assert_close, assert_scaled_close, randint, randn, to_np
 
 pytestmark = pytest.mark.gpu
 
@@ -42,19 +42,17 @@ def test_reference_test_case(device):
 @pytest.mark.parametrize("dtype", DTYPES, ids=DTYPE_IDS)
 @pytest.mark.parametrize("rows,hidden,vocab", [(5, 7, 11), (64, 64, 128), (300, 128, 1000), (1024, 256, 4096)])
 def test_parity_with_float64(device, rows, hidden, vocab, dtype):
-    if dtype == torch.float32 and rows * hidden * vocab > 300 * 128 * 1000:
-        pytest.skip("fp32 storage runs on the plain contraction kernel; large shapes are covered in 16-bit")
     x, c = randn((rows, hidden), dtype, 1), randn((vocab, hidden), dtype, 2, 0.05)
     targets = randint(vocab, (rows,), 3)
     l64, dx64, dc64 = oracle64.cut_cross_entropy(to_np(x), to_np(c), targets.numpy(), 1024.0)
     loss, dx, dc = run(device, x, c, targets, 1024.0)
     assert abs(loss - l64) <= (1e-4 if dtype == torch.float32 else 5e-3) * max(1.0, l64)
-    assert_close(dx, dx64, TOL[dtype] * max(1.0, np.abs(dx64).max()), "dX")
-    assert_close(dc, dc64, TOL[dtype] * max(1.0, np.abs(dc64).max()), "dC")
+    assert_scaled_close(dx, dx64, TOL[dtype], "dX")
+    assert_scaled_close(dc, dc64, TOL[dtype], "dC")
     base = randn((vocab, hidden), dtype, 4)
     _, _, dc2 = run(device, x, c, targets, 1024.0, True, base)
     want = dc64 + to_np(base)
-    assert_close(dc2, want, TOL[dtype] * max(1.0, np.abs(want).max()), "dC accumulate")
+    assert_scaled_close(dc2, want, TOL[dtype], "dC accumulate")
 
 
 def test_equivalent_to_dense_cross_entropy_plus_linear_backward(device):
@@ -72,8 +70,8 @@ def test_equivalent_to_dense_cross_entropy_plus_linear_backward(device):
     dx2, dc2 = torch.empty_like(x), torch.empty_like(c)
     ops.linear_backward(dx2, dc2, None, grad, x, c)
     assert abs(loss - dense_loss.item()) <= 1e-5 * dense_loss.item()
-    assert_close(dx, dx2, TOL[dtype] * max(1.0, float(dx2.float().abs().max())), "dX vs dense path")
-    assert_close(dc, dc2, TOL[dtype] * max(1.0, float(dc2.float().abs().max())), "dC vs dense path")
+    assert_scaled_close(dx, dx2, TOL[dtype], "dX vs dense path")
+    assert_scaled_close(dc, dc2, TOL[dtype], "dC vs dense path")
     again = run(device, x, c, targets, 1024.0)
     assert again[0] == loss and torch.equal(again[1], dx) and torch.equal(again[2], dc)
 

@@ -39,6 +39,22 @@ def assert_close(actual, expected, tol, what=""):
     assert err <= tol, f"{what}: max rel err {err:.3e} > {tol:.1e}"
 
 
+def assert_scaled_close(actual, expected, tol, what=""):
+    """One normalisation only: max |a-b| <= tol * max(1, max |expected|). For results that are sums of many
+    rounded terms (dK/dV, dW, dC), whose rounding error follows the tensor's scale and not each element's.
+    Prints the observed error so that a run shows how far inside the bound the kernels are."""
+    a = to_np(actual) if isinstance(actual, torch.Tensor) else np.asarray(actual, dtype=np.float64)
+    e = to_np(expected) if isinstance(expected, torch.Tensor) else np.asarray(expected, dtype=np.float64)
+    assert a.shape == e.shape, (a.shape, e.shape)
+    if a.size == 0:
+        return
+    assert np.isfinite(a).all(), f"{what}: non-finite values in result"
+    scale = max(1.0, float(np.abs(e).max()))
+    err = float(np.abs(a - e).max()) / scale
+    print(f"[parity] {what}: max|a-b|/max(1,max|w|) = {err:.3e} (bound {tol:.1e}, scale {scale:.3g})")
+    assert err <= tol, f"{what}: max abs err / scale {err:.3e} > {tol:.1e} (scale {scale:.3e})"
+
+
 def scaled_tol(dtype, expected, floor=1.0):
     """Tolerance for results that are sums of many rounded terms: TOL times the result's scale."""
     e = to_np(expected) if isinstance(expected, torch.Tensor) else np.asarray(expected, dtype=np.float64)
