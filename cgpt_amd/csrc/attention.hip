@@ -1234,6 +1234,138 @@ __global__ __launch_bounds__(kThreads, 1) void attention_dkv_wide_kernel(Params 
     }
 }
 
+
+// ============================================================================================
+// Scalar family: fp32 storage, head dimensions that are not multiples of 8, and tensors that are not
+// 16-byte aligned — what the reference serves with its warp-per-row kernels
+// (src/ops/backward/attention_backward.cu:352-504, dispatch 2044-2068). Correct, not fast: one
+// wavefront per output row, fp32 arithmetic throughout, lane l holding head-dim elements l and l + 64.
+// No atomics: dQ rows and (key, kv-head) rows each have one owner that adds its terms in a fixed order
+// (heads of the group ascending, queries ascending), so results do not depend on scheduling.
+template <typename T>
+struct RowPair {
+    float a, b;  // elements lane and lane + 64 of a head_dim-long row (0 past the end)
+    __device__ __forceinline__ static RowPair load(const T* row, int d) {
+        const int lane = threadIdx.x & 63;
+        RowPair r;
+        r.a = lane < d ? to_f32(row[lane]) : 0.0f;
+        r.b = lane + 64 < d ? to_f32(row[lane + 64]) : 0.0f;
+        return r;
+    }
+    __device__ __forceinline__ void store(T* row, int d, bool accumulate) const {
+        const int lane = threadIdx.x & 63;
+        if (lane < d) row[lane] = from_f32<T>(accumulate ? a + to_f32(row[lane]) : a);
+        if (lane + 64 < d) row[lane + 64] = from_f32<T>(accumulate ? b + to_f32(row[lane + 64]) : b);
+    }
+};
+template <typename T>
+__device__ __forceinline__ float row_dot(const RowPair<T>& x, const RowPair<T>& y) {
+    return wave_sum(fmaf(x.a, y.a, x.b * y.b));
+}
+
+constexpr int kScalarWaves = 4;  // rows per 256-thread block
+
+// O and LSE of one (batch, query, head) row per wavefront; lse_out and delta-style outputs are fp32.
+template <typename T>
+__global__ __launch_bounds__(kThreads) void attention_forward_scalar_kernel(Params p) {
+    const long row = static_cast<long>(blockIdx.x) * kScalarWaves + (threadIdx.x >> 6);
+    const long rows = static_cast<long>(p.batch) * p.qs * p.hq;
+    if (row >= rows) return;
+    const int h = static_cast<int>(row % p.hq);
+    const int q = static_cast<int>((row / p.hq) % p.qs);
+    const int b = static_cast<int>(row / (static_cast<long>(p.hq) * p.qs));
+    const int kvh = h / (p.hq / p.hkv);
+    const RowPair<T> qr = RowPair<T>::load(static_cast<const T*>(p.q) + row * p.d, p.d);
+    const T* k_base = static_cast<const T*>(p.k) + (static_cast<long>(b) * p.ks * p.hkv + kvh) * p.d;
+    const T* v_base = static_cast<const T*>(p.v) + (static_cast<long>(b) * p.ks * p.hkv + kvh) * p.d;
+    const long kv_stride = static_cast<long>(p.hkv) * p.d;
+    const int k_end = p.causal ? min(p.ks, p.offset + q + 1) : p.ks;
+    float m = -INFINITY, l = 0.0f;
+    RowPair<T> o{0.0f, 0.0f};
+    for (int j = 0; j < k_end; ++j) {
+        const float s = row_dot(qr, RowPair<T>::load(k_base + j * kv_stride, p.d)) * p.scale;
+        const float m_new = fmaxf(m, s);
+        const float alpha = expf(m - m_new), e = expf(s - m_new);  // exp(-inf) = 0 on the first key
+        const RowPair<T> vr = RowPair<T>::load(v_base + j * kv_stride, p.d);
+        l = l * alpha + e;
+        o.a = fmaf(e, vr.a, o.a * alpha);
+        o.b = fmaf(e, vr.b, o.b * alpha);
+        m = m_new;
+    }
+    const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+    o.a *= inv;
+    o.b *= inv;
+    o.store(static_cast<T*>(p.out0) + row * p.d, p.d, false);
+    if (p.lse_out != nullptr && (threadIdx.x & 63) == 0) p.lse_out[row] = m + logf(l);
+}
+
+// dQ of one (batch, query, head) row per wavefront; also leaves delta = rowsum(dO∘O) for the dK/dV pass.
+template <typename T>
+__global__ __launch_bounds__(kThreads) void attention_dq_scalar_kernel(Params p, const void* out, float* delta_out) {
+    const long row = static_cast<long>(blockIdx.x) * kScalarWaves + (threadIdx.x >> 6);
+    const long rows = static_cast<long>(p.batch) * p.qs * p.hq;
+    if (row >= rows) return;
+    const int h = static_cast<int>(row % p.hq);
+    const int q = static_cast<int>((row / p.hq) % p.qs);
+    const int b = static_cast<int>(row / (static_cast<long>(p.hq) * p.qs));
+    const int kvh = h / (p.hq / p.hkv);
+    const RowPair<T> qr = RowPair<T>::load(static_cast<const T*>(p.q) + row * p.d, p.d);
+    const RowPair<T> dor = RowPair<T>::load(static_cast<const T*>(p.dout) + row * p.d, p.d);
+    const float delta = row_dot(dor, RowPair<T>::load(static_cast<const T*>(out) + row * p.d, p.d));
+    if ((threadIdx.x & 63) == 0) delta_out[row] = delta;
+    const float lse = p.lse[row];
+    const T* k_base = static_cast<const T*>(p.k) + (static_cast<long>(b) * p.ks * p.hkv + kvh) * p.d;
+    const T* v_base = static_cast<const T*>(p.v) + (static_cast<long>(b) * p.ks * p.hkv + kvh) * p.d;
+    const long kv_stride = static_cast<long>(p.hkv) * p.d;
+    const int k_end = p.causal ? min(p.ks, p.offset + q + 1) : p.ks;
+    RowPair<T> dq{0.0f, 0.0f};
+    for (int j = 0; j < k_end; ++j) {
+        const RowPair<T> kr = RowPair<T>::load(k_base + j * kv_stride, p.d);
+        const float prob = expf(row_dot(qr, kr) * p.scale - lse);
+        const float ds = prob * (row_dot(dor, RowPair<T>::load(v_base + j * kv_stride, p.d)) - delta);
+        dq.a = fmaf(ds, kr.a, dq.a);
+        dq.b = fmaf(ds, kr.b, dq.b);
+    }
+    dq.a *= p.scale;
+    dq.b *= p.scale;
+    dq.store(static_cast<T*>(p.out0) + row * p.d, p.d, p.accumulate != 0);
+}
+
+// dK and dV of one (batch, key, kv-head) row per wavefront: the heads of the group in ascending order,
+// each over the queries that see the key in ascending order.
+template <typename T>
+__global__ __launch_bounds__(kThreads) void attention_dkv_scalar_kernel(Params p) {
+    const long row = static_cast<long>(blockIdx.x) * kScalarWaves + (threadIdx.x >> 6);
+    const long rows = static_cast<long>(p.batch) * p.ks * p.hkv;
+    if (row >= rows) return;
+    const int kvh = static_cast<int>(row % p.hkv);
+    const int j = static_cast<int>((row / p.hkv) % p.ks);
+    const int b = static_cast<int>(row / (static_cast<long>(p.hkv) * p.ks));
+    const int group = p.hq / p.hkv;
+    const RowPair<T> kr = RowPair<T>::load(static_cast<const T*>(p.k) + row * p.d, p.d);
+    const RowPair<T> vr = RowPair<T>::load(static_cast<const T*>(p.v) + row * p.d, p.d);
+    const int q_begin = p.causal ? max(0, j - p.offset) : 0;
+    RowPair<T> dk{0.0f, 0.0f}, dv{0.0f, 0.0f};
+    for (int g = 0; g < group; ++g) {
+        const int h = kvh * group + g;
+        for (int q = q_begin; q < p.qs; ++q) {
+            const long q_row = (static_cast<long>(b) * p.qs + q) * p.hq + h;
+            const RowPair<T> qr = RowPair<T>::load(static_cast<const T*>(p.q) + q_row * p.d, p.d);
+            const RowPair<T> dor = RowPair<T>::load(static_cast<const T*>(p.dout) + q_row * p.d, p.d);
+            const float prob = expf(row_dot(qr, kr) * p.scale - p.lse[q_row]);
+            const float ds = prob * (row_dot(dor, vr) - p.delta[q_row]);
+            dv.a = fmaf(prob, dor.a, dv.a);
+            dv.b = fmaf(prob, dor.b, dv.b);
+            dk.a = fmaf(ds, qr.a, dk.a);
+            dk.b = fmaf(ds, qr.b, dk.b);
+        }
+    }
+    dk.a *= p.scale;
+    dk.b *= p.scale;
+    dk.store(static_cast<T*>(p.out0) + row * p.d, p.d, p.accumulate != 0);
+    dv.store(static_cast<T*>(p.out1) + row * p.d, p.d, p.accumulate != 0);
+}
+
 // ---------------------------------------------------------------------- host
 struct Shape {
     std::size_t batch, qs, ks, hq, hkv, d;
@@ -1245,15 +1377,14 @@ struct Shape {
 
 int validate(const char* name, const Shape& s) {
     const std::string n(name);
-    if (s.dtype != CGPTX_F16 && s.dtype != CGPTX_BF16)
-        return fail(CGPTX_INVALID_ARGUMENT, n + ": only F16 and BF16 storage are supported by the MFMA kernels");
+    if (!valid_dtype(s.dtype)) return fail(CGPTX_INVALID_ARGUMENT, n + ": unsupported dtype");
     if (s.batch == 0 || s.qs == 0 || s.ks == 0 || s.hq == 0 || s.hkv == 0 || s.d == 0 || s.hq % s.hkv != 0)
         return fail(CGPTX_INVALID_ARGUMENT, n + ": invalid tensors or options");
     if (!std::isfinite(s.scale)) return fail(CGPTX_INVALID_ARGUMENT, n + ": attention scale must be finite");
     if (s.causal && (s.offset > s.ks || s.qs > s.ks - s.offset))
         return fail(CGPTX_INVALID_ARGUMENT, n + ": causal range exceeds the key sequence");
-    if (s.d % 8 != 0 || s.d > 128)
-        return fail(CGPTX_INVALID_ARGUMENT, n + ": head_dim must be a multiple of 8 up to 128");
+    if (s.d > 128)  // as src/ops/backward/attention_backward.cu:1886-1887
+        return fail(CGPTX_INVALID_ARGUMENT, n + ": head_dim must not exceed 128");
     constexpr std::size_t limit = 1u << 30;
     if (s.batch > 65535 || s.qs > limit || s.ks > limit || s.hq > 65535 || s.offset > limit ||
         s.hq * s.d > limit)
@@ -1302,7 +1433,30 @@ int dispatch_16bit(int dtype, Fn&& fn) {
     return dtype == CGPTX_F16 ? fn.template operator()<f16_t>() : fn.template operator()<bf16_t>();
 }
 
-int launch_forward(const Shape& s, Params p, hipStream_t stream) {
+bool aligned16_all(std::initializer_list<const void*> pointers) {
+    for (const void* ptr : pointers)
+        if (ptr != nullptr && !is_aligned16(ptr)) return false;
+    return true;
+}
+
+// The matrix-core kernels take 16-bit storage, head dimensions in multiples of 8 (128-bit row chunks) and
+// 16-byte aligned tensors; everything else the interface accepts runs on the scalar family.
+bool scalar_path(const Shape& s, std::initializer_list<const void*> pointers) {
+    return s.dtype == CGPTX_F32 || s.d % 8 != 0 || !aligned16_all(pointers);
+}
+
+unsigned int scalar_blocks(std::size_t rows) { return static_cast<unsigned int>((rows + kScalarWaves - 1) / kScalarWaves); }
+
+int launch_forward(const Shape& s, Params p, bool scalar, hipStream_t stream) {
+    if (scalar) {
+        const std::size_t rows = s.batch * s.qs * s.hq;
+        if (rows / kScalarWaves >= (std::size_t{1} << 31)) return fail(CGPTX_OVERFLOW, "attention: grid too large");
+        return dispatch_dtype(s.dtype, [&]<typename T>() -> int {
+            hipLaunchKernelGGL((attention_forward_scalar_kernel<T>), dim3(scalar_blocks(rows)), dim3(kThreads), 0, stream, p);
+            CGPTX_LAUNCH_CHECK();
+            return CGPTX_OK;
+        });
+    }
     const dim3 grid(static_cast<unsigned int>((s.qs + kBlockRows - 1) / kBlockRows), static_cast<unsigned int>(s.hq),
                     static_cast<unsigned int>(s.batch));
     return dispatch_16bit(s.dtype, [&]<typename T>() -> int {
@@ -1321,7 +1475,7 @@ int launch_forward(const Shape& s, Params p, hipStream_t stream) {
 }
 
 int launch_backward(const Shape& s, Params p, void* dq, void* dk, void* dv, const void* dout, const void* out,
-                    const float* lse, int accumulate, hipStream_t stream) {
+                    const float* lse, int accumulate, bool scalar, hipStream_t stream) {
     const std::size_t rows = s.batch * s.qs * s.hq;
     const std::size_t stat_bytes = stat_block_bytes(rows);
     void* mem = nullptr;
@@ -1332,6 +1486,24 @@ int launch_backward(const Shape& s, Params p, void* dq, void* dk, void* dv, cons
     p.lse = lse;
     p.delta = delta;
     p.accumulate = accumulate;
+    if (scalar) {
+        const std::size_t key_rows = s.batch * s.ks * s.hkv;
+        if (rows / kScalarWaves >= (std::size_t{1} << 31) || key_rows / kScalarWaves >= (std::size_t{1} << 31))
+            return fail(CGPTX_OVERFLOW, "attention: grid too large");
+        return dispatch_dtype(s.dtype, [&]<typename T>() -> int {
+            Params pq = p;
+            pq.out0 = dq;
+            hipLaunchKernelGGL((attention_dq_scalar_kernel<T>), dim3(scalar_blocks(rows)), dim3(kThreads), 0, stream, pq,
+                               out, delta);
+            CGPTX_LAUNCH_CHECK();
+            Params pk = p;
+            pk.out0 = dk;
+            pk.out1 = dv;
+            hipLaunchKernelGGL((attention_dkv_scalar_kernel<T>), dim3(scalar_blocks(key_rows)), dim3(kThreads), 0, stream, pk);
+            CGPTX_LAUNCH_CHECK();
+            return CGPTX_OK;
+        });
+    }
     return dispatch_16bit(s.dtype, [&]<typename T>() -> int {
         const int lpr = s.d <= 32 ? 4 : (s.d <= 64 ? 8 : 16);
         const unsigned int delta_blocks = static_cast<unsigned int>((rows * lpr + kThreads - 1) / kThreads);
@@ -1392,12 +1564,6 @@ int launch_backward(const Shape& s, Params p, void* dq, void* dk, void* dv, cons
     });
 }
 
-bool aligned16_all(std::initializer_list<const void*> pointers) {
-    for (const void* ptr : pointers)
-        if (ptr != nullptr && !is_aligned16(ptr)) return false;
-    return true;
-}
-
 }  // namespace
 }  // namespace cgptx
 
@@ -1413,15 +1579,13 @@ extern "C" int cgptx_flash_gqa_attention_forward(void* output, float* logsumexp,
     if (int st = validate(name, s)) return st;
     if (output == nullptr || query == nullptr || key == nullptr || value == nullptr)
         return fail(CGPTX_INVALID_ARGUMENT, std::string(name) + ": null tensor");
-    if (!aligned16_all({output, query, key, value}))
-        return fail(CGPTX_INVALID_ARGUMENT, std::string(name) + ": tensors must be 16-byte aligned");
     Params p = make_params(s);
     p.out0 = output;
     p.lse_out = logsumexp;
     p.q = query;
     p.k = key;
     p.v = value;
-    return launch_forward(s, p, static_cast<hipStream_t>(stream));
+    return launch_forward(s, p, scalar_path(s, {output, query, key, value}), static_cast<hipStream_t>(stream));
 }
 
 extern "C" int cgptx_flash_gqa_attention_backward_with_lse(
@@ -1438,14 +1602,13 @@ extern "C" int cgptx_flash_gqa_attention_backward_with_lse(
     if (grad_query == nullptr || grad_key == nullptr || grad_value == nullptr || grad_output == nullptr ||
         output == nullptr || logsumexp == nullptr || query == nullptr || key == nullptr || value == nullptr)
         return fail(CGPTX_INVALID_ARGUMENT, std::string(name) + ": null tensor");
-    if (!aligned16_all({grad_query, grad_key, grad_value, grad_output, output, query, key, value}))
-        return fail(CGPTX_INVALID_ARGUMENT, std::string(name) + ": tensors must be 16-byte aligned");
     Params p = make_params(s);
     p.q = query;
     p.k = key;
     p.v = value;
+    const bool scalar = scalar_path(s, {grad_query, grad_key, grad_value, grad_output, output, query, key, value});
     return launch_backward(s, p, grad_query, grad_key, grad_value, grad_output, output, logsumexp,
-                           accumulate_grads != 0, static_cast<hipStream_t>(stream));
+                           accumulate_grads != 0, scalar, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int cgptx_flash_gqa_attention_backward(void* grad_query, void* grad_key, void* grad_value,
@@ -1463,15 +1626,14 @@ extern "C" int cgptx_flash_gqa_attention_backward(void* grad_query, void* grad_k
     if (grad_query == nullptr || grad_key == nullptr || grad_value == nullptr || grad_output == nullptr ||
         query == nullptr || key == nullptr || value == nullptr)
         return fail(CGPTX_INVALID_ARGUMENT, std::string(name) + ": null tensor");
-    if (!aligned16_all({grad_query, grad_key, grad_value, grad_output, query, key, value}))
-        return fail(CGPTX_INVALID_ARGUMENT, std::string(name) + ": tensors must be 16-byte aligned");
+    const bool scalar = scalar_path(s, {grad_query, grad_key, grad_value, grad_output, query, key, value});
     auto stream = static_cast<hipStream_t>(stream_);
     // Recompute the output and the log-sum-exp into scratch, then run the LSE path. The scratch
     // block is laid out [delta | LSE·log2 e | lse | output] so that launch_backward's request for
     // the two-block prefix returns the same base pointer.
     const std::size_t rows = batch * query_sequence * query_heads;
     const std::size_t stat_bytes = stat_block_bytes(rows);
-    const std::size_t out_bytes = rows * head_dim * 2;
+    const std::size_t out_bytes = rows * head_dim * dtype_size(dtype);
     void* mem = nullptr;
     if (int st = scratch(stream, 3 * stat_bytes + out_bytes, &mem)) return st;
     auto* lse = reinterpret_cast<float*>(static_cast<char*>(mem) + 2 * stat_bytes);
@@ -1483,7 +1645,7 @@ extern "C" int cgptx_flash_gqa_attention_backward(void* grad_query, void* grad_k
     Params fwd = p;
     fwd.out0 = out;
     fwd.lse_out = lse;
-    if (int st = launch_forward(s, fwd, stream)) return st;
+    if (int st = launch_forward(s, fwd, scalar, stream)) return st;
     return launch_backward(s, p, grad_query, grad_key, grad_value, grad_output, out, lse, accumulate_grads != 0,
-                           stream);
+                           scalar, stream);
 }

@@ -506,6 +506,8 @@ int validate_config(const cgptx_model_config& c, std::size_t batch, std::size_t 
     const std::size_t rotary = c.rotary_dim == 0 ? c.head_dim : c.rotary_dim;
     if ((rotary & 1) != 0 || rotary > c.head_dim || (c.head_dim & 1) != 0)
         return fail(CGPTX_INVALID_ARGUMENT, "model: head_dim and rotary_dim must be even, rotary_dim <= head_dim");
+    if (c.head_dim > 128)  // the attention operators' limit (src/ops/backward/attention_backward.cu:1886-1887)
+        return fail(CGPTX_INVALID_ARGUMENT, "model: head_dim must not exceed 128");
     if (!std::isfinite(c.rms_epsilon) || c.rms_epsilon <= 0.0f || !std::isfinite(c.rope_base) || c.rope_base <= 0.0f)
         return fail(CGPTX_INVALID_ARGUMENT, "model: invalid epsilon or rope base");
     return CGPTX_OK;

@@ -40,14 +40,16 @@ def rope_cache(sequence, rotary_dim, base=10000.0):
     return torch.cos(theta).contiguous(), torch.sin(theta).contiguous()
 
 
-def train_step(w, tokens, targets, cfg, loss_scale=1.0, optimizer=None, step=1):
-    """One float32 CPU step. Returns (loss, grads). `optimizer` = dict of AdamW options to also update."""
+def forward(w, tokens, cfg):
+    """The reference's CPU forward for whole sequences (src/core/generation_cpu.cpp:323-379: embedding, per layer
+    {RMSNorm, q/k/v projections, per-head RMSNorm, RoPE, attention, o-projection, RMSNorm, gate/up, SwiGLU, down,
+    two adds}, final norm, classifier). Returns (hidden states entering each layer + the last one, the tensors the
+    backward pass needs, normalized, logits)."""
     B, T = tokens.shape
     N, H, I, D, HQ, HKV, V = B * T, cfg["hidden"], cfg["inter"], cfg["d"], cfg["hq"], cfg["hkv"], cfg["vocab"]
     QW, KW, eps = HQ * D, HKV * D, cfg["eps"]
     cos, sin = rope_cache(T, D)
     ids = tokens.reshape(-1).to(torch.int32).contiguous()
-    tg = targets.reshape(-1).to(torch.int32).contiguous()
     E = w["embedding"]
     x = torch.empty(N, H)
     c.embedding_forward(x, ids, E)
@@ -85,6 +87,40 @@ def train_step(w, tokens, targets, cfg, loss_scale=1.0, optimizer=None, step=1):
     normalized, logits = torch.empty(N, H), torch.empty(N, V)
     c.rmsnorm_forward(normalized, x, w["final_norm"], eps)
     c.linear_forward(logits, normalized, E)
+    return [s["x"] for s in saved] + [x], saved, normalized, logits
+
+
+def forward_loss(w, tokens, targets, cfg):
+    """Forward + cross_entropy_forward_cpu (src/ops/cpu/cross_entropy_cpu.cpp): the reference's CPU-runnable
+    configuration. Returns (loss, hidden states [layers + 1], float64 sum of the logits as a checksum)."""
+    hidden, _, _, logits = forward(w, tokens, cfg)
+    loss = torch.empty(1)
+    c.cross_entropy_forward(loss, logits, targets.reshape(-1).to(torch.int32).contiguous())
+    return loss.item(), hidden, float(logits.double().sum())
+
+
+def timed_forward_loss(cfg, batch, sequence, seed=0):
+    """Seconds, loss and logits checksum of one CPU forward + loss on a seeded random batch."""
+    w = make_weights(cfg, seed)
+    g = torch.Generator().manual_seed(seed + 1)
+    tokens = torch.randint(0, cfg["vocab"], (batch, sequence), generator=g)
+    targets = torch.randint(0, cfg["vocab"], (batch, sequence), generator=g)
+    start = time.perf_counter()
+    loss, _, checksum = forward_loss(w, tokens, targets, cfg)
+    return time.perf_counter() - start, loss, checksum
+
+
+def train_step(w, tokens, targets, cfg, loss_scale=1.0, optimizer=None, step=1):
+    """One float32 CPU step. Returns (loss, grads). `optimizer` = dict of AdamW options to also update."""
+    B, T = tokens.shape
+    N, H, I, D, HQ, HKV, V = B * T, cfg["hidden"], cfg["inter"], cfg["d"], cfg["hq"], cfg["hkv"], cfg["vocab"]
+    QW, KW, eps = HQ * D, HKV * D, cfg["eps"]
+    cos, sin = rope_cache(T, D)
+    ids = tokens.reshape(-1).to(torch.int32).contiguous()
+    tg = targets.reshape(-1).to(torch.int32).contiguous()
+    E = w["embedding"]
+    hidden, saved, normalized, logits = forward(w, tokens, cfg)
+    x = hidden[-1]
     loss, dlogits = torch.empty(1), torch.empty(N, V)
     c.cross_entropy_forward_backward(loss, dlogits, logits, tg, loss_scale)
 

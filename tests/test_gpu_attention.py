@@ -222,6 +222,70 @@ def test_long_context_variant(device):
         assert_scaled_close(g, w, TOL[dtype], name)
 
 
+SCALAR_CASES = [  # served by the scalar family: fp32 storage, head_dim not a multiple of 8, unaligned tensors
+    (torch.float32, dict(b=2, qs=40, ks=40, hq=8, hkv=2, d=128)),
+    (torch.float32, dict(b=1, qs=33, ks=70, hq=6, hkv=2, d=64, off=37, scale=0.2)),
+    (torch.float32, dict(b=1, qs=50, ks=90, hq=2, hkv=1, d=20, causal=False)),
+    (torch.float32, dict(b=3, qs=1, ks=1, hq=2, hkv=1, d=128)),
+    (torch.float16, dict(b=1, qs=48, ks=48, hq=4, hkv=2, d=36)),
+    (torch.bfloat16, dict(b=2, qs=30, ks=45, hq=3, hkv=1, d=100, off=15)),
+    (torch.bfloat16, dict(b=1, qs=20, ks=20, hq=2, hkv=2, d=7)),
+    (torch.float32, dict(b=1, qs=3, ks=35, hq=4, hkv=1, d=128, off=32, scale=0.11)),  # flash_attention_test.cu:382-388 in fp32
+]
+
+
+@pytest.mark.parametrize("case", range(len(SCALAR_CASES)))
+@pytest.mark.parametrize("with_lse", [True, False])
+def test_scalar_family_parity(device, case, with_lse):
+    """What the reference serves with its warp-per-row kernels (src/ops/backward/attention_backward.cu:352-504,
+    2044-2068): fp32 storage and any head_dim up to 128. fp32 storage: max |a-b| / max(1, |b|) <= 1e-4 against
+    the float64 formulas; 16-bit storage: 2e-2 of the result's scale."""
+    dtype, c = SCALAR_CASES[case]
+    q, k, v, do = make_inputs(c, dtype, 100 + case)
+    out, lse = run_forward(device, q, k, v, c)
+    want_out, want_lse = oracle64.attention_forward(to_np(q), to_np(k), to_np(v), *oracle_args(c))
+    assert_close(out, want_out, TOL[dtype], "O")
+    assert_close(lse, want_lse, 1e-4 if dtype == torch.float32 else 1e-3, "LSE")
+    want = oracle64.attention_backward(to_np(do), to_np(q), to_np(k), to_np(v), *oracle_args(c))
+    got = run_backward(device, do, q, k, v, c, with_lse)
+    for g, w, name in zip(got, want, ("dQ", "dK", "dV")):
+        if dtype == torch.float32:
+            assert_close(g, w, TOL[dtype], f"{name} scalar case {case}")
+        else:
+            assert_scaled_close(g, w, TOL[dtype], f"{name} scalar case {case}")
+    base = (randn(q.shape, dtype, 91), randn(k.shape, dtype, 92), randn(v.shape, dtype, 93))
+    acc = run_backward(device, do, q, k, v, c, with_lse, accumulate=True, base=base)
+    for a, w, b_, name in zip(acc, want, base, ("dQ", "dK", "dV")):
+        assert_scaled_close(a, w + to_np(b_), TOL[dtype], f"{name} accumulate")
+    again = run_backward(device, do, q, k, v, c, with_lse)
+    for a, b_ in zip(got, again):
+        assert torch.equal(a, b_)   # no atomics: results do not depend on scheduling
+
+
+def test_unaligned_tensors_take_the_scalar_family(device):
+    """Views that start 2 bytes into an allocation are not 16-byte aligned: same results as the aligned call
+    to storage precision (the two families round differently)."""
+    c = dict(b=1, qs=64, ks=64, hq=4, hkv=2, d=64)
+    dtype = torch.float16
+    q, k, v, do = make_inputs(c, dtype, 3)
+
+    def shifted(t):
+        flat = torch.empty(t.numel() + 1, dtype=t.dtype, device=device)
+        view = flat[1:].view(t.shape)
+        view.copy_(t)
+        assert view.data_ptr() % 16 != 0
+        return view
+
+    out, lse = torch.empty_like(q, device=device), torch.empty(q.shape[:3], device=device)
+    ops.flash_gqa_attention_forward_with_lse(out, lse, shifted(q), shifted(k), shifted(v), None, options(c))
+    dq, dk, dv = torch.empty_like(out), torch.empty_like(k, device=device), torch.empty_like(v, device=device)
+    ops.flash_gqa_attention_backward_with_lse(dq, dk, dv, shifted(do), out, lse, shifted(q), shifted(k), shifted(v), None,
+                                              options(c))
+    want = oracle64.attention_backward(to_np(do), to_np(q), to_np(k), to_np(v), *oracle_args(c))
+    for g, w, name in zip((dq, dk, dv), want, ("dQ", "dK", "dV")):
+        assert_scaled_close(g, w, TOL[dtype], name)
+
+
 def test_argument_errors(device):
     q = torch.zeros(1, 4, 4, 32, dtype=torch.float16, device=device)
     k = torch.zeros(1, 4, 2, 32, dtype=torch.float16, device=device)
@@ -238,3 +302,7 @@ def test_argument_errors(device):
                                                   good)
     with pytest.raises(ValueError):  # gradient shape mismatch
         ops.flash_gqa_attention_backward(q.clone(), q.clone(), k.clone(), q, q, k, k, None, good)
+    wide_q = torch.zeros(1, 4, 2, 136, device=device)  # src/ops/backward/attention_backward.cu:1886-1887
+    with pytest.raises(ValueError):
+        ops.flash_gqa_attention_backward(wide_q.clone(), wide_q.clone(), wide_q.clone(), wide_q, wide_q, wide_q, wide_q, None,
+                                         ops.FlashAttentionOptions(2, 2, 136))

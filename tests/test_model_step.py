@@ -328,18 +328,22 @@ def test_block_norms_in_one_pass_match_the_separate_operators(device, monkeypatc
         assert (fused - separate).abs().max().item() <= 2e-2 * scale, name
 
 
+HEADLINE = dict(vocabulary_size=32000, num_layers=8, hidden_size=1024, intermediate_size=2048, num_query_heads=8,
+                num_kv_heads=2, head_dim=128, rotary_dim=128)
+HEADLINE_CFG = dict(vocab=32000, layers=8, hidden=1024, inter=2048, hq=8, hkv=2, d=128, eps=1e-5)
+
+
 @pytest.mark.gpu
-def test_headline_configuration_scales_exactly_replays_exactly_and_starts_at_the_closed_form_loss(device):
-    """The 104m preset at the benchmark's size (B=32, T=1024, bf16), where no CPU composition finishes
-    in test time: properties that hold at any size. The backward pass is linear in the loss scale, and
-    a factor of two is exact in binary floating point, so every gradient at scale 2048 is exactly twice
-    the one at 1024; a hipGraph replay repeats the eager pass bit for bit; the two loss paths agree;
-    a random-init model starts at the closed-form loss of Gaussian logits."""
+@pytest.mark.parametrize("batch,seq", [(32, 1024), (8, 4096)], ids=["b32-t1024", "long-context-b8-t4096"])
+def test_headline_configuration_scales_exactly_replays_exactly_and_starts_at_the_closed_form_loss(device, batch, seq):
+    """The 104m preset at the benchmark's sizes (B=32, T=1024 and the long-context variant B=8, T=4096, bf16),
+    where no CPU composition finishes in test time: properties that hold at any size. The backward pass is
+    linear in the loss scale, and a factor of two is exact in binary floating point, so every gradient at scale
+    2048 is exactly twice the one at 1024; a hipGraph replay repeats the eager pass bit for bit; the two loss
+    paths agree; a random-init model starts at the closed-form loss of Gaussian logits."""
     from cgpt_amd.model import LOSS_CUT, LOSS_DENSE, Model, ModelConfig
 
-    config = ModelConfig(vocabulary_size=32000, num_layers=8, hidden_size=1024, intermediate_size=2048,
-                         num_query_heads=8, num_kv_heads=2, head_dim=128, rotary_dim=128, dtype=torch.bfloat16)
-    batch, seq = 32, 1024
+    config = ModelConfig(dtype=torch.bfloat16, **HEADLINE)
     model = Model(config, batch, seq, seed=0, device=device)
     assert model.num_parameters == 104_090_624
     rng = np.random.default_rng(0)
@@ -376,4 +380,150 @@ def test_headline_configuration_scales_exactly_replays_exactly_and_starts_at_the
     for (name, _, g), b in zip(model.parameters(), base):
         scale = max(float(b.float().abs().max()), 1e-6)
         assert float((g.float() - b.float()).abs().max()) <= 3e-2 * scale, name
+    model.close()
+
+
+@pytest.mark.gpu
+def test_adamw_over_all_104m_parameters_matches_the_float64_update(device):
+    """Two full train steps of the 104m preset at B=32, T=1024 (hipGraph step + adamw_step_many_async over the 90
+    tensors / 104,090,624 parameters: src/optim/adamw.cu:276-346). After each step the master copies, both
+    moments and the 16-bit parameters of every tensor are compared with the float64 update
+    (oracle64.adamw: unscale by the loss scale, one global norm over all tensors, clip to 1, bias correction)
+    applied to the gradients the step left on the device."""
+    from cgpt_amd.model import LOSS_CUT, Model, ModelConfig
+    from cgpt_amd.ops import AdamWOptions
+    from oracle import oracle64
+
+    batch, seq = 32, 1024
+    model = Model(ModelConfig(dtype=torch.bfloat16, **HEADLINE), batch, seq, seed=0, device=device)
+    rng = np.random.default_rng(1)
+    model.set_tokens(rng.integers(0, 32000, size=(batch, seq)), rng.integers(0, 32000, size=(batch, seq)))
+    stream = torch.cuda.Stream(device=device)
+    opt = dict(lr=3e-4, beta1=0.9, beta2=0.95, eps=1e-8, wd=0.1, loss_scale=1024.0, max_grad_norm=1.0)
+    options = AdamWOptions(learning_rate=opt["lr"], beta1=opt["beta1"], beta2=opt["beta2"], epsilon=opt["eps"],
+                           weight_decay=opt["wd"], loss_scale=opt["loss_scale"], max_grad_norm=opt["max_grad_norm"])
+    tensors = model.parameters()
+    assert len(tensors) == 90 and sum(p.numel() for _, p, _ in tensors) == 104_090_624
+    state = [tuple(to_np(t) for t in model.optimizer_state(i)) for i in range(len(tensors))]
+    for (name, p, _), (master, m, v) in zip(tensors, state):   # masters start as the 16-bit parameters, moments at 0
+        assert np.array_equal(master, to_np(p)), name
+        assert not m.any() and not v.any(), name
+    step = 0
+    eps32 = float(np.finfo(np.float32).eps)
+    for _ in range(2):
+        model.train_step(options, LOSS_CUT, use_graph=True, stream=stream)
+        loss, finite, steps = model.status(stream)
+        grads = [to_np(g) for _, _, g in tensors]
+        norm = np.sqrt(sum(((g / opt["loss_scale"]) ** 2).sum() for g in grads))
+        applied, masters, ms, vs, step = oracle64.adamw(
+            None, grads, [s[0] for s in state], [s[1] for s in state], [s[2] for s in state], step, opt["lr"],
+            opt["beta1"], opt["beta2"], opt["eps"], opt["wd"], opt["loss_scale"], opt["max_grad_norm"])
+        assert applied and finite and steps == step, (loss, finite, steps)
+        print(f"[parity] AdamW step {step}: loss {loss:.4f}, unscaled gradient norm {norm:.4f} "
+              f"({'clipped' if norm > opt['max_grad_norm'] else 'not clipped'})")
+        worst = dict(master=0.0, m=0.0, v=0.0)
+        for i, (name, p, _) in enumerate(tensors):
+            got_master, got_m, got_v = (to_np(t) for t in model.optimizer_state(i))
+            # master: the update is lr-sized on parameters up to 1 (norm weights): a thousandth of lr plus the
+            # fp32 representation of the value itself
+            bound = 1e-3 * opt["lr"] + 2 * eps32 * np.abs(masters[i])
+            err = np.abs(got_master - masters[i])
+            assert (err <= bound).all(), f"{name}: master differs by {err.max():.3e}"
+            worst["master"] = max(worst["master"], float(err.max()))
+            for key, got, want in (("m", got_m, ms[i]), ("v", got_v, vs[i])):
+                scale = max(float(np.abs(want).max()), 1e-30)
+                rel = float(np.abs(got - want).max()) / scale
+                assert rel <= 2e-5, f"{name}: {key} differs by {rel:.3e} of its largest entry"
+                worst[key] = max(worst[key], rel)
+            # the 16-bit parameter is the master copy rounded to nearest even
+            assert torch.equal(p, model.optimizer_state(i)[0].to(torch.bfloat16)), name
+            state[i] = (got_master, got_m, got_v)   # the next step starts from what the device holds
+        print(f"[parity] AdamW step {step}: worst master error {worst['master']:.3e} (lr {opt['lr']:.0e}), "
+              f"worst m {worst['m']:.3e}, v {worst['v']:.3e} of the tensor's largest entry")
+    model.close()
+
+
+def cpu_weights_from_model(model, cfg):
+    """The library's weights as the float32 tensors oracle/cpu_model.py takes."""
+    params, _ = params_from_model(model, cfg)
+    as_f32 = lambda a: torch.from_numpy(np.ascontiguousarray(a)).float().contiguous()
+    return {"embedding": as_f32(params["embedding"]), "final_norm": as_f32(params["final_norm"]),
+            "layers": [{k: as_f32(v) for k, v in lw.items()} for lw in params["layers"]]}
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype,tol", [(torch.bfloat16, 4e-2), (torch.float32, 1e-4)], ids=["bf16", "f32"])
+def test_cpu_plumbing_configuration_forward_and_loss_against_the_cpu_port(device, dtype, tol):
+    """The reference's CPU-runnable configuration: 104m dims, B=1, T=256, forward + cross-entropy loss in the
+    order of src/core/generation_cpu.cpp:323-379 + cross_entropy_forward_cpu (oracle/cpu_model.forward_loss, the
+    float32 port; about 40 s on one core, since linear_forward_cpu is serial for more than one row). The GPU
+    forward runs on the same weights (the CPU side reads the library's rounded weights back): the hidden state
+    entering every layer and leaving the last one, and the loss, must agree. bf16 rounds every operator output
+    (2e-2 each, several operators deep: 4e-2 of the state's scale); fp32 storage accumulates in a different
+    order only (1e-4 of the scale; 2e-6 observed)."""
+    from cgpt_amd.model import LOSS_DENSE, Model, ModelConfig
+    from oracle import cpu_model
+
+    cfg, batch, seq = HEADLINE_CFG, 1, 256
+    model = Model(ModelConfig(dtype=dtype, **HEADLINE), batch, seq, seed=0, device=device)
+    g = torch.Generator().manual_seed(1)
+    tokens = torch.randint(0, cfg["vocab"], (batch, seq), generator=g)
+    targets = torch.randint(0, cfg["vocab"], (batch, seq), generator=g)
+    model.set_tokens(tokens.numpy(), targets.numpy())
+    model.forward_backward(1.0, LOSS_DENSE, use_graph=False)
+    loss, _, _ = model.status()
+    want_loss, want_hidden, want_checksum = cpu_model.forward_loss(cpu_weights_from_model(model, cfg), tokens, targets, cfg)
+    print(f"[parity] configuration 1 ({dtype}): GPU loss {loss:.6f}, CPU port {want_loss:.6f}, logits checksum {want_checksum:.4f}")
+    assert abs(loss - want_loss) <= (5e-3 if dtype == torch.bfloat16 else 1e-4) * want_loss
+    for l, want in enumerate(want_hidden):
+        got = to_np(model.activation(f"hidden.{l}")).reshape(batch * seq, cfg["hidden"])
+        scale = max(1.0, float(want.abs().max()))
+        err = float(np.abs(got - to_np(want)).max()) / scale
+        print(f"[parity] hidden.{l}: {err:.3e} of scale {scale:.3g}")
+        assert err <= tol, f"hidden state {l}: {err:.3e}"
+    # the checksum follows from logits that agree element by element: N*V terms with errors below tol each
+    logits = to_np(model.activation("logits"))
+    assert abs(logits.sum() - want_checksum) <= tol * np.abs(logits).sum()
+    model.close()
+
+
+@pytest.mark.gpu
+def test_graph_is_recorded_again_after_the_scratch_arena_moves(device):
+    """A recorded step holds addresses inside the stream's scratch arena. Releasing the arena
+    (cgptx_release_scratch), or an operator on the same stream that needs a larger one, frees that block: the
+    next graph step must notice, run eagerly and record again, and give the same bits as before."""
+    from cgpt_amd import capi, ops
+
+    cfg, dtype, batch, seq = MODEL_CFG, torch.bfloat16, 2, 40
+    rng = np.random.default_rng(8)
+    model = build(device, dtype, batch, seq, cfg)
+    model.set_tokens(rng.integers(0, cfg["vocab"], size=(batch, seq)), rng.integers(0, cfg["vocab"], size=(batch, seq)))
+    stream = torch.cuda.Stream(device=device)
+
+    def step():
+        for _, _, g in model.parameters():
+            g.zero_()
+        torch.cuda.synchronize()
+        model.forward_backward(64.0, 1, use_graph=True, stream=stream)
+        return model.status(stream)[0], [g.clone() for _, _, g in model.parameters()]
+
+    step()                      # eager + capture
+    want = step()               # replay
+    capi.call("cgptx_release_scratch")
+    # fill the freed block with other data so that a stale replay could not pass by accident
+    junk = [torch.full((1 << 20,), 1e30, device=device) for _ in range(8)]
+    after_release = step()
+    with torch.cuda.stream(stream):   # a larger request on the same stream reallocates the arena
+        big_rows = 1 << 16
+        x = torch.randn(big_rows, 1024, device=device).to(dtype)
+        dx, dw = torch.empty_like(x), torch.empty(1024, dtype=dtype, device=device)
+        ops.rmsnorm_backward(dx, dw, x, x, torch.ones(1024, dtype=dtype, device=device), 1e-5, stream=stream)
+    torch.cuda.synchronize()
+    after_growth = step()
+    replay = step()
+    del junk
+    for name, (loss, grads) in (("release", after_release), ("growth", after_growth), ("replay", replay)):
+        assert loss == want[0], name
+        for a, b in zip(grads, want[1]):
+            assert torch.equal(a, b), name
     model.close()
