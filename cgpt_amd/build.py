@@ -72,19 +72,20 @@ def build(force: bool = True, jobs: int | None = None) -> pathlib.Path:
     return LIB_PATH
 
 
-INTERFACE_TEST_SOURCE = ROOT / "tests" / "cpp" / "ops_interface_test.cpp"
+INTERFACE_TEST_SOURCES = [ROOT / "tests" / "cpp" / "ops_interface_test.cpp", ROOT / "tests" / "cpp" / "block_backward_test.cpp"]
 INTERFACE_TEST_BINARY = ROOT / "tests" / "cpp" / "ops_interface_test.bin"
 
 
 def build_interface_test() -> pathlib.Path:
-    """Compiles the C++ program that drives include/ops/**, include/optim/** against the library.
-    Host code only (the headers are inline wrappers over the C-ABI); linked with an rpath relative to
-    the binary so that it runs from any checkout location."""
-    cmd = [HIPCC, "-std=c++20", "-O1", f"-I{ROOT / 'include'}", str(INTERFACE_TEST_SOURCE), "-o",
-           str(INTERFACE_TEST_BINARY), f"-L{LIB_DIR}", "-lcgptx", "-Wl,-rpath,$ORIGIN/../../cgpt_amd/lib"]
-    proc = subprocess.run(cmd, capture_output=True, text=True)
-    if proc.returncode != 0:
-        raise RuntimeError(f"interface test build failed:\n{proc.stderr}")
+    """Compiles the C++ programs that drive include/core, include/ops/**, include/optim/** against the library
+    (tests/cpp/*.cpp -> *.bin). Host code only (the headers are inline wrappers over the C-ABI); linked with an
+    rpath relative to the binary so that they run from any checkout location."""
+    for source in INTERFACE_TEST_SOURCES:
+        cmd = [HIPCC, "-std=c++20", "-O1", f"-I{ROOT / 'include'}", str(source), "-o", str(source.with_suffix(".bin")),
+               f"-L{LIB_DIR}", "-lcgptx", "-Wl,-rpath,$ORIGIN/../../cgpt_amd/lib"]
+        proc = subprocess.run(cmd, capture_output=True, text=True)
+        if proc.returncode != 0:
+            raise RuntimeError(f"interface test build failed ({source.name}):\n{proc.stderr}")
     return INTERFACE_TEST_BINARY
 
 

@@ -347,7 +347,108 @@ bool fused_swiglu() {
     return text == nullptr || text[0] != '0';
 }
 
+// CGPTX_FUSE=0: the step as the reference's own call sequence, one public operator per call — forward in the
+// order of src/core/transformer_block.cu:466-595, backward in the order of :663-747 and
+// src/core/transformer_model.cu:360-380 (separate q / k / v and gate / up projections with accumulating input
+// gradients, separate SwiGLU and RoPE passes, residual additions as `add` calls). It is what a caller of
+// include/ops/** executes, so its results are the yardstick for the fused step and for callers' own block code.
+// The halves of the [rows, 2I] gate_up buffers serve as the separate [rows, I] gate and up tensors.
+bool reference_call_sequence() {
+    const char* text = std::getenv("CGPTX_FUSE");  // read per enqueue
+    return text != nullptr && text[0] == '0';
+}
+
+int enqueue_reference_sequence(cgptx_model* m, float loss_scale, int loss_mode, hipStream_t stream) {
+    const auto& c = m->config;
+    const int dt = c.dtype;
+    const std::size_t N = m->rows, H = c.hidden_size, I = c.intermediate_size;
+    const std::size_t HQ = c.num_query_heads, HKV = c.num_kv_heads, D = c.head_dim;
+    const std::size_t QW = HQ * D, KW = HKV * D, elem = dtype_size(dt);
+    const float eps = c.rms_epsilon;
+    auto* s = static_cast<cgptx_stream>(stream);
+    auto second_half = [&](void* gate_up) { return static_cast<void*>(static_cast<char*>(gate_up) + N * I * elem); };
+
+    CGPTX_OP("embedding_fwd", cgptx_embedding_forward(m->hidden[0], m->tokens, N, m->embedding.value, c.vocabulary_size, H, dt, s));
+    for (std::size_t l = 0; l < c.num_layers; ++l) {
+        const auto& w = m->layers[l];
+        const auto& a = m->acts[l];
+        void *x = m->hidden[l], *out = m->hidden[l + 1];
+        void *projected = m->d_norm_in, *ffn = m->d_norm_in_f;  // backward workspace, free during the forward pass
+        void *gate = a.gate_up, *up = second_half(a.gate_up);
+        CGPTX_OP("rmsnorm_fwd", cgptx_rmsnorm_forward(a.norm_a, x, w.attention_norm.value, N, H, eps, dt, s));
+        CGPTX_OP("gemm_fwd", cgptx_linear_forward(a.q_pre, a.norm_a, w.q.value, nullptr, N, H, QW, dt, s));
+        CGPTX_OP("gemm_fwd", cgptx_linear_forward(a.k_pre, a.norm_a, w.k.value, nullptr, N, H, KW, dt, s));
+        CGPTX_OP("gemm_fwd", cgptx_linear_forward(a.v, a.norm_a, w.v.value, nullptr, N, H, KW, dt, s));
+        CGPTX_OP("rmsnorm_fwd", cgptx_rmsnorm_forward(a.q, a.q_pre, w.q_norm.value, N * HQ, D, eps, dt, s));
+        CGPTX_OP("rmsnorm_fwd", cgptx_rmsnorm_forward(a.k, a.k_pre, w.k_norm.value, N * HKV, D, eps, dt, s));
+        CGPTX_OP("rope_fwd", cgptx_rope_forward(a.q, a.k, m->cos_cache, m->sin_cache, m->batch, m->sequence, HQ, HKV, D,
+                                                c.rotary_dim, 0, m->sequence, dt, s));
+        CGPTX_OP("attn_fwd", cgptx_flash_gqa_attention_forward(a.attn_out, a.lse, a.q, a.k, a.v, m->batch, m->sequence,
+                                                               m->sequence, HQ, HKV, D, 0.0f, 1, 0, dt, s));
+        CGPTX_OP("gemm_fwd", cgptx_linear_forward(projected, a.attn_out, w.o.value, nullptr, N, QW, H, dt, s));
+        CGPTX_OP("rmsnorm_fwd", cgptx_rmsnorm_forward(a.norm_f, x, w.ffn_norm.value, N, H, eps, dt, s));
+        CGPTX_OP("gemm_fwd", cgptx_linear_forward(gate, a.norm_f, w.gate.value, nullptr, N, H, I, dt, s));
+        CGPTX_OP("gemm_fwd", cgptx_linear_forward(up, a.norm_f, w.up.value, nullptr, N, H, I, dt, s));
+        CGPTX_OP("swiglu_fwd", cgptx_swiglu_forward(a.act, gate, up, N * I, dt, s));
+        CGPTX_OP("gemm_fwd", cgptx_linear_forward(ffn, a.act, w.down.value, nullptr, N, I, H, dt, s));
+        CGPTX_OP("add", cgptx_add(out, x, projected, N * H, dt, s));
+        CGPTX_OP("add", cgptx_add(out, out, ffn, N * H, dt, s));
+    }
+    void* last = m->hidden[c.num_layers];
+    CGPTX_OP("rmsnorm_fwd", cgptx_rmsnorm_forward(m->normalized, last, m->final_norm.value, N, H, eps, dt, s));
+    if (loss_mode == CGPTX_LOSS_CUT) {
+        CGPTX_OP("cut_ce", cgptx_cut_cross_entropy_forward_backward(m->loss, m->d_normalized, m->embedding.gradient, m->normalized,
+                                                                    m->embedding.value, m->targets, N, H, c.vocabulary_size,
+                                                                    loss_scale, 0, dt, s));
+    } else {
+        CGPTX_OP("gemm_fwd", cgptx_linear_forward(m->logits, m->normalized, m->embedding.value, nullptr, N, H, c.vocabulary_size, dt, s));
+        CGPTX_OP("dense_ce", cgptx_cross_entropy_forward_backward(m->loss, m->grad_logits, m->logits, m->targets, N,
+                                                                  c.vocabulary_size, loss_scale, dt, s));
+        CGPTX_TRY(linear_backward_split(m, m->d_normalized, m->embedding.gradient, m->grad_logits, m->normalized,
+                                        m->embedding.value, N, H, c.vocabulary_size, 0, dt, stream));
+    }
+
+    void *current = m->grad_a, *previous = m->grad_b;
+    CGPTX_OP("rmsnorm_bwd", cgptx_rmsnorm_backward(current, m->final_norm.gradient, m->d_normalized, last, m->final_norm.value, N,
+                                                   H, eps, dt, s));
+    for (std::size_t reverse = c.num_layers; reverse-- > 0;) {
+        const auto& w = m->layers[reverse];
+        const auto& a = m->acts[reverse];
+        void* x = m->hidden[reverse];
+        void *gate = a.gate_up, *up = second_half(a.gate_up);
+        void *d_gate = m->d_gate_up, *d_up = second_half(m->d_gate_up);
+        void* grad_residual = m->d_norm_in_f;
+        CGPTX_TRY(linear_backward_split(m, m->d_act, w.down.gradient, current, a.act, w.down.value, N, I, H, 0, dt, stream));
+        CGPTX_OP("swiglu_bwd", cgptx_swiglu_backward(d_gate, d_up, m->d_act, gate, up, N * I, 0, 0, dt, s));
+        CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.gate.gradient, d_gate, a.norm_f, w.gate.value, N, H, I, 0, dt, stream));
+        CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.up.gradient, d_up, a.norm_f, w.up.value, N, H, I, 1, dt, stream));
+        CGPTX_OP("rmsnorm_bwd", cgptx_rmsnorm_backward(grad_residual, w.ffn_norm.gradient, m->d_norm_in, x, w.ffn_norm.value, N, H,
+                                                       eps, dt, s));
+        CGPTX_OP("add", cgptx_add(previous, current, grad_residual, N * H, dt, s));  // grad_input = grad_output + grad_residual
+        CGPTX_TRY(linear_backward_split(m, m->d_attn_out, w.o.gradient, current, a.attn_out, w.o.value, N, QW, H, 0, dt, stream));
+        CGPTX_OP("attn_bwd", cgptx_flash_gqa_attention_backward_with_lse(m->d_q, m->d_k, m->d_v, m->d_attn_out, a.attn_out, a.lse,
+                                                                         a.q, a.k, a.v, m->batch, m->sequence, m->sequence, HQ,
+                                                                         HKV, D, 0.0f, 1, 0, 0, dt, s));
+        CGPTX_OP("rope_bwd", cgptx_rope_backward(m->d_q_pre, m->d_k_pre, m->d_q, m->d_k, m->cos_cache, m->sin_cache, m->batch,
+                                                 m->sequence, HQ, HKV, D, c.rotary_dim, 0, m->sequence, dt, s));
+        CGPTX_OP("rmsnorm_bwd", cgptx_rmsnorm_backward(m->d_q, w.q_norm.gradient, m->d_q_pre, a.q_pre, w.q_norm.value, N * HQ, D,
+                                                       eps, dt, s));
+        CGPTX_OP("rmsnorm_bwd", cgptx_rmsnorm_backward(m->d_k, w.k_norm.gradient, m->d_k_pre, a.k_pre, w.k_norm.value, N * HKV, D,
+                                                       eps, dt, s));
+        CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.q.gradient, m->d_q, a.norm_a, w.q.value, N, H, QW, 0, dt, stream));
+        CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.k.gradient, m->d_k, a.norm_a, w.k.value, N, H, KW, 1, dt, stream));
+        CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.v.gradient, m->d_v, a.norm_a, w.v.value, N, H, KW, 1, dt, stream));
+        CGPTX_OP("rmsnorm_bwd", cgptx_rmsnorm_backward(grad_residual, w.attention_norm.gradient, m->d_norm_in, x,
+                                                       w.attention_norm.value, N, H, eps, dt, s));
+        CGPTX_OP("add", cgptx_add(previous, previous, grad_residual, N * H, dt, s));
+        std::swap(current, previous);
+    }
+    CGPTX_OP("embedding_bwd", cgptx_embedding_backward(m->embedding.gradient, current, m->tokens, N, c.vocabulary_size, H, 1, 1, dt, s));
+    return CGPTX_OK;
+}
+
 int enqueue_forward_backward(cgptx_model* m, float loss_scale, int loss_mode, hipStream_t stream) {
+    if (reference_call_sequence()) return enqueue_reference_sequence(m, loss_scale, loss_mode, stream);
     const auto& c = m->config;
     const int dt = c.dtype;
     const std::size_t N = m->rows, H = c.hidden_size, I = c.intermediate_size;
@@ -931,6 +1032,11 @@ extern "C" int cgptx_model_activation(const cgptx_model* m, const char* name, vo
     const std::size_t NH = m->rows * m->config.hidden_size;
     if (n == "normalized") { *data = m->normalized; *count = NH; return CGPTX_OK; }
     if (n == "loss") { *data = m->loss; *count = 1; return CGPTX_OK; }
+    if (n == "rope.cos" || n == "rope.sin") {  // [sequence, rotary_dim / 2] in the storage dtype
+        *data = n == "rope.cos" ? m->cos_cache : m->sin_cache;
+        *count = m->sequence * (m->config.rotary_dim / 2);
+        return CGPTX_OK;
+    }
     if (n == "logits" && m->logits != nullptr) {
         *data = m->logits;
         *count = m->rows * m->config.vocabulary_size;
@@ -939,6 +1045,36 @@ extern "C" int cgptx_model_activation(const cgptx_model* m, const char* name, vo
     if (n.rfind("hidden.", 0) == 0) {
         const std::size_t l = std::stoul(n.substr(7));
         if (l < m->hidden.size()) { *data = m->hidden[l]; *count = NH; return CGPTX_OK; }
+    }
+    // Gradient of the loss with respect to hidden.0 / hidden.1 as the last backward pass left them (the two
+    // residual-stream gradient buffers alternate per block, so only the first block's pair survives a step).
+    if (n == "grad.hidden.0" || n == "grad.hidden.1") {
+        const bool even = m->config.num_layers % 2 == 0;  // d hidden[L] is in grad_a; each block switches buffers
+        const bool in_a = (n == "grad.hidden.0") ? even : !even;
+        *data = in_a ? m->grad_a : m->grad_b;
+        *count = NH;
+        return CGPTX_OK;
+    }
+    // Saved tensors of one block: "layer.<l>.<name>".
+    if (n.rfind("layer.", 0) == 0) {
+        const std::size_t dot = n.find('.', 6);
+        if (dot != std::string::npos) {
+            const std::size_t l = std::stoul(n.substr(6, dot - 6));
+            const std::string what = n.substr(dot + 1);
+            const auto& c = m->config;
+            const std::size_t QW = m->rows * c.num_query_heads * c.head_dim, KW = m->rows * c.num_kv_heads * c.head_dim;
+            const std::size_t NI = m->rows * c.intermediate_size;
+            if (l < m->acts.size()) {
+                const auto& a = m->acts[l];
+                const struct { const char* name; void* ptr; std::size_t elements; } table[] = {
+                    {"attention_norm_output", a.norm_a, NH}, {"query_pre_norm", a.q_pre, QW}, {"key_pre_norm", a.k_pre, KW},
+                    {"query", a.q, QW}, {"key", a.k, KW}, {"value", a.v, KW}, {"attention_output", a.attn_out, QW},
+                    {"logsumexp", a.lse, m->rows * c.num_query_heads}, {"ffn_norm_output", a.norm_f, NH},
+                    {"gate_up", a.gate_up, 2 * NI}, {"activated", a.act, NI}};
+                for (const auto& entry : table)
+                    if (what == entry.name) { *data = entry.ptr; *count = entry.elements; return CGPTX_OK; }
+            }
+        }
     }
     return fail(CGPTX_INVALID_ARGUMENT, "model_activation: unknown activation " + n);
 }

@@ -125,8 +125,19 @@ int cgptx_model_load_checkpoint(cgptx_model* model, const char* directory);
 int cgptx_model_save_optimizer(const cgptx_model* model, const char* path, uint64_t step);
 int cgptx_model_load_optimizer(cgptx_model* model, const char* path, uint64_t* step);
 
-/* Device pointer to a named saved activation of the last forward ("hidden.<l>", "logits" ...);
- * used by tests. Returns INVALID_ARGUMENT for unknown names. */
+/* Device pointer to a named tensor of the last step, for tests and for callers that run their own block code
+ * on the saved state: "hidden.<l>" (input of block l; l = num_layers: the last block's output), "normalized",
+ * "loss", "logits" (dense loss only), "rope.cos" / "rope.sin" ([sequence, rotary_dim/2]),
+ * "layer.<l>.<name>" with name one of attention_norm_output, query_pre_norm, key_pre_norm, query, key, value,
+ * attention_output, logsumexp (fp32), ffn_norm_output, gate_up ([rows, 2I] = [gate | up]; with CGPTX_FUSE=0 its two
+ * halves are the separate [rows, I] gate and up tensors), activated; "grad.hidden.0" / "grad.hidden.1" (the
+ * residual-stream gradients the first block's backward read and wrote). *count is in elements. Returns
+ * INVALID_ARGUMENT for unknown names.
+ *
+ * Environment switches read at every enqueue (a recorded graph keeps what it was recorded with):
+ * CGPTX_FUSE=0 runs the step as the reference's own call sequence, one public operator per call
+ * (src/core/transformer_block.cu:466-595, 663-747); CGPTX_FUSE_QK=0, CGPTX_FUSE_NORMS=0 and CGPTX_FUSE_SWIGLU=0
+ * switch single fusions of the default step off. */
 int cgptx_model_activation(const cgptx_model* model, const char* name, void** data, size_t* count);
 
 #ifdef __cplusplus

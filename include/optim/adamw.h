@@ -85,8 +85,8 @@ inline AdamWState AdamWState::for_parameter(const Tensor& parameter, hipStream_t
     if (stream != nullptr && hipStreamSynchronize(stream) != hipSuccess) throw std::runtime_error("AdamWState: sync failed");
     AdamWState state;
     state.master_parameter = Tensor(parameter.shape(), DeviceType::GPU, Dtype::F32);
-    state.first_moment = Tensor::zeros(parameter.shape(), DeviceType::GPU, Dtype::F32);
-    state.second_moment = Tensor::zeros(parameter.shape(), DeviceType::GPU, Dtype::F32);
+    state.first_moment = Tensor::zeros(parameter.shape(), DeviceType::GPU, stream, Dtype::F32);
+    state.second_moment = Tensor::zeros(parameter.shape(), DeviceType::GPU, stream, Dtype::F32);
     const std::size_t count = parameter.numel();
     std::vector<std::uint8_t> raw(parameter.nbytes());
     parameter.copy_raw_to_host(raw);

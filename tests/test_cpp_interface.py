@@ -66,3 +66,15 @@ def test_interface_program_replays_reference_known_answers():
     proc = subprocess.run([str(binary)], capture_output=True, text=True, timeout=120)
     assert proc.returncode == 0, proc.stdout + proc.stderr
     assert "0 failure(s)" in proc.stdout
+
+
+@pytest.mark.gpu
+def test_block_backward_written_against_the_headers_matches_the_library_step():
+    """tests/cpp/block_backward_test.cpp: the reference's transformer_block_backward call sequence
+    (src/core/transformer_block.cu:644-748) against include/ only, eagerly and from a HipGraph capture, bit for bit
+    equal to the library's step run as the reference's call sequence (CGPTX_FUSE=0)."""
+    binary = ROOT / "tests" / "cpp" / "block_backward_test.bin"
+    assert binary.exists(), "build it with `python -m cgpt_amd.build` (there is no fallback)"
+    proc = subprocess.run([str(binary)], capture_output=True, text=True, timeout=120)
+    assert proc.returncode == 0, proc.stdout + proc.stderr
+    assert "0 failure(s)" in proc.stdout

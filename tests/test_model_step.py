@@ -527,3 +527,31 @@ def test_graph_is_recorded_again_after_the_scratch_arena_moves(device):
         for a, b in zip(grads, want[1]):
             assert torch.equal(a, b), name
     model.close()
+
+
+@pytest.mark.gpu
+def test_step_as_the_reference_call_sequence_agrees_with_the_fused_step(device, monkeypatch):
+    """CGPTX_FUSE=0 runs the step as the reference's own call sequence (one public operator per call: separate
+    q / k / v and gate / up projections with accumulating input gradients, separate SwiGLU, RoPE and residual
+    additions). The default step fuses across those boundaries and rounds less often: the two agree to storage
+    precision, the loss almost exactly."""
+    from cgpt_amd.model import LOSS_CUT, Model, ModelConfig
+    config = ModelConfig(vocabulary_size=512, num_layers=2, hidden_size=256, intermediate_size=512, num_query_heads=2,
+                         num_kv_heads=2, head_dim=128, rotary_dim=128, dtype=torch.bfloat16)
+    rng = np.random.default_rng(9)
+    inputs, targets = rng.integers(0, 512, size=(2, 64)), rng.integers(0, 512, size=(2, 64))
+    results = []
+    for fuse in ("1", "0"):
+        monkeypatch.setenv("CGPTX_FUSE", fuse)
+        model = Model(config, 2, 64, seed=6, device=device)
+        model.set_tokens(inputs, targets)
+        model.forward_backward(loss_scale=64.0, loss_mode=LOSS_CUT)
+        results.append((model.status()[0], {n: g.float().cpu() for n, _, g in model.parameters()},
+                        model.activation("hidden.2").float().cpu()))
+        model.close()
+    assert abs(results[0][0] - results[1][0]) <= 1e-3 * results[1][0]
+    assert (results[0][2] - results[1][2]).abs().max().item() <= 4e-2 * max(1.0, results[1][2].abs().max().item())
+    for name, fused in results[0][1].items():
+        separate = results[1][1][name]
+        scale = separate.abs().max().item() + 1e-12
+        assert (fused - separate).abs().max().item() <= 3e-2 * scale, name
