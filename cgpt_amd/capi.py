@@ -49,6 +49,7 @@ class ModelConfig(ctypes.Structure):
 PROTOTYPES = {
     "cgptx_release_scratch": [],
     "cgptx_rmsnorm_backward": [_vp, _vp, _vp, _vp, _vp, _sz, _sz, _f, _i, _vp],
+    "cgptx_rmsnorm_backward_static": [_vp, _vp, _vp, _vp, _vp, _sz, _sz, _f, _i, _vp],
     "cgptx_rope_backward": [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz, _sz, _sz, _sz, _i, _vp],
     "cgptx_swiglu_backward": [_vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _vp],
     "cgptx_swiglu_backward_packed": [_vp, _vp, _vp, _sz, _sz, _i, _i, _vp],

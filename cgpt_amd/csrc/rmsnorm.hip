@@ -710,9 +710,27 @@ int rmsnorm_backward_dual(void* grad_input, void* grad_weight_a, void* grad_weig
     });
 }
 
-int rmsnorm_backward_residual(void* grad_input, void* grad_weight, const void* grad_output, const void* input,
-                              const void* weight, const void* residual, std::size_t rows, std::size_t hidden,
-                              float epsilon, int dtype, hipStream_t stream) {
+namespace {
+// Where rmsnorm_backward's partial sums go: the per-stream arena (fixed == nullptr), or a caller-provided block
+// of `fixed_bytes` that is never exceeded (a larger need is an error, nothing is allocated).
+struct Workspace {
+    hipStream_t stream;
+    void* fixed;
+    std::size_t fixed_bytes;
+    int get(std::size_t bytes, void** out) const {
+        if (fixed == nullptr) return scratch(stream, bytes, out);
+        if (bytes > fixed_bytes)
+            return fail(CGPTX_INVALID_ARGUMENT, "rmsnorm_backward_static: the shape needs " + std::to_string(bytes) +
+                                                    " bytes of working memory, the built-in block holds " +
+                                                    std::to_string(fixed_bytes));
+        *out = fixed;
+        return CGPTX_OK;
+    }
+};
+
+int rmsnorm_backward_impl(void* grad_input, void* grad_weight, const void* grad_output, const void* input,
+                          const void* weight, const void* residual, std::size_t rows, std::size_t hidden,
+                          float epsilon, int dtype, hipStream_t stream, const Workspace& workspace) {
     if (int s = validate(grad_input, grad_output, input, rows, hidden, epsilon, dtype, "rmsnorm_backward")) return s;
     if (grad_weight == nullptr || weight == nullptr)
         return fail(CGPTX_INVALID_ARGUMENT, "rmsnorm_backward: null weight tensor");
@@ -732,7 +750,7 @@ int rmsnorm_backward_residual(void* grad_input, void* grad_weight, const void* g
             const int slices = wide_reduce_slices(blocks, h, compute_units());
             void* mem = nullptr;
             const std::size_t partial_bytes = static_cast<std::size_t>(blocks) * hidden * sizeof(float);
-            if (int s = scratch(stream, partial_bytes + static_cast<std::size_t>(slices) * hidden * sizeof(float), &mem))
+            if (int s = workspace.get(partial_bytes + static_cast<std::size_t>(slices) * hidden * sizeof(float), &mem))
                 return s;
             auto* partial = static_cast<float*>(mem);
             if (int s = launch_fast<T, true>(shape, dx, partial, dy, res, x, w, r, h, epsilon, blocks, stream)) return s;
@@ -755,7 +773,7 @@ int rmsnorm_backward_residual(void* grad_input, void* grad_weight, const void* g
         const int rows_per_slice = (r + slices - 1) / slices;
         void* mem = nullptr;
         const std::size_t inv_bytes = (rows * sizeof(float) + 255) & ~std::size_t{255};
-        if (int s = scratch(stream, inv_bytes + static_cast<std::size_t>(slices) * hidden * sizeof(float), &mem))
+        if (int s = workspace.get(inv_bytes + static_cast<std::size_t>(slices) * hidden * sizeof(float), &mem))
             return s;
         auto* inv_rms = static_cast<float*>(mem);
         auto* partial = reinterpret_cast<float*>(static_cast<char*>(mem) + inv_bytes);
@@ -773,8 +791,57 @@ int rmsnorm_backward_residual(void* grad_input, void* grad_weight, const void* g
         return CGPTX_OK;
     });
 }
+}  // namespace
+
+int rmsnorm_backward_residual(void* grad_input, void* grad_weight, const void* grad_output, const void* input,
+                              const void* weight, const void* residual, std::size_t rows, std::size_t hidden,
+                              float epsilon, int dtype, hipStream_t stream) {
+    return rmsnorm_backward_impl(grad_input, grad_weight, grad_output, input, weight, residual, rows, hidden, epsilon, dtype,
+                                 stream, Workspace{stream, nullptr, 0});
+}
 
 }  // namespace cgptx
+
+// ---- rmsnorm_backward without any allocation ------------------------------------------------------------------
+// The partial sums of the weight gradient live in a block that is part of the library's device image: every
+// GPU the library runs on holds its own copy, at its own address, until the process ends. Host code reaches it
+// only through the address hipGetSymbolAddress returns for the current device (the array's name is a host-side
+// stand-in, not a device address), looked up once per device and kept.
+namespace {
+constexpr std::size_t kStaticScratchBytes = std::size_t{16} << 20;
+static __device__ __align__(256) unsigned char g_static_scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_static_scratch_mutex;
+void* g_static_scratch_address[kMaxDevices] = {};  // per device; null until first use on that device
+
+int static_scratch_address(void** out) {
+    int device = 0;
+    CGPTX_HIP(hipGetDevice(&device));
+    if (device < 0 || device >= kMaxDevices) return cgptx::fail(CGPTX_RUNTIME, "rmsnorm_backward_static: device index out of range");
+    std::lock_guard<std::mutex> lock(g_static_scratch_mutex);
+    if (g_static_scratch_address[device] == nullptr) {
+        void* address = nullptr;
+        CGPTX_HIP(hipGetSymbolAddress(&address, HIP_SYMBOL(g_static_scratch)));
+        if (address == nullptr) return cgptx::fail(CGPTX_RUNTIME, "rmsnorm_backward_static: no device address for the working block");
+        g_static_scratch_address[device] = address;
+    }
+    *out = g_static_scratch_address[device];
+    return CGPTX_OK;
+}
+}  // namespace
+
+extern "C" int cgptx_rmsnorm_backward_static(void* grad_input, void* grad_weight, const void* grad_output, const void* input,
+                                             const void* weight, size_t rows, size_t hidden, float epsilon, int dtype,
+                                             cgptx_stream stream_) {
+    void* block = nullptr;
+    if (int s = static_scratch_address(&block)) return s;
+    auto stream = static_cast<hipStream_t>(stream_);
+    // Nothing in the block has to start at zero: the row kernel writes every partial-sum row it is launched
+    // with before the reduction kernels, later on the same stream, read them.
+    return cgptx::rmsnorm_backward_impl(grad_input, grad_weight, grad_output, input, weight, nullptr, rows, hidden, epsilon,
+                                        dtype, stream, cgptx::Workspace{stream, block, kStaticScratchBytes});
+}
 
 extern "C" int cgptx_rmsnorm_backward(void* grad_input, void* grad_weight, const void* grad_output, const void* input,
                                       const void* weight, size_t rows, size_t hidden, float epsilon, int dtype,

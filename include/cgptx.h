@@ -61,6 +61,21 @@ int cgptx_rmsnorm_backward(void* grad_input, void* grad_weight,
                            const void* weight, size_t rows, size_t hidden,
                            float epsilon, int dtype, cgptx_stream stream);
 
+/* rmsnorm_backward that allocates nothing. No counterpart in the reference: it is for callers that cannot
+ * allocate device memory — code under hipGraph capture that has not run eagerly first, tight serving loops,
+ * harnesses that forbid hipMalloc. Same arguments, kernels and results (bit for bit) as cgptx_rmsnorm_backward;
+ * the partial sums of the weight gradient go to a 16 MiB block built into the library's device image (each GPU
+ * the library runs on holds one until the process ends) instead of the per-stream arena. A shape that needs
+ * more (4 bytes x hidden x the blocks resident on the device, at most a few thousand, for hidden sizes the row
+ * kernel takes: multiples of 8 up to 2048 in 16-bit storage; else 4 bytes x rows + 1 KiB x hidden) returns
+ * CGPTX_INVALID_ARGUMENT with both sizes in the message, before anything is launched. Calls no hipMalloc / hipFree. Every call on a GPU
+ * shares that GPU's block: calls that overlap on one GPU (different streams or threads) race; calls on one
+ * stream are ordered. */
+int cgptx_rmsnorm_backward_static(void* grad_input, void* grad_weight,
+                                  const void* grad_output, const void* input,
+                                  const void* weight, size_t rows, size_t hidden,
+                                  float epsilon, int dtype, cgptx_stream stream);
+
 /* rope_backward — include/ops/backward/rope_backward.h:22-31.
  * q grads [batch, sequence, query_heads, head_dim], k grads [.., kv_heads, ..],
  * caches [cache_positions, rotary_dim/2]; adjacent pairs (2p, 2p+1) rotate by

@@ -1,0 +1,50 @@
+"""cgptx_rmsnorm_backward_static — the entry point that allocates nothing (its working memory is a block inside
+the library's device image) — against cgptx_rmsnorm_backward, through the C-ABI, bit for bit: the two share
+their kernels and launch shapes, so any difference is a fault in how the built-in block is addressed. Two calls
+in a row, the second with a smaller input (the block keeps the first call's contents), then a shape whose
+partial sums exceed the block, which must be refused before anything is launched."""
+import ctypes
+
+import pytest
+import torch
+
+from cgpt_amd import capi
+from tests.util import bits, randn
+
+pytestmark = pytest.mark.gpu
+
+
+def _call(name, dx, dw, dy, x, w, eps, stream):
+    code = {torch.float16: capi.F16, torch.bfloat16: capi.BF16, torch.float32: capi.F32}[x.dtype]
+    capi.call(name, ctypes.c_void_p(dx.data_ptr()), ctypes.c_void_p(dw.data_ptr()), ctypes.c_void_p(dy.data_ptr()),
+              ctypes.c_void_p(x.data_ptr()), ctypes.c_void_p(w.data_ptr()), x.shape[0], x.shape[1], eps, code,
+              ctypes.c_void_p(stream.cuda_stream))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=["bf16", "f32"])
+def test_static_entry_point_matches_the_allocating_one_on_two_calls_in_a_row(device, dtype):
+    stream = torch.cuda.Stream(device=device)
+    # [rows, hidden]: the training shape's row count, then smaller inputs (row kernel and generic kernels)
+    for call, (rows, hidden) in enumerate([(32768, 1024), (4096, 128), (777, 200), (5, 1024)]):
+        x, dy = randn((rows, hidden), dtype, 10 + call).to(device), randn((rows, hidden), dtype, 20 + call).to(device)
+        w = (1 + 0.1 * randn((hidden,), torch.float32, 30 + call)).to(dtype).to(device)
+        want_dx, want_dw = torch.full_like(x, 3.0), torch.full_like(w, 3.0)
+        got_dx, got_dw = torch.full_like(x, 5.0), torch.full_like(w, 5.0)
+        torch.cuda.synchronize()
+        _call("cgptx_rmsnorm_backward", want_dx, want_dw, dy, x, w, 1e-5, stream)
+        _call("cgptx_rmsnorm_backward_static", got_dx, got_dw, dy, x, w, 1e-5, stream)
+        stream.synchronize()
+        assert (bits(got_dx) == bits(want_dx)).all(), f"dx differs on call {call} [{rows}, {hidden}]"
+        assert (bits(got_dw) == bits(want_dw)).all(), f"dgamma differs on call {call} [{rows}, {hidden}]"
+
+
+def test_static_entry_point_refuses_what_does_not_fit(device):
+    stream = torch.cuda.Stream(device=device)
+    rows, hidden = 4_300_000, 9   # off the row kernel's shapes: one fp32 statistic per row, 17.2 MB > 16 MiB
+    x = torch.zeros(rows, hidden, dtype=torch.bfloat16, device=device)
+    w = torch.ones(hidden, dtype=torch.bfloat16, device=device)
+    dx, dw = torch.empty_like(x), torch.empty_like(w)
+    with pytest.raises(ValueError, match="working memory"):
+        _call("cgptx_rmsnorm_backward_static", dx, dw, x, x, w, 1e-5, stream)
+    with pytest.raises(ValueError):   # the shared validation still runs first
+        _call("cgptx_rmsnorm_backward_static", dx, dw, x, x, w, 0.0, stream)
