@@ -36,6 +36,12 @@ DEVICE_FLAGS = [
 ]
 
 
+# Per-file additions. attention.hip: MFMA results in vector registers by default (the softmax arithmetic reads
+# them in place); the kernels pin the accumulators that never leave the matrix pipeline to the accumulation
+# registers themselves.
+FILE_FLAGS = {"attention.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]}
+
+
 def sources() -> list[pathlib.Path]:
     return sorted(CSRC.glob("*.hip")) + sorted(CSRC.glob("*.cpp"))
 
@@ -45,7 +51,7 @@ def _compile(src: pathlib.Path, force: bool) -> pathlib.Path:
     deps = [src] + list(CSRC.glob("*.hpp")) + list((ROOT / "include").glob("*.h"))
     if not force and obj.exists() and all(obj.stat().st_mtime >= d.stat().st_mtime for d in deps):
         return obj
-    cmd = [HIPCC, *DEVICE_FLAGS, "-c", str(src), "-o", str(obj)]
+    cmd = [HIPCC, *DEVICE_FLAGS, *FILE_FLAGS.get(src.name, []), "-c", str(src), "-o", str(obj)]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     noise = "is not a recognized feature for this target"
     err = "\n".join(line for line in proc.stderr.splitlines() if noise not in line)

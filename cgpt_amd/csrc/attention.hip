@@ -36,6 +36,7 @@
 #include <cmath>
 #include <cstdlib>
 #include <limits>
+#include <utility>
 
 namespace cgptx {
 namespace {
@@ -51,11 +52,20 @@ using s16x4 = vec_t<short, 4>;
 
 template <typename T>
 struct Mma;
+// run(): the compiler places result and addend (this file is built with MFMA results in vector registers,
+// where the VALU reads them without a copy). accumulate(): the accumulator is pinned to the accumulation
+// registers, for tiles that only ever feed the next MFMA of their chain (dK, dV) — with both kinds in one
+// kernel nothing is copied between the two register files inside the loops. The operands of accumulate() come
+// from LDS reads and VALU converts (the compiler waits for both); its result is read again only by the next
+// accumulate() on the same registers (no wait states needed) and, after drain(), by the epilogue.
 template <>
 struct Mma<bf16_t> {
     using frag = vec_t<bf16_t, 8>;
     __device__ static __forceinline__ acc_t run(frag a, frag b, acc_t c) {
         return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+    }
+    __device__ static __forceinline__ void accumulate(frag a, frag b, acc_t& c) {
+        asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
     }
 };
 template <>
@@ -64,7 +74,12 @@ struct Mma<f16_t> {
     __device__ static __forceinline__ acc_t run(frag a, frag b, acc_t c) {
         return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
     }
+    __device__ static __forceinline__ void accumulate(frag a, frag b, acc_t& c) {
+        asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+    }
 };
+// Enough independent cycles after the last accumulate() for its result to be readable by any instruction.
+__device__ __forceinline__ void drain_accumulators() { asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); }
 
 struct Params {
     void* out0;  // forward: O      | dq: dQ | dkv: dK
@@ -627,6 +642,23 @@ __device__ __forceinline__ void sched_reads_under_mfmas() {
     }
 }
 
+// MFMAS matrix instructions with READS LDS reads, VALU vector and TRANS transcendental instructions of
+// independent work dealt out evenly between them (reads lead by a few so that operands arrive in time).
+constexpr int kSchedValu = 0x002, kSchedTrans = 0x400;
+template <int MFMAS, int READS, int VALU, int TRANS, int I = 0>
+__device__ __forceinline__ void sched_pipeline() {
+    if constexpr (I == 0) sched_group<kSchedDsRead, (READS < 6 ? READS : 6)>();
+    if constexpr (I < MFMAS) {
+        constexpr int kLead = READS < 6 ? READS : 6;
+        constexpr int kRest = READS - kLead;
+        sched_group<kSchedMfma, 1>();
+        sched_group<kSchedDsRead, ((I + 1) * kRest) / MFMAS - (I * kRest) / MFMAS>();
+        sched_group<kSchedValu, ((I + 1) * VALU) / MFMAS - (I * VALU) / MFMAS>();
+        sched_group<kSchedTrans, ((I + 1) * TRANS) / MFMAS - (I * TRANS) / MFMAS>();
+        sched_pipeline<MFMAS, READS, VALU, TRANS, I + 1>();
+    }
+}
+
 template <int W>
 __device__ __forceinline__ int swizzle(int row) {
     static_assert(W == 64 || W == 128, "padded widths of the LDS-direct kernels");
@@ -1094,118 +1126,181 @@ __global__ __launch_bounds__(kThreads, 1) void attention_dkv_wide_kernel(Params 
         const int wave_first_key = k_block + wave * 32;
         const int wave_last_key = wave_first_key + 31;
 
-        auto issue = [&](int tile) {
-            const int h = kvh * group + tile / tiles_per_head;
-            const int q0 = q_begin + (tile % tiles_per_head) * kStream;
-            T* stage = lds + (tile & 1) * 2 * kWideTile<W>;
-            const int head_bytes = h * p.d * static_cast<int>(sizeof(T));
-            constexpr int kRowsPerLoad = 64 / (W / 8), kLoads = kStream / (4 * kRowsPerLoad);
-#pragma unroll
-            for (int i = 0; i < kLoads; ++i) {
-                const int soffset = (q0 + i * 4 * kRowsPerLoad) * q_src.row_bytes + head_bytes;
-                T* rows = stage + (i * 4 + wave) * kRowsPerLoad * W;
+        // Where the next tile comes from (requested during the current tile's first MFMAs).
+        struct NextTile {
+            bool live;
+            int soffset;  // bytes: first row of the tile + head
+            T* stage;
+            int stat_soffset;
+            float* stat_stage;
+        };
+        auto next_tile = [&](int tile) {
+            NextTile n;
+            n.live = tile < total_tiles;
+            const int h = kvh * group + tile / max(tiles_per_head, 1);
+            const int q0 = q_begin + (tile % max(tiles_per_head, 1)) * kStream;
+            n.soffset = q0 * q_src.row_bytes + h * p.d * static_cast<int>(sizeof(T));
+            n.stage = lds + (tile & 1) * 2 * kWideTile<W>;
+            n.stat_soffset = (q0 * p.hq + h) * static_cast<int>(sizeof(float));
+            n.stat_stage = stats + (tile & 1) * 2 * kStream + wave * kStream;
+            return n;
+        };
+        constexpr int kRowsPerLoad = 64 / (W / 8), kLoads = kStream / (4 * kRowsPerLoad);
+        // Part `i` of a tile request: rows 4 R i + R w .. of Q and dO (i < kLoads), then the statistics.
+        auto request_part = [&](const NextTile& n, int i) {
+            if (!n.live) return;
+            if (i < kLoads) {
+                const int soffset = n.soffset + i * 4 * kRowsPerLoad * q_src.row_bytes;
+                T* rows = n.stage + (i * 4 + wave) * kRowsPerLoad * W;
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(q_src.rsrc, (lds_void_ptr)(rows), 16, q_src.voffset, soffset, 0, 0);
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(do_src.rsrc, (lds_void_ptr)(rows + kWideTile<W>), 16, do_src.voffset,
                                                          soffset, 0, 0);
-            }
-            if (wave < 2)
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(
-                    stat_rsrc, (lds_void_ptr)(stats + (tile & 1) * 2 * kStream + wave * kStream), 4, stat_voffset,
-                    (q0 * p.hq + h) * static_cast<int>(sizeof(float)), 0, 0);
-        };
-
-        // One 64-query tile. masked: some (query, key) pairs of this wavefront are hidden (causal
-        // mask, keys past the end); first = first visible register coordinate for this lane's key.
-        auto tile_body = [&](const T* q_tile, const T* do_tile, const float* stat, bool masked, int first) {
-            acc_t s_acc[2] = {acc_t(0.0f), acc_t(0.0f)}, dp_acc[2] = {acc_t(0.0f), acc_t(0.0f)};
-            frag pf[2][2], dsf[2][2];
-            auto scores = [&](int sub) {
-                frag qa[STEPS], da[STEPS];
-#pragma unroll
-                for (int s = 0; s < STEPS; ++s) {
-                    qa[s] = *reinterpret_cast<const frag*>(q_tile + sub * 32 * W + q_off[s]);
-                    da[s] = *reinterpret_cast<const frag*>(do_tile + sub * 32 * W + q_off[s]);
-                }
-#pragma unroll
-                for (int s = 0; s < STEPS; ++s) {
-                    s_acc[sub] = Mma<T>::run(qa[s], kf[s], s_acc[sub]);
-                    dp_acc[sub] = Mma<T>::run(da[s], vf[s], dp_acc[sub]);
-                }
-            };
-            auto softmax = [&](int sub) {
-                vec_t<float, 4> lse_q[4], delta_q[4];
-#pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    const int local = sub * 32 + 8 * g + 4 * (lane >> 5);
-                    lse_q[g] = *reinterpret_cast<const vec_t<float, 4>*>(stat + local);
-                    delta_q[g] = *reinterpret_cast<const vec_t<float, 4>*>(stat + kStream + local);
-                }
-                acc_t prob, ds;
-#pragma unroll
-                for (int i = 0; i < 16; ++i)
-                    prob[i] = __builtin_amdgcn_exp2f(fmaf(s_acc[sub][i], scale2, -lse_q[i >> 2][i & 3]));
-                if (masked) {
-                    asm volatile("" ::: "memory");  // keeps the masking out of the common path (no if-conversion)
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) prob[i] = (sub * 32 + 8 * (i >> 2) + (i & 3) >= first) ? prob[i] : 0.0f;
-                }
-#pragma unroll
-                for (int i = 0; i < 16; ++i) ds[i] = prob[i] * (dp_acc[sub][i] - delta_q[i >> 2][i & 3]);
-#pragma unroll
-                for (int s = 0; s < 2; ++s) {
-                    pf[sub][s] = acc_frag<T>(prob, s);
-                    dsf[sub][s] = acc_frag<T>(ds, s);
-                }
-            };
-            auto gradients = [&](int sub) {
-                frag dot[2][DT], qt[2][DT];
-#pragma unroll
-                for (int s = 0; s < 2; ++s) {
-                    const int block = (sub * 32 + s * 16) * W;
-#pragma unroll
-                    for (int t = 0; t < DT; ++t) {
-                        dot[s][t] = wide_transposed_frag<T>(do_tile + block, t_off[t][0], t_off[t][1]);
-                        qt[s][t] = wide_transposed_frag<T>(q_tile + block, t_off[t][0], t_off[t][1]);
-                    }
-                }
-#pragma unroll
-                for (int s = 0; s < 2; ++s)
-#pragma unroll
-                    for (int t = 0; t < DT; ++t) {
-                        dv[t] = Mma<T>::run(dot[s][t], pf[sub][s], dv[t]);
-                        dk[t] = Mma<T>::run(qt[s][t], dsf[sub][s], dk[t]);
-                    }
-            };
-#pragma unroll
-            for (int sub = 0; sub < 2; ++sub) {
-                scores(sub);
-                sched_reads_under_mfmas<2 * STEPS, 2 * STEPS, 4>();
-                __builtin_amdgcn_sched_barrier(0);
-                softmax(sub);
-                __builtin_amdgcn_sched_barrier(0);
-                gradients(sub);
-                sched_reads_under_mfmas<4 * DT, 8 * DT, 8>();
-                __builtin_amdgcn_sched_barrier(0);
+            } else if (i == kLoads && wave < 2) {
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(stat_rsrc, (lds_void_ptr)(n.stat_stage), 4, stat_voffset, n.stat_soffset, 0,
+                                                         0);
             }
         };
 
-        if (total_tiles > 0) issue(0);
-        for (int tile = 0; tile < total_tiles; ++tile) {
-            const int q0 = q_begin + (tile % tiles_per_head) * kStream;
-            const T* q_tile = lds + (tile & 1) * 2 * kWideTile<W>;
-            const float* stat = stats + (tile & 1) * 2 * kStream;
+        // One 64-query tile = 4 N MFMAs (N = W / 8) in four phases over its two 32-query halves:
+        //   Sᵀ,dPᵀ(0) | Sᵀ,dPᵀ(1) + P,dS(0) | dV,dK(0) + P,dS(1) | dV,dK(1)
+        // A wavefront's VALU instructions run in the shadow of its own MFMAs when they do not depend on them,
+        // but only if they stand between them in program order (an MFMA waits at issue for the previous one,
+        // and everything behind it waits too). So the tile is written as 4 N slots of one MFMA each, with a
+        // scheduling fence after every slot; a slot also carries the LDS reads of the operand needed kLookAhead
+        // slots later, and its share of what else the tile has to do: the requests for the next tile and the
+        // reads of LSE·log2 e and delta in phase 0, the exponentials and products of half 0 in phase 1, of half 1
+        // in phase 2 (two scores per slot pair: fma, exp | subtract, multiply, packed converts).
+        // MASKED: some (query, key) pairs of this wavefront are hidden (causal mask, keys past the end);
+        // first = first visible register coordinate for this lane's key. Two separate straight-line bodies.
+        auto tile_body = [&]<bool MASKED>(const T* q_tile, const T* do_tile, const float* stat, int first, const NextTile& next) {
+            constexpr int N = W / 8, kLookAhead = 4;
+            acc_t s_acc[2], dp_acc[2];
+            vec_t<unsigned int, 4> p_words[2][2], ds_words[2][2];  // [half][16-query step]: the k-operands of dV, dK
+            vec_t<float, 4> lse_q[2][4], delta_q[2][4];
+            float prob_pair[2][16];
+            frag operand[4 * N];
+            auto read_operand = [&]<int K>() {
+                constexpr int phase = K / N, j = K % N;
+                if constexpr (phase < 2) {
+                    const T* tile = (j & 1) ? do_tile : q_tile;
+                    operand[K] = *reinterpret_cast<const frag*>(tile + phase * 32 * W + q_off[j >> 1]);
+                } else {
+                    constexpr int s = j / (2 * DT), t = (j / 2) % DT;
+                    const T* tile = (j & 1) ? q_tile : do_tile;
+                    operand[K] = wide_transposed_frag<T>(tile + ((phase - 2) * 32 + s * 16) * W, t_off[t][0], t_off[t][1]);
+                }
+            };
+            auto multiply = [&]<int K>() {
+                constexpr int phase = K / N, j = K % N;
+                if constexpr (phase < 2) {
+                    constexpr int s = j >> 1;
+                    if constexpr (j & 1) dp_acc[phase] = Mma<T>::run(operand[K], vf[s], s == 0 ? acc_t(0.0f) : dp_acc[phase]);
+                    else s_acc[phase] = Mma<T>::run(operand[K], kf[s], s == 0 ? acc_t(0.0f) : s_acc[phase]);
+                } else {
+                    constexpr int s = j / (2 * DT), t = (j / 2) % DT;
+                    if constexpr (j & 1) dk[t] = Mma<T>::run(operand[K], __builtin_bit_cast(frag, ds_words[phase - 2][s]), dk[t]);
+                    else dv[t] = Mma<T>::run(operand[K], __builtin_bit_cast(frag, p_words[phase - 2][s]), dv[t]);
+                }
+            };
+            auto statistics = [&]<int SUB, int I>() {  // read I of 8
+                constexpr int g = I >> 1;
+                const int local = SUB * 32 + 8 * g + 4 * (lane >> 5);
+                if constexpr (I & 1) delta_q[SUB][g] = *reinterpret_cast<const vec_t<float, 4>*>(stat + kStream + local);
+                else lse_q[SUB][g] = *reinterpret_cast<const vec_t<float, 4>*>(stat + local);
+            };
+            // Half-slice H of 16 for half SUB: scores 2 (H/2), 2 (H/2) + 1. Even H: P; odd H: dS and both packs.
+            auto softmax_part = [&]<int SUB, int H>() {
+                constexpr int i0 = 2 * (H / 2), i1 = i0 + 1;
+                if constexpr ((H & 1) == 0) {
+                    float a = __builtin_amdgcn_exp2f(fmaf(s_acc[SUB][i0], scale2, -lse_q[SUB][i0 >> 2][i0 & 3]));
+                    float c = __builtin_amdgcn_exp2f(fmaf(s_acc[SUB][i1], scale2, -lse_q[SUB][i1 >> 2][i1 & 3]));
+                    if constexpr (MASKED) {
+                        a = (SUB * 32 + 8 * (i0 >> 2) + (i0 & 3) >= first) ? a : 0.0f;
+                        c = (SUB * 32 + 8 * (i1 >> 2) + (i1 & 3) >= first) ? c : 0.0f;
+                    }
+                    prob_pair[SUB][i0] = a;
+                    prob_pair[SUB][i1] = c;
+                } else {
+                    const float a = prob_pair[SUB][i0], c = prob_pair[SUB][i1];
+                    vec_t<float, 2> pv, dsv;
+                    pv[0] = a;
+                    pv[1] = c;
+                    dsv[0] = a * (dp_acc[SUB][i0] - delta_q[SUB][i0 >> 2][i0 & 3]);
+                    dsv[1] = c * (dp_acc[SUB][i1] - delta_q[SUB][i1 >> 2][i1 & 3]);
+                    constexpr int word = i0 / 2;  // 8 words per half: 4 per 16-query step
+                    p_words[SUB][word / 4][word % 4] = __builtin_bit_cast(unsigned int, vec_from_f32<T, 2>(pv));
+                    ds_words[SUB][word / 4][word % 4] = __builtin_bit_cast(unsigned int, vec_from_f32<T, 2>(dsv));
+                }
+            };
+            auto slot = [&]<int K>() {
+                constexpr int phase = K / N, j = K % N;
+                if constexpr (K + kLookAhead < 4 * N) read_operand.template operator()<K + kLookAhead>();
+                multiply.template operator()<K>();
+                if constexpr (phase == 0) {
+                    if constexpr (j <= kLoads) request_part(next, j);
+                }
+                if constexpr (phase < 2) {  // statistics of half `phase`, read while its scores are multiplied
+                    constexpr int per_slot = 8 / N > 0 ? 8 / N : 1;
+                    if constexpr (j * per_slot < 8) {
+                        statistics.template operator()<phase, j * per_slot>();
+                        if constexpr (per_slot == 2) statistics.template operator()<phase, j * per_slot + 1>();
+                    }
+                }
+                if constexpr (phase == 1 || phase == 2) {  // P, dS of half phase - 1
+                    constexpr int per_slot = 16 / N;
+#pragma unroll
+                    for (int unused = 0; unused < 1; ++unused) {
+                        softmax_part.template operator()<phase - 1, j * per_slot>();
+                        if constexpr (per_slot == 2) softmax_part.template operator()<phase - 1, j * per_slot + 1>();
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            };
+            [&]<int... K>(std::integer_sequence<int, K...>) {
+                (read_operand.template operator()<K>(), ...);
+            }(std::make_integer_sequence<int, kLookAhead>{});
+            __builtin_amdgcn_sched_barrier(0);
+            [&]<int... K>(std::integer_sequence<int, K...>) { (slot.template operator()<K>(), ...); }(
+                std::make_integer_sequence<int, 4 * N>{});
+        };
+
+        // Every wavefront runs every tile (no divergent paths around the accumulators): pairs the causal mask
+        // hides, and keys past the end of the sequence, get P = 0. Register i of half `sub` holds query
+        // q0 + 32 sub + 8 (i/4) + 4 (lane/32) + i%4; this lane's key sees it iff that query is >= key - offset.
+        // Per head the tiles that need the mask come first (the ones on the diagonal; all of them for a
+        // wavefront with keys past the end): two loops with one straight-line body each, so that the
+        // accumulators stay where they are from tile to tile.
+        int masked_per_head = 0;
+        if (wave_last_key >= p.ks) masked_per_head = tiles_per_head;
+        else if (p.causal) masked_per_head = min(tiles_per_head, max(0, (wave_last_key - p.offset - q_begin + kStream - 1) / kStream));
+        auto arrive = [&]() {
             __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wavefront's part of the tile is in LDS
             __syncthreads();                     // ... and everybody else's; the other stage is free
-            if (tile + 1 < total_tiles) issue(tile + 1);
-            // Every wavefront runs every tile (no divergent paths around the accumulators): pairs the
-            // causal mask hides, and keys past the end of the sequence, get P = 0.
-            // Register i of half `sub` holds query q0 + 32 sub + 8 (i/4) + 4 (lane/32) + i%4; this lane's
-            // key sees it iff that query is >= key - offset.
-            const bool masked = (p.causal && wave_last_key > p.offset + q0) || wave_last_key >= p.ks;
-            const int causal_first = p.causal ? k_row - p.offset - q0 - 4 * (lane >> 5) : -(1 << 30);
-            const int first = k_live ? causal_first : (1 << 30);
-            tile_body(q_tile, q_tile + kWideTile<W>, stat, masked, first);
+        };
+        {
+            const NextTile first_tile = next_tile(0);
+#pragma unroll
+            for (int i = 0; i <= kLoads; ++i) request_part(first_tile, i);
         }
+        for (int head = 0; head < group; ++head) {
+            const int tile0 = head * tiles_per_head;
+            for (int t = 0; t < masked_per_head; ++t) {
+                const int tile = tile0 + t, q0 = q_begin + t * kStream;
+                const T* q_tile = lds + (tile & 1) * 2 * kWideTile<W>;
+                arrive();
+                const int causal_first = p.causal ? k_row - p.offset - q0 - 4 * (lane >> 5) : -(1 << 30);
+                tile_body.template operator()<true>(q_tile, q_tile + kWideTile<W>, stats + (tile & 1) * 2 * kStream,
+                                                    k_live ? causal_first : (1 << 30), next_tile(tile + 1));
+            }
+            for (int t = masked_per_head; t < tiles_per_head; ++t) {
+                const int tile = tile0 + t;
+                const T* q_tile = lds + (tile & 1) * 2 * kWideTile<W>;
+                arrive();
+                tile_body.template operator()<false>(q_tile, q_tile + kWideTile<W>, stats + (tile & 1) * 2 * kStream, 0,
+                                                     next_tile(tile + 1));
+            }
+        }
+        drain_accumulators();
         __syncthreads();  // the next key block's first loads overwrite stage 0
         if (k_live) {
             T* dk_out = static_cast<T*>(p.out0) + k_offset;

@@ -209,7 +209,8 @@ void collect(cgptx_model* m, std::vector<Parameter*>& out) {
         if (int status_ = (expr)) return status_; \
     } while (0)
 
-// Runs one operator call; when profiling, brackets it with events on the same stream.
+// Runs one operator call; when profiling, brackets it with events on the same stream. Labels are "kind" or
+// "kind.part" (the contractions carry the projection they belong to: qkv, o, gate_up, down, classifier).
 #define CGPTX_OP(label, expr)                                                   \
     do {                                                                        \
         cgptx_model::Timed t_{label, nullptr, nullptr};                         \
@@ -228,11 +229,11 @@ void collect(cgptx_model* m, std::vector<Parameter*>& out) {
 // linear_backward as two single-kernel calls so that each can be timed on its own.
 int linear_backward_split(cgptx_model* m, void* dx, void* dw, const void* dy, const void* x, const void* w,
                           std::size_t rows, std::size_t in_features, std::size_t out_features, int accumulate_input,
-                          int dt, hipStream_t stream, const char* dx_label = "gemm_dx") {
+                          int dt, hipStream_t stream, const char* dx_label, const char* dw_label) {
     auto* s = static_cast<cgptx_stream>(stream);
     CGPTX_OP(dx_label, cgptx_linear_backward(dx, nullptr, nullptr, dy, x, w, rows, in_features, out_features,
                                               accumulate_input, 0, 0, dt, s));
-    CGPTX_OP("gemm_dw", cgptx_linear_backward(nullptr, dw, nullptr, dy, x, w, rows, in_features, out_features, 0, 0,
+    CGPTX_OP(dw_label, cgptx_linear_backward(nullptr, dw, nullptr, dy, x, w, rows, in_features, out_features, 0, 0,
                                               0, dt, s));
     return CGPTX_OK;
 }
@@ -376,21 +377,21 @@ int enqueue_reference_sequence(cgptx_model* m, float loss_scale, int loss_mode, 
         void *projected = m->d_norm_in, *ffn = m->d_norm_in_f;  // backward workspace, free during the forward pass
         void *gate = a.gate_up, *up = second_half(a.gate_up);
         CGPTX_OP("rmsnorm_fwd", cgptx_rmsnorm_forward(a.norm_a, x, w.attention_norm.value, N, H, eps, dt, s));
-        CGPTX_OP("gemm_fwd", cgptx_linear_forward(a.q_pre, a.norm_a, w.q.value, nullptr, N, H, QW, dt, s));
-        CGPTX_OP("gemm_fwd", cgptx_linear_forward(a.k_pre, a.norm_a, w.k.value, nullptr, N, H, KW, dt, s));
-        CGPTX_OP("gemm_fwd", cgptx_linear_forward(a.v, a.norm_a, w.v.value, nullptr, N, H, KW, dt, s));
+        CGPTX_OP("gemm_fwd.qkv", cgptx_linear_forward(a.q_pre, a.norm_a, w.q.value, nullptr, N, H, QW, dt, s));
+        CGPTX_OP("gemm_fwd.qkv", cgptx_linear_forward(a.k_pre, a.norm_a, w.k.value, nullptr, N, H, KW, dt, s));
+        CGPTX_OP("gemm_fwd.qkv", cgptx_linear_forward(a.v, a.norm_a, w.v.value, nullptr, N, H, KW, dt, s));
         CGPTX_OP("rmsnorm_fwd", cgptx_rmsnorm_forward(a.q, a.q_pre, w.q_norm.value, N * HQ, D, eps, dt, s));
         CGPTX_OP("rmsnorm_fwd", cgptx_rmsnorm_forward(a.k, a.k_pre, w.k_norm.value, N * HKV, D, eps, dt, s));
         CGPTX_OP("rope_fwd", cgptx_rope_forward(a.q, a.k, m->cos_cache, m->sin_cache, m->batch, m->sequence, HQ, HKV, D,
                                                 c.rotary_dim, 0, m->sequence, dt, s));
         CGPTX_OP("attn_fwd", cgptx_flash_gqa_attention_forward(a.attn_out, a.lse, a.q, a.k, a.v, m->batch, m->sequence,
                                                                m->sequence, HQ, HKV, D, 0.0f, 1, 0, dt, s));
-        CGPTX_OP("gemm_fwd", cgptx_linear_forward(projected, a.attn_out, w.o.value, nullptr, N, QW, H, dt, s));
+        CGPTX_OP("gemm_fwd.o", cgptx_linear_forward(projected, a.attn_out, w.o.value, nullptr, N, QW, H, dt, s));
         CGPTX_OP("rmsnorm_fwd", cgptx_rmsnorm_forward(a.norm_f, x, w.ffn_norm.value, N, H, eps, dt, s));
-        CGPTX_OP("gemm_fwd", cgptx_linear_forward(gate, a.norm_f, w.gate.value, nullptr, N, H, I, dt, s));
-        CGPTX_OP("gemm_fwd", cgptx_linear_forward(up, a.norm_f, w.up.value, nullptr, N, H, I, dt, s));
+        CGPTX_OP("gemm_fwd.gate_up", cgptx_linear_forward(gate, a.norm_f, w.gate.value, nullptr, N, H, I, dt, s));
+        CGPTX_OP("gemm_fwd.gate_up", cgptx_linear_forward(up, a.norm_f, w.up.value, nullptr, N, H, I, dt, s));
         CGPTX_OP("swiglu_fwd", cgptx_swiglu_forward(a.act, gate, up, N * I, dt, s));
-        CGPTX_OP("gemm_fwd", cgptx_linear_forward(ffn, a.act, w.down.value, nullptr, N, I, H, dt, s));
+        CGPTX_OP("gemm_fwd.down", cgptx_linear_forward(ffn, a.act, w.down.value, nullptr, N, I, H, dt, s));
         CGPTX_OP("add", cgptx_add(out, x, projected, N * H, dt, s));
         CGPTX_OP("add", cgptx_add(out, out, ffn, N * H, dt, s));
     }
@@ -401,11 +402,12 @@ int enqueue_reference_sequence(cgptx_model* m, float loss_scale, int loss_mode, 
                                                                     m->embedding.value, m->targets, N, H, c.vocabulary_size,
                                                                     loss_scale, 0, dt, s));
     } else {
-        CGPTX_OP("gemm_fwd", cgptx_linear_forward(m->logits, m->normalized, m->embedding.value, nullptr, N, H, c.vocabulary_size, dt, s));
+        CGPTX_OP("gemm_fwd.classifier", cgptx_linear_forward(m->logits, m->normalized, m->embedding.value, nullptr, N, H, c.vocabulary_size, dt, s));
         CGPTX_OP("dense_ce", cgptx_cross_entropy_forward_backward(m->loss, m->grad_logits, m->logits, m->targets, N,
                                                                   c.vocabulary_size, loss_scale, dt, s));
         CGPTX_TRY(linear_backward_split(m, m->d_normalized, m->embedding.gradient, m->grad_logits, m->normalized,
-                                        m->embedding.value, N, H, c.vocabulary_size, 0, dt, stream));
+                                        m->embedding.value, N, H, c.vocabulary_size, 0, dt, stream, "gemm_dx.classifier",
+                                        "gemm_dw.classifier"));
     }
 
     void *current = m->grad_a, *previous = m->grad_b;
@@ -418,14 +420,14 @@ int enqueue_reference_sequence(cgptx_model* m, float loss_scale, int loss_mode, 
         void *gate = a.gate_up, *up = second_half(a.gate_up);
         void *d_gate = m->d_gate_up, *d_up = second_half(m->d_gate_up);
         void* grad_residual = m->d_norm_in_f;
-        CGPTX_TRY(linear_backward_split(m, m->d_act, w.down.gradient, current, a.act, w.down.value, N, I, H, 0, dt, stream));
+        CGPTX_TRY(linear_backward_split(m, m->d_act, w.down.gradient, current, a.act, w.down.value, N, I, H, 0, dt, stream, "gemm_dx.down", "gemm_dw.down"));
         CGPTX_OP("swiglu_bwd", cgptx_swiglu_backward(d_gate, d_up, m->d_act, gate, up, N * I, 0, 0, dt, s));
-        CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.gate.gradient, d_gate, a.norm_f, w.gate.value, N, H, I, 0, dt, stream));
-        CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.up.gradient, d_up, a.norm_f, w.up.value, N, H, I, 1, dt, stream));
+        CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.gate.gradient, d_gate, a.norm_f, w.gate.value, N, H, I, 0, dt, stream, "gemm_dx.gate_up", "gemm_dw.gate_up"));
+        CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.up.gradient, d_up, a.norm_f, w.up.value, N, H, I, 1, dt, stream, "gemm_dx.gate_up", "gemm_dw.gate_up"));
         CGPTX_OP("rmsnorm_bwd", cgptx_rmsnorm_backward(grad_residual, w.ffn_norm.gradient, m->d_norm_in, x, w.ffn_norm.value, N, H,
                                                        eps, dt, s));
         CGPTX_OP("add", cgptx_add(previous, current, grad_residual, N * H, dt, s));  // grad_input = grad_output + grad_residual
-        CGPTX_TRY(linear_backward_split(m, m->d_attn_out, w.o.gradient, current, a.attn_out, w.o.value, N, QW, H, 0, dt, stream));
+        CGPTX_TRY(linear_backward_split(m, m->d_attn_out, w.o.gradient, current, a.attn_out, w.o.value, N, QW, H, 0, dt, stream, "gemm_dx.o", "gemm_dw.o"));
         CGPTX_OP("attn_bwd", cgptx_flash_gqa_attention_backward_with_lse(m->d_q, m->d_k, m->d_v, m->d_attn_out, a.attn_out, a.lse,
                                                                          a.q, a.k, a.v, m->batch, m->sequence, m->sequence, HQ,
                                                                          HKV, D, 0.0f, 1, 0, 0, dt, s));
@@ -435,9 +437,9 @@ int enqueue_reference_sequence(cgptx_model* m, float loss_scale, int loss_mode, 
                                                        eps, dt, s));
         CGPTX_OP("rmsnorm_bwd", cgptx_rmsnorm_backward(m->d_k, w.k_norm.gradient, m->d_k_pre, a.k_pre, w.k_norm.value, N * HKV, D,
                                                        eps, dt, s));
-        CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.q.gradient, m->d_q, a.norm_a, w.q.value, N, H, QW, 0, dt, stream));
-        CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.k.gradient, m->d_k, a.norm_a, w.k.value, N, H, KW, 1, dt, stream));
-        CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.v.gradient, m->d_v, a.norm_a, w.v.value, N, H, KW, 1, dt, stream));
+        CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.q.gradient, m->d_q, a.norm_a, w.q.value, N, H, QW, 0, dt, stream, "gemm_dx.qkv", "gemm_dw.qkv"));
+        CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.k.gradient, m->d_k, a.norm_a, w.k.value, N, H, KW, 1, dt, stream, "gemm_dx.qkv", "gemm_dw.qkv"));
+        CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.v.gradient, m->d_v, a.norm_a, w.v.value, N, H, KW, 1, dt, stream, "gemm_dx.qkv", "gemm_dw.qkv"));
         CGPTX_OP("rmsnorm_bwd", cgptx_rmsnorm_backward(grad_residual, w.attention_norm.gradient, m->d_norm_in, x,
                                                        w.attention_norm.value, N, H, eps, dt, s));
         CGPTX_OP("add", cgptx_add(previous, previous, grad_residual, N * H, dt, s));
@@ -475,11 +477,11 @@ int enqueue_forward_backward(cgptx_model* m, float loss_scale, int loss_mode, hi
             CGPTX_OP("rmsnorm_fwd", cgptx_rmsnorm_forward(a.norm_a, x, w.attention_norm.value, N, H, eps, dt, s));
         }
         if (fused_qkv) {
-            CGPTX_OP("gemm_fwd", qkv_forward(a.q_pre, a.k_pre, a.v, a.norm_a, w.q.value, N, H, QW, KW, dt, stream));
+            CGPTX_OP("gemm_fwd.qkv", qkv_forward(a.q_pre, a.k_pre, a.v, a.norm_a, w.q.value, N, H, QW, KW, dt, stream));
         } else {
-            CGPTX_OP("gemm_fwd", cgptx_linear_forward(a.q_pre, a.norm_a, w.q.value, nullptr, N, H, QW, dt, s));
-            CGPTX_OP("gemm_fwd", cgptx_linear_forward(a.k_pre, a.norm_a, w.k.value, nullptr, N, H, KW, dt, s));
-            CGPTX_OP("gemm_fwd", cgptx_linear_forward(a.v, a.norm_a, w.v.value, nullptr, N, H, KW, dt, s));
+            CGPTX_OP("gemm_fwd.qkv", cgptx_linear_forward(a.q_pre, a.norm_a, w.q.value, nullptr, N, H, QW, dt, s));
+            CGPTX_OP("gemm_fwd.qkv", cgptx_linear_forward(a.k_pre, a.norm_a, w.k.value, nullptr, N, H, KW, dt, s));
+            CGPTX_OP("gemm_fwd.qkv", cgptx_linear_forward(a.v, a.norm_a, w.v.value, nullptr, N, H, KW, dt, s));
         }
         if (fused_qk_norm_rope(m, a.q, a.q_pre, nullptr, w.q_norm.value) && fused_qk_norm_rope(m, a.k, a.k_pre, nullptr, w.k_norm.value)) {
             CGPTX_OP("rmsnorm_fwd", rmsnorm_rope_forward(a.q, a.q_pre, w.q_norm.value, m->cos_cache, m->sin_cache, N * HQ, D, HQ,
@@ -495,15 +497,15 @@ int enqueue_forward_backward(cgptx_model* m, float loss_scale, int loss_mode, hi
         CGPTX_OP("attn_fwd", cgptx_flash_gqa_attention_forward(a.attn_out, a.lse, a.q, a.k, a.v, m->batch, m->sequence,
                                                     m->sequence, HQ, HKV, D, 0.0f, 1, 0, dt, s));
         // out = x + attention_projection, then out += ffn_output (src/core/transformer_block.cu:594-595)
-        CGPTX_OP("gemm_fwd", linear_forward_residual(out, a.attn_out, w.o.value, x, false, N, QW, H, dt, stream));
+        CGPTX_OP("gemm_fwd.o", linear_forward_residual(out, a.attn_out, w.o.value, x, false, N, QW, H, dt, stream));
         if (!dual_norms) CGPTX_OP("rmsnorm_fwd", cgptx_rmsnorm_forward(a.norm_f, x, w.ffn_norm.value, N, H, eps, dt, s));
         if (fused_swiglu()) {
-            CGPTX_OP("gemm_fwd", cgptx_linear_swiglu_forward(a.gate_up, a.act, a.norm_f, w.gate.value, N, H, I, dt, s));
+            CGPTX_OP("gemm_fwd.gate_up", cgptx_linear_swiglu_forward(a.gate_up, a.act, a.norm_f, w.gate.value, N, H, I, dt, s));
         } else {
-            CGPTX_OP("gemm_fwd", cgptx_linear_forward(a.gate_up, a.norm_f, w.gate.value, nullptr, N, H, 2 * I, dt, s));
+            CGPTX_OP("gemm_fwd.gate_up", cgptx_linear_forward(a.gate_up, a.norm_f, w.gate.value, nullptr, N, H, 2 * I, dt, s));
             CGPTX_OP("swiglu_fwd", cgptx_swiglu_forward_packed(a.act, a.gate_up, N, I, dt, s));
         }
-        CGPTX_OP("gemm_fwd", linear_forward_residual(out, a.act, w.down.value, nullptr, true, N, I, H, dt, stream));
+        CGPTX_OP("gemm_fwd.down", linear_forward_residual(out, a.act, w.down.value, nullptr, true, N, I, H, dt, stream));
     }
     void* last = m->hidden[c.num_layers];
     CGPTX_OP("rmsnorm_fwd", cgptx_rmsnorm_forward(m->normalized, last, m->final_norm.value, N, H, eps, dt, s));
@@ -514,11 +516,11 @@ int enqueue_forward_backward(cgptx_model* m, float loss_scale, int loss_mode, hi
                                                            m->normalized, m->embedding.value, m->targets, N, H,
                                                            c.vocabulary_size, loss_scale, 0, dt, s));
     } else {
-        CGPTX_OP("gemm_fwd", cgptx_linear_forward(m->logits, m->normalized, m->embedding.value, nullptr, N, H,
+        CGPTX_OP("gemm_fwd.classifier", cgptx_linear_forward(m->logits, m->normalized, m->embedding.value, nullptr, N, H,
                                        c.vocabulary_size, dt, s));
         CGPTX_OP("dense_ce", cgptx_cross_entropy_forward_backward(m->loss, m->grad_logits, m->logits, m->targets, N,
                                                        c.vocabulary_size, loss_scale, dt, s));
-        CGPTX_TRY(linear_backward_split(m, m->d_normalized, m->embedding.gradient, m->grad_logits, m->normalized, m->embedding.value, N, H, c.vocabulary_size, 0, dt, stream));
+        CGPTX_TRY(linear_backward_split(m, m->d_normalized, m->embedding.gradient, m->grad_logits, m->normalized, m->embedding.value, N, H, c.vocabulary_size, 0, dt, stream, "gemm_dx.classifier", "gemm_dw.classifier"));
     }
 
     // ----------------------------------------------------------------- backward
@@ -532,10 +534,10 @@ int enqueue_forward_backward(cgptx_model* m, float loss_scale, int loss_mode, hi
         void* x = m->hidden[reverse];
         if (fused_swiglu()) {
             // The SwiGLU gradient rides in the epilogue of the down projection's input gradient.
-            CGPTX_OP("gemm_dx", cgptx_linear_swiglu_backward(m->d_gate_up, m->d_act, current, w.down.value, a.gate_up, N, I, H, dt, s));
-            CGPTX_OP("gemm_dw", cgptx_linear_backward(nullptr, w.down.gradient, nullptr, current, a.act, w.down.value, N, I, H, 0, 0, 0, dt, s));
+            CGPTX_OP("gemm_dx.down", cgptx_linear_swiglu_backward(m->d_gate_up, m->d_act, current, w.down.value, a.gate_up, N, I, H, dt, s));
+            CGPTX_OP("gemm_dw.down", cgptx_linear_backward(nullptr, w.down.gradient, nullptr, current, a.act, w.down.value, N, I, H, 0, 0, 0, dt, s));
         } else {
-            CGPTX_TRY(linear_backward_split(m, m->d_act, w.down.gradient, current, a.act, w.down.value, N, I, H, 0, dt, stream));
+            CGPTX_TRY(linear_backward_split(m, m->d_act, w.down.gradient, current, a.act, w.down.value, N, I, H, 0, dt, stream, "gemm_dx.down", "gemm_dw.down"));
             CGPTX_OP("swiglu_bwd", cgptx_swiglu_backward_packed(m->d_gate_up, m->d_act, a.gate_up, N, I, 0, dt, s));
         }
         // The gradient of the residual stream collects the two norm branches: in one pass at the end of
@@ -544,15 +546,13 @@ int enqueue_forward_backward(cgptx_model* m, float loss_scale, int loss_mode, hi
         const bool dual_norms = fused_block_norms(m, previous, m->d_norm_in, m->d_norm_in_f, x, current) &&
                                 is_aligned16(w.attention_norm.value) && is_aligned16(w.ffn_norm.value);
         void* d_norm_f = dual_norms ? m->d_norm_in_f : m->d_norm_in;
-        // The input gradient of the gate/up projection is labelled on its own ("kind.part"): the launch
-        // the kernel roofline of the benchmark is quoted on.
         CGPTX_TRY(linear_backward_split(m, d_norm_f, w.gate.gradient, m->d_gate_up, a.norm_f, w.gate.value, N, H, 2 * I, 0, dt, stream,
-                                        "gemm_dx.gate_up"));
+                                        "gemm_dx.gate_up", "gemm_dw.gate_up"));
         if (!dual_norms) {
             CGPTX_OP("rmsnorm_bwd", rmsnorm_backward_residual(previous, w.ffn_norm.gradient, m->d_norm_in, x, w.ffn_norm.value,
                                                               current, N, H, eps, dt, stream));
         }
-        CGPTX_TRY(linear_backward_split(m, m->d_attn_out, w.o.gradient, current, a.attn_out, w.o.value, N, QW, H, 0, dt, stream));
+        CGPTX_TRY(linear_backward_split(m, m->d_attn_out, w.o.gradient, current, a.attn_out, w.o.value, N, QW, H, 0, dt, stream, "gemm_dx.o", "gemm_dw.o"));
         CGPTX_OP("attn_bwd", cgptx_flash_gqa_attention_backward_with_lse(m->d_q, m->d_k, m->d_v, m->d_attn_out, a.attn_out,
                                                               a.lse, a.q, a.k, a.v, m->batch, m->sequence,
                                                               m->sequence, HQ, HKV, D, 0.0f, 1, 0, 0, dt, s));
@@ -572,12 +572,12 @@ int enqueue_forward_backward(cgptx_model* m, float loss_scale, int loss_mode, hi
                                              eps, dt, s));
         }
         if (fused_qkv) {
-            CGPTX_OP("gemm_dx", qkv_backward_input(m->d_norm_in, m->d_q, m->d_k, m->d_v, w.q.value, N, H, QW, KW, dt, stream));
-            CGPTX_OP("gemm_dw", qkv_backward_weight(w.q.gradient, m->d_q, m->d_k, m->d_v, a.norm_a, N, H, QW, KW, dt, stream));
+            CGPTX_OP("gemm_dx.qkv", qkv_backward_input(m->d_norm_in, m->d_q, m->d_k, m->d_v, w.q.value, N, H, QW, KW, dt, stream));
+            CGPTX_OP("gemm_dw.qkv", qkv_backward_weight(w.q.gradient, m->d_q, m->d_k, m->d_v, a.norm_a, N, H, QW, KW, dt, stream));
         } else {
-            CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.q.gradient, m->d_q, a.norm_a, w.q.value, N, H, QW, 0, dt, stream));
-            CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.k.gradient, m->d_k, a.norm_a, w.k.value, N, H, KW, 1, dt, stream));
-            CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.v.gradient, m->d_v, a.norm_a, w.v.value, N, H, KW, 1, dt, stream));
+            CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.q.gradient, m->d_q, a.norm_a, w.q.value, N, H, QW, 0, dt, stream, "gemm_dx.qkv", "gemm_dw.qkv"));
+            CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.k.gradient, m->d_k, a.norm_a, w.k.value, N, H, KW, 1, dt, stream, "gemm_dx.qkv", "gemm_dw.qkv"));
+            CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.v.gradient, m->d_v, a.norm_a, w.v.value, N, H, KW, 1, dt, stream, "gemm_dx.qkv", "gemm_dw.qkv"));
         }
         if (dual_norms) {
             CGPTX_OP("rmsnorm_bwd", rmsnorm_backward_dual(previous, w.attention_norm.gradient, w.ffn_norm.gradient, m->d_norm_in,
