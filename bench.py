@@ -3,7 +3,7 @@
 at B=32, T=1024 on one MI355X, bf16 storage with fp32 accumulation, synthetic seeded token ids
 and random-init weights.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--loss cut|dense] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--loss cut|dense] [--dtype bf16|f16] [--no-cpu-baseline]
 
 Prints ONE JSON line. Besides the contract fields it carries
   roofline     – the kernel that takes the most time in the step, on the launch it spends most
@@ -11,8 +11,15 @@ Prints ONE JSON line. Besides the contract fields it carries
                  duration inside the step (HIP events around every operator call of one eager
                  pass on the step's stream), against the 2.5 PFLOP/s dense bf16 MFMA peak; the
                  same launch timed 20 times back to back; the per-kind breakdown of the step;
+                 `gemm_launches` (every contraction of the step by position: shape, microseconds, fraction) and
+                 `kernels` (every backward operator alone at the configuration's shape, HIP events on the launch
+                 stream, against its HBM or MFMA roofline);
   cpu_baseline – the float32 CPU restatement of the reference's operators (oracle/, "port")
-                 timed on this host on a bounded sample of the same workload.
+                 timed on this host on bounded samples of the same workload: one full train step, the
+                 reference's CPU-runnable configuration (forward + loss at B=1, T=256) and each backward
+                 operator alone.
+--dtype f16 --loss dense is the configuration of the reference's own published run (F16 storage, dense
+cross-entropy over materialised logits: train/train.cpp:59, 436-440).
 This run uses one GPU; --gpus above 1 exits with a message.
 """
 from __future__ import annotations
@@ -69,16 +76,17 @@ TRAFFIC_FILE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profile
                             "gemm_dx_256x256_gate_projection_pmc.txt")
 
 
-def kernel_probe(torch, cfg, batch, seq, stream, launches, seed):
+def kernel_probe(torch, cfg, batch, seq, stream, launches, seed, dtype=None):
     """Average duration of one launch of the dominant kernel: HIP events on the launch stream."""
     from cgpt_amd import ops
 
+    dtype = dtype or torch.bfloat16
     rows, hidden, inter = batch * seq, cfg.hidden_size, 2 * cfg.intermediate_size  # [gate; up] as one weight
     generator = torch.Generator(device="cuda").manual_seed(seed)
-    dy = torch.randn(rows, inter, device="cuda", generator=generator).to(torch.bfloat16)
-    x = torch.empty(rows, hidden, device="cuda", dtype=torch.bfloat16)  # shape only: no weight gradient is asked for
-    w = (torch.randn(inter, hidden, device="cuda", generator=generator) * 0.02).to(torch.bfloat16)
-    dx = torch.empty(rows, hidden, device="cuda", dtype=torch.bfloat16)
+    dy = torch.randn(rows, inter, device="cuda", generator=generator).to(dtype)
+    x = torch.empty(rows, hidden, device="cuda", dtype=dtype)  # shape only: no weight gradient is asked for
+    w = (torch.randn(inter, hidden, device="cuda", generator=generator) * 0.02).to(dtype)
+    dx = torch.empty(rows, hidden, device="cuda", dtype=dtype)
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     with torch.cuda.stream(stream):
         for _ in range(3):
@@ -95,6 +103,121 @@ def kernel_probe(torch, cfg, batch, seq, stream, launches, seed):
             "shape": f"[{rows}, {inter}] x [{inter}, {hidden}]"}
 
 
+def gemm_shapes(cfg, batch, seq):
+    """(M, N, K) of every contraction label of the step profile ("kind.position")."""
+    N, H, I, V = batch * seq, cfg.hidden_size, cfg.intermediate_size, cfg.vocabulary_size
+    QKV = (cfg.num_query_heads + 2 * cfg.num_kv_heads) * cfg.head_dim
+    QW = cfg.num_query_heads * cfg.head_dim
+    outs = {"qkv": (QKV, H), "o": (H, QW), "gate_up": (2 * I, H), "down": (H, I), "classifier": (V, H)}  # (out, in)
+    shapes = {}
+    for name, (o, i) in outs.items():
+        shapes[f"gemm_fwd.{name}"] = (N, o, i)   # Y[N, out] = X[N, in] W^T
+        shapes[f"gemm_dx.{name}"] = (N, i, o)    # dX[N, in] = dY[N, out] W
+        shapes[f"gemm_dw.{name}"] = (o, i, N)    # dW[out, in] = dY^T X
+    return shapes
+
+
+def timed(torch, stream, fn, launches=20, warm=3):
+    """Average seconds per call of fn(), HIP events recorded on the stream the kernels are launched on."""
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    with torch.cuda.stream(stream):
+        for _ in range(warm):
+            fn()
+        start.record(stream)
+        for _ in range(launches):
+            fn()
+        stop.record(stream)
+    stop.synchronize()
+    return start.elapsed_time(stop) * 1e-3 / launches
+
+
+def isolated_kernels(torch, cfg, batch, seq, dtype, stream, seed, only=""):
+    """Every backward operator alone at the configuration's shape: algorithmic bytes or FLOPs of one call /
+    its average duration over 20 back-to-back calls. `only`: run just the sections whose name contains it."""
+    from cgpt_amd import ops
+
+    N, H, I, V = batch * seq, cfg.hidden_size, cfg.intermediate_size, cfg.vocabulary_size
+    HQ, HKV, D = cfg.num_query_heads, cfg.num_kv_heads, cfg.head_dim
+    e = 2
+    gen = torch.Generator(device="cuda").manual_seed(seed)
+
+    def rnd(*shape, scale=1.0):
+        return (torch.randn(*shape, device="cuda", generator=gen) * scale).to(dtype)
+
+    out = {}
+
+    def want(section):
+        return only in section
+
+    def record(name, bound, amount, seconds, shape):
+        rate = amount / seconds / (1e12 if bound == "mfma" else 1e9)
+        peak = PEAK_BF16_TFLOPS if bound == "mfma" else PEAK_HBM_GBS
+        out[name] = {"shape": shape, "bound": bound, "us": round(seconds * 1e6, 1), "rate": round(rate, 1),
+                     "unit": "TFLOP/s" if bound == "mfma" else "GB/s", "frac": round(rate / peak, 4)}
+
+    for rows, hidden in ((N, H), (N * HQ, D), (N * HKV, D)) if want("rmsnorm") else ():
+        x, dy, w = rnd(rows, hidden), rnd(rows, hidden), rnd(hidden)
+        dx, dw = torch.empty_like(x), torch.empty_like(w)
+        t = timed(torch, stream, lambda: ops.rmsnorm_backward(dx, dw, dy, x, w, 1e-5, stream))
+        record(f"rmsnorm_backward[{rows},{hidden}]", "hbm", 3 * rows * hidden * e, t, f"x, dy read, dx written")
+        del x, dy, dx
+    ids = torch.randint(0, V, (N,), device="cuda", generator=gen, dtype=torch.int32)
+    if not (want("rope") or want("attention")):
+        return _isolated_rest(torch, ops, want, record, rnd, timed, stream, out, N, H, I, V, e, ids)
+    q, k = rnd(batch, seq, HQ, D), rnd(batch, seq, HKV, D)
+    pos = torch.arange(seq, device="cuda", dtype=torch.float32)[:, None]
+    theta = pos / torch.pow(torch.tensor(10000.0, device="cuda"), torch.arange(D // 2, device="cuda") * 2.0 / D)[None, :]
+    cos, sin = torch.cos(theta).to(dtype), torch.sin(theta).to(dtype)
+    gq, gk = torch.empty_like(q), torch.empty_like(k)
+    if want("rope"):
+        t = timed(torch, stream, lambda: ops.rope_backward(gq, gk, q, k, cos, sin, stream))
+        record(f"rope_backward q[{batch},{seq},{HQ},{D}] k[..,{HKV},..]", "hbm", 2 * (q.numel() + k.numel()) * e, t, "read + write")
+    if not want("attention"):
+        return _isolated_rest(torch, ops, want, record, rnd, timed, stream, out, N, H, I, V, e, ids)
+    v = rnd(batch, seq, HKV, D)
+    o, lse = torch.empty_like(q), torch.empty(batch, seq, HQ, device="cuda")
+    do = rnd(batch, seq, HQ, D)
+    opt = ops.FlashAttentionOptions(HQ, HKV, D)
+    causal_matmul = 2.0 * batch * HQ * seq * seq * D / 2
+    t = timed(torch, stream, lambda: ops.flash_gqa_attention_forward_with_lse(o, lse, q, k, v, stream, opt))
+    record("flash_gqa_attention_forward_with_lse", "mfma", 2 * causal_matmul, t, f"B={batch} T={seq} {HQ}:{HKV} heads D={D}, 2 causal matmuls")
+    gv = torch.empty_like(k)
+    t = timed(torch, stream, lambda: ops.flash_gqa_attention_backward_with_lse(gq, gk, gv, do, o, lse, q, k, v, stream, opt))
+    record("flash_gqa_attention_backward_with_lse", "mfma", 5 * causal_matmul, t,
+           f"B={batch} T={seq} {HQ}:{HKV} heads D={D}, 5 causal matmuls counted (7 executed)")
+    del q, k, v, o, do, gq, gk, gv
+    return _isolated_rest(torch, ops, want, record, rnd, timed, stream, out, N, H, I, V, e, ids)
+
+
+def _isolated_rest(torch, ops, want, record, rnd, timed, stream, out, N, H, I, V, e, ids):
+    dtype = rnd(1).dtype
+    if want("swiglu"):
+        gate_up, dy = rnd(N, 2 * I), rnd(N, I)
+        g_gate_up = torch.empty_like(gate_up)
+        t = timed(torch, stream, lambda: ops.swiglu_backward_packed(g_gate_up, dy, gate_up, stream))
+        record(f"swiglu_backward[{N},{I}]", "hbm", 5 * N * I * e, t, "dy, gate, up read; dgate, dup written")
+        del gate_up, dy, g_gate_up
+    if want("embedding"):
+        dy, table = rnd(N, H), torch.zeros(V, H, device="cuda", dtype=dtype)
+        t = timed(torch, stream, lambda: ops.embedding_backward(table, dy, ids, N, stream, ops.EmbeddingBackwardOptions(accumulate_weight=True)))
+        record(f"embedding_backward {N} tokens into [{V},{H}]", "hbm", 3 * N * H * e, t, "dy read, table rows read and written")
+        del dy, table
+    if want("cut_cross_entropy"):
+        x, c = rnd(N, H), rnd(V, H, scale=0.02)
+        dx, dc, loss = torch.empty_like(x), torch.empty_like(c), torch.zeros(1, device="cuda")
+        t = timed(torch, stream, lambda: ops.cut_cross_entropy_forward_backward(loss, dx, dc, x, c, ids, N, stream, 1024.0), launches=5, warm=2)
+        record(f"cut_cross_entropy_forward_backward [{N},{H}] x [{V},{H}]", "mfma", 3 * 2.0 * N * V * H, t,
+               "3 vocabulary contractions executed (logits, dX, dC); 4 in a recompute formulation")
+        del x, c, dx, dc
+    if want("dense_cross_entropy"):
+        rows = N // 2
+        logits = rnd(rows, V)
+        grad, loss = torch.empty_like(logits), torch.zeros(1, device="cuda")
+        t = timed(torch, stream, lambda: ops.cross_entropy_forward_backward(loss, grad, logits, ids[:rows], rows, stream, 1024.0), launches=10)
+        record(f"cross_entropy_forward_backward[{rows},{V}]", "hbm", 2 * rows * V * e, t, "logits read once, gradient written once")
+    return out
+
+
 def measured_traffic():
     """HBM bytes per launch of the probe kernel from the committed counter summary, or None."""
     try:
@@ -107,11 +230,74 @@ def measured_traffic():
     return None
 
 
+def cpu_model_name():
+    try:
+        with open("/proc/cpuinfo") as handle:
+            for line in handle:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def cpu_operator_samples(seed):
+    """Each backward operator of the CPU port alone, at the largest shape of the configuration that stays within
+    a few seconds on this host (seconds and the same algorithmic rate the GPU table uses)."""
+    import torch
+
+    from oracle import cpu_ops as c
+
+    g = torch.Generator().manual_seed(seed)
+    out = {}
+
+    def sample(name, amount, unit, shape, fn):
+        start = time.perf_counter()
+        fn()
+        seconds = time.perf_counter() - start
+        out[name] = {"shape": shape, "seconds": round(seconds, 3), "rate": round(amount / seconds / 1e9, 2), "unit": unit}
+
+    rows, hidden = 32768, 1024
+    x, dy, w = torch.randn(rows, hidden, generator=g), torch.randn(rows, hidden, generator=g), torch.ones(hidden)
+    dx, dw = torch.empty_like(x), torch.empty_like(w)
+    sample("rmsnorm_backward", 3 * rows * hidden * 4, "GB/s", f"[{rows},{hidden}] fp32", lambda: c.rmsnorm_backward(dx, dw, dy, x, w, 1e-5))
+    q, k = torch.randn(8, 1024, 8, 128, generator=g), torch.randn(8, 1024, 2, 128, generator=g)
+    cos, sin = torch.rand(1024, 64, generator=g), torch.rand(1024, 64, generator=g)
+    gq, gk = torch.empty_like(q), torch.empty_like(k)
+    sample("rope_backward", 2 * (q.numel() + k.numel()) * 4, "GB/s", "q[8,1024,8,128] k[8,1024,2,128] fp32", lambda: c.rope_backward(gq, gk, q, k, cos, sin))
+    gate, up, dyi = (torch.randn(8192, 2048, generator=g) for _ in range(3))
+    dg, du = torch.empty_like(gate), torch.empty_like(up)
+    sample("swiglu_backward", 5 * gate.numel() * 4, "GB/s", "[8192,2048] fp32", lambda: c.swiglu_backward(dg, du, dyi, gate, up))
+    rows, fin, fout = 1024, 1024, 1024
+    x, wt, dy = torch.randn(rows, fin, generator=g), torch.randn(fout, fin, generator=g), torch.randn(rows, fout, generator=g)
+    gi, gw, gb = torch.empty_like(x), torch.empty_like(wt), torch.empty(fout)
+    sample("linear_backward", 2 * 2.0 * rows * fin * fout, "GFLOP/s", f"rows {rows}, {fout}x{fin} fp32 (dX and dW)", lambda: c.linear_backward(gi, gw, gb, dy, x, wt))
+    tokens = torch.randint(0, 32000, (32768,), generator=g, dtype=torch.int32)
+    dy, table = torch.randn(32768, 1024, generator=g), torch.zeros(32000, 1024)
+    sample("embedding_backward", 3 * dy.numel() * 4, "GB/s", "32768 tokens into [32000,1024] fp32", lambda: c.embedding_backward(table, dy, tokens, True, True))
+    logits, targets = torch.randn(1024, 32000, generator=g), torch.randint(0, 32000, (1024,), generator=g, dtype=torch.int32)
+    grad, loss = torch.empty_like(logits), torch.empty(1)
+    sample("cross_entropy_forward_backward", 2 * logits.numel() * 4, "GB/s", "[1024,32000] fp32", lambda: c.cross_entropy_forward_backward(loss, grad, logits, targets, 1024.0))
+    T = 64
+    q, k, v = torch.randn(1, T, 8, 128, generator=g), torch.randn(1, T, 2, 128, generator=g), torch.randn(1, T, 2, 128, generator=g)
+    do = torch.randn(1, T, 8, 128, generator=g)
+    gq, gk, gv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    sample("flash_gqa_attention_backward", 5 * 2.0 * 8 * T * T * 128 / 2, "GFLOP/s",
+           f"B=1 T={T} 8:2 heads D=128 fp32; NOT extrapolable: the operator recomputes the softmax row per output element "
+           "(cost grows with T^3)", lambda: c.attention_backward(gq, gk, gv, do, q, k, v, 8, 2, 128))
+    n = 104_090_624
+    p_, g_, m_, a_, b_ = torch.zeros(n), torch.full((n,), 1e-3), torch.zeros(n), torch.zeros(n), torch.zeros(n)
+    sample("adamw", 30.0 * n, "GB/s", f"{n} parameters fp32 (rate on the 30 B/parameter the 16-bit GPU update moves)",
+           lambda: c.adamw(p_, g_, m_, a_, b_, 1, 3e-4, 0.9, 0.95, 1e-8, 0.1, 1024.0, 1.0, parallel=True))
+    return out
+
+
 def cpu_baseline(seed):
-    """Times the CPU port on one step of the same 104m model (forward + loss + backward + AdamW) at B=1
-    and the longest sequence that keeps the sample near 10-30 s on this host: T doubles from 16 while the
-    last step took under 8 s and four times as long (the port's attention backward grows faster than
-    linearly in T) would still stay under 40 s. The last timing is the sample."""
+    """The CPU port on this host: (1) `value`: one full step of the same 104m model (forward + loss + backward +
+    AdamW) at B=1 and the longest sequence that keeps the sample near 10-30 s (T doubles from 16 while the last step
+    took under 8 s and four times as long would still stay under 40 s); (2) the reference's CPU-runnable
+    configuration: forward + cross-entropy loss at B=1, T=256, fp32, with its loss and logits checksum; (3) each
+    backward operator alone."""
     from oracle import cpu_model, cpu_ops
 
     cfg = dict(vocab=32000, layers=8, hidden=1024, inter=2048, hq=8, hkv=2, d=128, eps=1e-5)
@@ -120,10 +306,18 @@ def cpu_baseline(seed):
     while seconds < 8.0 and 4.0 * seconds < 40.0 and seq < 128:
         seq *= 2
         seconds, loss = cpu_model.timed_train_step(cfg, batch, seq, seed)
+    forward_seconds, forward_loss, checksum = cpu_model.timed_forward_loss(cfg, 1, 256, seed)
     return {"value": batch * seq / seconds, "unit": "tokens/s", "cores": cpu_ops.max_threads(), "kind": "port",
+            "cpu": cpu_model_name(),
             "sample": f"one full 104m train step (fwd+loss+bwd+AdamW, fp32) at B={batch}, T={seq}: "
                       f"{seconds:.1f} s, loss {loss:.3f}; the fixed AdamW pass over 104M parameters is part of "
-                      "the sample, the contractions are unblocked loops"}
+                      "the sample, the contractions are unblocked loops",
+            "configuration_1": {"workload": "forward + cross-entropy loss, 104m dims, fp32, B=1, T=256 "
+                                            "(src/core/generation_cpu.cpp:323-379 order; linear_forward_cpu is "
+                                            "serial for more than one row)",
+                                "seconds": round(forward_seconds, 2), "tokens_per_s": round(256 / forward_seconds, 2),
+                                "loss": forward_loss, "logits_checksum": checksum},
+            "operators": cpu_operator_samples(seed)}
 
 
 def main() -> int:
@@ -134,9 +328,15 @@ def main() -> int:
     parser.add_argument("--batch", type=int, default=32)
     parser.add_argument("--seq", type=int, default=1024)
     parser.add_argument("--loss", choices=["cut", "dense"], default="cut")
+    parser.add_argument("--dtype", choices=["bf16", "f16"], default="bf16")
+    parser.add_argument("--no-kernel-table", action="store_true", help="skip the isolated per-operator launches")
     parser.add_argument("--no-graph", action="store_true")
     parser.add_argument("--no-cpu-baseline", action="store_true")
     parser.add_argument("--seed", type=int, default=0)
+    parser.add_argument("--kernels-only", metavar="NAME", default=None,
+                        help="run only the isolated operator launches whose name contains NAME (rmsnorm, rope, "
+                             "attention, swiglu, embedding, cut_cross_entropy, dense_cross_entropy; '' = all) and print "
+                             "their table: the target of per-kernel rocprofv3 runs")
     parser.add_argument("--probe-only", action="store_true",
                         help="launch only the dominant kernel (20x) and a 1 GiB device copy: the target of the "
                              "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs behind roofline.traffic")
@@ -155,7 +355,13 @@ def main() -> int:
         print("bench.py: no GPU visible", file=sys.stderr)
         return 3
     device = torch.device("cuda:0")
-    cfg = ModelConfig()  # the reference's 104m preset
+    dtype = torch.bfloat16 if args.dtype == "bf16" else torch.float16
+    cfg = ModelConfig(dtype=dtype)  # the reference's 104m preset
+    if args.kernels_only is not None:
+        stream = torch.cuda.Stream(device=device)
+        print(json.dumps({"kernels": isolated_kernels(torch, cfg, args.batch, args.seq, dtype, stream, args.seed,
+                                                      args.kernels_only)}))
+        return 0
     if args.probe_only:
         stream = torch.cuda.Stream(device=device)
         probe = kernel_probe(torch, cfg, args.batch, args.seq, stream, 20, args.seed)
@@ -178,7 +384,7 @@ def main() -> int:
 
     for _ in range(args.warmup):
         model.train_step(options, loss_mode, use_graph, stream)
-    first_loss, finite, _ = model.status(stream)
+    loss_after_warmup, finite, _ = model.status(stream)
     torch.cuda.synchronize()
     start = time.perf_counter()
     for _ in range(args.steps):
@@ -190,7 +396,7 @@ def main() -> int:
     tokens = args.batch * args.seq
     ms_per_step = elapsed / max(args.steps, 1) * 1e3
 
-    probe = kernel_probe(torch, cfg, args.batch, args.seq, stream, 20, args.seed)
+    probe = kernel_probe(torch, cfg, args.batch, args.seq, stream, 20, args.seed, dtype)
     labelled = model.profile(options.loss_scale, loss_mode, stream)
     # Labels are "kind" or "kind.part"; the parts of a kind add up in the breakdown.
     breakdown = {}
@@ -208,10 +414,32 @@ def main() -> int:
     back_to_back = probe["flops"] / probe["seconds"] / 1e12
     per_kind = {}
     for kind, ms in sorted(breakdown.items(), key=lambda kv: -kv[1]):
+        if kind not in work:
+            continue
         b, amt = work[kind]
         rate = amt / (ms * 1e-3) / (1e12 if b == "mfma" else 1e9)
         per_kind[kind] = {"ms": round(ms, 3), "rate": round(rate, 1), "unit": "TFLOP/s" if b == "mfma" else "GB/s",
                           "frac": round(rate / (PEAK_BF16_TFLOPS if b == "mfma" else PEAK_HBM_GBS), 4)}
+    # Every contraction of the step by position: one launch per layer (the classifier's: one per step).
+    shapes = gemm_shapes(cfg, args.batch, args.seq)
+    launches = {}
+    for label, ms in labelled.items():
+        if label in shapes:
+            m_, n_, k_ = shapes[label]
+            calls = 1 if label.endswith("classifier") else cfg.num_layers
+            tflops = 2.0 * m_ * n_ * k_ * calls / (ms * 1e-3) / 1e12
+            launches[label] = {"m": m_, "n": n_, "k": k_, "calls": calls, "us_per_call": round(ms * 1e3 / calls, 1),
+                               "tflops": round(tflops, 1), "frac": round(tflops / PEAK_BF16_TFLOPS, 4)}
+    family = {kind: per_kind[kind]["frac"] for kind in ("gemm_fwd", "gemm_dx", "gemm_dw") if kind in per_kind}
+    kernels = {} if args.no_kernel_table else isolated_kernels(torch, cfg, args.batch, args.seq, dtype, stream, args.seed)
+    # AdamW over all parameters (3 launches for the 90 tensors): 30 B/parameter with 16-bit gradients and parameters.
+    options_probe = options
+    adamw_seconds = timed(torch, stream, lambda: model.optimizer_step(options_probe, stream), launches=5, warm=1)
+    adamw_bytes = 30.0 * model.num_parameters
+    kernels["adamw_step_many_async"] = {
+        "shape": f"{model.num_parameters} parameters in 90 tensors", "bound": "hbm", "us": round(adamw_seconds * 1e6, 1),
+        "rate": round(adamw_bytes / adamw_seconds / 1e9, 1), "unit": "GB/s",
+        "frac": round(adamw_bytes / adamw_seconds / 1e9 / PEAK_HBM_GBS, 4)}
 
     result = {
         "metric": f"train tokens/sec, 104m fwd+bwd+AdamW B={args.batch} T={args.seq}",
@@ -224,13 +452,13 @@ def main() -> int:
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "bf16",
+        "dtype": args.dtype,
         "data": "synthetic",
         "config": {"workload": f"full 104m train step (embedding, 8 blocks, {args.loss} cross-entropy, backward, "
                                f"AdamW), B={args.batch}, T={args.seq}, hipGraph={'on' if use_graph else 'off'}",
                    "parameters": model.num_parameters, "global_batch": args.batch, "seq_len": args.seq,
                    "loss_scale": 1024.0},
-        "loss_first": first_loss, "loss_last": last_loss, "all_finite": bool(finite and finite_after),
+        "loss_after_warmup": loss_after_warmup, "loss_last": last_loss, "all_finite": bool(finite and finite_after),
         "optimizer_steps": steps_done,
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / PEAK_BF16_TFLOPS, "traffic": measured_traffic(),
@@ -245,8 +473,13 @@ def main() -> int:
                              "row on random bf16 data, where the chip's power limit lowers the clock; traffic = "
                              "HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE, calibrated on a "
                              "1 GiB copy; breakdown = per operator kind, algorithmic work of one step / summed "
-                             "event-timed duration of its calls (the same eager pass)",
-                     "breakdown": per_kind},
+                             "event-timed duration of its calls (the same eager pass); "
+                             "family_step_wide = the contraction family's fractions over the whole step (from "
+                             "breakdown), next to the best launch quoted as `frac`; gemm_launches = every contraction "
+                             "by position in that pass; kernels = each backward operator alone at the configuration's "
+                             "shape, 20 back-to-back launches between HIP events on the launch stream",
+                     "family_step_wide": family,
+                     "breakdown": per_kind, "gemm_launches": launches, "kernels": kernels},
     }
     model.close()
     if not args.no_cpu_baseline:
