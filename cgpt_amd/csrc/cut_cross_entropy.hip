@@ -20,6 +20,7 @@
 
 #include <algorithm>
 #include <cmath>
+#include <cstdlib>
 #include <limits>
 
 namespace cgptx {
@@ -62,17 +63,24 @@ extern "C" int cgptx_cut_cross_entropy_forward_backward(float* loss, void* input
         return fail(CGPTX_OVERFLOW, std::string(name) + ": dimension exceeds int range");
     auto stream = static_cast<hipStream_t>(stream_);
     const std::size_t elem = dtype_size(dtype);
-    // Chunk so that the logits scratch stays near 1 GiB whatever the number of rows, while each
-    // chunk still gives the three contractions enough 256x256 tiles to fill the chip. The rows are
-    // split evenly over the chunks (32768 rows at V=32000: 2 x 16384, so that the input-gradient
-    // contraction has 64 x 4 tiles, one per CU; 16640 + 16128 would cost it a second round for 4 tiles).
-    std::size_t limit = (std::size_t{1} << 30) / (vocab * elem);
+    // Chunk so that the logits scratch stays within 2 GiB whatever the number of rows (a small fraction of this
+    // GPU's memory; CGPTX_CUT_CE_LOGITS_BYTES, read per call, sets another bound), while each chunk still gives
+    // the three contractions enough 256x256 tiles to fill the chip. The rows are split evenly over the chunks.
+    // 32768 rows at V=32000 are one chunk: the classifier gradient then comes straight out of its contraction,
+    // rounded once, without the fp32 accumulator and the pass that folds it into the gradient.
+    std::size_t logits_bytes = std::size_t{1} << 31;
+    if (const char* text = std::getenv("CGPTX_CUT_CE_LOGITS_BYTES")) {
+        const unsigned long long asked = std::strtoull(text, nullptr, 0);
+        if (asked > 0) logits_bytes = static_cast<std::size_t>(asked);
+    }
+    std::size_t limit = logits_bytes / (vocab * elem);
     limit = std::max<std::size_t>(256, limit / 256 * 256);
     const std::size_t pieces = (rows + limit - 1) / limit;
     std::size_t chunk = ((rows + pieces - 1) / pieces + 255) / 256 * 256;
     chunk = std::min(chunk, rows);
+    const bool single = chunk >= rows;
     const std::size_t loss_bytes = (rows * sizeof(float) + 255) & ~std::size_t{255};
-    const std::size_t acc_bytes = (vocab * hidden * sizeof(float) + 255) & ~std::size_t{255};
+    const std::size_t acc_bytes = single ? 0 : (vocab * hidden * sizeof(float) + 255) & ~std::size_t{255};
     const std::size_t logit_bytes = (chunk * vocab * elem + 255) & ~std::size_t{255};
     void* mem = nullptr;
     // Arena layout: [row_loss | acc | logits]. The contractions below run with no_split, so they
@@ -115,10 +123,10 @@ extern "C" int cgptx_cut_cross_entropy_forward_backward(float* loss, void* input
         dx.dtype = dtype;
         dx.no_split = true;
         if (int s = gemm(dx, stream)) return s;
-        GemmArgs dc;  // acc[V, H] (+)= dZᵀ[V, r]·X[r, H], fp32
+        GemmArgs dc;  // acc[V, H] (+)= dZᵀ[V, r]·X[r, H], fp32; a single chunk writes the gradient itself
         dc.a = logits;
         dc.b = x;
-        dc.c = acc;
+        dc.c = single ? classifier_gradient : static_cast<void*>(acc);
         dc.m = vocab;
         dc.n = hidden;
         dc.k = r;
@@ -127,13 +135,14 @@ extern "C" int cgptx_cut_cross_entropy_forward_backward(float* loss, void* input
         dc.ldc = hidden;
         dc.a_k_contiguous = false;
         dc.b_k_contiguous = false;
-        dc.accumulate = r0 != 0;
-        dc.c_is_f32 = true;
+        dc.accumulate = single ? accumulate_classifier != 0 : r0 != 0;
+        dc.c_is_f32 = !single;
         dc.dtype = dtype;
         dc.no_split = true;
         if (int s = gemm(dc, stream)) return s;
     }
     if (int s = mean_reduce(loss, row_loss, rows, stream)) return s;
+    if (single) return CGPTX_OK;
     const std::size_t count = vocab * hidden;
     const std::size_t blocks = std::min<std::size_t>((count + kThreads - 1) / kThreads,
                                                      static_cast<std::size_t>(compute_units()) * 16);

@@ -55,8 +55,13 @@ def test_parity_with_float64(device, rows, hidden, vocab, dtype):
     assert_scaled_close(dc2, want, TOL[dtype], "dC accumulate")
 
 
-def test_equivalent_to_dense_cross_entropy_plus_linear_backward(device):
-    """Several row chunks (rows > the chunk derived from 128 MiB / vocab): bf16, [6000, 256] x [32000, 256]."""
+@pytest.mark.parametrize("logits_bytes", [None, 128 << 20], ids=["one-chunk", "three-chunks"])
+def test_equivalent_to_dense_cross_entropy_plus_linear_backward(device, monkeypatch, logits_bytes):
+    """bf16, [6000, 256] x [32000, 256], as one chunk of logits (the classifier gradient straight out of its
+    contraction) and as several row chunks (CGPTX_CUT_CE_LOGITS_BYTES = 128 MiB: 3 chunks of 2048 rows, the
+    classifier gradient accumulated in fp32 across them)."""
+    if logits_bytes is not None:
+        monkeypatch.setenv("CGPTX_CUT_CE_LOGITS_BYTES", str(logits_bytes))
     dtype = torch.bfloat16
     rows, hidden, vocab = 6000, 256, 32000
     x, c = randn((rows, hidden), dtype, 5).to(device), randn((vocab, hidden), dtype, 6, 0.05).to(device)
