@@ -209,6 +209,12 @@ def _isolated_rest(torch, ops, want, record, rnd, timed, stream, out, N, H, I, V
         record(f"cut_cross_entropy_forward_backward [{N},{H}] x [{V},{H}]", "mfma", 3 * 2.0 * N * V * H, t,
                "3 vocabulary contractions executed (logits, dX, dC); 4 in a recompute formulation")
         del x, c, dx, dc
+    if want("copy"):  # calibration of the profiler's FETCH_SIZE / WRITE_SIZE counters: reads and writes 1 GiB
+        source = torch.empty(1 << 30, dtype=torch.uint8, device="cuda")
+        target = torch.empty_like(source)
+        t = timed(torch, torch.cuda.current_stream(), lambda: target.copy_(source), launches=5, warm=1)
+        record("copy 1 GiB (torch)", "hbm", 2.0 * (1 << 30), t, "1 GiB read, 1 GiB written")
+        del source, target
     if want("dense_cross_entropy"):
         rows = N // 2
         logits = rnd(rows, V)
@@ -335,7 +341,7 @@ def main() -> int:
     parser.add_argument("--seed", type=int, default=0)
     parser.add_argument("--kernels-only", metavar="NAME", default=None,
                         help="run only the isolated operator launches whose name contains NAME (rmsnorm, rope, "
-                             "attention, swiglu, embedding, cut_cross_entropy, dense_cross_entropy; '' = all) and print "
+                             "attention, swiglu, embedding, cut_cross_entropy, dense_cross_entropy, copy; '' = all) and print "
                              "their table: the target of per-kernel rocprofv3 runs")
     parser.add_argument("--probe-only", action="store_true",
                         help="launch only the dominant kernel (20x) and a 1 GiB device copy: the target of the "

@@ -197,19 +197,37 @@ __device__ __forceinline__ int acc_row(int i) { return 8 * (i >> 2) + 4 * ((thre
 // to the 8 XCDs round-robin. Under a causal mask a query block's work grows with its position, so
 // the linear id is read position-major with the last (longest) query blocks first: the work that
 // is handed out last is the shortest, which keeps the tail of the launch short, and every XCD
-// receives the same mix of lengths (heads x batch workgroups of each).
+// receives the same mix of lengths.
+// Each XCD has its own L2, and the workgroups that stream the same K and V are the heads of one GQA group
+// at every query position: when the (batch, kv-head) pairs divide evenly over the 8 XCDs, XCD x (linear id
+// mod 8) takes pairs x, x + 8, ... and walks positions (longest first) x its pairs x the heads of the group,
+// so that the workgroups resident on an XCD at any time share a few K/V streams instead of each bringing
+// its own from memory.
 struct BlockCoordinates {
     int q_block;  // first query row
     int h, b;
 };
-__device__ __forceinline__ BlockCoordinates block_coordinates() {
+__device__ __forceinline__ BlockCoordinates block_coordinates(int hkv) {
+    constexpr unsigned int kXcds = 8;
     const unsigned int linear = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
-    const unsigned int per_position = gridDim.y * gridDim.z;
-    const unsigned int position = linear / per_position, rest = linear - position * per_position;
+    const unsigned int heads = gridDim.y, batch = gridDim.z, positions = gridDim.x;
+    const unsigned int pairs = batch * static_cast<unsigned int>(hkv), group = heads / static_cast<unsigned int>(hkv);
     BlockCoordinates c;
-    c.q_block = static_cast<int>(gridDim.x - 1 - position) * kBlockRows;
-    c.h = static_cast<int>(rest % gridDim.y);
-    c.b = static_cast<int>(rest / gridDim.y);
+    if (pairs % kXcds == 0) {
+        const unsigned int xcd = linear % kXcds, local = linear / kXcds;
+        const unsigned int per_position = (pairs / kXcds) * group;
+        const unsigned int position = local / per_position, rest = local - position * per_position;
+        const unsigned int pair = xcd + kXcds * (rest / group), head_in_group = rest % group;
+        c.q_block = static_cast<int>(positions - 1 - position) * kBlockRows;
+        c.b = static_cast<int>(pair / static_cast<unsigned int>(hkv));
+        c.h = static_cast<int>((pair % static_cast<unsigned int>(hkv)) * group + head_in_group);
+        return c;
+    }
+    const unsigned int per_position = heads * batch;
+    const unsigned int position = linear / per_position, rest = linear - position * per_position;
+    c.q_block = static_cast<int>(positions - 1 - position) * kBlockRows;
+    c.h = static_cast<int>(rest % heads);
+    c.b = static_cast<int>(rest / heads);
     return c;
 }
 
@@ -220,7 +238,7 @@ __global__ __launch_bounds__(kThreads) void attention_forward_kernel(Params p) {
     __shared__ __align__(16) T k_lds[kStream * lds_stride<DP>()];
     __shared__ __align__(16) T v_lds[kStream * lds_stride<DP>()];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const BlockCoordinates where = block_coordinates();
+    const BlockCoordinates where = block_coordinates(p.hkv);
     const int b = where.b, h = where.h, kvh = h / (p.hq / p.hkv);
     const int q_block = where.q_block;
     const int q_row = q_block + wave * 32 + (lane & 31);
@@ -365,7 +383,7 @@ __global__ __launch_bounds__(kThreads) void attention_dq_kernel(Params p) {
     __shared__ __align__(16) T k_lds[kStream * lds_stride<DP>()];
     __shared__ __align__(16) T v_lds[kStream * lds_stride<DP>()];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const BlockCoordinates where = block_coordinates();
+    const BlockCoordinates where = block_coordinates(p.hkv);
     const int b = where.b, h = where.h, kvh = h / (p.hq / p.hkv);
     const int q_block = where.q_block;
     const int q_row = q_block + wave * 32 + (lane & 31);
@@ -755,7 +773,7 @@ __global__ __launch_bounds__(kThreads, 2) void attention_forward_wide_kernel(Par
     __shared__ __align__(1024) T lds[4 * kWideTile<W>];  // [stage][K | V]
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const BlockCoordinates where = block_coordinates();
+    const BlockCoordinates where = block_coordinates(p.hkv);
     const int b = where.b, h = where.h, kvh = h / (p.hq / p.hkv);
     const int q_block = where.q_block;
     const int q_row = q_block + wave * 32 + (lane & 31);
@@ -923,7 +941,7 @@ __global__ __launch_bounds__(kThreads, 2) void attention_dq_wide_kernel(Params p
     __shared__ __align__(1024) T lds[4 * kWideTile<W>];  // [stage][K | V]
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const BlockCoordinates where = block_coordinates();
+    const BlockCoordinates where = block_coordinates(p.hkv);
     const int b = where.b, h = where.h, kvh = h / (p.hq / p.hkv);
     const int q_block = where.q_block;
     const int q_row = q_block + wave * 32 + (lane & 31);
@@ -1074,7 +1092,24 @@ __global__ __launch_bounds__(kThreads, 1) void attention_dkv_wide_kernel(Params 
     float* stats = reinterpret_cast<float*>(wide_smem + 4 * kWideTile<W> * sizeof(T));  // [stage][lse2 | delta][64]
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int b = blockIdx.z, kvh = blockIdx.y, group = p.hq / p.hkv;
+    // Workgroup -> (key-block pair, kv head, batch entry). The pairs of one (batch, kv-head) stream the same Q and
+    // dO rows: when the (batch, kv-head) pairs divide evenly over the 8 XCDs (workgroups go to them round-robin by
+    // linear id), XCD x takes pairs x, x + 8, ... with all key-block pairs of each next to each other, so that they
+    // run at the same time behind the same L2.
+    int pair_x = static_cast<int>(blockIdx.x), b = static_cast<int>(blockIdx.z), kvh = static_cast<int>(blockIdx.y);
+    {
+        constexpr unsigned int kXcds = 8;
+        const unsigned int linear = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+        const unsigned int owners = gridDim.y * gridDim.z;
+        if (owners % kXcds == 0) {
+            const unsigned int xcd = linear % kXcds, local = linear / kXcds;
+            const unsigned int owner = xcd + kXcds * (local / gridDim.x);
+            pair_x = static_cast<int>(local % gridDim.x);
+            kvh = static_cast<int>(owner % gridDim.y);
+            b = static_cast<int>(owner / gridDim.y);
+        }
+    }
+    const int group = p.hq / p.hkv;
     const long q_stride = static_cast<long>(p.hq) * p.d, kv_stride = static_cast<long>(p.hkv) * p.d;
     const float scale2 = p.scale * kLog2e;
 
@@ -1100,8 +1135,8 @@ __global__ __launch_bounds__(kThreads, 1) void attention_dkv_wide_kernel(Params 
 
     const int key_blocks = (p.ks + kBlockRows - 1) / kBlockRows;
     for (int half = 0; half < 2; ++half) {
-        const int block_index = half == 0 ? static_cast<int>(blockIdx.x) : key_blocks - 1 - static_cast<int>(blockIdx.x);
-        if (half == 1 && block_index <= static_cast<int>(blockIdx.x)) break;
+        const int block_index = half == 0 ? pair_x : key_blocks - 1 - pair_x;
+        if (half == 1 && block_index <= pair_x) break;
         const int k_block = block_index * kBlockRows;
         const int k_row = k_block + wave * 32 + (lane & 31);
         const bool k_live = k_row < p.ks;
