@@ -131,7 +131,7 @@ def timed(torch, stream, fn, launches=20, warm=3):
     return start.elapsed_time(stop) * 1e-3 / launches
 
 
-def isolated_kernels(torch, cfg, batch, seq, dtype, stream, seed, only=""):
+def isolated_kernels(torch, cfg, batch, seq, dtype, stream, seed, only="", secondary=True):
     """Every backward operator alone at the configuration's shape: algorithmic bytes or FLOPs of one call /
     its average duration over 20 back-to-back calls. `only`: run just the sections whose name contains it."""
     from cgpt_amd import ops
@@ -161,6 +161,13 @@ def isolated_kernels(torch, cfg, batch, seq, dtype, stream, seed, only=""):
         t = timed(torch, stream, lambda: ops.rmsnorm_backward(dx, dw, dy, x, w, 1e-5, stream))
         record(f"rmsnorm_backward[{rows},{hidden}]", "hbm", 3 * rows * hidden * e, t, f"x, dy read, dx written")
         del x, dy, dx
+    if secondary and want("secondary"):
+        # The 12 x 768 shape named beside the preset (12:4 heads of 64): norm, rotary, attention and cut cross-entropy.
+        import dataclasses
+        second = dataclasses.replace(cfg, hidden_size=768, num_query_heads=12, num_kv_heads=4, head_dim=64, rotary_dim=64)
+        for section in ("rmsnorm", "rope", "attention", "cut_cross_entropy"):
+            for name, entry in isolated_kernels(torch, second, batch, seq, dtype, stream, seed, section, False).items():
+                out["secondary: " + name] = entry
     ids = torch.randint(0, V, (N,), device="cuda", generator=gen, dtype=torch.int32)
     if not (want("rope") or want("attention")):
         return _isolated_rest(torch, ops, want, record, rnd, timed, stream, out, N, H, I, V, e, ids)
@@ -221,6 +228,58 @@ def _isolated_rest(torch, ops, want, record, rnd, timed, stream, out, N, H, I, V
         grad, loss = torch.empty_like(logits), torch.zeros(1, device="cuda")
         t = timed(torch, stream, lambda: ops.cross_entropy_forward_backward(loss, grad, logits, ids[:rows], rows, stream, 1024.0), launches=10)
         record(f"cross_entropy_forward_backward[{rows},{V}]", "hbm", 2 * rows * V * e, t, "logits read once, gradient written once")
+    return out
+
+
+def published_kernel_shapes(torch, stream, seed):
+    """The launches of the reference's own kernel table (kernel_profile.md:9-25: B = 1, T = 512, 32:8 heads, D = 128,
+    hidden 4096, measured by its authors on a 192 GB/s GPU) on this GPU: average us over 50 back-to-back calls beside
+    the published milliseconds. These launches are small (2 to 100 MB): they measure launch latency as much as rate."""
+    from cgpt_amd import ops
+
+    gen = torch.Generator(device="cuda").manual_seed(seed)
+
+    def rnd(*shape, dtype=torch.float16):
+        return torch.randn(*shape, device="cuda", generator=gen).to(dtype)
+
+    out = {}
+
+    def record(name, published_ms, seconds):
+        out[name] = {"us": round(seconds * 1e6, 1), "published_ms": published_ms,
+                     "speedup": round(published_ms * 1e-3 / seconds, 1)}
+
+    for dtype, label, ms in ((torch.float16, "F16", 0.1228), (torch.bfloat16, "BF16", 0.1230)):
+        x, dy, w = rnd(512, 4096, dtype=dtype), rnd(512, 4096, dtype=dtype), rnd(4096, dtype=dtype)
+        dx, dw = torch.empty_like(x), torch.empty_like(w)
+        record(f"rmsnorm_backward {label} [512,4096]", ms,
+               timed(torch, stream, lambda: ops.rmsnorm_backward(dx, dw, dy, x, w, 1e-5, stream), launches=50))
+    B, T, HQ, HKV, D = 1, 512, 32, 8, 128
+    q, k, v, do = rnd(B, T, HQ, D), rnd(B, T, HKV, D), rnd(B, T, HKV, D), rnd(B, T, HQ, D)
+    pos = torch.arange(T, device="cuda", dtype=torch.float32)[:, None]
+    theta = pos / torch.pow(torch.tensor(10000.0, device="cuda"), torch.arange(D // 2, device="cuda") * 2.0 / D)[None, :]
+    cos, sin = torch.cos(theta).to(torch.float16), torch.sin(theta).to(torch.float16)
+    gq, gk, gv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(k)
+    record("rope_backward F16 q[1,512,32,128] k[1,512,8,128]", 0.0640,
+           timed(torch, stream, lambda: ops.rope_backward(gq, gk, q, k, cos, sin, stream), launches=50))
+    opt = ops.FlashAttentionOptions(HQ, HKV, D, causal=False)
+    o, lse = torch.empty_like(q), torch.empty(B, T, HQ, device="cuda")
+    ops.flash_gqa_attention_forward_with_lse(o, lse, q, k, v, stream, opt)
+    record("flash_gqa_attention_backward F16 B=1 T=512 32:8 D=128 non-causal", 1.9464,
+           timed(torch, stream, lambda: ops.flash_gqa_attention_backward(gq, gk, gv, do, q, k, v, stream, opt), launches=50))
+    record("flash_gqa_attention_backward_with_lse, same shape", 1.6369,
+           timed(torch, stream, lambda: ops.flash_gqa_attention_backward_with_lse(gq, gk, gv, do, o, lse, q, k, v, stream, opt),
+                 launches=50))
+    ids = torch.arange(512, device="cuda", dtype=torch.int32)  # embedding_test.cu:205-230: distinct ids, accumulating
+    dy, table = rnd(512, 4096), torch.zeros(32000, 4096, device="cuda", dtype=torch.float16)
+    accumulate = ops.EmbeddingBackwardOptions(accumulate_weight=True)
+    record("embedding_backward F16 512 tokens into [32000,4096]", 0.0766,
+           timed(torch, stream, lambda: ops.embedding_backward(table, dy, ids, 512, stream, accumulate), launches=50))
+    del table
+    logits = rnd(512, 50257, dtype=torch.float32)
+    grad, loss = torch.empty_like(logits), torch.zeros(1, device="cuda")
+    targets = torch.randint(0, 50257, (512,), device="cuda", generator=gen, dtype=torch.int32)
+    record("cross_entropy_forward_backward F32 [512,50257]", 2.3196,
+           timed(torch, stream, lambda: ops.cross_entropy_forward_backward(loss, grad, logits, targets, 512, stream), launches=50))
     return out
 
 
@@ -365,8 +424,10 @@ def main() -> int:
     cfg = ModelConfig(dtype=dtype)  # the reference's 104m preset
     if args.kernels_only is not None:
         stream = torch.cuda.Stream(device=device)
-        print(json.dumps({"kernels": isolated_kernels(torch, cfg, args.batch, args.seq, dtype, stream, args.seed,
-                                                      args.kernels_only)}))
+        shown = {"kernels": isolated_kernels(torch, cfg, args.batch, args.seq, dtype, stream, args.seed, args.kernels_only)}
+        if "published" in args.kernels_only or args.kernels_only == "":
+            shown["published_kernel_shapes"] = published_kernel_shapes(torch, stream, args.seed)
+        print(json.dumps(shown))
         return 0
     if args.probe_only:
         stream = torch.cuda.Stream(device=device)
@@ -438,6 +499,7 @@ def main() -> int:
                                "tflops": round(tflops, 1), "frac": round(tflops / PEAK_BF16_TFLOPS, 4)}
     family = {kind: per_kind[kind]["frac"] for kind in ("gemm_fwd", "gemm_dx", "gemm_dw") if kind in per_kind}
     kernels = {} if args.no_kernel_table else isolated_kernels(torch, cfg, args.batch, args.seq, dtype, stream, args.seed)
+    published = {} if args.no_kernel_table else published_kernel_shapes(torch, stream, args.seed)
     # AdamW over all parameters (3 launches for the 90 tensors): 30 B/parameter with 16-bit gradients and parameters.
     options_probe = options
     adamw_seconds = timed(torch, stream, lambda: model.optimizer_step(options_probe, stream), launches=5, warm=1)
@@ -483,9 +545,12 @@ def main() -> int:
                              "family_step_wide = the contraction family's fractions over the whole step (from "
                              "breakdown), next to the best launch quoted as `frac`; gemm_launches = every contraction "
                              "by position in that pass; kernels = each backward operator alone at the configuration's "
-                             "shape, 20 back-to-back launches between HIP events on the launch stream",
+                             "shape, 20 back-to-back launches between HIP events on the launch stream; "
+                             "published_kernel_shapes = the launches of the reference's own kernel table "
+                             "(kernel_profile.md:9-25, other hardware) on this GPU",
                      "family_step_wide": family,
-                     "breakdown": per_kind, "gemm_launches": launches, "kernels": kernels},
+                     "breakdown": per_kind, "gemm_launches": launches, "kernels": kernels,
+                     "published_kernel_shapes": published},
     }
     model.close()
     if not args.no_cpu_baseline:

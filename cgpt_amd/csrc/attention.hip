@@ -94,6 +94,7 @@ struct Params {
     int batch, qs, ks, hq, hkv, d;
     float scale;
     int causal, offset, accumulate;
+    int paired;  // dK/dV, LDS-direct family: a workgroup takes key blocks (i, last - i) instead of one
 };
 
 template <int DP>
@@ -1134,7 +1135,7 @@ __global__ __launch_bounds__(kThreads, 1) void attention_dkv_wide_kernel(Params 
     }
 
     const int key_blocks = (p.ks + kBlockRows - 1) / kBlockRows;
-    for (int half = 0; half < 2; ++half) {
+    for (int half = 0; half < (p.paired ? 2 : 1); ++half) {
         const int block_index = half == 0 ? pair_x : key_blocks - 1 - pair_x;
         if (half == 1 && block_index <= pair_x) break;
         const int k_block = block_index * kBlockRows;
@@ -1670,7 +1671,12 @@ int launch_backward(const Shape& s, Params p, void* dq, void* dk, void* dv, cons
             const unsigned int key_blocks = static_cast<unsigned int>((s.ks + kBlockRows - 1) / kBlockRows);
             if (wide_path(s)) {
                 pk.lse = lse2;
-                const dim3 pair_grid((key_blocks + 1) / 2, static_cast<unsigned int>(s.hkv),
+                // Pairs equalise the work under a causal mask; without one every block carries the same work, and a
+                // grid that leaves compute units idle is better off with twice the workgroups (the longest single
+                // block is shorter than the pair that contains it).
+                const std::size_t single_blocks = static_cast<std::size_t>(key_blocks) * s.hkv * s.batch;
+                pk.paired = s.causal && single_blocks > static_cast<std::size_t>(compute_units());
+                const dim3 pair_grid(pk.paired ? (key_blocks + 1) / 2 : key_blocks, static_cast<unsigned int>(s.hkv),
                                      static_cast<unsigned int>(s.batch));
                 auto launch = [&]<int W>() -> int {
                     auto kernel = attention_dkv_wide_kernel<T, W>;

@@ -48,6 +48,10 @@ __device__ __forceinline__ MaxSum block_combine(MaxSum v, MaxSum* stage) {
     return total;
 }
 
+// Streaming kernel for rows that are too long to hold or not 16-byte aligned (a vocabulary that is not a
+// multiple of the vector width moves every row's start): each row is split into the elements before its first
+// 16-byte boundary, whole 128-bit vectors, and the rest. vector_ok: logits and gradient rows have the same
+// alignment phase (or there is no gradient).
 template <typename T, bool WithGradient>
 __global__ __launch_bounds__(kThreads) void cross_entropy_row_kernel(float* __restrict__ row_loss,
                                                                     T* gradient,  // may alias logits (in place)
@@ -59,14 +63,20 @@ __global__ __launch_bounds__(kThreads) void cross_entropy_row_kernel(float* __re
     __shared__ MaxSum stage[kWaves];
     const std::size_t base = static_cast<std::size_t>(blockIdx.x) * vocab;
     const T* row = logits + base;
-    const unsigned int vectors = vector_ok ? vocab / VEC : 0;
+    const unsigned int to_boundary =
+        static_cast<unsigned int>(((16u - (reinterpret_cast<std::uintptr_t>(row) & 15u)) & 15u) / sizeof(T));
+    const unsigned int head = vector_ok ? (to_boundary < vocab ? to_boundary : vocab) : vocab;
+    const unsigned int vectors = (vocab - head) / VEC;
+    const unsigned int body_end = head + vectors * VEC;
+    const unsigned int edge = head + (vocab - body_end);  // elements handled one by one
+    const T* body = row + head;
     const std::uint32_t target = targets[blockIdx.x];
     // Read before the barrier below: in-place use overwrites the row in pass 2.
     const float target_logit = (threadIdx.x == 0 && target < vocab) ? to_f32(row[target]) : 0.0f;
 
     MaxSum acc{-INFINITY, 0.0f};
     for (unsigned int v = threadIdx.x; v < vectors; v += kThreads) {
-        const vec_t<float, VEC> x = vec_to_f32<T, VEC>(load_vec<T, VEC>(row + v * VEC));
+        const vec_t<float, VEC> x = vec_to_f32<T, VEC>(load_vec<T, VEC>(body + v * VEC));
         float vmax = x[0];
 #pragma unroll
         for (int e = 1; e < VEC; ++e) vmax = fmaxf(vmax, x[e]);
@@ -79,7 +89,8 @@ __global__ __launch_bounds__(kThreads) void cross_entropy_row_kernel(float* __re
             for (int e = 0; e < VEC; ++e) acc.s += __expf(x[e] - acc.m);
         }
     }
-    for (unsigned int i = vectors * VEC + threadIdx.x; i < vocab; i += kThreads) {
+    for (unsigned int k = threadIdx.x; k < edge; k += kThreads) {
+        const unsigned int i = k < head ? k : body_end + (k - head);
         const float x = to_f32(row[i]);
         if (x > acc.m) {
             acc.s *= __expf(acc.m - x);
@@ -97,17 +108,18 @@ __global__ __launch_bounds__(kThreads) void cross_entropy_row_kernel(float* __re
         const float inv = 1.0f / total.s;
         T* out = gradient + base;
         for (unsigned int v = threadIdx.x; v < vectors; v += kThreads) {
-            const vec_t<float, VEC> x = vec_to_f32<T, VEC>(load_vec<T, VEC>(row + v * VEC));
+            const vec_t<float, VEC> x = vec_to_f32<T, VEC>(load_vec<T, VEC>(body + v * VEC));
             vec_t<float, VEC> g;
 #pragma unroll
             for (int e = 0; e < VEC; ++e) {
                 float value = __expf(x[e] - total.m) * inv;
-                if (v * VEC + e == target) value -= 1.0f;
+                if (head + v * VEC + e == target) value -= 1.0f;
                 g[e] = value * factor;
             }
-            store_vec<T, VEC>(out + v * VEC, vec_from_f32<T, VEC>(g));
+            store_vec<T, VEC>(out + head + v * VEC, vec_from_f32<T, VEC>(g));
         }
-        for (unsigned int i = vectors * VEC + threadIdx.x; i < vocab; i += kThreads) {
+        for (unsigned int k = threadIdx.x; k < edge; k += kThreads) {
+            const unsigned int i = k < head ? k : body_end + (k - head);
             float value = __expf(to_f32(row[i]) - total.m) * inv;
             if (i == target) value -= 1.0f;
             out[i] = from_f32<T>(value * factor);
@@ -232,6 +244,9 @@ int cross_entropy_rows(float* row_loss, void* gradient, const void* logits, cons
     return dispatch_dtype(dtype, [&]<typename T>() -> int {
         const bool vector_ok = vocab % kVec128<T> == 0 && is_aligned16(logits) &&
                                (!with_gradient || is_aligned16(gradient));
+        // The streaming kernel finds each row's own 16-byte boundary; logits and gradient rows must share it.
+        const bool same_phase = !with_gradient || ((reinterpret_cast<std::uintptr_t>(logits) ^
+                                                    reinterpret_cast<std::uintptr_t>(gradient)) & 15u) == 0;
         const unsigned int vectors = v / kVec128<T>;
         if (vector_ok && vectors <= 16u * kResidentThreads) {
             auto* g = static_cast<T*>(gradient);
@@ -241,10 +256,10 @@ int cross_entropy_rows(float* row_loss, void* gradient, const void* logits, cons
             else launch_resident<T, 16>(row_loss, g, z, targets, r, v, factor, stream);
         } else if (with_gradient) {
             hipLaunchKernelGGL((cross_entropy_row_kernel<T, true>), dim3(r), dim3(kThreads), 0, stream, row_loss,
-                               static_cast<T*>(gradient), static_cast<const T*>(logits), targets, v, factor, vector_ok);
+                               static_cast<T*>(gradient), static_cast<const T*>(logits), targets, v, factor, same_phase);
         } else {
             hipLaunchKernelGGL((cross_entropy_row_kernel<T, false>), dim3(r), dim3(kThreads), 0, stream, row_loss,
-                               static_cast<T*>(nullptr), static_cast<const T*>(logits), targets, v, factor, vector_ok);
+                               static_cast<T*>(nullptr), static_cast<const T*>(logits), targets, v, factor, same_phase);
         }
         CGPTX_LAUNCH_CHECK();
         return CGPTX_OK;

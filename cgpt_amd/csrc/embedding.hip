@@ -81,6 +81,61 @@ __global__ __launch_bounds__(kThreads) void embedding_segment_kernel(T* __restri
     }
 }
 
+// Short token lists (up to kDirectTokens) skip the sort: one wavefront per token compares its id with all the
+// others. The first occurrence of an id owns the row and adds the later occurrences in ascending token order —
+// the segment kernel's arithmetic, in one launch instead of six. Lane c keeps the 64-bit match mask of tokens
+// 64 c .. 64 c + 63.
+constexpr unsigned int kDirectTokens = 4096;
+template <typename T, bool Vector>
+__global__ __launch_bounds__(kThreads) void embedding_direct_kernel(T* __restrict__ grad_weight,
+                                                                   const T* __restrict__ grad_output,
+                                                                   const std::uint32_t* __restrict__ ids,
+                                                                   unsigned int count, unsigned int vocab,
+                                                                   unsigned int hidden, bool accumulate) {
+    constexpr int VEC = Vector ? kVec128<T> : 1;
+    const unsigned int lane = threadIdx.x & (kWave - 1);
+    const unsigned int token = blockIdx.x * kWavesPerBlock + threadIdx.x / kWave;
+    if (token >= count) return;
+    const std::uint32_t id = ids[token];
+    if (id >= vocab) return;
+    for (unsigned int first = 0; first < token; first += kWave) {
+        const unsigned int j = first + lane;
+        if (__ballot(j < token && ids[j] == id) != 0) return;  // an earlier token owns this row
+    }
+    const unsigned int chunks = (count + kWave - 1) / kWave, own_chunk = token / kWave;
+    unsigned long long later = 0;
+    for (unsigned int c = own_chunk; c < chunks; ++c) {
+        const unsigned int j = c * kWave + lane;
+        const unsigned long long mask = __ballot(j > token && j < count && ids[j] == id);
+        if (lane == c) later = mask;
+    }
+    T* row = grad_weight + static_cast<std::size_t>(id) * hidden;
+    for (unsigned int col = lane * VEC; col < hidden; col += kWave * VEC) {
+        vec_t<float, VEC> acc;
+        if (accumulate) {
+            acc = vec_to_f32<T, VEC>(load_vec<T, VEC>(row + col));
+        } else {
+            acc = vec_t<float, VEC>(0.0f);
+        }
+        const vec_t<float, VEC> own = vec_to_f32<T, VEC>(load_vec<T, VEC>(grad_output + static_cast<std::size_t>(token) * hidden + col));
+        acc = vec_to_f32<T, VEC>(vec_from_f32<T, VEC>(acc + own));  // one rounding to the storage dtype per add
+        for (unsigned int c = own_chunk; c < chunks; ++c) {
+            // v_readlane reads any lane, active or not (the lanes past the row's width are inactive here).
+            const int holder = __builtin_amdgcn_readfirstlane(static_cast<int>(c));
+            unsigned long long mask =
+                static_cast<unsigned long long>(static_cast<unsigned int>(__builtin_amdgcn_readlane(static_cast<int>(later), holder))) |
+                (static_cast<unsigned long long>(static_cast<unsigned int>(__builtin_amdgcn_readlane(static_cast<int>(later >> 32), holder))) << 32);
+            while (mask != 0) {
+                const unsigned int j = c * kWave + static_cast<unsigned int>(__builtin_ctzll(mask));
+                mask &= mask - 1;
+                const vec_t<float, VEC> dy = vec_to_f32<T, VEC>(load_vec<T, VEC>(grad_output + static_cast<std::size_t>(j) * hidden + col));
+                acc = vec_to_f32<T, VEC>(vec_from_f32<T, VEC>(acc + dy));
+            }
+        }
+        store_vec<T, VEC>(row + col, vec_from_f32<T, VEC>(acc));
+    }
+}
+
 template <typename T, bool Vector>
 __global__ __launch_bounds__(kThreads) void embedding_gather_kernel(T* __restrict__ out,
                                                                    const std::uint32_t* __restrict__ ids,
@@ -129,26 +184,31 @@ extern "C" int cgptx_embedding_backward(void* grad_weight, const void* grad_outp
     const auto v = static_cast<unsigned int>(vocab);
     const int end_bit = bits_for(v);
 
-    // Scratch: keys_in | keys_out | values_in | values_out | rocPRIM temporary storage.
-    const std::size_t array_bytes = (token_count * sizeof(unsigned int) + 255) & ~std::size_t{255};
-    std::size_t temp_bytes = 0;
-    CGPTX_HIP(rocprim::radix_sort_pairs(nullptr, temp_bytes, static_cast<unsigned int*>(nullptr),
-                                        static_cast<unsigned int*>(nullptr), static_cast<unsigned int*>(nullptr),
-                                        static_cast<unsigned int*>(nullptr), token_count, 0, end_bit, stream));
-    void* mem = nullptr;
-    if (int s = scratch(stream, 4 * array_bytes + temp_bytes + 256, &mem)) return s;
-    auto* base = static_cast<char*>(mem);
-    auto* keys_in = reinterpret_cast<unsigned int*>(base);
-    auto* keys_out = reinterpret_cast<unsigned int*>(base + array_bytes);
-    auto* values_in = reinterpret_cast<unsigned int*>(base + 2 * array_bytes);
-    auto* values_out = reinterpret_cast<unsigned int*>(base + 3 * array_bytes);
-    void* temp = base + 4 * array_bytes;
+    const bool direct = token_count <= kDirectTokens;
+    unsigned int* keys_out = nullptr;
+    unsigned int* values_out = nullptr;
+    if (!direct) {
+        // Scratch: keys_in | keys_out | values_in | values_out | rocPRIM temporary storage.
+        const std::size_t array_bytes = (token_count * sizeof(unsigned int) + 255) & ~std::size_t{255};
+        std::size_t temp_bytes = 0;
+        CGPTX_HIP(rocprim::radix_sort_pairs(nullptr, temp_bytes, static_cast<unsigned int*>(nullptr),
+                                            static_cast<unsigned int*>(nullptr), static_cast<unsigned int*>(nullptr),
+                                            static_cast<unsigned int*>(nullptr), token_count, 0, end_bit, stream));
+        void* mem = nullptr;
+        if (int s = scratch(stream, 4 * array_bytes + temp_bytes + 256, &mem)) return s;
+        auto* base = static_cast<char*>(mem);
+        auto* keys_in = reinterpret_cast<unsigned int*>(base);
+        keys_out = reinterpret_cast<unsigned int*>(base + array_bytes);
+        auto* values_in = reinterpret_cast<unsigned int*>(base + 2 * array_bytes);
+        values_out = reinterpret_cast<unsigned int*>(base + 3 * array_bytes);
+        void* temp = base + 4 * array_bytes;
 
-    hipLaunchKernelGGL(embedding_keys_kernel, dim3((count + kThreads - 1) / kThreads), dim3(kThreads), 0, stream,
-                       keys_in, values_in, token_ids, count, v);
-    CGPTX_LAUNCH_CHECK();
-    CGPTX_HIP(rocprim::radix_sort_pairs(temp, temp_bytes, keys_in, keys_out, values_in, values_out, token_count, 0,
-                                        end_bit, stream));
+        hipLaunchKernelGGL(embedding_keys_kernel, dim3((count + kThreads - 1) / kThreads), dim3(kThreads), 0, stream,
+                           keys_in, values_in, token_ids, count, v);
+        CGPTX_LAUNCH_CHECK();
+        CGPTX_HIP(rocprim::radix_sort_pairs(temp, temp_bytes, keys_in, keys_out, values_in, values_out, token_count, 0,
+                                            end_bit, stream));
+    }
     return dispatch_dtype(dtype, [&]<typename T>() -> int {
         auto* dw = static_cast<T*>(grad_weight);
         auto* dy = static_cast<const T*>(grad_output);
@@ -163,7 +223,15 @@ extern "C" int cgptx_embedding_backward(void* grad_weight, const void* grad_outp
         }
         const dim3 grid((count + kWavesPerBlock - 1) / kWavesPerBlock);
         const auto h = static_cast<unsigned int>(hidden);
-        if (vector_ok) {
+        if (direct) {
+            if (vector_ok) {
+                hipLaunchKernelGGL((embedding_direct_kernel<T, true>), grid, dim3(kThreads), 0, stream, dw, dy, token_ids,
+                                   count, v, h, accumulate_weight != 0);
+            } else {
+                hipLaunchKernelGGL((embedding_direct_kernel<T, false>), grid, dim3(kThreads), 0, stream, dw, dy, token_ids,
+                                   count, v, h, accumulate_weight != 0);
+            }
+        } else if (vector_ok) {
             hipLaunchKernelGGL((embedding_segment_kernel<T, true>), grid, dim3(kThreads), 0, stream, dw, dy, keys_out,
                                values_out, count, v, h, accumulate_weight != 0);
         } else {

@@ -30,7 +30,7 @@ def test_embedding_backward_repeated_tokens_known_answer(device, dtype, tol):
 @pytest.mark.parametrize("dtype", DTYPES, ids=DTYPE_IDS)
 @pytest.mark.parametrize("tokens,vocab,hidden,accumulate", [
     (64, 7, 16, False), (64, 7, 16, True), (1000, 50, 24, True), (4096, 1000, 128, False), (300, 5, 7, True),
-    (1, 3, 8, False),
+    (1, 3, 8, False), (4097, 900, 40, True), (6000, 50, 24, False),
 ])
 def test_embedding_backward_bit_exact(device, tokens, vocab, hidden, accumulate, dtype):
     """Heavy id collisions, out-of-range ids, odd widths: which rows receive which tokens is integer work
@@ -145,6 +145,25 @@ def test_cross_entropy_parity(device, rows, vocab, dtype):
     only = torch.zeros(1, device=device)
     ops.cross_entropy_forward(only, dev(logits, device), dev(targets, device), rows)
     assert abs(only.item() - l64) <= 1e-4 * max(1.0, abs(l64))
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=DTYPE_IDS)
+def test_cross_entropy_rows_that_start_off_a_16_byte_boundary(device, dtype):
+    """A vocabulary that is not a multiple of the vector width: every row starts at another offset from a 16-byte
+    boundary. In place (gradient = logits), and with a gradient whose rows have a different offset than the logits'."""
+    rows, vocab = 9, 50257
+    logits = randn((rows, vocab), dtype, 21, 3.0)
+    targets = randint(vocab, (rows,), 22)
+    l64, g64 = oracle64.cross_entropy(to_np(logits), targets.numpy(), 8.0)
+    d_targets = dev(targets, device)
+    in_place, loss = dev(logits, device).clone(), torch.zeros(1, device=device)
+    ops.cross_entropy_forward_backward(loss, in_place, in_place, d_targets, rows, None, 8.0)
+    assert abs(loss.item() - l64) <= 1e-4 * max(1.0, abs(l64))
+    assert_close(in_place, g64, TOL[dtype], "in place")
+    storage = torch.empty(rows * vocab + 1, dtype=dtype, device=device)
+    shifted = storage[1:].view(rows, vocab)  # one element off the logits' alignment
+    ops.cross_entropy_forward_backward(loss, shifted, dev(logits, device), d_targets, rows, None, 8.0)
+    assert_close(shifted, g64, TOL[dtype], "gradient rows at another offset")
 
 
 def test_cross_entropy_training_shape_rows_sum_to_zero(device):
