@@ -133,7 +133,8 @@ def timed(torch, stream, fn, launches=20, warm=3):
 
 def isolated_kernels(torch, cfg, batch, seq, dtype, stream, seed, only="", secondary=True):
     """Every backward operator alone at the configuration's shape: algorithmic bytes or FLOPs of one call /
-    its average duration over 20 back-to-back calls. `only`: run just the sections whose name contains it."""
+    its average duration over 20 back-to-back calls. `only`: run just the sections whose name contains it (or one
+    of several, separated by commas)."""
     from cgpt_amd import ops
 
     N, H, I, V = batch * seq, cfg.hidden_size, cfg.intermediate_size, cfg.vocabulary_size
@@ -147,7 +148,7 @@ def isolated_kernels(torch, cfg, batch, seq, dtype, stream, seed, only="", secon
     out = {}
 
     def want(section):
-        return only in section
+        return any(part in section for part in only.split(","))
 
     def record(name, bound, amount, seconds, shape):
         rate = amount / seconds / (1e12 if bound == "mfma" else 1e9)
@@ -400,7 +401,8 @@ def main() -> int:
     parser.add_argument("--seed", type=int, default=0)
     parser.add_argument("--kernels-only", metavar="NAME", default=None,
                         help="run only the isolated operator launches whose name contains NAME (rmsnorm, rope, "
-                             "attention, swiglu, embedding, cut_cross_entropy, dense_cross_entropy, copy; '' = all) and print "
+                             "attention, swiglu, embedding, cut_cross_entropy, dense_cross_entropy, copy, secondary, published; several "
+                             "separated by commas; '' = all) and print "
                              "their table: the target of per-kernel rocprofv3 runs")
     parser.add_argument("--probe-only", action="store_true",
                         help="launch only the dominant kernel (20x) and a 1 GiB device copy: the target of the "
