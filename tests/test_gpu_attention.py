@@ -186,10 +186,12 @@ def test_causal_horizon_and_value_gradient_identity(device):
     assert np.abs(lhs - rhs).max() <= 2e-2 * np.abs(rhs).max()
 
 
-def test_training_shape_against_float64_and_determinism(device):
-    """B=32, T=1024, 8:2 heads, D=128, bf16: two runs are bit-identical, the Σ dV identity holds for every
-    batch, and two batches are compared element-wise with the float64 formulas."""
-    c = dict(b=32, qs=1024, ks=1024, hq=8, hkv=2, d=128)
+@pytest.mark.parametrize("hq,hkv,d", [(8, 2, 128), (12, 4, 64)], ids=["preset-8:2x128", "secondary-12:4x64"])
+def test_training_shape_against_float64_and_determinism(device, hq, hkv, d):
+    """B=32, T=1024, bf16, the preset's 8:2 heads of 128 and the 12:4 heads of 64 of the 768-wide shape: two runs are
+    bit-identical, the Σ dV identity holds for every batch, and two batches are compared element-wise with the float64
+    formulas."""
+    c = dict(b=32, qs=1024, ks=1024, hq=hq, hkv=hkv, d=d)
     dtype = torch.bfloat16
     q, k, v, do = make_inputs(c, dtype, 1234)
     first = run_backward(device, do, q, k, v, c)
@@ -198,15 +200,15 @@ def test_training_shape_against_float64_and_determinism(device):
         assert torch.equal(a, b_)
     dq, dk, dv = (t.cpu() for t in first)
     lhs = to_np(dv).sum(axis=1)
-    rhs = to_np(do).reshape(32, 1024, 2, 4, 128).sum(axis=(1, 3))
+    rhs = to_np(do).reshape(32, 1024, hkv, hq // hkv, d).sum(axis=(1, 3))
     assert np.abs(lhs - rhs).max() <= 2e-2 * np.abs(rhs).max()
     for bi in (0, 31):
         sl = slice(bi, bi + 1)
-        want = oracle64.attention_backward(to_np(do[sl]), to_np(q[sl]), to_np(k[sl]), to_np(v[sl]), 8, 2, 128)
+        want = oracle64.attention_backward(to_np(do[sl]), to_np(q[sl]), to_np(k[sl]), to_np(v[sl]), hq, hkv, d)
         for g, w, name in zip((dq[sl], dk[sl], dv[sl]), want, ("dQ", "dK", "dV")):
             assert_scaled_close(g, w, TOL[dtype], f"{name} batch {bi}")
         out, lse = run_forward(device, q[sl].contiguous(), k[sl].contiguous(), v[sl].contiguous(), dict(c, b=1))
-        wo, wl = oracle64.attention_forward(to_np(q[sl]), to_np(k[sl]), to_np(v[sl]), 8, 2, 128)
+        wo, wl = oracle64.attention_forward(to_np(q[sl]), to_np(k[sl]), to_np(v[sl]), hq, hkv, d)
         assert_close(out, wo, TOL[dtype], "O")
         assert_close(lse, wl, 1e-3, "LSE")
 

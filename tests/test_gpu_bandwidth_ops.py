@@ -54,9 +54,9 @@ def test_rmsnorm_backward_reference_test_inputs(device, dtype, tol):
 
 
 def test_rmsnorm_backward_is_deterministic_and_full_size(device):
-    """[32768, 1024] bf16 (the training shape) and the QK-norm shape [65536, 128]: run twice, bit-identical,
-    and equal to the CPU checker."""
-    for rows, hidden in ((32768, 1024), (65536, 128)):
+    """[32768, 1024] bf16 (the training shape), the QK-norm shape [65536, 128] and the 768-wide shapes ([32768, 768];
+    [131072, 64] for its 4 kv-heads of 64): run twice, bit-identical, and equal to the CPU checker."""
+    for rows, hidden in ((32768, 1024), (65536, 128), (32768, 768), (131072, 64)):
         dtype = torch.bfloat16
         x, dy = randn((rows, hidden), dtype, 11), randn((rows, hidden), dtype, 12)
         w = (1.0 + 0.1 * randn((hidden,), torch.float32, 13)).to(dtype)
@@ -150,12 +150,13 @@ def test_rope_backward_known_answer(device, dtype, tol):
     assert np.abs(to_np(gk).reshape(-1) - [1, -2, 30, 40, -6, -5, 70, 80]).max() <= tol
 
 
-def test_rope_backward_full_size_bit_exact_vs_checker(device):
-    """q[32,1024,8,128] + k[32,1024,2,128] bf16: same fp32 arithmetic and one rounding as the CPU
-    checker, so the result is compared bit for bit."""
+@pytest.mark.parametrize("hq,hkv,d", [(8, 2, 128), (12, 4, 64)], ids=["preset-8:2x128", "secondary-12:4x64"])
+def test_rope_backward_full_size_bit_exact_vs_checker(device, hq, hkv, d):
+    """q[32,1024,8,128] + k[32,1024,2,128] and q[32,1024,12,64] + k[32,1024,4,64], bf16: same fp32 arithmetic and one
+    rounding as the CPU checker, so the result is compared bit for bit."""
     dtype = torch.bfloat16
-    cos, sin = rope_cache(1024, 128, dtype)
-    q, k = randn((32, 1024, 8, 128), dtype, 21), randn((32, 1024, 2, 128), dtype, 22)
+    cos, sin = rope_cache(1024, d, dtype)
+    q, k = randn((32, 1024, hq, d), dtype, 21), randn((32, 1024, hkv, d), dtype, 22)
     gq, gk = torch.empty_like(q), torch.empty_like(k)
     cpu_ops.rope_backward(gq, gk, q, k, cos, sin)
     dq, dk = torch.empty_like(q, device=device), torch.empty_like(k, device=device)

@@ -81,6 +81,39 @@ def test_equivalent_to_dense_cross_entropy_plus_linear_backward(device, monkeypa
     assert again[0] == loss and torch.equal(again[1], dx) and torch.equal(again[2], dc)
 
 
+@pytest.mark.parametrize("hidden", [1024, 768], ids=["preset-1024", "secondary-768"])
+def test_training_shape_against_the_dense_path_and_float64_rows(device, hidden):
+    """[32768, hidden] x [32000, hidden] bf16, loss scale 1024: loss, dX and dC against the dense path (logits
+    contraction, cross-entropy operator, linear_backward), the dX rows of 256 rows against float64 (a row's gradient
+    does not depend on the other rows), and two runs are bit-identical."""
+    dtype = torch.bfloat16
+    rows, vocab = 32768, 32000
+    x, c = randn((rows, hidden), dtype, 31), randn((vocab, hidden), dtype, 32, 0.02)
+    targets = randint(vocab, (rows,), 33)
+    dx_, dc_, dt = x.to(device), c.to(device), targets.to(device)
+    loss, dx, dc = run(device, dx_, dc_, dt, 1024.0)
+    logits = torch.empty(rows, vocab, dtype=dtype, device=device)
+    ops.linear_forward(logits, dx_, dc_)
+    dense_loss, grad = torch.zeros(1, device=device), torch.empty_like(logits)
+    ops.cross_entropy_forward_backward(dense_loss, grad, logits, dt, rows, None, 1024.0)
+    dx2, dc2 = torch.empty_like(dx_), torch.empty_like(dc_)
+    ops.linear_backward(dx2, dc2, None, grad, dx_, dc_)
+    del logits, grad
+    assert abs(loss - dense_loss.item()) <= 1e-5 * dense_loss.item()
+    assert_scaled_close(dx, dx2, TOL[dtype], "dX vs dense path")
+    assert_scaled_close(dc, dc2, TOL[dtype], "dC vs dense path")
+    # float64 on a slice: the per-row loss terms and the dX rows do not depend on the other rows
+    pick = np.arange(0, rows, rows // 256)
+    z = to_np(x)[pick].astype(np.float64) @ to_np(c).astype(np.float64).T
+    lse = np.log(np.exp(z - z.max(axis=1, keepdims=True)).sum(axis=1)) + z.max(axis=1)
+    prob = np.exp(z - lse[:, None])
+    prob[np.arange(len(pick)), targets.numpy()[pick]] -= 1.0
+    dx64 = prob @ to_np(c).astype(np.float64) * (1024.0 / rows)
+    assert_scaled_close(dx.cpu()[pick], dx64, TOL[dtype], "dX rows vs float64")
+    again = run(device, dx_, dc_, dt, 1024.0)
+    assert again[0] == loss and torch.equal(again[1], dx) and torch.equal(again[2], dc)
+
+
 def test_argument_errors(device):
     x, c = torch.zeros(4, 8, device=device), torch.zeros(5, 8, device=device)
     t = torch.zeros(4, dtype=torch.int32, device=device)
