@@ -395,6 +395,9 @@ def main() -> int:
     parser.add_argument("--seq", type=int, default=1024)
     parser.add_argument("--loss", choices=["cut", "dense"], default="cut")
     parser.add_argument("--dtype", choices=["bf16", "f16"], default="bf16")
+    parser.add_argument("--shape", choices=["104m", "12x768"], default="104m",
+                        help="104m = the reference's preset (8 layers, hidden 1024, 8:2 heads of 128); 12x768 = the "
+                             "12-layer, 768-wide decoder with 12:4 heads of 64 (a parity shape, not the bench line)")
     parser.add_argument("--no-kernel-table", action="store_true", help="skip the isolated per-operator launches")
     parser.add_argument("--no-graph", action="store_true")
     parser.add_argument("--no-cpu-baseline", action="store_true")
@@ -424,6 +427,9 @@ def main() -> int:
     device = torch.device("cuda:0")
     dtype = torch.bfloat16 if args.dtype == "bf16" else torch.float16
     cfg = ModelConfig(dtype=dtype)  # the reference's 104m preset
+    if args.shape == "12x768":
+        cfg = ModelConfig(dtype=dtype, num_layers=12, hidden_size=768, num_query_heads=12, num_kv_heads=4, head_dim=64,
+                          rotary_dim=64)
     if args.kernels_only is not None:
         stream = torch.cuda.Stream(device=device)
         shown = {"kernels": isolated_kernels(torch, cfg, args.batch, args.seq, dtype, stream, args.seed, args.kernels_only)}
@@ -502,17 +508,17 @@ def main() -> int:
     family = {kind: per_kind[kind]["frac"] for kind in ("gemm_fwd", "gemm_dx", "gemm_dw") if kind in per_kind}
     kernels = {} if args.no_kernel_table else isolated_kernels(torch, cfg, args.batch, args.seq, dtype, stream, args.seed)
     published = {} if args.no_kernel_table else published_kernel_shapes(torch, stream, args.seed)
-    # AdamW over all parameters (3 launches for the 90 tensors): 30 B/parameter with 16-bit gradients and parameters.
+    # AdamW over all parameters (3 launches for all tensors): 30 B/parameter with 16-bit gradients and parameters.
     options_probe = options
     adamw_seconds = timed(torch, stream, lambda: model.optimizer_step(options_probe, stream), launches=5, warm=1)
     adamw_bytes = 30.0 * model.num_parameters
     kernels["adamw_step_many_async"] = {
-        "shape": f"{model.num_parameters} parameters in 90 tensors", "bound": "hbm", "us": round(adamw_seconds * 1e6, 1),
+        "shape": f"{model.num_parameters} parameters in {2 + 11 * cfg.num_layers} tensors", "bound": "hbm", "us": round(adamw_seconds * 1e6, 1),
         "rate": round(adamw_bytes / adamw_seconds / 1e9, 1), "unit": "GB/s",
         "frac": round(adamw_bytes / adamw_seconds / 1e9 / PEAK_HBM_GBS, 4)}
 
     result = {
-        "metric": f"train tokens/sec, 104m fwd+bwd+AdamW B={args.batch} T={args.seq}",
+        "metric": f"train tokens/sec, {args.shape} fwd+bwd+AdamW B={args.batch} T={args.seq}",
         "value": tokens * args.steps / elapsed,
         "unit": "tokens/s",
         "n_gpus": 1,
@@ -524,7 +530,7 @@ def main() -> int:
         "vs_baseline": None,
         "dtype": args.dtype,
         "data": "synthetic",
-        "config": {"workload": f"full 104m train step (embedding, 8 blocks, {args.loss} cross-entropy, backward, "
+        "config": {"workload": f"full {args.shape} train step (embedding, {cfg.num_layers} blocks, {args.loss} cross-entropy, backward, "
                                f"AdamW), B={args.batch}, T={args.seq}, hipGraph={'on' if use_graph else 'off'}",
                    "parameters": model.num_parameters, "global_batch": args.batch, "seq_len": args.seq,
                    "loss_scale": 1024.0},

@@ -333,19 +333,25 @@ HEADLINE = dict(vocabulary_size=32000, num_layers=8, hidden_size=1024, intermedi
 HEADLINE_CFG = dict(vocab=32000, layers=8, hidden=1024, inter=2048, hq=8, hkv=2, d=128, eps=1e-5)
 
 
+# The 12-layer, 768-wide decoder with 12:4 heads of 64 that is named beside the preset as the 104m shape.
+SECONDARY = dict(vocabulary_size=32000, num_layers=12, hidden_size=768, intermediate_size=2048, num_query_heads=12,
+                 num_kv_heads=4, head_dim=64, rotary_dim=64)
+
+
 @pytest.mark.gpu
-@pytest.mark.parametrize("batch,seq", [(32, 1024), (8, 4096)], ids=["b32-t1024", "long-context-b8-t4096"])
-def test_headline_configuration_scales_exactly_replays_exactly_and_starts_at_the_closed_form_loss(device, batch, seq):
-    """The 104m preset at the benchmark's sizes (B=32, T=1024 and the long-context variant B=8, T=4096, bf16),
-    where no CPU composition finishes in test time: properties that hold at any size. The backward pass is
-    linear in the loss scale, and a factor of two is exact in binary floating point, so every gradient at scale
-    2048 is exactly twice the one at 1024; a hipGraph replay repeats the eager pass bit for bit; the two loss
-    paths agree; a random-init model starts at the closed-form loss of Gaussian logits."""
+@pytest.mark.parametrize("dims,batch,seq", [(HEADLINE, 32, 1024), (HEADLINE, 8, 4096), (SECONDARY, 32, 1024)],
+                         ids=["b32-t1024", "long-context-b8-t4096", "12x768-b32-t1024"])
+def test_headline_configuration_scales_exactly_replays_exactly_and_starts_at_the_closed_form_loss(device, dims, batch, seq):
+    """The 104m preset at the benchmark's sizes (B=32, T=1024 and the long-context variant B=8, T=4096, bf16) and the
+    12 x 768 shape at B=32, T=1024, where no CPU composition finishes in test time: properties that hold at any size.
+    The backward pass is linear in the loss scale, and a factor of two is exact in binary floating point, so every
+    gradient at scale 2048 is exactly twice the one at 1024; a hipGraph replay repeats the eager pass bit for bit; the
+    two loss paths agree; a random-init model starts at the closed-form loss of Gaussian logits."""
     from cgpt_amd.model import LOSS_CUT, LOSS_DENSE, Model, ModelConfig
 
-    config = ModelConfig(dtype=torch.bfloat16, **HEADLINE)
+    config = ModelConfig(dtype=torch.bfloat16, **dims)
     model = Model(config, batch, seq, seed=0, device=device)
-    assert model.num_parameters == 104_090_624
+    assert model.num_parameters == (104_090_624 if dims is HEADLINE else 100_094_208)
     rng = np.random.default_rng(0)
     model.set_tokens(rng.integers(0, 32000, size=(batch, seq)), rng.integers(0, 32000, size=(batch, seq)))
     stream = torch.cuda.Stream(device=device)
@@ -354,7 +360,7 @@ def test_headline_configuration_scales_exactly_replays_exactly_and_starts_at_the
     loss, _, _ = model.status(stream)
     # Rows leave the final norm with unit RMS and the tied classifier is N(0, 0.02^2): logits are close to
     # N(0, H * 0.02^2) and independent of the target, so E[loss] = ln V + variance / 2.
-    assert abs(loss - (np.log(32000.0) + 0.5 * 1024 * 0.02 ** 2)) < 0.02
+    assert abs(loss - (np.log(32000.0) + 0.5 * dims["hidden_size"] * 0.02 ** 2)) < 0.02
     base = [g.clone() for _, _, g in model.parameters()]
     for (name, _, _), g in zip(model.parameters(), base):
         assert bool(torch.isfinite(g.float()).all()), name
