@@ -9,6 +9,7 @@
 #include <cstdint>
 #include <cstdio>
 #include <string>
+#include <vector>
 
 #include "cgptx.h"
 
@@ -99,12 +100,53 @@ int dispatch_dtype(int dtype, Fn&& fn) {
     }
 }
 
+// ---- weight-gradient reductions of several norm-backward passes as one pair of launches ----------
+// A norm-backward pass leaves per-workgroup partial sums of the weight gradient [parts, hidden] and reduces them
+// over the parts in two small launches. A caller that runs many such passes (the train step: four per block) may
+// hand them a sink instead: the pass then takes its partial-sum memory from the sink (which must outlive the pass,
+// unlike the per-stream arena that the next operator reuses), records what is to be reduced, and the caller runs
+// all recorded reductions with run_column_reductions — the same arithmetic in the same order, two launches in all.
+struct ColumnReduceEntry {
+    const float* partial;  // [parts, hidden]
+    float* second;         // [slices, hidden] (used when slices > 1)
+    void* out;             // T[hidden]
+    int parts, hidden, slices, dtype;
+    bool operator==(const ColumnReduceEntry& o) const {
+        return partial == o.partial && second == o.second && out == o.out && parts == o.parts && hidden == o.hidden &&
+               slices == o.slices && dtype == o.dtype;
+    }
+};
+struct ColumnReduceSink {
+    char* memory = nullptr;      // device memory owned by the caller
+    std::size_t capacity = 0;    // bytes behind `memory`
+    std::size_t used = 0;        // bytes handed out since begin()
+    std::size_t wanted = 0;      // bytes asked for since begin(), served or not
+    std::vector<ColumnReduceEntry> entries;
+    void begin() {
+        used = 0;
+        wanted = 0;
+        entries.clear();
+    }
+    // 256-byte aligned block, or nullptr when it does not fit (the pass then reduces at once, from the arena).
+    void* take(std::size_t bytes) {
+        bytes = (bytes + 255) & ~std::size_t{255};
+        wanted += bytes;
+        if (memory == nullptr || used + bytes > capacity) return nullptr;
+        void* block = memory + used;
+        used += bytes;
+        return block;
+    }
+};
+// Runs the reductions recorded in `table` (device copy of `count` entries). max_hidden / max_slices: the largest
+// values among the entries (they size the grid).
+int run_column_reductions(const ColumnReduceEntry* table, int count, int max_hidden, int max_slices, hipStream_t stream);
+
 // ---- fused variants used by the composed train step --------------------------
 // rmsnorm backward with grad_input = (norm gradient) + residual; residual may be null or alias
 // grad_input. Same validation and results as cgptx_rmsnorm_backward otherwise.
 int rmsnorm_backward_residual(void* grad_input, void* grad_weight, const void* grad_output, const void* input,
                               const void* weight, const void* residual, std::size_t rows, std::size_t hidden,
-                              float epsilon, int dtype, hipStream_t stream);
+                              float epsilon, int dtype, hipStream_t stream, ColumnReduceSink* sink = nullptr);
 
 // Per-head RMSNorm and rotary embedding in one pass over [rows = tokens x heads, head_dim]:
 //   forward   output = rope(rmsnorm(input));   backward   the gradient of that, with the weight gradient.
@@ -119,7 +161,8 @@ int rmsnorm_rope_forward(void* output, const void* input, const void* weight, co
 int rmsnorm_rope_backward(void* grad_input, void* grad_weight, const void* grad_output, const void* input,
                           const void* weight, const void* cos_cache, const void* sin_cache, std::size_t rows,
                           std::size_t head_dim, std::size_t heads, std::size_t sequence, std::size_t rotary_dim,
-                          std::size_t position_offset, float epsilon, int dtype, hipStream_t stream);
+                          std::size_t position_offset, float epsilon, int dtype, hipStream_t stream,
+                          ColumnReduceSink* sink = nullptr);
 
 // Two RMSNorms of the same rows with different weights in one pass (x is read once):
 //   forward   output_a = rmsnorm(input; weight_a), output_f = rmsnorm(input; weight_f)
@@ -133,7 +176,7 @@ int rmsnorm_forward_dual(void* output_a, void* output_f, const void* input, cons
 int rmsnorm_backward_dual(void* grad_input, void* grad_weight_a, void* grad_weight_f, const void* grad_output_a,
                           const void* grad_output_f, const void* input, const void* weight_a, const void* weight_f,
                           const void* residual, std::size_t rows, std::size_t hidden, float epsilon, int dtype,
-                          hipStream_t stream);
+                          hipStream_t stream, ColumnReduceSink* sink = nullptr);
 
 // ---- scratch arena ----------------------------------------------------------
 // Returns `bytes` of device scratch bound to (current device, stream), 256-byte

@@ -8,14 +8,14 @@ namespace cgptx {
 constexpr int kReduceThreads = 256;
 constexpr int kReduceWaves = kReduceThreads / kWave;
 
-// Sums partial[P, H] over P in a fixed order and stores (or adds) in T.
+// Sums partial[P, H] over P in a fixed order and stores (or adds) in T; `group` = which 64 columns.
 template <typename T>
-__global__ __launch_bounds__(kReduceThreads) void column_partial_reduce_kernel(
-    T* __restrict__ out, const float* __restrict__ partial, int parts, int hidden, int accumulate) {
+__device__ __forceinline__ void column_partial_reduce_body(T* __restrict__ out, const float* __restrict__ partial,
+                                                           int parts, int hidden, int accumulate, int group) {
     __shared__ float stage[kReduceWaves][kWave];
     const int lane = threadIdx.x & (kWave - 1);
     const int slice = threadIdx.x / kWave;
-    const int col = blockIdx.x * kWave + lane;
+    const int col = group * kWave + lane;
     float v0 = 0.0f, v1 = 0.0f, v2 = 0.0f, v3 = 0.0f;
     if (col < hidden) {
         int p = slice;
@@ -37,22 +37,24 @@ __global__ __launch_bounds__(kReduceThreads) void column_partial_reduce_kernel(
         out[col] = from_f32<T>(v);
     }
 }
+template <typename T>
+__global__ __launch_bounds__(kReduceThreads) void column_partial_reduce_kernel(
+    T* __restrict__ out, const float* __restrict__ partial, int parts, int hidden, int accumulate) {
+    column_partial_reduce_body<T>(out, partial, parts, hidden, accumulate, static_cast<int>(blockIdx.x));
+}
 
-
-// First level for many parts: block (x, y) of a (column groups, slices) grid folds the parts of
-// slice y for its 64 columns into second[y, col]; column_partial_reduce_kernel over the `slices`
+// First level for many parts: block (group, index) of a (column groups, slices) grid folds the parts of
+// slice `index` for its 64 columns into second[index, col]; column_partial_reduce_kernel over the `slices`
 // rows of `second` finishes. (A single launch whose last block finishes would need device-scope
 // fences, which cost more here than the second launch.)
-static __global__ __launch_bounds__(kReduceThreads) void column_partial_fold_kernel(float* __restrict__ second,
-                                                                            const float* __restrict__ partial,
-                                                                            int parts, int hidden) {
+__device__ __forceinline__ void column_partial_fold_body(float* __restrict__ second, const float* __restrict__ partial,
+                                                         int parts, int hidden, int slices, int index, int group) {
     __shared__ float stage[kReduceWaves][kWave];
     const int lane = threadIdx.x & (kWave - 1);
     const int slice = threadIdx.x / kWave;
-    const int col = blockIdx.x * kWave + lane;
-    const int slices = gridDim.y;
+    const int col = group * kWave + lane;
     const int chunk = (parts + slices - 1) / slices;
-    const int begin = blockIdx.y * chunk;
+    const int begin = index * chunk;
     const int end = begin + chunk < parts ? begin + chunk : parts;
     float v0 = 0.0f, v1 = 0.0f;
     if (col < hidden) {
@@ -69,7 +71,36 @@ static __global__ __launch_bounds__(kReduceThreads) void column_partial_fold_ker
         float v = 0.0f;
 #pragma unroll
         for (int s = 0; s < kReduceWaves; ++s) v += stage[s][lane];
-        second[static_cast<std::size_t>(blockIdx.y) * hidden + col] = v;
+        second[static_cast<std::size_t>(index) * hidden + col] = v;
+    }
+}
+static __global__ __launch_bounds__(kReduceThreads) void column_partial_fold_kernel(float* __restrict__ second,
+                                                                            const float* __restrict__ partial,
+                                                                            int parts, int hidden) {
+    column_partial_fold_body(second, partial, parts, hidden, static_cast<int>(gridDim.y), static_cast<int>(blockIdx.y),
+                             static_cast<int>(blockIdx.x));
+}
+
+// The two kernels above over a table of reductions (blockIdx.z, or blockIdx.y of the second, picks the entry):
+// the same additions in the same order for every entry, whatever else is in the table.
+static __global__ __launch_bounds__(kReduceThreads) void column_partial_fold_table_kernel(
+    const ColumnReduceEntry* __restrict__ table) {
+    const ColumnReduceEntry e = table[blockIdx.z];
+    if (e.slices <= 1 || static_cast<int>(blockIdx.y) >= e.slices || static_cast<int>(blockIdx.x) * kWave >= e.hidden) return;
+    column_partial_fold_body(e.second, e.partial, e.parts, e.hidden, e.slices, static_cast<int>(blockIdx.y),
+                             static_cast<int>(blockIdx.x));
+}
+static __global__ __launch_bounds__(kReduceThreads) void column_partial_reduce_table_kernel(
+    const ColumnReduceEntry* __restrict__ table) {
+    const ColumnReduceEntry e = table[blockIdx.y];
+    if (static_cast<int>(blockIdx.x) * kWave >= e.hidden) return;
+    const float* source = e.slices > 1 ? e.second : e.partial;
+    const int parts = e.slices > 1 ? e.slices : e.parts;
+    const int group = static_cast<int>(blockIdx.x);
+    switch (e.dtype) {
+        case CGPTX_F16: column_partial_reduce_body<f16_t>(static_cast<f16_t*>(e.out), source, parts, e.hidden, 0, group); break;
+        case CGPTX_BF16: column_partial_reduce_body<bf16_t>(static_cast<bf16_t*>(e.out), source, parts, e.hidden, 0, group); break;
+        default: column_partial_reduce_body<float>(static_cast<float*>(e.out), source, parts, e.hidden, 0, group); break;
     }
 }
 

@@ -529,6 +529,49 @@ RopeArgs make_rope(const void* cos_cache, const void* sin_cache, std::size_t hea
 }
 }  // namespace
 
+// Memory for a pass's partial sums: from the sink when one is given and has room (the reductions are then recorded
+// and run later by the caller), else from the per-stream arena (the reductions then run at once).
+int partial_memory(ColumnReduceSink* sink, hipStream_t stream, std::size_t bytes, void** out, bool* deferred) {
+    *out = sink != nullptr ? sink->take(bytes) : nullptr;
+    *deferred = *out != nullptr;
+    return *deferred ? CGPTX_OK : scratch(stream, bytes, out);
+}
+
+// dw[h] = column sums of partial[blocks, h]: two small launches now, or an entry in the sink.
+template <typename T>
+int reduce_columns(ColumnReduceSink* sink, bool deferred, T* dw, float* partial, float* second, int blocks, int h,
+                   int slices, int dtype, hipStream_t stream) {
+    if (deferred) {
+        sink->entries.push_back(ColumnReduceEntry{partial, second, dw, blocks, h, slices, dtype});
+        return CGPTX_OK;
+    }
+    const int reduce_blocks = (h + kWave - 1) / kWave;
+    if (slices > 1) {
+        hipLaunchKernelGGL(column_partial_fold_kernel, dim3(reduce_blocks, slices), dim3(kThreads), 0, stream, second,
+                           partial, blocks, h);
+        CGPTX_LAUNCH_CHECK();
+        hipLaunchKernelGGL((column_partial_reduce_kernel<T>), dim3(reduce_blocks), dim3(kThreads), 0, stream, dw, second,
+                           slices, h, 0);
+    } else {
+        hipLaunchKernelGGL((column_partial_reduce_kernel<T>), dim3(reduce_blocks), dim3(kThreads), 0, stream, dw, partial,
+                           blocks, h, 0);
+    }
+    CGPTX_LAUNCH_CHECK();
+    return CGPTX_OK;
+}
+
+int run_column_reductions(const ColumnReduceEntry* table, int count, int max_hidden, int max_slices, hipStream_t stream) {
+    if (count <= 0) return CGPTX_OK;
+    const int groups = (max_hidden + kWave - 1) / kWave;
+    if (max_slices > 1) {
+        hipLaunchKernelGGL(column_partial_fold_table_kernel, dim3(groups, max_slices, count), dim3(kThreads), 0, stream, table);
+        CGPTX_LAUNCH_CHECK();
+    }
+    hipLaunchKernelGGL(column_partial_reduce_table_kernel, dim3(groups, count), dim3(kThreads), 0, stream, table);
+    CGPTX_LAUNCH_CHECK();
+    return CGPTX_OK;
+}
+
 int rmsnorm_rope_forward(void* output, const void* input, const void* weight, const void* cos_cache, const void* sin_cache,
                          std::size_t rows, std::size_t head_dim, std::size_t heads, std::size_t sequence,
                          std::size_t rotary_dim, std::size_t position_offset, float epsilon, int dtype, hipStream_t stream) {
@@ -552,7 +595,7 @@ int rmsnorm_rope_forward(void* output, const void* input, const void* weight, co
 int rmsnorm_rope_backward(void* grad_input, void* grad_weight, const void* grad_output, const void* input,
                           const void* weight, const void* cos_cache, const void* sin_cache, std::size_t rows,
                           std::size_t head_dim, std::size_t heads, std::size_t sequence, std::size_t rotary_dim,
-                          std::size_t position_offset, float epsilon, int dtype, hipStream_t stream) {
+                          std::size_t position_offset, float epsilon, int dtype, hipStream_t stream, ColumnReduceSink* sink) {
     if (int s = validate(grad_input, grad_output, input, rows, head_dim, epsilon, dtype, "rmsnorm_rope_backward")) return s;
     if (grad_weight == nullptr || weight == nullptr || cos_cache == nullptr || sin_cache == nullptr || heads == 0 ||
         sequence == 0 ||
@@ -563,30 +606,23 @@ int rmsnorm_rope_backward(void* grad_input, void* grad_weight, const void* grad_
     return dispatch_dtype(dtype, [&]<typename T>() -> int {
         const FastShape shape = pick_fast_shape<T>(h);
         const int blocks = fast_blocks(shape, r, fast_kernel<T, true>(shape, true));
-        const int reduce_blocks = (h + kWave - 1) / kWave;
         const int slices = wide_reduce_slices(blocks, h, compute_units());
         void* mem = nullptr;
+        bool deferred = false;
         const std::size_t partial_bytes = static_cast<std::size_t>(blocks) * head_dim * sizeof(float);
-        if (int s = scratch(stream, partial_bytes + static_cast<std::size_t>(slices) * head_dim * sizeof(float), &mem)) return s;
+        if (int s = partial_memory(sink, stream, partial_bytes + static_cast<std::size_t>(slices) * head_dim * sizeof(float), &mem,
+                                   &deferred))
+            return s;
         auto* partial = static_cast<float*>(mem);
         if (int s = launch_fast<T, true>(shape, static_cast<T*>(grad_input), partial, static_cast<const T*>(grad_output),
                                          nullptr, static_cast<const T*>(input), static_cast<const T*>(weight), r, h, epsilon,
                                          blocks, stream, &rope))
             return s;
         CGPTX_LAUNCH_CHECK();
-        auto* dw = static_cast<T*>(grad_weight);
-        if (slices > 1) {
-            auto* second = reinterpret_cast<float*>(static_cast<char*>(mem) + partial_bytes);
-            hipLaunchKernelGGL(column_partial_fold_kernel, dim3(reduce_blocks, slices), dim3(kThreads), 0, stream, second,
-                               partial, blocks, h);
-            CGPTX_LAUNCH_CHECK();
-            hipLaunchKernelGGL((column_partial_reduce_kernel<T>), dim3(reduce_blocks), dim3(kThreads), 0, stream, dw, second,
-                               slices, h, 0);
-        } else {
-            hipLaunchKernelGGL((column_partial_reduce_kernel<T>), dim3(reduce_blocks), dim3(kThreads), 0, stream, dw, partial,
-                               blocks, h, 0);
-        }
-        CGPTX_LAUNCH_CHECK();
+        auto* second = reinterpret_cast<float*>(static_cast<char*>(mem) + partial_bytes);
+        if (int s = reduce_columns<T>(sink, deferred, static_cast<T*>(grad_weight), partial, second, blocks, h, slices, dtype,
+                                      stream))
+            return s;
         return CGPTX_OK;
     });
 }
@@ -662,7 +698,7 @@ int rmsnorm_forward_dual(void* output_a, void* output_f, const void* input, cons
 int rmsnorm_backward_dual(void* grad_input, void* grad_weight_a, void* grad_weight_f, const void* grad_output_a,
                           const void* grad_output_f, const void* input, const void* weight_a, const void* weight_f,
                           const void* residual, std::size_t rows, std::size_t hidden, float epsilon, int dtype,
-                          hipStream_t stream) {
+                          hipStream_t stream, ColumnReduceSink* sink) {
     if (int s = validate(grad_input, grad_output_a, input, rows, hidden, epsilon, dtype, "rmsnorm_backward_dual")) return s;
     if (grad_weight_a == nullptr || grad_weight_f == nullptr || weight_a == nullptr || weight_f == nullptr ||
         grad_output_f == nullptr ||
@@ -673,15 +709,16 @@ int rmsnorm_backward_dual(void* grad_input, void* grad_weight_a, void* grad_weig
     return dispatch_dtype(dtype, [&]<typename T>() -> int {
         const FastShape shape = pick_fast_shape<T>(h);
         const int blocks = fast_blocks(shape, r, dual_kernel<T, true>(shape));
-        const int reduce_blocks = (h + kWave - 1) / kWave;
         const int slices = wide_reduce_slices(blocks, h, compute_units());
         void* mem = nullptr;
+        bool deferred = false;
         const std::size_t partial_bytes = static_cast<std::size_t>(blocks) * hidden * sizeof(float);
-        const std::size_t second_bytes = static_cast<std::size_t>(slices) * hidden * sizeof(float);
-        if (int s = scratch(stream, 2 * partial_bytes + second_bytes, &mem)) return s;
+        const std::size_t second_bytes = (static_cast<std::size_t>(slices) * hidden * sizeof(float) + 255) & ~std::size_t{255};
+        if (int s = partial_memory(sink, stream, 2 * partial_bytes + 2 * second_bytes, &mem, &deferred)) return s;
         auto* partial_a = static_cast<float*>(mem);
         auto* partial_f = reinterpret_cast<float*>(static_cast<char*>(mem) + partial_bytes);
-        auto* second = reinterpret_cast<float*>(static_cast<char*>(mem) + 2 * partial_bytes);
+        auto* second_a = reinterpret_cast<float*>(static_cast<char*>(mem) + 2 * partial_bytes);
+        auto* second_f = reinterpret_cast<float*>(static_cast<char*>(mem) + 2 * partial_bytes + second_bytes);
         if (int s = launch_dual<T, true>(shape, static_cast<T*>(grad_input), nullptr, partial_a, partial_f,
                                          static_cast<const T*>(grad_output_a), static_cast<const T*>(grad_output_f),
                                          static_cast<const T*>(residual), static_cast<const T*>(input),
@@ -689,23 +726,12 @@ int rmsnorm_backward_dual(void* grad_input, void* grad_weight_a, void* grad_weig
                                          stream))
             return s;
         CGPTX_LAUNCH_CHECK();
-        // The two weight gradients are reduced one after the other through the same second-stage buffer
-        // (launches on one stream run in order).
-        for (int which = 0; which < 2; ++which) {
-            float* partial = which == 0 ? partial_a : partial_f;
-            auto* dw = static_cast<T*>(which == 0 ? grad_weight_a : grad_weight_f);
-            if (slices > 1) {
-                hipLaunchKernelGGL(column_partial_fold_kernel, dim3(reduce_blocks, slices), dim3(kThreads), 0, stream, second,
-                                   partial, blocks, h);
-                CGPTX_LAUNCH_CHECK();
-                hipLaunchKernelGGL((column_partial_reduce_kernel<T>), dim3(reduce_blocks), dim3(kThreads), 0, stream, dw, second,
-                                   slices, h, 0);
-            } else {
-                hipLaunchKernelGGL((column_partial_reduce_kernel<T>), dim3(reduce_blocks), dim3(kThreads), 0, stream, dw, partial,
-                                   blocks, h, 0);
-            }
-            CGPTX_LAUNCH_CHECK();
-        }
+        if (int s = reduce_columns<T>(sink, deferred, static_cast<T*>(grad_weight_a), partial_a, second_a, blocks, h, slices,
+                                      dtype, stream))
+            return s;
+        if (int s = reduce_columns<T>(sink, deferred, static_cast<T*>(grad_weight_f), partial_f, second_f, blocks, h, slices,
+                                      dtype, stream))
+            return s;
         return CGPTX_OK;
     });
 }
@@ -717,6 +743,7 @@ struct Workspace {
     hipStream_t stream;
     void* fixed;
     std::size_t fixed_bytes;
+    ColumnReduceSink* sink = nullptr;  // when given and roomy enough, the weight-gradient reduction is recorded there
     int get(std::size_t bytes, void** out) const {
         if (fixed == nullptr) return scratch(stream, bytes, out);
         if (bytes > fixed_bytes)
@@ -750,24 +777,17 @@ int rmsnorm_backward_impl(void* grad_input, void* grad_weight, const void* grad_
             const int slices = wide_reduce_slices(blocks, h, compute_units());
             void* mem = nullptr;
             const std::size_t partial_bytes = static_cast<std::size_t>(blocks) * hidden * sizeof(float);
-            if (int s = workspace.get(partial_bytes + static_cast<std::size_t>(slices) * hidden * sizeof(float), &mem))
-                return s;
+            const std::size_t bytes = partial_bytes + static_cast<std::size_t>(slices) * hidden * sizeof(float);
+            if (workspace.sink != nullptr) mem = workspace.sink->take(bytes);
+            const bool deferred = mem != nullptr;
+            if (!deferred) {
+                if (int s = workspace.get(bytes, &mem)) return s;
+            }
             auto* partial = static_cast<float*>(mem);
             if (int s = launch_fast<T, true>(shape, dx, partial, dy, res, x, w, r, h, epsilon, blocks, stream)) return s;
             CGPTX_LAUNCH_CHECK();
-            if (slices > 1) {
-                auto* second = reinterpret_cast<float*>(static_cast<char*>(mem) + partial_bytes);
-                hipLaunchKernelGGL(column_partial_fold_kernel, dim3(reduce_blocks, slices), dim3(kThreads), 0, stream,
-                                   second, partial, blocks, h);
-                CGPTX_LAUNCH_CHECK();
-                hipLaunchKernelGGL((column_partial_reduce_kernel<T>), dim3(reduce_blocks), dim3(kThreads), 0, stream, dw,
-                                   second, slices, h, 0);
-            } else {
-                hipLaunchKernelGGL((column_partial_reduce_kernel<T>), dim3(reduce_blocks), dim3(kThreads), 0, stream, dw,
-                                   partial, blocks, h, 0);
-            }
-            CGPTX_LAUNCH_CHECK();
-            return CGPTX_OK;
+            auto* second = reinterpret_cast<float*>(static_cast<char*>(mem) + partial_bytes);
+            return reduce_columns<T>(workspace.sink, deferred, dw, partial, second, blocks, h, slices, dtype, stream);
         }
         const int slices = r < 256 ? 1 : (r < 65536 ? 64 : 256);
         const int rows_per_slice = (r + slices - 1) / slices;
@@ -795,9 +815,9 @@ int rmsnorm_backward_impl(void* grad_input, void* grad_weight, const void* grad_
 
 int rmsnorm_backward_residual(void* grad_input, void* grad_weight, const void* grad_output, const void* input,
                               const void* weight, const void* residual, std::size_t rows, std::size_t hidden,
-                              float epsilon, int dtype, hipStream_t stream) {
+                              float epsilon, int dtype, hipStream_t stream, ColumnReduceSink* sink) {
     return rmsnorm_backward_impl(grad_input, grad_weight, grad_output, input, weight, residual, rows, hidden, epsilon, dtype,
-                                 stream, Workspace{stream, nullptr, 0});
+                                 stream, Workspace{stream, nullptr, 0, sink});
 }
 
 }  // namespace cgptx

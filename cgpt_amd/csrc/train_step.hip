@@ -116,6 +116,12 @@ struct cgptx_model {
     int graph_loss_mode = -1;
     hipStream_t graph_stream = nullptr;
     std::uint64_t graph_scratch_generation = 0;  // scratch arena block the recorded kernels point into
+    // weight-gradient reductions of the norm-backward passes, run as one pair of launches per step
+    cgptx::ColumnReduceSink norm_reductions;
+    cgptx::ColumnReduceEntry* norm_reduction_table = nullptr;       // device copy of the entries
+    std::vector<cgptx::ColumnReduceEntry> norm_reduction_uploaded;  // what the device copy holds
+    std::size_t norm_reduction_table_capacity = 0;                  // entries
+    bool norm_reductions_resized = false;                           // the last pass grew the sink's memory
     // optional per-operator timing of one eager pass
     struct Timed {
         const char* label;
@@ -348,6 +354,69 @@ bool fused_swiglu() {
     return text == nullptr || text[0] != '0';
 }
 
+// Whether the norm-backward passes of the step leave their weight-gradient reductions to one pair of launches at
+// the end of the backward pass (CGPTX_FUSE_DGAMMA=0 keeps the two small launches after each pass, for comparisons:
+// same additions in the same order, same bits).
+cgptx::ColumnReduceSink* norm_reduction_sink(cgptx_model* m) {
+    const char* text = std::getenv("CGPTX_FUSE_DGAMMA");  // read per enqueue
+    return (text == nullptr || text[0] != '0') ? &m->norm_reductions : nullptr;
+}
+
+// Runs what the passes recorded. The entries are the same from pass to pass (same buffers, same shapes), so the
+// device copy of the table is written once, outside any capture; the sink's memory is sized after the first pass
+// that found it too small (that pass reduced at once, from the arena).
+int finish_norm_reductions(cgptx_model* m, hipStream_t stream) {
+    auto& sink = m->norm_reductions;
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    if (stream != nullptr) CGPTX_HIP(hipStreamIsCapturing(stream, &capture));
+    const bool capturing = capture != hipStreamCaptureStatusNone;
+    // A recorded step holds the addresses of the table and of the sink's memory and the number of entries: it is
+    // recorded again after any of them changes.
+    auto drop_recorded_step = [&]() {
+        if (m->graph_exec != nullptr) {
+            (void)hipGraphExecDestroy(m->graph_exec);
+            m->graph_exec = nullptr;
+        }
+    };
+    if (!sink.entries.empty()) {
+        if (!(sink.entries == m->norm_reduction_uploaded)) {
+            if (capturing) return fail(CGPTX_RUNTIME, "model: the table of norm reductions changed under graph capture");
+            CGPTX_HIP(hipStreamSynchronize(stream));  // earlier launches may still read the table
+            drop_recorded_step();
+            if (sink.entries.size() > m->norm_reduction_table_capacity) {
+                if (m->norm_reduction_table != nullptr) CGPTX_HIP(hipFree(m->norm_reduction_table));
+                m->norm_reduction_table = nullptr;
+                CGPTX_HIP(hipMalloc(reinterpret_cast<void**>(&m->norm_reduction_table),
+                                    sink.entries.size() * sizeof(ColumnReduceEntry)));
+                m->norm_reduction_table_capacity = sink.entries.size();
+            }
+            CGPTX_HIP(hipMemcpy(m->norm_reduction_table, sink.entries.data(), sink.entries.size() * sizeof(ColumnReduceEntry),
+                                hipMemcpyHostToDevice));
+            m->norm_reduction_uploaded = sink.entries;
+        }
+        int max_hidden = 0, max_slices = 0;
+        for (const ColumnReduceEntry& e : sink.entries) {
+            max_hidden = std::max(max_hidden, e.hidden);
+            max_slices = std::max(max_slices, e.slices);
+        }
+        if (int s = run_column_reductions(m->norm_reduction_table, static_cast<int>(sink.entries.size()), max_hidden,
+                                          max_slices, stream))
+            return s;
+    }
+    m->norm_reductions_resized = false;
+    if (sink.wanted > sink.capacity && !capturing) {
+        CGPTX_HIP(hipStreamSynchronize(stream));
+        drop_recorded_step();
+        if (sink.memory != nullptr) CGPTX_HIP(hipFree(sink.memory));
+        sink.memory = nullptr;
+        sink.capacity = 0;
+        CGPTX_HIP(hipMalloc(reinterpret_cast<void**>(&sink.memory), sink.wanted));
+        sink.capacity = sink.wanted;
+        m->norm_reductions_resized = true;
+    }
+    return CGPTX_OK;
+}
+
 // CGPTX_FUSE=0: the step as the reference's own call sequence, one public operator per call — forward in the
 // order of src/core/transformer_block.cu:466-595, backward in the order of :663-747 and
 // src/core/transformer_model.cu:360-380 (separate q / k / v and gate / up projections with accumulating input
@@ -526,8 +595,10 @@ int enqueue_forward_backward(cgptx_model* m, float loss_scale, int loss_mode, hi
     // ----------------------------------------------------------------- backward
     void* current = m->grad_a;
     void* previous = m->grad_b;
-    CGPTX_OP("rmsnorm_bwd", cgptx_rmsnorm_backward(current, m->final_norm.gradient, m->d_normalized, last, m->final_norm.value, N,
-                                     H, eps, dt, s));
+    ColumnReduceSink* sink = norm_reduction_sink(m);
+    m->norm_reductions.begin();
+    CGPTX_OP("rmsnorm_bwd", rmsnorm_backward_residual(current, m->final_norm.gradient, m->d_normalized, last, m->final_norm.value,
+                                                      nullptr, N, H, eps, dt, stream, sink));
     for (std::size_t reverse = c.num_layers; reverse-- > 0;) {
         const auto& w = m->layers[reverse];
         const auto& a = m->acts[reverse];
@@ -550,7 +621,7 @@ int enqueue_forward_backward(cgptx_model* m, float loss_scale, int loss_mode, hi
                                         "gemm_dx.gate_up", "gemm_dw.gate_up"));
         if (!dual_norms) {
             CGPTX_OP("rmsnorm_bwd", rmsnorm_backward_residual(previous, w.ffn_norm.gradient, m->d_norm_in, x, w.ffn_norm.value,
-                                                              current, N, H, eps, dt, stream));
+                                                              current, N, H, eps, dt, stream, sink));
         }
         CGPTX_TRY(linear_backward_split(m, m->d_attn_out, w.o.gradient, current, a.attn_out, w.o.value, N, QW, H, 0, dt, stream, "gemm_dx.o", "gemm_dw.o"));
         CGPTX_OP("attn_bwd", cgptx_flash_gqa_attention_backward_with_lse(m->d_q, m->d_k, m->d_v, m->d_attn_out, a.attn_out,
@@ -560,16 +631,16 @@ int enqueue_forward_backward(cgptx_model* m, float loss_scale, int loss_mode, hi
         if (fused_qk_norm_rope(m, m->d_q, m->d_q, a.q_pre, w.q_norm.value) &&
             fused_qk_norm_rope(m, m->d_k, m->d_k, a.k_pre, w.k_norm.value)) {
             CGPTX_OP("rmsnorm_bwd", rmsnorm_rope_backward(m->d_q, w.q_norm.gradient, m->d_q, a.q_pre, w.q_norm.value, m->cos_cache,
-                                                          m->sin_cache, N * HQ, D, HQ, m->sequence, c.rotary_dim, 0, eps, dt, stream));
+                                                          m->sin_cache, N * HQ, D, HQ, m->sequence, c.rotary_dim, 0, eps, dt, stream, sink));
             CGPTX_OP("rmsnorm_bwd", rmsnorm_rope_backward(m->d_k, w.k_norm.gradient, m->d_k, a.k_pre, w.k_norm.value, m->cos_cache,
-                                                          m->sin_cache, N * HKV, D, HKV, m->sequence, c.rotary_dim, 0, eps, dt, stream));
+                                                          m->sin_cache, N * HKV, D, HKV, m->sequence, c.rotary_dim, 0, eps, dt, stream, sink));
         } else {
             CGPTX_OP("rope_bwd", cgptx_rope_backward(m->d_q_pre, m->d_k_pre, m->d_q, m->d_k, m->cos_cache, m->sin_cache, m->batch,
                                           m->sequence, HQ, HKV, D, c.rotary_dim, 0, m->sequence, dt, s));
-            CGPTX_OP("rmsnorm_bwd", cgptx_rmsnorm_backward(m->d_q, w.q_norm.gradient, m->d_q_pre, a.q_pre, w.q_norm.value, N * HQ, D,
-                                             eps, dt, s));
-            CGPTX_OP("rmsnorm_bwd", cgptx_rmsnorm_backward(m->d_k, w.k_norm.gradient, m->d_k_pre, a.k_pre, w.k_norm.value, N * HKV, D,
-                                             eps, dt, s));
+            CGPTX_OP("rmsnorm_bwd", rmsnorm_backward_residual(m->d_q, w.q_norm.gradient, m->d_q_pre, a.q_pre, w.q_norm.value, nullptr,
+                                                              N * HQ, D, eps, dt, stream, sink));
+            CGPTX_OP("rmsnorm_bwd", rmsnorm_backward_residual(m->d_k, w.k_norm.gradient, m->d_k_pre, a.k_pre, w.k_norm.value, nullptr,
+                                                              N * HKV, D, eps, dt, stream, sink));
         }
         if (fused_qkv) {
             CGPTX_OP("gemm_dx.qkv", qkv_backward_input(m->d_norm_in, m->d_q, m->d_k, m->d_v, w.q.value, N, H, QW, KW, dt, stream));
@@ -582,16 +653,17 @@ int enqueue_forward_backward(cgptx_model* m, float loss_scale, int loss_mode, hi
         if (dual_norms) {
             CGPTX_OP("rmsnorm_bwd", rmsnorm_backward_dual(previous, w.attention_norm.gradient, w.ffn_norm.gradient, m->d_norm_in,
                                                           m->d_norm_in_f, x, w.attention_norm.value, w.ffn_norm.value, current, N, H,
-                                                          eps, dt, stream));
+                                                          eps, dt, stream, sink));
         } else {
             CGPTX_OP("rmsnorm_bwd", rmsnorm_backward_residual(previous, w.attention_norm.gradient, m->d_norm_in, x,
-                                                              w.attention_norm.value, previous, N, H, eps, dt, stream));
+                                                              w.attention_norm.value, previous, N, H, eps, dt, stream, sink));
         }
         std::swap(current, previous);
     }
     // Tied embedding: the classifier gradient is already in place; add the lookup's gradient
     // (src/core/transformer_model.cu:375-380).
     CGPTX_OP("embedding_bwd", cgptx_embedding_backward(m->embedding.gradient, current, m->tokens, N, c.vocabulary_size, H, 1, 1, dt, s));
+    CGPTX_OP("rmsnorm_bwd", finish_norm_reductions(m, stream));
     return CGPTX_OK;
 }
 
@@ -623,6 +695,8 @@ extern "C" int cgptx_model_destroy(cgptx_model* m) {
     if (m->graph_exec != nullptr) (void)hipGraphExecDestroy(m->graph_exec);
     if (m->optimizer != nullptr) (void)cgptx_adamw_workspace_destroy(m->optimizer);
     for (void* p : m->allocations) (void)hipFree(p);
+    if (m->norm_reductions.memory != nullptr) (void)hipFree(m->norm_reductions.memory);
+    if (m->norm_reduction_table != nullptr) (void)hipFree(m->norm_reduction_table);
     delete m;
     return CGPTX_OK;
 }
@@ -878,6 +952,11 @@ extern "C" int cgptx_model_forward_backward(cgptx_model* m, float loss_scale, in
     // Eager run first: it sizes every scratch arena and does this call's work. Then record the
     // same sequence for the following calls.
     if (int s = enqueue_forward_backward(m, loss_scale, loss_mode, stream)) return s;
+    if (m->norm_reductions_resized) {
+        // The pass above sized the memory of the deferred norm reductions (and reduced at once): one more eager
+        // pass records them and writes their table, which a capture cannot do.
+        if (int s = enqueue_forward_backward(m, loss_scale, loss_mode, stream)) return s;
+    }
     CGPTX_HIP(hipStreamSynchronize(stream));
     if (m->graph_exec != nullptr) {
         CGPTX_HIP(hipGraphExecDestroy(m->graph_exec));

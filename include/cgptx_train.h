@@ -136,8 +136,9 @@ int cgptx_model_load_optimizer(cgptx_model* model, const char* path, uint64_t* s
  *
  * Environment switches read at every enqueue (a recorded graph keeps what it was recorded with):
  * CGPTX_FUSE=0 runs the step as the reference's own call sequence, one public operator per call
- * (src/core/transformer_block.cu:466-595, 663-747); CGPTX_FUSE_QK=0, CGPTX_FUSE_NORMS=0 and CGPTX_FUSE_SWIGLU=0
- * switch single fusions of the default step off. */
+ * (src/core/transformer_block.cu:466-595, 663-747); CGPTX_FUSE_QK=0, CGPTX_FUSE_NORMS=0, CGPTX_FUSE_SWIGLU=0 and
+ * CGPTX_FUSE_DGAMMA=0 (the norm weight-gradient reductions after each pass instead of once per step) switch single
+ * fusions of the default step off. */
 int cgptx_model_activation(const cgptx_model* model, const char* name, void** data, size_t* count);
 
 #ifdef __cplusplus

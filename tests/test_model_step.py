@@ -275,6 +275,46 @@ def test_fused_qk_norm_rope_is_bit_identical_to_the_separate_operators(device, m
 
 
 @pytest.mark.gpu
+def test_norm_weight_gradients_reduced_at_the_end_of_the_backward_pass_are_bit_identical(device, monkeypatch):
+    """The norm-backward passes of a step leave the reduction of their weight-gradient partial sums to one pair of
+    launches at the end of the backward pass (same additions, same order); CGPTX_FUSE_DGAMMA=0 reduces after each
+    pass. Eager passes (the first sizes the memory for the partial sums and still reduces at once, the later ones
+    defer) and graph replays all give the same bits, with the block norms fused and separate."""
+    from cgpt_amd.model import LOSS_CUT, Model, ModelConfig
+    config = ModelConfig(vocabulary_size=512, num_layers=3, hidden_size=1024, intermediate_size=512, num_query_heads=8,
+                         num_kv_heads=2, head_dim=128, rotary_dim=128, dtype=torch.bfloat16)
+    batch, seq = 4, 512
+    rng = np.random.default_rng(5)
+    inputs = rng.integers(0, 512, size=batch * seq).astype(np.uint32)
+    targets = rng.integers(0, 512, size=batch * seq).astype(np.uint32)
+    stream = torch.cuda.Stream(device=device)
+
+    def gradients(model):
+        stream.synchronize()
+        return [g.clone() for _, _, g in model.parameters()]
+
+    for norms in ("1", "0"):
+        monkeypatch.setenv("CGPTX_FUSE_NORMS", norms)
+        monkeypatch.setenv("CGPTX_FUSE_DGAMMA", "0")
+        model = Model(config, batch, seq, seed=6, device=device)
+        model.set_tokens(inputs, targets)
+        model.forward_backward(8.0, LOSS_CUT, use_graph=False, stream=stream)
+        want = gradients(model)
+        model.close()
+        monkeypatch.setenv("CGPTX_FUSE_DGAMMA", "1")
+        model = Model(config, batch, seq, seed=6, device=device)
+        model.set_tokens(inputs, targets)
+        for use_graph in (False, False, True, True, True, False):
+            for _, _, g in model.parameters():
+                g.zero_()
+            torch.cuda.synchronize()
+            model.forward_backward(8.0, LOSS_CUT, use_graph=use_graph, stream=stream)
+            for (name, _, _), a, b in zip(model.parameters(), gradients(model), want):
+                assert torch.equal(a, b), f"{name} (block norms fused: {norms}, graph: {use_graph})"
+        model.close()
+
+
+@pytest.mark.gpu
 def test_swiglu_in_the_projection_epilogues_is_bit_identical_to_the_separate_operators(device, monkeypatch):
     """The SwiGLU product rides in the gate/up projection's epilogue and its gradient in the epilogue of the
     down projection's input gradient when the shapes fill the chip (here 4096 rows x 3328 feed-forward
