@@ -76,8 +76,10 @@ TRAFFIC_FILE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profile
                             "gemm_dx_256x256_gate_projection_pmc.txt")
 
 
-def kernel_probe(torch, cfg, batch, seq, stream, launches, seed, dtype=None):
-    """Average duration of one launch of the dominant kernel: HIP events on the launch stream."""
+def kernel_probe(torch, cfg, batch, seq, stream, launches, seed, dtype=None, data="random"):
+    """Average duration of one launch of the dominant kernel: HIP events on the launch stream. data = "zeros" runs the
+    same launch on all-zero operands (same instructions, same memory traffic, no switching in the multipliers): the
+    difference to random data is what the chip's power limit costs."""
     from cgpt_amd import ops
 
     dtype = dtype or torch.bfloat16
@@ -87,6 +89,9 @@ def kernel_probe(torch, cfg, batch, seq, stream, launches, seed, dtype=None):
     x = torch.empty(rows, hidden, device="cuda", dtype=dtype)  # shape only: no weight gradient is asked for
     w = (torch.randn(inter, hidden, device="cuda", generator=generator) * 0.02).to(dtype)
     dx = torch.empty(rows, hidden, device="cuda", dtype=dtype)
+    if data == "zeros":
+        dy.zero_()
+        w.zero_()
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     with torch.cuda.stream(stream):
         for _ in range(3):
@@ -407,6 +412,10 @@ def main() -> int:
                              "attention, swiglu, embedding, cut_cross_entropy, dense_cross_entropy, copy, secondary, published; several "
                              "separated by commas; '' = all) and print "
                              "their table: the target of per-kernel rocprofv3 runs")
+    parser.add_argument("--probe-data", choices=["random", "zeros"], default="random",
+                        help="operands of --probe-only: random bf16 values, or zeros (same launch without switching "
+                             "activity in the multipliers, to show what the power limit costs)")
+    parser.add_argument("--probe-launches", type=int, default=20, help="timed launches of --probe-only")
     parser.add_argument("--probe-only", action="store_true",
                         help="launch only the dominant kernel (20x) and a 1 GiB device copy: the target of the "
                              "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs behind roofline.traffic")
@@ -439,13 +448,13 @@ def main() -> int:
         return 0
     if args.probe_only:
         stream = torch.cuda.Stream(device=device)
-        probe = kernel_probe(torch, cfg, args.batch, args.seq, stream, 20, args.seed)
+        probe = kernel_probe(torch, cfg, args.batch, args.seq, stream, args.probe_launches, args.seed, None, args.probe_data)
         source = torch.empty(1 << 30, dtype=torch.uint8, device=device)
         target = torch.empty_like(source)
         for _ in range(5):
             target.copy_(source)  # calibration: reads 1 GiB and writes 1 GiB per launch
         torch.cuda.synchronize()
-        print(json.dumps({"probe": PROBE_KERNEL, **probe, "copy_bytes": 1 << 30}))
+        print(json.dumps({"probe": PROBE_KERNEL, "data": args.probe_data, **probe, "copy_bytes": 1 << 30}))
         return 0
     model = Model(cfg, args.batch, args.seq, seed=args.seed, device=device)
     rng = np.random.default_rng(args.seed)
