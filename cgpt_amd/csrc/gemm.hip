@@ -958,11 +958,12 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
     // (k = 32) of TM x TN MFMAs, taken as two column halves (all rows x the left TN/2 blocks, then
     // all rows x the right ones) so that one set of fragment registers suffices: a fragment is read
     // for the next tile as soon as its last MFMA of this tile has been issued.
-    //   left half    MFMAs ‖ LDS reads of this tile's right-half B fragments
+    //   left half    MFMAs ‖ LDS reads of this tile's right-half B fragments ‖ the second half of the loads of
+    //                tile t+kStages-2 (into the stage freed one tile ago)
     //   wait         this wavefront's loads of tile t+1 have landed; barrier: everybody's have, and
     //                nobody reads stage (t-1) % kStages any more
-    //   right half   MFMAs ‖ loads of tile t+kStages-1 into that stage ‖ tile t+1's left-half B
-    //                fragments (first thing) and its A fragment i after row i
+    //   right half   MFMAs ‖ the first half of the loads of tile t+kStages-1 into that stage ‖ tile t+1's
+    //                left-half B fragments (first thing) and its A fragment i after row i
     // so LDS latency and kStages-2 K tiles of global latency sit in the shadow of MFMAs. With one
     // wavefront per SIMD nothing else hides an instruction that is not next to an MFMA, so every
     // MFMA is followed by its share of the loads and fragment reads and a scheduling fence keeps
@@ -987,7 +988,16 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
                 // was in the left half), A fragment i after the last MFMA of row i.
                 if constexpr (jj == 0 && i < kHalf) read_frag.template operator()<TM + i>(tile);
                 if constexpr (jj == kHalf - 1) read_frag.template operator()<i>(tile);
-                static_for<(m * kTileLoads) / (kMfmas / 2), ((m + 1) * kTileLoads) / (kMfmas / 2)>(
+                // The first half of the loads of tile t+kStages-1 (one load per kMfmas / kTileLoads MFMAs).
+                static_for<(m * (kTileLoads / 2)) / (kMfmas / 2), ((m + 1) * (kTileLoads / 2)) / (kMfmas / 2)>(
+                    [&](auto l) { issue_one(l, free_lds, ca, cb); });
+            }
+            if constexpr (HALF == 0 && !FIRST) {
+                // The second half of the loads that the previous tile's right half began: a wavefront's load
+                // instruction keeps it from issuing for about as long as an MFMA runs, so the loads are dealt out
+                // evenly over the whole tile instead of twice as densely over one half.
+                static_for<kTileLoads / 2 + (m * (kTileLoads / 2)) / (kMfmas / 2),
+                           kTileLoads / 2 + ((m + 1) * (kTileLoads / 2)) / (kMfmas / 2)>(
                     [&](auto l) { issue_one(l, free_lds, ca, cb); });
             }
             __builtin_amdgcn_sched_barrier(0);
@@ -1012,8 +1022,11 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
         int free_stage = kStages - 1;  // of tile t-1, refilled with tile t+kStages-1
         auto multiply_tile = [&]<bool FIRST>(int t) __attribute__((always_inline)) {
             const int next_stage = stage + 1 == kStages ? 0 : stage + 1;
+            // The left half finishes the requests of tile t+kStages-2 (cursors and stage of the previous tile: the
+            // stage before free_stage), then the cursors move on to tile t+kStages-1.
+            const int previous_free = free_stage == 0 ? kStages - 1 : free_stage - 1;
+            multiply_half.template operator()<0, FIRST>(smem + stage * kStage, lds_wave + previous_free * kStageBytes);
             cursors(t + kStages - 1, ca, cb);
-            multiply_half.template operator()<0, FIRST>(smem + stage * kStage, 0u);
             __builtin_amdgcn_s_waitcnt(vmcnt_immediate((kStages - 3) * kTileLoads));
             barrier_only();
             multiply_half.template operator()<1, FIRST>(smem + next_stage * kStage, lds_wave + free_stage * kStageBytes);
