@@ -155,6 +155,46 @@ def test_gpu_step_matches_float64_composition(device, dtype, loss_mode, shape):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("seed", range(16))
+def test_gpu_step_matches_float64_composition_on_random_configurations(device, seed):
+    """Seeded random small models — 1 to 3 layers, 1 to 4 kv-heads with groups of 1 to 4, heads of 16 to 128, odd
+    feed-forward widths, every storage dtype, both loss paths, eager and recorded — against the float64 composition:
+    the shape classes in which the step falls back from its fused launches to the separate operators are exactly
+    the ones fixed shape lists tend to miss."""
+    rng = np.random.default_rng(700 + seed)
+    dtype = [torch.bfloat16, torch.float16, torch.float32][int(rng.integers(0, 3))]
+    hkv = int(rng.integers(1, 5))
+    hq = hkv * int(rng.integers(1, 5))
+    d = [16, 32, 64, 128][int(rng.integers(0, 4))]
+    if hq * d > 1024:
+        d = 32
+    cfg = dict(vocab=int(rng.integers(40, 300)), layers=int(rng.integers(1, 4)), hidden=hq * d,
+               inter=int(rng.integers(1, 40)) * 8 if rng.integers(0, 2) else int(rng.integers(8, 300)), hq=hq, hkv=hkv, d=d,
+               eps=1e-5)
+    batch, seq = int(rng.integers(1, 4)), int(rng.integers(2, 70))
+    loss_mode, use_graph = int(rng.integers(0, 2)), bool(rng.integers(0, 2))
+    loss_scale = 64.0
+    print(f"model {cfg} batch={batch} seq={seq} loss_mode={loss_mode} graph={use_graph} {dtype}", flush=True)
+    model = build(device, dtype, batch, seq, cfg, seed=seed)
+    tokens = rng.integers(0, cfg["vocab"], size=(batch, seq))
+    targets = rng.integers(0, cfg["vocab"], size=(batch, seq))
+    model.set_tokens(tokens, targets)
+    stream = torch.cuda.Stream(device=device)
+    for _ in range(2 if use_graph else 1):  # the second call replays the recorded step
+        model.forward_backward(loss_scale, loss_mode, use_graph=use_graph, stream=stream)
+    loss, _, _ = model.status(stream)
+    params, grads = params_from_model(model, cfg)
+    want_loss, want, saved = model64.forward_backward(params, tokens, targets, cfg, loss_scale, torch_round(dtype))
+    sixteen = dtype != torch.float32
+    assert abs(loss - want_loss) <= (2e-2 if sixteen else 1e-4) * want_loss
+    for l in range(cfg["layers"] + 1):
+        hidden = to_np(model.activation(f"hidden.{l}")).reshape(batch * seq, cfg["hidden"])
+        assert np.abs(hidden - saved["hidden"][l]).max() <= (4e-2 if sixteen else 1e-4) * max(1.0, np.abs(saved["hidden"][l]).max())
+    compare_gradients(grads, want, 5e-2 if sixteen else 1e-3, loss_scale)
+    model.close()
+
+
+@pytest.mark.gpu
 def test_graph_replay_equals_eager_and_losses_agree_between_modes(device):
     cfg = MODEL_CFG
     dtype = torch.bfloat16
