@@ -182,3 +182,48 @@ def test_embedding_and_cross_entropy_random_shapes(device, seed):
     assert abs(closs.item() - cl64) <= (1e-4 if dtype == torch.float32 else 5e-3) * max(1.0, cl64)
     assert_scaled_close(dx, dx64, TOL[dtype], "dX")
     assert_scaled_close(dc, dc64, TOL[dtype], "dC")
+
+
+@pytest.mark.parametrize("seed", SEEDS[:16])
+def test_adamw_many_random_tensor_lists(device, seed):
+    """Random lists of 1 to 12 tensors of 1 to 40000 elements each (mixed storage dtypes within a list), random
+    hyper-parameters, clipping on or off, three steps of which one may carry a non-finite gradient (skipped as a
+    whole: no tensor changes, the step counter stays), against the float64 update of src/optim/adamw.cu:148-187."""
+    rng = np.random.default_rng(6000 + seed)
+    count = int(rng.integers(1, 13))
+    sizes = [int(rng.integers(1, 40000)) if rng.integers(0, 4) else int(rng.integers(1, 9)) for _ in range(count)]
+    dtypes = [DTYPES[int(rng.integers(0, 3))] for _ in range(count)]
+    lr, wd = float(10 ** rng.uniform(-4, -2)), float(rng.uniform(0, 0.2))
+    beta1, beta2 = float(rng.uniform(0.8, 0.95)), float(rng.uniform(0.9, 0.999))
+    loss_scale = float(pick(rng, [1.0, 64.0, 1024.0]))
+    max_norm = float(pick(rng, [float("inf"), 1.0, 0.05]))
+    bad_step = int(rng.integers(0, 6))  # 0..2: that step's gradients hold an Inf or NaN somewhere
+    print(f"adamw sizes={sizes} lr={lr:.2e} wd={wd:.3f} betas=({beta1:.3f},{beta2:.4f}) scale={loss_scale} "
+          f"max_norm={max_norm} bad_step={bad_step}", flush=True)
+    params = [randn((n,), t, seed * 100 + i, 0.5) for i, (n, t) in enumerate(zip(sizes, dtypes))]
+    d_params = [dev(p, device).clone() for p in params]
+    states = [ops.AdamWState.for_parameter(p) for p in d_params]
+    d_grads = [torch.empty_like(p) for p in d_params]
+    entries = [ops.AdamWBatchEntry(p, g, s) for p, g, s in zip(d_params, d_grads, states)]
+    ws = ops.AdamWWorkspace()
+    options = ops.AdamWOptions(learning_rate=lr, beta1=beta1, beta2=beta2, epsilon=1e-8, weight_decay=wd,
+                               loss_scale=loss_scale, max_grad_norm=max_norm)
+    masters = [to_np(p) for p in params]
+    ms, vs, step = [np.zeros(n) for n in sizes], [np.zeros(n) for n in sizes], 0
+    for it in range(3):
+        grads = [randn((n,), t, seed * 1000 + 10 * it + i, loss_scale * 0.02) for i, (n, t) in enumerate(zip(sizes, dtypes))]
+        if it == bad_step:
+            victim = int(rng.integers(0, count))
+            grads[victim][int(rng.integers(0, sizes[victim]))] = float("inf") if rng.integers(0, 2) else float("nan")
+        for dg, g in zip(d_grads, grads):
+            dg.copy_(g)
+        ops.adamw_step_many_async(entries, options, ws)
+        ok, masters, ms, vs, step = oracle64.adamw(None, [to_np(g) for g in grads], masters, ms, vs, step, lr, beta1, beta2,
+                                                   1e-8, wd, loss_scale, max_norm)
+        assert ops.adamw_check(ws) == ok
+        assert states[0].step == step
+    for p, s, m64, mm, vv, t in zip(d_params, states, masters, ms, vs, dtypes):
+        assert_close(s.master_parameter, m64, 1e-5, "master")
+        assert_close(s.first_moment, mm, 1e-5, "m")
+        assert np.abs(to_np(s.second_moment) - vv).max() <= 1e-5 * max(1e-12, np.abs(vv).max()) + 1e-12
+        assert torch.equal(p, s.master_parameter.to(t))
