@@ -36,10 +36,28 @@ DEVICE_FLAGS = [
 ]
 
 
-# Per-file additions. attention.hip: MFMA results in vector registers by default (the softmax arithmetic reads
-# them in place); the kernels pin the accumulators that never leave the matrix pipeline to the accumulation
-# registers themselves.
+# Per-file additions. attention.hip: MFMA results in vector registers (the softmax arithmetic reads them in
+# place). The option belongs to the compiler's backend, not to its documented interface: it is probed once and
+# left out, with a warning, when this hipcc does not know it (the kernels are correct either way, the
+# accumulators are then copied between the two register files).
 FILE_FLAGS = {"attention.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]}
+_probed_flags: dict[tuple[str, ...], bool] = {}
+
+
+def _compiler_accepts(flags: list[str]) -> bool:
+    key = tuple(flags)
+    if key not in _probed_flags:
+        proc = subprocess.run([HIPCC, "--offload-arch=gfx950", "-x", "hip", "-c", "/dev/null", "-o", "/dev/null", *flags],
+                              capture_output=True, text=True)
+        _probed_flags[key] = proc.returncode == 0
+        if proc.returncode != 0:
+            print(f"cgpt_amd.build: {HIPCC} rejects {' '.join(flags)}; building without it", file=sys.stderr)
+    return _probed_flags[key]
+
+
+def file_flags(name: str) -> list[str]:
+    flags = FILE_FLAGS.get(name, [])
+    return flags if not flags or _compiler_accepts(flags) else []
 
 
 def sources() -> list[pathlib.Path]:
@@ -51,7 +69,7 @@ def _compile(src: pathlib.Path, force: bool) -> pathlib.Path:
     deps = [src] + list(CSRC.glob("*.hpp")) + list((ROOT / "include").glob("*.h"))
     if not force and obj.exists() and all(obj.stat().st_mtime >= d.stat().st_mtime for d in deps):
         return obj
-    cmd = [HIPCC, *DEVICE_FLAGS, *FILE_FLAGS.get(src.name, []), "-c", str(src), "-o", str(obj)]
+    cmd = [HIPCC, *DEVICE_FLAGS, *file_flags(src.name), "-c", str(src), "-o", str(obj)]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     noise = "is not a recognized feature for this target"
     err = "\n".join(line for line in proc.stderr.splitlines() if noise not in line)
@@ -78,7 +96,8 @@ def build(force: bool = True, jobs: int | None = None) -> pathlib.Path:
     return LIB_PATH
 
 
-INTERFACE_TEST_SOURCES = [ROOT / "tests" / "cpp" / "ops_interface_test.cpp", ROOT / "tests" / "cpp" / "block_backward_test.cpp"]
+INTERFACE_TEST_SOURCES = [ROOT / "tests" / "cpp" / name
+                          for name in ("ops_interface_test.cpp", "block_backward_test.cpp", "data_upload_test.cpp")]
 INTERFACE_TEST_BINARY = ROOT / "tests" / "cpp" / "ops_interface_test.bin"
 
 

@@ -100,12 +100,21 @@ PROTOTYPES = {
     "cgptx_token_upload_acquire": [_vp, ctypes.POINTER(_vp), ctypes.POINTER(_vp)],
     "cgptx_token_upload_submit": [_vp, _vp, _vp, _vp],
     "cgptx_model_upload_tokens": [_vp, _vp, _vp],
+    "cgptx_pinned_allocate": [ctypes.POINTER(_vp), _sz],
+    "cgptx_pinned_release": [_vp],
+    "cgptx_device_allocate": [ctypes.POINTER(_vp), _sz],
+    "cgptx_device_release": [_vp],
+    "cgptx_upload_fence_wait": [_vp],
+    "cgptx_upload_fence_destroy": [_vp],
+    "cgptx_token_upload_async": [_vp, _vp, _vp, _vp, _sz, ctypes.POINTER(_vp), _vp],
     "cgptx_model_profile": [_vp, _f, _i, _vp],
     "cgptx_model_profile_entry": [_vp, _sz, ctypes.POINTER(ctypes.c_char_p), ctypes.POINTER(_f)],
+    "cgptx_model_record_calls": [_vp, _i],
+    "cgptx_model_call": [_vp, _sz, _vp],
 }
 
 SIZE_FUNCTIONS = {"cgptx_model_parameter_count": [_vp], "cgptx_model_num_parameters": [_vp],
-                  "cgptx_model_profile_count": [_vp]}
+                  "cgptx_model_profile_count": [_vp], "cgptx_model_call_count": [_vp]}
 
 STRING_FUNCTIONS = ("cgptx_last_error", "cgptx_version")
 

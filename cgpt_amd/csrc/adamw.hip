@@ -195,44 +195,51 @@ __device__ __forceinline__ void update_chunk(const DeviceEntry& entry, unsigned 
                            reinterpret_cast<std::uintptr_t>(entry.second + begin)) & 15u) == 0;
     const unsigned long long count = end - begin;
     const unsigned long long vectors = aligned ? count / VEC : 0;
-    for (unsigned long long vi = threadIdx.x; vi < vectors; vi += kThreads) {
-        const unsigned long long at = begin + vi * VEC;
-        const vec_t<float, VEC> gr = vec_to_f32<T, VEC>(load_vec<T, VEC>(g + at));
-        vec_t<float, VEC> mm, vv, ww;
+    // A thread requests everything it will touch in the chunk (kPasses vectors of the gradient and of the three fp32
+    // state tensors: 7 kPasses 128-bit loads with 16-bit gradients) before it computes anything.
+    constexpr int kPasses = kChunk / (kThreads * VEC) > 0 ? kChunk / (kThreads * VEC) : 1;
+    constexpr int kQuads = VEC / 4;
+    for (unsigned long long v0 = 0; v0 < vectors; v0 += static_cast<unsigned long long>(kPasses) * kThreads) {
+        vec_t<T, VEC> gr[kPasses];
+        vec_t<float, 4> mm[kPasses][kQuads], vv[kPasses][kQuads], ww[kPasses][kQuads];
+        bool live[kPasses];
 #pragma unroll
-        for (int q = 0; q < VEC / 4; ++q) {
-            const vec_t<float, 4> a = load_vec<float, 4>(entry.first + at + 4 * q);
-            const vec_t<float, 4> b = load_vec<float, 4>(entry.second + at + 4 * q);
-            const vec_t<float, 4> c = load_vec<float, 4>(entry.master + at + 4 * q);
+        for (int k = 0; k < kPasses; ++k) {
+            const unsigned long long vi = v0 + static_cast<unsigned long long>(k) * kThreads + threadIdx.x;
+            live[k] = vi < vectors;
+            if (!live[k]) continue;
+            const unsigned long long at = begin + vi * VEC;
+            gr[k] = load_vec<T, VEC>(g + at);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                mm[4 * q + e] = a[e];
-                vv[4 * q + e] = b[e];
-                ww[4 * q + e] = c[e];
+            for (int q = 0; q < kQuads; ++q) {
+                mm[k][q] = load_vec<float, 4>(entry.first + at + 4 * q);
+                vv[k][q] = load_vec<float, 4>(entry.second + at + 4 * q);
+                ww[k][q] = load_vec<float, 4>(entry.master + at + 4 * q);
             }
         }
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) {
-            float m = mm[e], v = vv[e], w = ww[e];
-            adamw_element(gr[e], m, v, w, h, bc1, bc2, clip);
-            mm[e] = m;
-            vv[e] = v;
-            ww[e] = w;
-        }
+        for (int k = 0; k < kPasses; ++k) {
+            if (!live[k]) continue;
+            const unsigned long long at = begin + (v0 + static_cast<unsigned long long>(k) * kThreads + threadIdx.x) * VEC;
+            const vec_t<float, VEC> grad = vec_to_f32<T, VEC>(gr[k]);
+            vec_t<float, VEC> updated;
 #pragma unroll
-        for (int q = 0; q < VEC / 4; ++q) {
-            vec_t<float, 4> a, b, c;
+            for (int q = 0; q < kQuads; ++q) {
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                a[e] = mm[4 * q + e];
-                b[e] = vv[4 * q + e];
-                c[e] = ww[4 * q + e];
+                for (int e = 0; e < 4; ++e) {
+                    float m = mm[k][q][e], v = vv[k][q][e], w = ww[k][q][e];
+                    adamw_element(grad[4 * q + e], m, v, w, h, bc1, bc2, clip);
+                    mm[k][q][e] = m;
+                    vv[k][q][e] = v;
+                    ww[k][q][e] = w;
+                    updated[4 * q + e] = w;
+                }
+                store_vec<float, 4>(entry.first + at + 4 * q, mm[k][q]);
+                store_vec<float, 4>(entry.second + at + 4 * q, vv[k][q]);
+                store_vec<float, 4>(entry.master + at + 4 * q, ww[k][q]);
             }
-            store_vec<float, 4>(entry.first + at + 4 * q, a);
-            store_vec<float, 4>(entry.second + at + 4 * q, b);
-            store_vec<float, 4>(entry.master + at + 4 * q, c);
+            store_vec<T, VEC>(p + at, vec_from_f32<T, VEC>(updated));
         }
-        store_vec<T, VEC>(p + at, vec_from_f32<T, VEC>(ww));
     }
     for (unsigned long long i = begin + vectors * VEC + threadIdx.x; i < end; i += kThreads) {
         float m = entry.first[i], v = entry.second[i], w = entry.master[i];

@@ -52,20 +52,13 @@ using s16x4 = vec_t<short, 4>;
 
 template <typename T>
 struct Mma;
-// run(): the compiler places result and addend (this file is built with MFMA results in vector registers,
-// where the VALU reads them without a copy). accumulate(): the accumulator is pinned to the accumulation
-// registers, for tiles that only ever feed the next MFMA of their chain (dK, dV) — with both kinds in one
-// kernel nothing is copied between the two register files inside the loops. The operands of accumulate() come
-// from LDS reads and VALU converts (the compiler waits for both); its result is read again only by the next
-// accumulate() on the same registers (no wait states needed) and, after drain(), by the epilogue.
+// The compiler places result and addend (this file is built with MFMA results in vector registers, where the
+// softmax arithmetic reads them without a copy).
 template <>
 struct Mma<bf16_t> {
     using frag = vec_t<bf16_t, 8>;
     __device__ static __forceinline__ acc_t run(frag a, frag b, acc_t c) {
         return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
-    }
-    __device__ static __forceinline__ void accumulate(frag a, frag b, acc_t& c) {
-        asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
     }
 };
 template <>
@@ -74,12 +67,7 @@ struct Mma<f16_t> {
     __device__ static __forceinline__ acc_t run(frag a, frag b, acc_t c) {
         return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
     }
-    __device__ static __forceinline__ void accumulate(frag a, frag b, acc_t& c) {
-        asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
-    }
 };
-// Enough independent cycles after the last accumulate() for its result to be readable by any instruction.
-__device__ __forceinline__ void drain_accumulators() { asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); }
 
 struct Params {
     void* out0;  // forward: O      | dq: dQ | dkv: dK
@@ -1336,7 +1324,6 @@ __global__ __launch_bounds__(kThreads, 1) void attention_dkv_wide_kernel(Params 
                                                      next_tile(tile + 1));
             }
         }
-        drain_accumulators();
         __syncthreads();  // the next key block's first loads overwrite stage 0
         if (k_live) {
             T* dk_out = static_cast<T*>(p.out0) + k_offset;

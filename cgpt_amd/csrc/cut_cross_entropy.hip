@@ -68,10 +68,13 @@ extern "C" int cgptx_cut_cross_entropy_forward_backward(float* loss, void* input
     // the three contractions enough 256x256 tiles to fill the chip. The rows are split evenly over the chunks.
     // 32768 rows at V=32000 are one chunk: the classifier gradient then comes straight out of its contraction,
     // rounded once, without the fp32 accumulator and the pass that folds it into the gradient.
-    std::size_t logits_bytes = std::size_t{1} << 31;
+    // The bound itself stays 1 MiB under 2^31: the streamed contraction kernels address an operand with 32-bit
+    // byte offsets below that, and a chunk beyond it would fall back to the plain kernels.
+    constexpr std::size_t kMaxLogitsBytes = (std::size_t{1} << 31) - (std::size_t{1} << 20);
+    std::size_t logits_bytes = kMaxLogitsBytes;
     if (const char* text = std::getenv("CGPTX_CUT_CE_LOGITS_BYTES")) {
         const unsigned long long asked = std::strtoull(text, nullptr, 0);
-        if (asked > 0) logits_bytes = static_cast<std::size_t>(asked);
+        if (asked > 0) logits_bytes = std::min<std::size_t>(static_cast<std::size_t>(asked), kMaxLogitsBytes);
     }
     std::size_t limit = logits_bytes / (vocab * elem);
     limit = std::max<std::size_t>(256, limit / 256 * 256);

@@ -184,41 +184,64 @@ __device__ __forceinline__ float sigmoid_f32(float x) { return 1.0f / (1.0f + __
 
 // Packed: row-major [rows, 2*hidden] with gate in the first half of each row.
 // Separate layout is the special case handled by passing distinct pointers.
+// A workgroup takes tiles of kSwigluUnroll x 256 consecutive vectors: a thread requests its kSwigluUnroll
+// vectors of all three inputs (and of the old gradients when accumulating) before it computes anything, so that
+// twelve 128-bit loads per lane are in flight, and the position inside a packed row comes from 32-bit
+// arithmetic (a shift when a row holds a power-of-two number of vectors).
+constexpr int kSwigluUnroll = 4;
 template <typename T, bool AccGate, bool AccUp>
 __global__ __launch_bounds__(kThreads) void swiglu_backward_vec_kernel(
     T* grad_gate, T* grad_up, const T* __restrict__ grad_output, const T* __restrict__ gate,
-    const T* __restrict__ up, std::size_t vectors, std::size_t row_vectors, std::size_t packed_row_stride) {
+    const T* __restrict__ up, std::size_t vectors, unsigned int row_vectors, int row_shift,
+    std::size_t packed_row_stride) {
     // packed_row_stride == 0: flat separate tensors. Otherwise gate/up/grad_* are
-    // views into [rows, 2*hidden] and index = row * stride + col.
+    // views into [rows, 2*hidden] and index = row * stride + col. row_shift >= 0: row_vectors == 1 << row_shift.
     constexpr int VEC = kVec128<T>;
-    for (std::size_t v = static_cast<std::size_t>(blockIdx.x) * kThreads + threadIdx.x; v < vectors;
-         v += static_cast<std::size_t>(gridDim.x) * kThreads) {
-        const std::size_t flat = v * VEC;
-        std::size_t index = flat;
-        if (packed_row_stride != 0) {
-            const std::size_t row = v / row_vectors;
-            index = row * packed_row_stride + (v - row * row_vectors) * VEC;
-        }
-        const vec_t<float, VEC> dy = vec_to_f32<T, VEC>(load_vec<T, VEC>(grad_output + flat));
-        const vec_t<float, VEC> g = vec_to_f32<T, VEC>(load_vec<T, VEC>(gate + index));
-        const vec_t<float, VEC> u = vec_to_f32<T, VEC>(load_vec<T, VEC>(up + index));
-        vec_t<float, VEC> dg, du;
+    constexpr std::size_t kTile = static_cast<std::size_t>(kThreads) * kSwigluUnroll;
+    for (std::size_t base = static_cast<std::size_t>(blockIdx.x) * kTile; base < vectors;
+         base += static_cast<std::size_t>(gridDim.x) * kTile) {
+        vec_t<T, VEC> dy_raw[kSwigluUnroll], g_raw[kSwigluUnroll], u_raw[kSwigluUnroll], og_raw[kSwigluUnroll],
+            ou_raw[kSwigluUnroll];
+        std::size_t index[kSwigluUnroll];
+        bool live[kSwigluUnroll];
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) {
-            const float s = sigmoid_f32(g[e]);
-            dg[e] = dy[e] * u[e] * (s * (1.0f + g[e] * (1.0f - s)));
-            du[e] = dy[e] * (g[e] * s);
+        for (int k = 0; k < kSwigluUnroll; ++k) {
+            const std::size_t v = base + static_cast<std::size_t>(k) * kThreads + threadIdx.x;
+            live[k] = v < vectors;
+            index[k] = v * VEC;
+            if (packed_row_stride != 0) {
+                std::size_t row;
+                if (row_shift >= 0) row = v >> row_shift;
+                else if (vectors <= 0xFFFFFFFFull) row = static_cast<unsigned int>(v) / row_vectors;
+                else row = v / row_vectors;
+                index[k] = row * packed_row_stride + (v - row * row_vectors) * VEC;
+            }
+            if (live[k]) {
+                dy_raw[k] = load_vec<T, VEC>(grad_output + v * VEC);
+                g_raw[k] = load_vec<T, VEC>(gate + index[k]);
+                u_raw[k] = load_vec<T, VEC>(up + index[k]);
+                if constexpr (AccGate) og_raw[k] = load_vec<T, VEC>(grad_gate + index[k]);
+                if constexpr (AccUp) ou_raw[k] = load_vec<T, VEC>(grad_up + index[k]);
+            }
         }
-        if constexpr (AccGate) {
-            const vec_t<float, VEC> old = vec_to_f32<T, VEC>(load_vec<T, VEC>(grad_gate + index));
-            dg += old;
+#pragma unroll
+        for (int k = 0; k < kSwigluUnroll; ++k) {
+            if (!live[k]) continue;
+            const vec_t<float, VEC> dy = vec_to_f32<T, VEC>(dy_raw[k]);
+            const vec_t<float, VEC> g = vec_to_f32<T, VEC>(g_raw[k]);
+            const vec_t<float, VEC> u = vec_to_f32<T, VEC>(u_raw[k]);
+            vec_t<float, VEC> dg, du;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                const float s = sigmoid_f32(g[e]);
+                dg[e] = dy[e] * u[e] * (s * (1.0f + g[e] * (1.0f - s)));
+                du[e] = dy[e] * (g[e] * s);
+            }
+            if constexpr (AccGate) dg += vec_to_f32<T, VEC>(og_raw[k]);
+            if constexpr (AccUp) du += vec_to_f32<T, VEC>(ou_raw[k]);
+            store_vec<T, VEC>(grad_gate + index[k], vec_from_f32<T, VEC>(dg));
+            store_vec<T, VEC>(grad_up + index[k], vec_from_f32<T, VEC>(du));
         }
-        if constexpr (AccUp) {
-            const vec_t<float, VEC> old = vec_to_f32<T, VEC>(load_vec<T, VEC>(grad_up + index));
-            du += old;
-        }
-        store_vec<T, VEC>(grad_gate + index, vec_from_f32<T, VEC>(dg));
-        store_vec<T, VEC>(grad_up + index, vec_from_f32<T, VEC>(du));
     }
 }
 
@@ -316,12 +339,17 @@ int launch_swiglu_backward(T* grad_gate, T* grad_up, const T* grad_output, const
         return CGPTX_OK;
     }
     const std::size_t vectors = count / VEC;
-    const std::size_t row_vectors = row_elems / VEC;
-    const dim3 grid(grid_for(vectors)), block(kThreads);
+    if (packed_row_stride != 0 && row_elems / VEC > 0xFFFFFFFFull)
+        return fail(CGPTX_OVERFLOW, "swiglu_backward: row length exceeds uint32_t range");
+    const auto row_vectors = packed_row_stride != 0 ? static_cast<unsigned int>(row_elems / VEC) : 0u;
+    int row_shift = -1;
+    if (row_vectors != 0 && (row_vectors & (row_vectors - 1)) == 0) row_shift = __builtin_ctz(row_vectors);
+    // One tile per workgroup and pass; the grid is capped like the other streaming kernels'.
+    const dim3 grid(grid_for((vectors + kSwigluUnroll - 1) / kSwigluUnroll)), block(kThreads);
 #define CGPTX_SWIGLU_CASE(G, U)                                                                               \
     if (acc_gate == G && acc_up == U)                                                                         \
         hipLaunchKernelGGL((swiglu_backward_vec_kernel<T, G, U>), grid, block, 0, stream, grad_gate, grad_up, \
-                           grad_output, gate, up, vectors, row_vectors, packed_row_stride);
+                           grad_output, gate, up, vectors, row_vectors, row_shift, packed_row_stride);
     CGPTX_SWIGLU_CASE(false, false)
     CGPTX_SWIGLU_CASE(true, false)
     CGPTX_SWIGLU_CASE(false, true)

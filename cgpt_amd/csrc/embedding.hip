@@ -2,19 +2,17 @@
 //
 // Backward semantics: include/ops/backward/embedding_backward.h:35-42. The
 // reference scatters with storage-dtype atomics (src/ops/backward/embedding_backward.cu:68-92),
-// so its rounding depends on arrival order. Here the token list is stably sorted
-// by id (integer work, order-independent), then one wavefront per distinct id
-// walks that id's tokens in ascending token order and adds their rows with one
-// rounding to the storage dtype per add — the arithmetic of the reference's CPU
-// operator (src/ops/cpu/backward/embedding_backward_cpu.cpp:99-112). The result is
-// deterministic and no float atomics are used. Lanes cover the hidden dimension
-// with 128-bit accesses, so each token row is read once, fully coalesced.
+// so its rounding depends on arrival order. Here the tokens are grouped by id with a counting
+// sort over the vocabulary (integer work: histogram, scan, fill — one launch), then one wavefront
+// per vocabulary row adds that row's tokens in ascending token order with one rounding to the
+// storage dtype per add — the arithmetic of the reference's CPU operator
+// (src/ops/cpu/backward/embedding_backward_cpu.cpp:99-112). The result is deterministic and no
+// float atomics are used. Lanes cover the hidden dimension with 128-bit accesses, so each token
+// row is read once, fully coalesced; rows that no token names are zero-filled by the same launch
+// when the gradient is not accumulated.
 #include "common.hpp"
 
 #include <cstring>
-
-#include <rocprim/device/device_radix_sort.hpp>
-
 #include <limits>
 
 namespace cgptx {
@@ -23,116 +21,144 @@ namespace {
 constexpr int kThreads = 256;
 constexpr int kWavesPerBlock = kThreads / kWave;
 
-__global__ __launch_bounds__(kThreads) void embedding_keys_kernel(unsigned int* __restrict__ keys,
-                                                                 unsigned int* __restrict__ values,
+// ---- grouping: counting sort of the token positions by id -------------------------------------------
+// Workgroup b owns the ids [b R, (b+1) R) and reads the whole id list twice: first it counts its ids in an
+// LDS histogram and, on the side, the tokens with smaller ids (which is where its part of the output begins:
+// no workgroup waits for another); after an exclusive scan of the histogram it hands every token of its range
+// the next free slot of its id's segment. Slots are handed out with LDS integer atomics, so the order inside a
+// segment is whatever order the lanes arrived in: the row kernel puts each segment into ascending order itself.
+// offsets[id] .. offsets[id + 1] is id's segment of `order`; ids >= vocab belong to nobody and are skipped.
+constexpr int kGroupThreads = 1024;
+constexpr unsigned int kGroupMaxIds = 32768;  // LDS histogram entries of one workgroup (128 KiB)
+
+__global__ __launch_bounds__(kGroupThreads) void embedding_group_kernel(unsigned int* __restrict__ offsets,
+                                                                       unsigned int* __restrict__ order,
+                                                                       const std::uint32_t* __restrict__ ids,
+                                                                       unsigned int count, unsigned int vocab,
+                                                                       unsigned int ids_per_group) {
+    extern __shared__ unsigned int bins[];  // [ids_per_group]
+    __shared__ unsigned int wave_totals[kGroupThreads / kWave];
+    __shared__ unsigned int smaller_total;
+    const unsigned int lo = blockIdx.x * ids_per_group;
+    const unsigned int width = min(ids_per_group, vocab - lo);
+    const unsigned int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    for (unsigned int i = tid; i < width; i += kGroupThreads) bins[i] = 0;
+    if (tid == 0) smaller_total = 0;
+    __syncthreads();
+    unsigned int smaller = 0;
+    for (unsigned int t = tid; t < count; t += kGroupThreads) {
+        const unsigned int id = ids[t];
+        if (id < lo) ++smaller;
+        else if (id - lo < width) atomicAdd(&bins[id - lo], 1u);
+    }
+#pragma unroll
+    for (int offset = kWave / 2; offset > 0; offset >>= 1) smaller += __shfl_xor(smaller, offset, kWave);
+    if (lane == 0 && smaller != 0) atomicAdd(&smaller_total, smaller);
+    __syncthreads();
+    // Exclusive scan of bins[0, width) in place, starting at the number of tokens with smaller ids: thread i
+    // owns the contiguous piece [i per, (i + 1) per).
+    const unsigned int per = (width + kGroupThreads - 1) / kGroupThreads;
+    const unsigned int first = min(tid * per, width), last = min(first + per, width);
+    unsigned int mine = 0;
+    for (unsigned int i = first; i < last; ++i) mine += bins[i];
+    unsigned int inclusive = mine;
+#pragma unroll
+    for (int offset = 1; offset < kWave; offset <<= 1) {
+        const unsigned int other = __shfl_up(inclusive, offset, kWave);
+        if (lane >= static_cast<unsigned int>(offset)) inclusive += other;
+    }
+    if (lane == kWave - 1) wave_totals[wave] = inclusive;
+    __syncthreads();
+    unsigned int before = smaller_total;
+    for (unsigned int w = 0; w < wave; ++w) before += wave_totals[w];
+    unsigned int running = before + inclusive - mine;
+    for (unsigned int i = first; i < last; ++i) {
+        const unsigned int n = bins[i];
+        bins[i] = running;
+        offsets[lo + i] = running;
+        running += n;
+    }
+    if (lo + width == vocab && tid == kGroupThreads - 1) offsets[vocab] = running;  // the piece that ends the last range
+    __syncthreads();
+    for (unsigned int t = tid; t < count; t += kGroupThreads) {
+        const unsigned int id = ids[t];
+        if (id >= lo && id - lo < width) order[atomicAdd(&bins[id - lo], 1u)] = t;
+    }
+}
+
+// ---- rows: one wavefront per vocabulary row -------------------------------------------------------
+// Adds, into row `id` of the table, the rows of grad_output of the tokens with that id, in ascending token
+// order with one rounding to the storage dtype per add. Segments of up to 64 tokens are ordered in registers
+// (lane i holds the token of rank i); longer ones are walked by scanning the id list itself, 64 tokens per
+// step, which yields them in ascending order by construction. Rows without tokens are zero-filled unless the
+// gradient is accumulated.
+template <typename T, bool Vector>
+__global__ __launch_bounds__(kThreads) void embedding_rows_kernel(T* __restrict__ grad_weight,
+                                                                 const T* __restrict__ grad_output,
                                                                  const std::uint32_t* __restrict__ ids,
-                                                                 unsigned int count, unsigned int vocab) {
-    const unsigned int t = blockIdx.x * kThreads + threadIdx.x;
-    if (t >= count) return;
-    const std::uint32_t id = ids[t];
-    keys[t] = id < vocab ? id : vocab;  // out-of-range ids sort to the end and are skipped
-    values[t] = t;
-}
-
-template <typename T>
-__global__ __launch_bounds__(kThreads) void fill_zero_kernel(T* __restrict__ out, std::size_t count, bool aligned) {
-    constexpr int VEC = kVec128<T>;
-    const std::size_t vectors = aligned ? count / VEC : 0;
-    for (std::size_t v = static_cast<std::size_t>(blockIdx.x) * kThreads + threadIdx.x; v < vectors;
-         v += static_cast<std::size_t>(gridDim.x) * kThreads)
-        store_vec<T, VEC>(out + v * VEC, vec_t<T, VEC>(0));
-    for (std::size_t i = vectors * VEC + static_cast<std::size_t>(blockIdx.x) * kThreads + threadIdx.x; i < count;
-         i += static_cast<std::size_t>(gridDim.x) * kThreads)
-        out[i] = from_f32<T>(0.0f);
-}
-
-// One wavefront per sorted position; only segment heads do work.
-template <typename T, bool Vector>
-__global__ __launch_bounds__(kThreads) void embedding_segment_kernel(T* __restrict__ grad_weight,
-                                                                    const T* __restrict__ grad_output,
-                                                                    const unsigned int* __restrict__ keys,
-                                                                    const unsigned int* __restrict__ tokens,
-                                                                    unsigned int count, unsigned int vocab,
-                                                                    unsigned int hidden, bool accumulate) {
+                                                                 const unsigned int* __restrict__ offsets,
+                                                                 const unsigned int* __restrict__ order,
+                                                                 unsigned int count, unsigned int vocab,
+                                                                 unsigned int hidden, bool accumulate) {
     constexpr int VEC = Vector ? kVec128<T> : 1;
+    using vec_f = vec_t<float, VEC>;
     const unsigned int lane = threadIdx.x & (kWave - 1);
-    const unsigned int position = blockIdx.x * kWavesPerBlock + threadIdx.x / kWave;
-    if (position >= count) return;
-    const unsigned int key = keys[position];
-    if (key >= vocab) return;
-    if (position > 0 && keys[position - 1] == key) return;
-    unsigned int end = position + 1;
-    while (end < count && keys[end] == key) ++end;
-    T* row = grad_weight + static_cast<std::size_t>(key) * hidden;
-    for (unsigned int col = lane * VEC; col < hidden; col += kWave * VEC) {
-        vec_t<float, VEC> acc;
-        if (accumulate) {
-            acc = vec_to_f32<T, VEC>(load_vec<T, VEC>(row + col));
-        } else {
-            acc = vec_t<float, VEC>(0.0f);
-        }
-        for (unsigned int j = position; j < end; ++j) {
-            const T* src = grad_output + static_cast<std::size_t>(tokens[j]) * hidden + col;
-            const vec_t<float, VEC> dy = vec_to_f32<T, VEC>(load_vec<T, VEC>(src));
-            // one rounding to the storage dtype per add
-            acc = vec_to_f32<T, VEC>(vec_from_f32<T, VEC>(acc + dy));
-        }
-        store_vec<T, VEC>(row + col, vec_from_f32<T, VEC>(acc));
-    }
-}
-
-// Short token lists (up to kDirectTokens) skip the sort: one wavefront per token compares its id with all the
-// others. The first occurrence of an id owns the row and adds the later occurrences in ascending token order —
-// the segment kernel's arithmetic, in one launch instead of six. Lane c keeps the 64-bit match mask of tokens
-// 64 c .. 64 c + 63.
-constexpr unsigned int kDirectTokens = 4096;
-template <typename T, bool Vector>
-__global__ __launch_bounds__(kThreads) void embedding_direct_kernel(T* __restrict__ grad_weight,
-                                                                   const T* __restrict__ grad_output,
-                                                                   const std::uint32_t* __restrict__ ids,
-                                                                   unsigned int count, unsigned int vocab,
-                                                                   unsigned int hidden, bool accumulate) {
-    constexpr int VEC = Vector ? kVec128<T> : 1;
-    const unsigned int lane = threadIdx.x & (kWave - 1);
-    const unsigned int token = blockIdx.x * kWavesPerBlock + threadIdx.x / kWave;
-    if (token >= count) return;
-    const std::uint32_t id = ids[token];
+    const unsigned int id = blockIdx.x * kWavesPerBlock + threadIdx.x / kWave;
     if (id >= vocab) return;
-    for (unsigned int first = 0; first < token; first += kWave) {
-        const unsigned int j = first + lane;
-        if (__ballot(j < token && ids[j] == id) != 0) return;  // an earlier token owns this row
-    }
-    const unsigned int chunks = (count + kWave - 1) / kWave, own_chunk = token / kWave;
-    unsigned long long later = 0;
-    for (unsigned int c = own_chunk; c < chunks; ++c) {
-        const unsigned int j = c * kWave + lane;
-        const unsigned long long mask = __ballot(j > token && j < count && ids[j] == id);
-        if (lane == c) later = mask;
-    }
+    const unsigned int begin = offsets[id], tokens = offsets[id + 1] - begin;
     T* row = grad_weight + static_cast<std::size_t>(id) * hidden;
-    for (unsigned int col = lane * VEC; col < hidden; col += kWave * VEC) {
-        vec_t<float, VEC> acc;
-        if (accumulate) {
-            acc = vec_to_f32<T, VEC>(load_vec<T, VEC>(row + col));
-        } else {
-            acc = vec_t<float, VEC>(0.0f);
+    if (tokens == 0) {
+        if (!accumulate)
+            for (unsigned int col = lane * VEC; col < hidden; col += kWave * VEC) store_vec<T, VEC>(row + col, vec_t<T, VEC>(0));
+        return;
+    }
+    auto add_row = [&](vec_f acc, unsigned int token, unsigned int col) {
+        const vec_f dy = vec_to_f32<T, VEC>(load_vec<T, VEC>(grad_output + static_cast<std::size_t>(token) * hidden + col));
+        return vec_to_f32<T, VEC>(vec_from_f32<T, VEC>(acc + dy));  // one rounding to the storage dtype per add
+    };
+    if (tokens <= kWave) {
+        const unsigned int mine = lane < tokens ? order[begin + lane] : 0xFFFFFFFFu;
+        // rank = number of tokens of the segment below mine; sorted = the token of rank `lane`.
+        unsigned int rank = 0;
+        for (unsigned int j = 0; j < tokens; ++j)
+            rank += static_cast<unsigned int>(__builtin_amdgcn_readlane(static_cast<int>(mine), static_cast<int>(j))) < mine ? 1u : 0u;
+        const unsigned int sorted = static_cast<unsigned int>(
+            __builtin_amdgcn_ds_permute(static_cast<int>(rank << 2), static_cast<int>(mine)));  // lane `rank` receives mine
+        for (unsigned int col = lane * VEC; col < hidden; col += kWave * VEC) {
+            vec_f acc = accumulate ? vec_to_f32<T, VEC>(load_vec<T, VEC>(row + col)) : vec_f(0.0f);
+            // Four token rows are requested at a time; the additions keep their order.
+            for (unsigned int j0 = 0; j0 < tokens; j0 += 4) {
+                vec_t<T, VEC> dy[4];
+#pragma unroll
+                for (unsigned int u = 0; u < 4; ++u)
+                    if (j0 + u < tokens) {
+                        const auto token = static_cast<unsigned int>(
+                            __builtin_amdgcn_readlane(static_cast<int>(sorted), static_cast<int>(j0 + u)));
+                        dy[u] = load_vec<T, VEC>(grad_output + static_cast<std::size_t>(token) * hidden + col);
+                    }
+#pragma unroll
+                for (unsigned int u = 0; u < 4; ++u)
+                    if (j0 + u < tokens)  // one rounding to the storage dtype per add
+                        acc = vec_to_f32<T, VEC>(vec_from_f32<T, VEC>(acc + vec_to_f32<T, VEC>(dy[u])));
+            }
+            store_vec<T, VEC>(row + col, vec_from_f32<T, VEC>(acc));
         }
-        const vec_t<float, VEC> own = vec_to_f32<T, VEC>(load_vec<T, VEC>(grad_output + static_cast<std::size_t>(token) * hidden + col));
-        acc = vec_to_f32<T, VEC>(vec_from_f32<T, VEC>(acc + own));  // one rounding to the storage dtype per add
-        for (unsigned int c = own_chunk; c < chunks; ++c) {
-            // v_readlane reads any lane, active or not (the lanes past the row's width are inactive here).
-            const int holder = __builtin_amdgcn_readfirstlane(static_cast<int>(c));
-            unsigned long long mask =
-                static_cast<unsigned long long>(static_cast<unsigned int>(__builtin_amdgcn_readlane(static_cast<int>(later), holder))) |
-                (static_cast<unsigned long long>(static_cast<unsigned int>(__builtin_amdgcn_readlane(static_cast<int>(later >> 32), holder))) << 32);
-            while (mask != 0) {
-                const unsigned int j = c * kWave + static_cast<unsigned int>(__builtin_ctzll(mask));
-                mask &= mask - 1;
-                const vec_t<float, VEC> dy = vec_to_f32<T, VEC>(load_vec<T, VEC>(grad_output + static_cast<std::size_t>(j) * hidden + col));
-                acc = vec_to_f32<T, VEC>(vec_from_f32<T, VEC>(acc + dy));
+        return;
+    }
+    for (unsigned int col0 = 0; col0 < hidden; col0 += kWave * VEC) {
+        const unsigned int col = col0 + lane * VEC;
+        const bool live = col < hidden;
+        vec_f acc = (accumulate && live) ? vec_to_f32<T, VEC>(load_vec<T, VEC>(row + col)) : vec_f(0.0f);
+        for (unsigned int first = 0; first < count; first += kWave) {
+            const unsigned int t = first + lane;
+            unsigned long long matches = __ballot(t < count && ids[t] == id);  // every lane takes part
+            while (matches != 0) {
+                const unsigned int token = first + static_cast<unsigned int>(__builtin_ctzll(matches));
+                matches &= matches - 1;
+                if (live) acc = add_row(acc, token, col);
             }
         }
-        store_vec<T, VEC>(row + col, vec_from_f32<T, VEC>(acc));
+        if (live) store_vec<T, VEC>(row + col, vec_from_f32<T, VEC>(acc));
     }
 }
 
@@ -157,12 +183,6 @@ __global__ __launch_bounds__(kThreads) void embedding_gather_kernel(T* __restric
     }
 }
 
-int bits_for(unsigned int max_value) {
-    int bits = 1;
-    while (bits < 32 && (max_value >> bits) != 0) ++bits;
-    return bits;
-}
-
 }  // namespace
 }  // namespace cgptx
 
@@ -182,61 +202,43 @@ extern "C" int cgptx_embedding_backward(void* grad_weight, const void* grad_outp
     auto stream = static_cast<hipStream_t>(stream_);
     const auto count = static_cast<unsigned int>(token_count);
     const auto v = static_cast<unsigned int>(vocab);
-    const int end_bit = bits_for(v);
 
-    const bool direct = token_count <= kDirectTokens;
-    unsigned int* keys_out = nullptr;
-    unsigned int* values_out = nullptr;
-    if (!direct) {
-        // Scratch: keys_in | keys_out | values_in | values_out | rocPRIM temporary storage.
-        const std::size_t array_bytes = (token_count * sizeof(unsigned int) + 255) & ~std::size_t{255};
-        std::size_t temp_bytes = 0;
-        CGPTX_HIP(rocprim::radix_sort_pairs(nullptr, temp_bytes, static_cast<unsigned int*>(nullptr),
-                                            static_cast<unsigned int*>(nullptr), static_cast<unsigned int*>(nullptr),
-                                            static_cast<unsigned int*>(nullptr), token_count, 0, end_bit, stream));
-        void* mem = nullptr;
-        if (int s = scratch(stream, 4 * array_bytes + temp_bytes + 256, &mem)) return s;
-        auto* base = static_cast<char*>(mem);
-        auto* keys_in = reinterpret_cast<unsigned int*>(base);
-        keys_out = reinterpret_cast<unsigned int*>(base + array_bytes);
-        auto* values_in = reinterpret_cast<unsigned int*>(base + 2 * array_bytes);
-        values_out = reinterpret_cast<unsigned int*>(base + 3 * array_bytes);
-        void* temp = base + 4 * array_bytes;
-
-        hipLaunchKernelGGL(embedding_keys_kernel, dim3((count + kThreads - 1) / kThreads), dim3(kThreads), 0, stream,
-                           keys_in, values_in, token_ids, count, v);
-        CGPTX_LAUNCH_CHECK();
-        CGPTX_HIP(rocprim::radix_sort_pairs(temp, temp_bytes, keys_in, keys_out, values_in, values_out, token_count, 0,
-                                            end_bit, stream));
+    // Scratch: offsets[vocab + 1] | order[token_count].
+    const std::size_t offsets_bytes = ((vocab + 1) * sizeof(unsigned int) + 255) & ~std::size_t{255};
+    void* mem = nullptr;
+    if (int s = scratch(stream, offsets_bytes + token_count * sizeof(unsigned int), &mem)) return s;
+    auto* offsets = static_cast<unsigned int*>(mem);
+    auto* order = reinterpret_cast<unsigned int*>(static_cast<char*>(mem) + offsets_bytes);
+    // Ranges of at least 1024 ids, at most one workgroup per compute unit, each histogram within the LDS.
+    unsigned int ids_per_group = 1024;
+    const unsigned int units = static_cast<unsigned int>(compute_units());
+    while (ids_per_group < kGroupMaxIds && (v + ids_per_group - 1) / ids_per_group > units) ids_per_group *= 2;
+    const unsigned int groups = (v + ids_per_group - 1) / ids_per_group;
+    const std::size_t group_lds = ids_per_group * sizeof(unsigned int);
+    {
+        static bool configured = false;
+        if (!configured) {
+            CGPTX_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(embedding_group_kernel),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize,
+                                          static_cast<int>(kGroupMaxIds * sizeof(unsigned int))));
+            configured = true;
+        }
     }
+    hipLaunchKernelGGL(embedding_group_kernel, dim3(groups), dim3(kGroupThreads), group_lds, stream, offsets, order, token_ids,
+                       count, v, ids_per_group);
+    CGPTX_LAUNCH_CHECK();
     return dispatch_dtype(dtype, [&]<typename T>() -> int {
         auto* dw = static_cast<T*>(grad_weight);
         auto* dy = static_cast<const T*>(grad_output);
         const bool vector_ok = hidden % kVec128<T> == 0 && is_aligned16(dw) && is_aligned16(dy);
-        if (!accumulate_weight) {
-            const std::size_t total = vocab * hidden;
-            const std::size_t blocks = (total / kVec128<T> + kThreads) / kThreads;
-            const std::size_t cap = static_cast<std::size_t>(compute_units()) * 16;
-            hipLaunchKernelGGL((fill_zero_kernel<T>), dim3(static_cast<unsigned int>(blocks < cap ? blocks : cap)),
-                               dim3(kThreads), 0, stream, dw, total, is_aligned16(dw));
-            CGPTX_LAUNCH_CHECK();
-        }
-        const dim3 grid((count + kWavesPerBlock - 1) / kWavesPerBlock);
+        const dim3 grid((v + kWavesPerBlock - 1) / kWavesPerBlock);
         const auto h = static_cast<unsigned int>(hidden);
-        if (direct) {
-            if (vector_ok) {
-                hipLaunchKernelGGL((embedding_direct_kernel<T, true>), grid, dim3(kThreads), 0, stream, dw, dy, token_ids,
-                                   count, v, h, accumulate_weight != 0);
-            } else {
-                hipLaunchKernelGGL((embedding_direct_kernel<T, false>), grid, dim3(kThreads), 0, stream, dw, dy, token_ids,
-                                   count, v, h, accumulate_weight != 0);
-            }
-        } else if (vector_ok) {
-            hipLaunchKernelGGL((embedding_segment_kernel<T, true>), grid, dim3(kThreads), 0, stream, dw, dy, keys_out,
-                               values_out, count, v, h, accumulate_weight != 0);
+        if (vector_ok) {
+            hipLaunchKernelGGL((embedding_rows_kernel<T, true>), grid, dim3(kThreads), 0, stream, dw, dy, token_ids, offsets,
+                               order, count, v, h, accumulate_weight != 0);
         } else {
-            hipLaunchKernelGGL((embedding_segment_kernel<T, false>), grid, dim3(kThreads), 0, stream, dw, dy,
-                               keys_out, values_out, count, v, h, accumulate_weight != 0);
+            hipLaunchKernelGGL((embedding_rows_kernel<T, false>), grid, dim3(kThreads), 0, stream, dw, dy, token_ids, offsets,
+                               order, count, v, h, accumulate_weight != 0);
         }
         CGPTX_LAUNCH_CHECK();
         return CGPTX_OK;

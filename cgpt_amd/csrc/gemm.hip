@@ -522,6 +522,7 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
         }
     };
     constexpr int kTileLoads = ATile::kLoads + BTile::kLoads;  // per wavefront and K tile
+    static_assert(kTileLoads % 2 == 0, "a K tile's loads are dealt out in two equal halves, and the vmcnt waits count both");
     const unsigned int lds_wave = lds_address_of(smem) + wave * kLoadBytes;
     TileCursor ca, cb;
     // Requests K tiles FIRST .. LAST-1 of the opened item into the stages of the same numbers.

@@ -17,6 +17,7 @@
 #include "common.hpp"
 #include "gemm.hpp"
 
+#include <charconv>
 #include <cmath>
 #include <cstdlib>
 #include <cstring>
@@ -129,6 +130,9 @@ struct cgptx_model {
     };
     bool profiling = false;
     std::vector<Timed> timed;
+    // optional table of the operator calls the reference call sequence makes (cgptx_model_record_calls)
+    bool recording_calls = false;
+    std::vector<cgptx_call_record> calls;
     std::vector<std::pair<std::string, float>> profile;  // label, milliseconds (summed per label)
 };
 
@@ -428,60 +432,108 @@ bool reference_call_sequence() {
     return text != nullptr && text[0] == '0';
 }
 
+// Adds one row to the model's call table (while cgptx_model_record_calls is on): the operator's name in
+// include/ops/**, its tensors in the operator's argument order, its sizes and flags in the order of the C-ABI
+// entry point, and its scalar (epsilon, attention scale or gradient scale).
+void note_call(cgptx_model* m, const char* op, std::initializer_list<const void*> tensors,
+               std::initializer_list<std::size_t> dims, std::initializer_list<int> flags = {}, float scalar = 0.0f) {
+    if (!m->recording_calls) return;
+    cgptx_call_record r{};
+    r.op = op;
+    std::size_t i = 0;
+    for (const void* t : tensors) r.tensors[i++] = t;
+    i = 0;
+    for (std::size_t d : dims) r.dims[i++] = d;
+    i = 0;
+    for (int f : flags) r.flags[i++] = f;
+    r.scalar = scalar;
+    r.dtype = m->config.dtype;
+    m->calls.push_back(r);
+}
+
 int enqueue_reference_sequence(cgptx_model* m, float loss_scale, int loss_mode, hipStream_t stream) {
     const auto& c = m->config;
     const int dt = c.dtype;
-    const std::size_t N = m->rows, H = c.hidden_size, I = c.intermediate_size;
-    const std::size_t HQ = c.num_query_heads, HKV = c.num_kv_heads, D = c.head_dim;
+    const std::size_t N = m->rows, H = c.hidden_size, I = c.intermediate_size, V = c.vocabulary_size;
+    const std::size_t HQ = c.num_query_heads, HKV = c.num_kv_heads, D = c.head_dim, B = m->batch, T = m->sequence;
     const std::size_t QW = HQ * D, KW = HKV * D, elem = dtype_size(dt);
     const float eps = c.rms_epsilon;
     auto* s = static_cast<cgptx_stream>(stream);
     auto second_half = [&](void* gate_up) { return static_cast<void*>(static_cast<char*>(gate_up) + N * I * elem); };
+    m->calls.clear();
 
-    CGPTX_OP("embedding_fwd", cgptx_embedding_forward(m->hidden[0], m->tokens, N, m->embedding.value, c.vocabulary_size, H, dt, s));
+    // One public operator per call; each is entered in the call table before it is enqueued.
+    auto norm_fwd = [&](void* out, const void* in, const void* w, std::size_t rows, std::size_t width) -> int {
+        note_call(m, "rmsnorm_forward", {out, in, w}, {rows, width}, {}, eps);
+        CGPTX_OP("rmsnorm_fwd", cgptx_rmsnorm_forward(out, in, w, rows, width, eps, dt, s));
+        return CGPTX_OK;
+    };
+    auto norm_bwd = [&](void* dx, void* dw, const void* dy, const void* x, const void* w, std::size_t rows, std::size_t width) -> int {
+        note_call(m, "rmsnorm_backward", {dx, dw, dy, x, w}, {rows, width}, {}, eps);
+        CGPTX_OP("rmsnorm_bwd", cgptx_rmsnorm_backward(dx, dw, dy, x, w, rows, width, eps, dt, s));
+        return CGPTX_OK;
+    };
+    auto project = [&](const char* label, void* out, const void* in, const void* w, std::size_t in_features, std::size_t out_features) -> int {
+        note_call(m, "linear_forward", {out, in, w}, {N, in_features, out_features});
+        CGPTX_OP(label, cgptx_linear_forward(out, in, w, nullptr, N, in_features, out_features, dt, s));
+        return CGPTX_OK;
+    };
+    auto project_bwd = [&](const char* dx_label, const char* dw_label, void* dx, void* dw, const void* dy, const void* x, const void* w,
+                           std::size_t in_features, std::size_t out_features, int accumulate_input) -> int {
+        note_call(m, "linear_backward", {dx, dw, dy, x, w}, {N, in_features, out_features}, {accumulate_input});
+        return linear_backward_split(m, dx, dw, dy, x, w, N, in_features, out_features, accumulate_input, dt, stream, dx_label, dw_label);
+    };
+    auto add = [&](void* out, const void* a, const void* b) -> int {
+        note_call(m, "add", {out, a, b}, {N * H});
+        CGPTX_OP("add", cgptx_add(out, a, b, N * H, dt, s));
+        return CGPTX_OK;
+    };
+
+    note_call(m, "embedding_forward", {m->hidden[0], m->tokens, m->embedding.value}, {N, V, H});
+    CGPTX_OP("embedding_fwd", cgptx_embedding_forward(m->hidden[0], m->tokens, N, m->embedding.value, V, H, dt, s));
     for (std::size_t l = 0; l < c.num_layers; ++l) {
         const auto& w = m->layers[l];
         const auto& a = m->acts[l];
         void *x = m->hidden[l], *out = m->hidden[l + 1];
         void *projected = m->d_norm_in, *ffn = m->d_norm_in_f;  // backward workspace, free during the forward pass
         void *gate = a.gate_up, *up = second_half(a.gate_up);
-        CGPTX_OP("rmsnorm_fwd", cgptx_rmsnorm_forward(a.norm_a, x, w.attention_norm.value, N, H, eps, dt, s));
-        CGPTX_OP("gemm_fwd.qkv", cgptx_linear_forward(a.q_pre, a.norm_a, w.q.value, nullptr, N, H, QW, dt, s));
-        CGPTX_OP("gemm_fwd.qkv", cgptx_linear_forward(a.k_pre, a.norm_a, w.k.value, nullptr, N, H, KW, dt, s));
-        CGPTX_OP("gemm_fwd.qkv", cgptx_linear_forward(a.v, a.norm_a, w.v.value, nullptr, N, H, KW, dt, s));
-        CGPTX_OP("rmsnorm_fwd", cgptx_rmsnorm_forward(a.q, a.q_pre, w.q_norm.value, N * HQ, D, eps, dt, s));
-        CGPTX_OP("rmsnorm_fwd", cgptx_rmsnorm_forward(a.k, a.k_pre, w.k_norm.value, N * HKV, D, eps, dt, s));
-        CGPTX_OP("rope_fwd", cgptx_rope_forward(a.q, a.k, m->cos_cache, m->sin_cache, m->batch, m->sequence, HQ, HKV, D,
-                                                c.rotary_dim, 0, m->sequence, dt, s));
-        CGPTX_OP("attn_fwd", cgptx_flash_gqa_attention_forward(a.attn_out, a.lse, a.q, a.k, a.v, m->batch, m->sequence,
-                                                               m->sequence, HQ, HKV, D, 0.0f, 1, 0, dt, s));
-        CGPTX_OP("gemm_fwd.o", cgptx_linear_forward(projected, a.attn_out, w.o.value, nullptr, N, QW, H, dt, s));
-        CGPTX_OP("rmsnorm_fwd", cgptx_rmsnorm_forward(a.norm_f, x, w.ffn_norm.value, N, H, eps, dt, s));
-        CGPTX_OP("gemm_fwd.gate_up", cgptx_linear_forward(gate, a.norm_f, w.gate.value, nullptr, N, H, I, dt, s));
-        CGPTX_OP("gemm_fwd.gate_up", cgptx_linear_forward(up, a.norm_f, w.up.value, nullptr, N, H, I, dt, s));
+        CGPTX_TRY(norm_fwd(a.norm_a, x, w.attention_norm.value, N, H));
+        CGPTX_TRY(project("gemm_fwd.qkv", a.q_pre, a.norm_a, w.q.value, H, QW));
+        CGPTX_TRY(project("gemm_fwd.qkv", a.k_pre, a.norm_a, w.k.value, H, KW));
+        CGPTX_TRY(project("gemm_fwd.qkv", a.v, a.norm_a, w.v.value, H, KW));
+        CGPTX_TRY(norm_fwd(a.q, a.q_pre, w.q_norm.value, N * HQ, D));
+        CGPTX_TRY(norm_fwd(a.k, a.k_pre, w.k_norm.value, N * HKV, D));
+        note_call(m, "rope_forward", {a.q, a.k, m->cos_cache, m->sin_cache}, {B, T, HQ, HKV, D, c.rotary_dim, 0, T});
+        CGPTX_OP("rope_fwd", cgptx_rope_forward(a.q, a.k, m->cos_cache, m->sin_cache, B, T, HQ, HKV, D, c.rotary_dim, 0, T, dt, s));
+        note_call(m, "flash_gqa_attention_forward_with_lse", {a.attn_out, a.lse, a.q, a.k, a.v}, {B, T, T, HQ, HKV, D, 0}, {1});
+        CGPTX_OP("attn_fwd", cgptx_flash_gqa_attention_forward(a.attn_out, a.lse, a.q, a.k, a.v, B, T, T, HQ, HKV, D, 0.0f, 1, 0, dt, s));
+        CGPTX_TRY(project("gemm_fwd.o", projected, a.attn_out, w.o.value, QW, H));
+        CGPTX_TRY(norm_fwd(a.norm_f, x, w.ffn_norm.value, N, H));
+        CGPTX_TRY(project("gemm_fwd.gate_up", gate, a.norm_f, w.gate.value, H, I));
+        CGPTX_TRY(project("gemm_fwd.gate_up", up, a.norm_f, w.up.value, H, I));
+        note_call(m, "swiglu_forward", {a.act, gate, up}, {N * I});
         CGPTX_OP("swiglu_fwd", cgptx_swiglu_forward(a.act, gate, up, N * I, dt, s));
-        CGPTX_OP("gemm_fwd.down", cgptx_linear_forward(ffn, a.act, w.down.value, nullptr, N, I, H, dt, s));
-        CGPTX_OP("add", cgptx_add(out, x, projected, N * H, dt, s));
-        CGPTX_OP("add", cgptx_add(out, out, ffn, N * H, dt, s));
+        CGPTX_TRY(project("gemm_fwd.down", ffn, a.act, w.down.value, I, H));
+        CGPTX_TRY(add(out, x, projected));
+        CGPTX_TRY(add(out, out, ffn));
     }
     void* last = m->hidden[c.num_layers];
-    CGPTX_OP("rmsnorm_fwd", cgptx_rmsnorm_forward(m->normalized, last, m->final_norm.value, N, H, eps, dt, s));
+    CGPTX_TRY(norm_fwd(m->normalized, last, m->final_norm.value, N, H));
     if (loss_mode == CGPTX_LOSS_CUT) {
+        note_call(m, "cut_cross_entropy_forward_backward", {m->loss, m->d_normalized, m->embedding.gradient, m->normalized,
+                                                            m->embedding.value, m->targets}, {N, H, V}, {}, loss_scale);
         CGPTX_OP("cut_ce", cgptx_cut_cross_entropy_forward_backward(m->loss, m->d_normalized, m->embedding.gradient, m->normalized,
-                                                                    m->embedding.value, m->targets, N, H, c.vocabulary_size,
-                                                                    loss_scale, 0, dt, s));
+                                                                    m->embedding.value, m->targets, N, H, V, loss_scale, 0, dt, s));
     } else {
-        CGPTX_OP("gemm_fwd.classifier", cgptx_linear_forward(m->logits, m->normalized, m->embedding.value, nullptr, N, H, c.vocabulary_size, dt, s));
-        CGPTX_OP("dense_ce", cgptx_cross_entropy_forward_backward(m->loss, m->grad_logits, m->logits, m->targets, N,
-                                                                  c.vocabulary_size, loss_scale, dt, s));
-        CGPTX_TRY(linear_backward_split(m, m->d_normalized, m->embedding.gradient, m->grad_logits, m->normalized,
-                                        m->embedding.value, N, H, c.vocabulary_size, 0, dt, stream, "gemm_dx.classifier",
-                                        "gemm_dw.classifier"));
+        CGPTX_TRY(project("gemm_fwd.classifier", m->logits, m->normalized, m->embedding.value, H, V));
+        note_call(m, "cross_entropy_forward_backward", {m->loss, m->grad_logits, m->logits, m->targets}, {N, V}, {}, loss_scale);
+        CGPTX_OP("dense_ce", cgptx_cross_entropy_forward_backward(m->loss, m->grad_logits, m->logits, m->targets, N, V, loss_scale, dt, s));
+        CGPTX_TRY(project_bwd("gemm_dx.classifier", "gemm_dw.classifier", m->d_normalized, m->embedding.gradient, m->grad_logits,
+                              m->normalized, m->embedding.value, H, V, 0));
     }
 
     void *current = m->grad_a, *previous = m->grad_b;
-    CGPTX_OP("rmsnorm_bwd", cgptx_rmsnorm_backward(current, m->final_norm.gradient, m->d_normalized, last, m->final_norm.value, N,
-                                                   H, eps, dt, s));
+    CGPTX_TRY(norm_bwd(current, m->final_norm.gradient, m->d_normalized, last, m->final_norm.value, N, H));
     for (std::size_t reverse = c.num_layers; reverse-- > 0;) {
         const auto& w = m->layers[reverse];
         const auto& a = m->acts[reverse];
@@ -489,32 +541,33 @@ int enqueue_reference_sequence(cgptx_model* m, float loss_scale, int loss_mode, 
         void *gate = a.gate_up, *up = second_half(a.gate_up);
         void *d_gate = m->d_gate_up, *d_up = second_half(m->d_gate_up);
         void* grad_residual = m->d_norm_in_f;
-        CGPTX_TRY(linear_backward_split(m, m->d_act, w.down.gradient, current, a.act, w.down.value, N, I, H, 0, dt, stream, "gemm_dx.down", "gemm_dw.down"));
+        CGPTX_TRY(project_bwd("gemm_dx.down", "gemm_dw.down", m->d_act, w.down.gradient, current, a.act, w.down.value, I, H, 0));
+        note_call(m, "swiglu_backward", {d_gate, d_up, m->d_act, gate, up}, {N * I}, {0, 0});
         CGPTX_OP("swiglu_bwd", cgptx_swiglu_backward(d_gate, d_up, m->d_act, gate, up, N * I, 0, 0, dt, s));
-        CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.gate.gradient, d_gate, a.norm_f, w.gate.value, N, H, I, 0, dt, stream, "gemm_dx.gate_up", "gemm_dw.gate_up"));
-        CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.up.gradient, d_up, a.norm_f, w.up.value, N, H, I, 1, dt, stream, "gemm_dx.gate_up", "gemm_dw.gate_up"));
-        CGPTX_OP("rmsnorm_bwd", cgptx_rmsnorm_backward(grad_residual, w.ffn_norm.gradient, m->d_norm_in, x, w.ffn_norm.value, N, H,
-                                                       eps, dt, s));
-        CGPTX_OP("add", cgptx_add(previous, current, grad_residual, N * H, dt, s));  // grad_input = grad_output + grad_residual
-        CGPTX_TRY(linear_backward_split(m, m->d_attn_out, w.o.gradient, current, a.attn_out, w.o.value, N, QW, H, 0, dt, stream, "gemm_dx.o", "gemm_dw.o"));
+        CGPTX_TRY(project_bwd("gemm_dx.gate_up", "gemm_dw.gate_up", m->d_norm_in, w.gate.gradient, d_gate, a.norm_f, w.gate.value, H, I, 0));
+        CGPTX_TRY(project_bwd("gemm_dx.gate_up", "gemm_dw.gate_up", m->d_norm_in, w.up.gradient, d_up, a.norm_f, w.up.value, H, I, 1));
+        CGPTX_TRY(norm_bwd(grad_residual, w.ffn_norm.gradient, m->d_norm_in, x, w.ffn_norm.value, N, H));
+        CGPTX_TRY(add(previous, current, grad_residual));  // grad_input = grad_output + grad_residual
+        CGPTX_TRY(project_bwd("gemm_dx.o", "gemm_dw.o", m->d_attn_out, w.o.gradient, current, a.attn_out, w.o.value, QW, H, 0));
+        note_call(m, "flash_gqa_attention_backward_with_lse", {m->d_q, m->d_k, m->d_v, m->d_attn_out, a.attn_out, a.lse, a.q, a.k, a.v},
+                  {B, T, T, HQ, HKV, D, 0}, {1, 0});
         CGPTX_OP("attn_bwd", cgptx_flash_gqa_attention_backward_with_lse(m->d_q, m->d_k, m->d_v, m->d_attn_out, a.attn_out, a.lse,
-                                                                         a.q, a.k, a.v, m->batch, m->sequence, m->sequence, HQ,
-                                                                         HKV, D, 0.0f, 1, 0, 0, dt, s));
-        CGPTX_OP("rope_bwd", cgptx_rope_backward(m->d_q_pre, m->d_k_pre, m->d_q, m->d_k, m->cos_cache, m->sin_cache, m->batch,
-                                                 m->sequence, HQ, HKV, D, c.rotary_dim, 0, m->sequence, dt, s));
-        CGPTX_OP("rmsnorm_bwd", cgptx_rmsnorm_backward(m->d_q, w.q_norm.gradient, m->d_q_pre, a.q_pre, w.q_norm.value, N * HQ, D,
-                                                       eps, dt, s));
-        CGPTX_OP("rmsnorm_bwd", cgptx_rmsnorm_backward(m->d_k, w.k_norm.gradient, m->d_k_pre, a.k_pre, w.k_norm.value, N * HKV, D,
-                                                       eps, dt, s));
-        CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.q.gradient, m->d_q, a.norm_a, w.q.value, N, H, QW, 0, dt, stream, "gemm_dx.qkv", "gemm_dw.qkv"));
-        CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.k.gradient, m->d_k, a.norm_a, w.k.value, N, H, KW, 1, dt, stream, "gemm_dx.qkv", "gemm_dw.qkv"));
-        CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.v.gradient, m->d_v, a.norm_a, w.v.value, N, H, KW, 1, dt, stream, "gemm_dx.qkv", "gemm_dw.qkv"));
-        CGPTX_OP("rmsnorm_bwd", cgptx_rmsnorm_backward(grad_residual, w.attention_norm.gradient, m->d_norm_in, x,
-                                                       w.attention_norm.value, N, H, eps, dt, s));
-        CGPTX_OP("add", cgptx_add(previous, previous, grad_residual, N * H, dt, s));
+                                                                         a.q, a.k, a.v, B, T, T, HQ, HKV, D, 0.0f, 1, 0, 0, dt, s));
+        note_call(m, "rope_backward", {m->d_q_pre, m->d_k_pre, m->d_q, m->d_k, m->cos_cache, m->sin_cache},
+                  {B, T, HQ, HKV, D, c.rotary_dim, 0, T});
+        CGPTX_OP("rope_bwd", cgptx_rope_backward(m->d_q_pre, m->d_k_pre, m->d_q, m->d_k, m->cos_cache, m->sin_cache, B, T, HQ, HKV, D,
+                                                 c.rotary_dim, 0, T, dt, s));
+        CGPTX_TRY(norm_bwd(m->d_q, w.q_norm.gradient, m->d_q_pre, a.q_pre, w.q_norm.value, N * HQ, D));
+        CGPTX_TRY(norm_bwd(m->d_k, w.k_norm.gradient, m->d_k_pre, a.k_pre, w.k_norm.value, N * HKV, D));
+        CGPTX_TRY(project_bwd("gemm_dx.qkv", "gemm_dw.qkv", m->d_norm_in, w.q.gradient, m->d_q, a.norm_a, w.q.value, H, QW, 0));
+        CGPTX_TRY(project_bwd("gemm_dx.qkv", "gemm_dw.qkv", m->d_norm_in, w.k.gradient, m->d_k, a.norm_a, w.k.value, H, KW, 1));
+        CGPTX_TRY(project_bwd("gemm_dx.qkv", "gemm_dw.qkv", m->d_norm_in, w.v.gradient, m->d_v, a.norm_a, w.v.value, H, KW, 1));
+        CGPTX_TRY(norm_bwd(grad_residual, w.attention_norm.gradient, m->d_norm_in, x, w.attention_norm.value, N, H));
+        CGPTX_TRY(add(previous, previous, grad_residual));
         std::swap(current, previous);
     }
-    CGPTX_OP("embedding_bwd", cgptx_embedding_backward(m->embedding.gradient, current, m->tokens, N, c.vocabulary_size, H, 1, 1, dt, s));
+    note_call(m, "embedding_backward", {m->embedding.gradient, current, m->tokens}, {N, V, H}, {1, 1});
+    CGPTX_OP("embedding_bwd", cgptx_embedding_backward(m->embedding.gradient, current, m->tokens, N, V, H, 1, 1, dt, s));
     return CGPTX_OK;
 }
 
@@ -923,6 +976,85 @@ extern "C" int cgptx_model_upload_tokens(cgptx_model* m, cgptx_token_upload* u, 
     return cgptx_token_upload_submit(u, m->tokens, m->targets, stream);
 }
 
+// ---- caller-owned batches: pinned and device blocks, one fence per host batch ----------------------
+struct cgptx_upload_fence {
+    hipEvent_t copied = nullptr;
+};
+
+extern "C" int cgptx_pinned_allocate(void** block, size_t bytes) {
+    using namespace cgptx;
+    clear_error();
+    if (block == nullptr) return fail(CGPTX_INVALID_ARGUMENT, "pinned_allocate: null argument");
+    *block = nullptr;
+    CGPTX_HIP(hipHostMalloc(block, std::max<std::size_t>(bytes, 1), hipHostMallocDefault));
+    return CGPTX_OK;
+}
+
+extern "C" int cgptx_pinned_release(void* block) {
+    using namespace cgptx;
+    clear_error();
+    if (block != nullptr) CGPTX_HIP(hipHostFree(block));
+    return CGPTX_OK;
+}
+
+extern "C" int cgptx_device_allocate(void** block, size_t bytes) {
+    using namespace cgptx;
+    clear_error();
+    if (block == nullptr || bytes == 0) return fail(CGPTX_INVALID_ARGUMENT, "device_allocate: null argument or no bytes");
+    *block = nullptr;
+    CGPTX_HIP(hipMalloc(block, bytes));
+    return CGPTX_OK;
+}
+
+extern "C" int cgptx_device_release(void* block) {
+    using namespace cgptx;
+    clear_error();
+    if (block != nullptr) CGPTX_HIP(hipFree(block));
+    return CGPTX_OK;
+}
+
+extern "C" int cgptx_upload_fence_wait(cgptx_upload_fence* fence) {
+    using namespace cgptx;
+    clear_error();
+    if (fence != nullptr) CGPTX_HIP(hipEventSynchronize(fence->copied));
+    return CGPTX_OK;
+}
+
+extern "C" int cgptx_upload_fence_destroy(cgptx_upload_fence* fence) {
+    if (fence == nullptr) return CGPTX_OK;
+    if (fence->copied != nullptr) (void)hipEventDestroy(fence->copied);
+    delete fence;
+    return CGPTX_OK;
+}
+
+extern "C" int cgptx_token_upload_async(uint32_t* device_inputs, uint32_t* device_targets, const uint32_t* inputs,
+                                        const uint32_t* targets, size_t count, cgptx_upload_fence** fence,
+                                        cgptx_stream stream_) {
+    using namespace cgptx;
+    clear_error();
+    if (fence == nullptr) return fail(CGPTX_INVALID_ARGUMENT, "token_upload_async: null fence slot");
+    if (count != 0 && (device_inputs == nullptr || device_targets == nullptr || inputs == nullptr || targets == nullptr))
+        return fail(CGPTX_INVALID_ARGUMENT, "token_upload_async: null buffer");
+    if (count > static_cast<std::size_t>(-1) / sizeof(std::uint32_t))
+        return fail(CGPTX_OVERFLOW, "token_upload_async: token count overflows");
+    auto stream = static_cast<hipStream_t>(stream_);
+    if (*fence == nullptr) {
+        auto* created = new cgptx_upload_fence();
+        if (int status = check_hip(hipEventCreateWithFlags(&created->copied, hipEventDisableTiming), "hipEventCreate")) {
+            delete created;
+            return status;
+        }
+        *fence = created;
+    }
+    const std::size_t bytes = count * sizeof(std::uint32_t);
+    if (bytes != 0) {
+        CGPTX_HIP(hipMemcpyAsync(device_inputs, inputs, bytes, hipMemcpyHostToDevice, stream));
+        CGPTX_HIP(hipMemcpyAsync(device_targets, targets, bytes, hipMemcpyHostToDevice, stream));
+    }
+    CGPTX_HIP(hipEventRecord((*fence)->copied, stream));
+    return CGPTX_OK;
+}
+
 extern "C" int cgptx_model_forward_backward(cgptx_model* m, float loss_scale, int loss_mode, int use_graph,
                                             cgptx_stream stream_) {
     using namespace cgptx;
@@ -1037,6 +1169,24 @@ extern "C" int cgptx_model_profile(cgptx_model* m, float loss_scale, int loss_mo
     return status;
 }
 
+extern "C" int cgptx_model_record_calls(cgptx_model* m, int enable) {
+    using namespace cgptx;
+    if (m == nullptr) return fail(CGPTX_INVALID_ARGUMENT, "model_record_calls: null model");
+    m->recording_calls = enable != 0;
+    if (!m->recording_calls) m->calls.clear();
+    return CGPTX_OK;
+}
+
+extern "C" size_t cgptx_model_call_count(const cgptx_model* m) { return m == nullptr ? 0 : m->calls.size(); }
+
+extern "C" int cgptx_model_call(const cgptx_model* m, size_t index, cgptx_call_record* record) {
+    using namespace cgptx;
+    if (m == nullptr || record == nullptr || index >= m->calls.size())
+        return fail(CGPTX_INVALID_ARGUMENT, "model_call: null argument or index out of range");
+    *record = m->calls[index];
+    return CGPTX_OK;
+}
+
 extern "C" size_t cgptx_model_profile_count(const cgptx_model* m) { return m == nullptr ? 0 : m->profile.size(); }
 
 extern "C" int cgptx_model_profile_entry(const cgptx_model* m, size_t index, const char** label, float* milliseconds) {
@@ -1121,9 +1271,16 @@ extern "C" int cgptx_model_activation(const cgptx_model* m, const char* name, vo
         *count = m->rows * m->config.vocabulary_size;
         return CGPTX_OK;
     }
+    // Decimal index at [first, last) of the name; anything else is no index.
+    auto index_at = [&](std::size_t first, std::size_t last, std::size_t* value) {
+        const char* begin = n.data() + first;
+        const char* end = n.data() + last;
+        const auto parsed = std::from_chars(begin, end, *value);
+        return first < last && parsed.ec == std::errc() && parsed.ptr == end;
+    };
     if (n.rfind("hidden.", 0) == 0) {
-        const std::size_t l = std::stoul(n.substr(7));
-        if (l < m->hidden.size()) { *data = m->hidden[l]; *count = NH; return CGPTX_OK; }
+        std::size_t l = 0;
+        if (index_at(7, n.size(), &l) && l < m->hidden.size()) { *data = m->hidden[l]; *count = NH; return CGPTX_OK; }
     }
     // Gradient of the loss with respect to hidden.0 / hidden.1 as the last backward pass left them (the two
     // residual-stream gradient buffers alternate per block, so only the first block's pair survives a step).
@@ -1138,7 +1295,8 @@ extern "C" int cgptx_model_activation(const cgptx_model* m, const char* name, vo
     if (n.rfind("layer.", 0) == 0) {
         const std::size_t dot = n.find('.', 6);
         if (dot != std::string::npos) {
-            const std::size_t l = std::stoul(n.substr(6, dot - 6));
+            std::size_t l = m->acts.size();
+            if (!index_at(6, dot, &l)) l = m->acts.size();
             const std::string what = n.substr(dot + 1);
             const auto& c = m->config;
             const std::size_t QW = m->rows * c.num_query_heads * c.head_dim, KW = m->rows * c.num_kv_heads * c.head_dim;

@@ -68,6 +68,29 @@ int cgptx_token_upload_submit(cgptx_token_upload* upload, uint32_t* device_input
  * upload's shape is not the model's ("Batch buffers do not match its declared shape"). */
 int cgptx_model_upload_tokens(cgptx_model* model, cgptx_token_upload* upload, cgptx_stream stream);
 
+/* The same upload for callers that own their batches (data::Batch / data::DeviceBatch,
+ * include/data/dataset_loader.h:111-170): page-locked host blocks for the token vectors
+ * (CudaHostAllocator::allocate / deallocate, include/data/dataset_loader.h:57-84; a request for 0 bytes
+ * gives a valid block), device blocks for the destination (DeviceBuffer::allocate / release,
+ * include/core/device_buffer.h:59-81), and the per-batch fence that says when the copies out of a host
+ * batch have finished (Batch::upload_complete_: mark_upload_complete / wait_until_reusable,
+ * src/data/dataset_loader.cpp:120-131). */
+int cgptx_pinned_allocate(void** block, size_t bytes);
+int cgptx_pinned_release(void* block);
+int cgptx_device_allocate(void** block, size_t bytes);
+int cgptx_device_release(void* block);
+typedef struct cgptx_upload_fence cgptx_upload_fence;
+/* Blocks the host until the copies recorded last on `fence` are done; a null fence has none. */
+int cgptx_upload_fence_wait(cgptx_upload_fence* fence);
+/* Does not wait; null is accepted. */
+int cgptx_upload_fence_destroy(cgptx_upload_fence* fence);
+/* data::upload_batch (src/data/dataset_loader.cpp:145-166) after its shape check: enqueues the copies of
+ * `count` input and `count` target ids from page-locked host memory to the device buffers on `stream`
+ * and records *fence behind them, creating the fence on first use. count == 0 only records. */
+int cgptx_token_upload_async(uint32_t* device_inputs, uint32_t* device_targets, const uint32_t* inputs,
+                             const uint32_t* targets, size_t count, cgptx_upload_fence** fence,
+                             cgptx_stream stream);
+
 /* Enqueues forward + loss + backward on `stream` (gradient of loss·loss_scale). With use_graph
  * the sequence is captured on first use (after one eager run) and replayed afterwards. */
 int cgptx_model_forward_backward(cgptx_model* model, float loss_scale, int loss_mode, int use_graph,
@@ -90,6 +113,27 @@ int cgptx_model_status(cgptx_model* model, float* loss, int* all_finite, uint64_
 int cgptx_model_profile(cgptx_model* model, float loss_scale, int loss_mode, cgptx_stream stream);
 size_t cgptx_model_profile_count(const cgptx_model* model);
 int cgptx_model_profile_entry(const cgptx_model* model, size_t index, const char** label, float* milliseconds);
+
+/* The operator calls of the step when it runs as the reference's own call sequence (environment
+ * CGPTX_FUSE=0: one public operator per call, forward in the order of src/core/transformer_block.cu:466-595,
+ * backward in the order of :663-747 and src/core/transformer_model.cu:360-380). While recording is on, every
+ * such step leaves the table of its calls: `op` is the operator's name in the headers under include/ops ("add" is the block's
+ * residual helper, src/core/transformer_block.cu:134-144), `tensors` its device tensors in the operator's
+ * argument order (outputs first; token ids and targets in their argument position), `dims` and `flags` its
+ * sizes and accumulate / causal / bounds-check switches in the order of the operator's C-ABI entry point,
+ * `scalar` its epsilon, attention scale or gradient scale. A caller written against those headers that walks
+ * the table reproduces the step's results bit for bit. */
+typedef struct cgptx_call_record {
+    const char* op;
+    const void* tensors[10];
+    size_t dims[8];
+    int flags[4];
+    float scalar;
+    int dtype;
+} cgptx_call_record;
+int cgptx_model_record_calls(cgptx_model* model, int enable);
+size_t cgptx_model_call_count(const cgptx_model* model);
+int cgptx_model_call(const cgptx_model* model, size_t index, cgptx_call_record* record);
 
 /* Number of parameter tensors and, per index, name / device pointers / element count. Names follow
  * the checkpoint names of src/core/huggingface_export.cpp:362-378 where one exists. */

@@ -1,154 +1,102 @@
-// A caller shaped like the reference's transformer_block_backward (src/core/transformer_block.cu:644-748),
-// written against include/ only: the same operator functions in the same order with the same argument
-// order, the metadata-only reshapes of saved tensors through const_cast, the accumulate flags, and the
-// block's own residual helper. It runs on the tensors a library step saved (a two-layer model stepped with
-// CGPTX_FUSE=0, i.e. as the reference's call sequence), eagerly and from a HipGraph capture
-// (include/core/hip_graph.h, the counterpart of the CudaGraph that train/train.cpp:536-548 uses), and every
-// gradient it produces must equal the library step's bit for bit.
+// Callers of include/ops/** get the library's results: two proofs against the headers only.
+//
+// (1) Compile-time: every operator wrapper is invocable with exactly the argument lists the reference's
+//     block and model code pass (src/core/transformer_block.cu:466-595, 663-747, src/core/transformer_model.cu:
+//     360-380): outputs, inputs, GEMM context, stream, options; defaults for the trailing ones; const saved
+//     tensors reshaped in place through const_cast and passed on as const references.
+// (2) Run-time: the library reports the operator calls of its own step when that step runs as the reference's
+//     call sequence (CGPTX_FUSE=0, cgptx_model_record_calls). This program walks that table and makes every
+//     call through the C++ wrapper of that operator, on Tensor views of the same buffers with all results
+//     overwritten beforehand — eagerly, and from a HipGraph capture (include/core/hip_graph.h, the counterpart
+//     of the CudaGraph train/train.cpp:536-548 uses). Every gradient must equal the library step's bit for bit.
 // Built with hipcc by __graft_entry__.build(); run by tests/test_cpp_interface.py on the GPU.
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <functional>
 #include <map>
 #include <stdexcept>
 #include <string>
+#include <type_traits>
 #include <vector>
 
 #include "cgptx_train.h"
 #include "core/hip_graph.h"
+#include "ops/attention.h"
 #include "ops/backward/attention_backward.h"
+#include "ops/backward/embedding_backward.h"
 #include "ops/backward/linear_backward.h"
 #include "ops/backward/rmsnorm_backward.h"
 #include "ops/backward/rope_backward.h"
 #include "ops/backward/swiglu_backward.h"
+#include "ops/cross_entropy.h"
+#include "ops/cut_cross_entropy.h"
+#include "ops/embedding.h"
+#include "ops/linear.h"
 #include "ops/rmsnorm.h"
+#include "ops/rope.h"
+#include "ops/swiglu.h"
 
 namespace {
 
-// The reference's option and workspace structs for one block (include/core/transformer_block.h), reduced to
-// the members transformer_block_backward touches.
-struct TransformerBlockOptions {
-    std::size_t hidden_size, intermediate_size, num_query_heads, num_kv_heads, head_dim, rotary_dim;
-    float rms_epsilon;
-    bool causal = true;
-    struct { ComputeType compute_type = ComputeType::F32; std::size_t workspace_bytes = 32ULL << 20; } linear_options;
-};
-struct TransformerBlockWeights {
-    const Tensor &attention_norm, &q_projection, &k_projection, &q_norm, &k_norm, &v_projection, &o_projection, &ffn_norm,
-        &gate_proj, &up_proj, &down_proj;
-};
-struct TransformerBlockGradients {
-    Tensor &attention_norm, &q_projection, &k_projection, &q_norm, &k_norm, &v_projection, &o_projection, &ffn_norm,
-        &gate_proj, &up_proj, &down_proj;
-};
-struct TransformerBlockWorkspace {
-    Tensor norm, query_pre_norm, key_pre_norm, query, key, value, attention_output, attention_logsumexp, gate, up, activated;
-};
-struct TransformerBlockBackwardWorkspace {
-    Tensor grad_activated, grad_gate, grad_up, grad_ffn_norm_input, grad_residual, grad_attention_projection,
-        grad_attention_output, grad_query, grad_key, grad_value, grad_query_pre_rope, grad_key_pre_rope,
-        attention_norm_output, grad_attention_norm_input, hidden_bias, intermediate_bias, kv_bias;
-};
+// ---- (1) argument lists -------------------------------------------------------------------------
+using T = Tensor&;
+using CT = const Tensor&;
+using Ids = const bpe::TokenId*;
+template <typename... Args>
+using op = void (*)(Args...);
+// Backward operators as the block calls them: with the stream and options, and with the defaults.
+static_assert(std::is_invocable_v<decltype(static_cast<op<T, T, T, CT, CT, CT, const GemmContext&, hipStream_t,
+                                                           const LinearBackwardOptions&>>(linear_backward)),
+                                  T, T, T, CT, CT, CT, const GemmContext&, hipStream_t, const LinearBackwardOptions&>);
+static_assert(std::is_invocable_v<decltype(static_cast<op<T, T, CT, CT, CT, float, hipStream_t>>(rmsnorm_backward)), T, T, CT, CT,
+                                  CT, float, hipStream_t>);
+static_assert(std::is_invocable_v<decltype(static_cast<op<T, T, CT, CT, CT, hipStream_t, const SwiGLUBackwardOptions&>>(swiglu_backward)),
+                                  T, T, CT, CT, CT, hipStream_t, const SwiGLUBackwardOptions&>);
+static_assert(std::is_invocable_v<decltype(static_cast<op<T, CT, CT, hipStream_t, const SwiGLUBackwardOptions&>>(swiglu_backward)), T,
+                                  CT, CT, hipStream_t, const SwiGLUBackwardOptions&>);  // concatenated gate_up overload
+static_assert(std::is_invocable_v<decltype(static_cast<op<T, T, CT, CT, CT, CT, hipStream_t, const RopeOptions&>>(rope_backward)), T,
+                                  T, CT, CT, CT, CT, hipStream_t, RopeOptions>);
+static_assert(std::is_invocable_v<decltype(static_cast<op<T, T, T, CT, CT, CT, CT, CT, CT, hipStream_t, const FlashAttentionOptions&,
+                                                           bool>>(flash_gqa_attention_backward_with_lse)),
+                                  T, T, T, CT, CT, CT, CT, CT, CT, hipStream_t, const FlashAttentionOptions&, bool>);
+static_assert(std::is_invocable_v<decltype(static_cast<op<T, T, T, CT, CT, CT, CT, hipStream_t, const FlashAttentionOptions&, bool>>(
+                                      flash_gqa_attention_backward)),
+                                  T, T, T, CT, CT, CT, CT, hipStream_t, const FlashAttentionOptions&, bool>);
+static_assert(std::is_invocable_v<decltype(static_cast<op<T, CT, Ids, std::size_t, hipStream_t, const EmbeddingBackwardOptions&>>(
+                                      embedding_backward)),
+                                  T, CT, Ids, std::size_t, hipStream_t, EmbeddingBackwardOptions>);
+static_assert(std::is_invocable_v<decltype(static_cast<op<T, T, CT, Ids, std::size_t, hipStream_t, float>>(cross_entropy_forward_backward)),
+                                  T, T, CT, Ids, std::size_t, hipStream_t, float>);
+static_assert(std::is_invocable_v<decltype(static_cast<op<T, T, T, CT, CT, Ids, std::size_t, hipStream_t>>(
+                                      cut_cross_entropy_forward_backward)),
+                                  T, T, T, CT, CT, Ids, std::size_t, hipStream_t>);
+// Trailing defaults: the stream, the options and the accumulate flag may be left out, as the reference's tests do.
+template <typename... Args>
+constexpr bool callable_linear_backward = requires(Args... a) { linear_backward(a...); };
+static_assert(callable_linear_backward<T, T, T, CT, CT, CT, const GemmContext&>);
+static_assert(callable_linear_backward<T, T, T, CT, CT, CT, const GemmContext&, hipStream_t>);
+static_assert(requires(T a, CT b, float e) { rmsnorm_backward(a, a, b, b, b, e); });
+static_assert(requires(T a, CT b) { swiglu_backward(a, a, b, b, b); });
+static_assert(requires(T a, CT b) { rope_backward(a, a, b, b, b, b); });
+static_assert(requires(T a, CT b) { flash_gqa_attention_backward_with_lse(a, a, a, b, b, b, b, b, b); });
+static_assert(requires(T a, CT b, Ids ids) { embedding_backward(a, b, ids, std::size_t{1}); });
+static_assert(requires(T a, CT b, Ids ids) { cross_entropy_forward_backward(a, a, b, ids, std::size_t{1}); });
+// Option structs carry the reference's fields with its defaults (include/ops/backward/*.h, include/ops/attention.h).
+static_assert(LinearBackwardOptions{}.compute_type == ComputeType::F32 && LinearBackwardOptions{}.workspace_bytes == (32ULL << 20) &&
+              !LinearBackwardOptions{}.accumulate_input && !LinearBackwardOptions{}.accumulate_weight &&
+              !LinearBackwardOptions{}.accumulate_bias);
+static_assert(!SwiGLUBackwardOptions{}.accumulate_gate && !SwiGLUBackwardOptions{}.accumulate_up &&
+              !SwiGLUBackwardOptions{}.accumulate_gate_up);
+static_assert(EmbeddingBackwardOptions{}.bounds_check && !EmbeddingBackwardOptions{}.accumulate_weight);
+static_assert(FlashAttentionOptions{}.causal && FlashAttentionOptions{}.attention_scale == 0.0F &&
+              FlashAttentionOptions{}.query_position_offset == 0);
+static_assert(RopeOptions{}.rotary_dim == 0 && RopeOptions{}.position_offset == 0);
+// A saved (const) tensor is reshaped in place through const_cast and handed on as a const reference; reshape is
+// metadata-only, so the view keeps its buffer.
+static_assert(requires(const Tensor& saved) { const_cast<Tensor&>(saved).reshape({std::size_t{1}, std::size_t{1}}); });
 
-void check_hip(hipError_t status, const char* what) {
-    if (status != hipSuccess) throw std::runtime_error(std::string(what) + ": " + hipGetErrorString(status));
-}
-
-// a += b, the block's residual helper (src/core/transformer_block.cu:134-144).
-void add_inplace(Tensor& a, const Tensor& b, hipStream_t stream) {
-    cgptx_detail::check(cgptx_add(a.raw_data(), a.raw_data(), b.raw_data(), a.numel(), cgptx_detail::dtype_code(a.dtype()), stream));
-}
-
-void transformer_block_backward(Tensor& grad_input, const Tensor& grad_output, const Tensor& input,
-                                const TransformerBlockWeights& weights, const TransformerBlockGradients gradients,
-                                const TransformerBlockWorkspace& forward_workspace, TransformerBlockBackwardWorkspace& backward,
-                                const Tensor& cos_cache, const Tensor& sin_cache, const GemmContext& gemm_context,
-                                hipStream_t stream, const TransformerBlockOptions& options, const std::size_t position_offset) {
-    if (input.shape() != grad_output.shape() || grad_input.shape() != input.shape() || input.dim() != 2)
-        throw std::invalid_argument("transformer block backward: invalid input or output gradient");
-    const std::size_t rows = input.size(0), hidden = options.hidden_size;
-    const std::size_t batch = forward_workspace.query.size(0), sequence = forward_workspace.query.size(1);
-
-    LinearBackwardOptions linear_options{options.linear_options.compute_type, options.linear_options.workspace_bytes};
-    linear_backward(backward.grad_activated, gradients.down_proj, backward.hidden_bias, grad_output,
-                    forward_workspace.activated, weights.down_proj, gemm_context, stream, linear_options);
-    swiglu_backward(backward.grad_gate, backward.grad_up, backward.grad_activated, forward_workspace.gate,
-                    forward_workspace.up, stream);
-    linear_backward(backward.grad_ffn_norm_input, gradients.gate_proj, backward.intermediate_bias, backward.grad_gate,
-                    forward_workspace.norm, weights.gate_proj, gemm_context, stream, linear_options);
-    linear_options.accumulate_input = true;
-    linear_backward(backward.grad_ffn_norm_input, gradients.up_proj, backward.intermediate_bias, backward.grad_up,
-                    forward_workspace.norm, weights.up_proj, gemm_context, stream, linear_options);
-    linear_options.accumulate_input = false;
-
-    rmsnorm_backward(backward.grad_residual, gradients.ffn_norm, backward.grad_ffn_norm_input, input, weights.ffn_norm,
-                     options.rms_epsilon, stream);
-
-    check_hip(hipMemcpyAsync(grad_input.raw_data(), grad_output.raw_data(), grad_output.nbytes(), hipMemcpyDeviceToDevice, stream),
-              "hipMemcpyAsync");
-    add_inplace(grad_input, backward.grad_residual, stream);
-    check_hip(hipMemcpyAsync(backward.grad_attention_projection.raw_data(), grad_output.raw_data(), grad_output.nbytes(),
-                             hipMemcpyDeviceToDevice, stream),
-              "hipMemcpyAsync");
-
-    backward.grad_attention_output.reshape({rows, hidden});
-    auto& saved_attention_output = const_cast<Tensor&>(forward_workspace.attention_output);
-    saved_attention_output.reshape({rows, hidden});
-    linear_backward(backward.grad_attention_output, gradients.o_projection, backward.hidden_bias,
-                    backward.grad_attention_projection, saved_attention_output, weights.o_projection, gemm_context, stream,
-                    linear_options);
-    saved_attention_output.reshape({batch, sequence, options.num_query_heads, options.head_dim});
-    backward.grad_attention_output.reshape({batch, sequence, options.num_query_heads, options.head_dim});
-    FlashAttentionOptions attention_options{};
-    attention_options.num_query_heads = options.num_query_heads;
-    attention_options.num_kv_heads = options.num_kv_heads;
-    attention_options.head_dim = options.head_dim;
-    attention_options.causal = options.causal;
-    attention_options.query_position_offset = position_offset;
-    flash_gqa_attention_backward_with_lse(backward.grad_query, backward.grad_key, backward.grad_value,
-                                          backward.grad_attention_output, forward_workspace.attention_output,
-                                          forward_workspace.attention_logsumexp, forward_workspace.query, forward_workspace.key,
-                                          forward_workspace.value, stream, attention_options);
-    rope_backward(backward.grad_query_pre_rope, backward.grad_key_pre_rope, backward.grad_query, backward.grad_key, cos_cache,
-                  sin_cache, stream, RopeOptions{options.rotary_dim, position_offset});
-
-    backward.grad_query_pre_rope.reshape({batch * sequence * options.num_query_heads, options.head_dim});
-    backward.grad_query.reshape({batch * sequence * options.num_query_heads, options.head_dim});
-    auto& saved_query_pre_norm = const_cast<Tensor&>(forward_workspace.query_pre_norm);
-    saved_query_pre_norm.reshape({batch * sequence * options.num_query_heads, options.head_dim});
-    rmsnorm_backward(backward.grad_query, gradients.q_norm, backward.grad_query_pre_rope, saved_query_pre_norm, weights.q_norm,
-                     options.rms_epsilon, stream);
-    backward.grad_key_pre_rope.reshape({batch * sequence * options.num_kv_heads, options.head_dim});
-    backward.grad_key.reshape({batch * sequence * options.num_kv_heads, options.head_dim});
-    auto& saved_key_pre_norm = const_cast<Tensor&>(forward_workspace.key_pre_norm);
-    saved_key_pre_norm.reshape({batch * sequence * options.num_kv_heads, options.head_dim});
-    rmsnorm_backward(backward.grad_key, gradients.k_norm, backward.grad_key_pre_rope, saved_key_pre_norm, weights.k_norm,
-                     options.rms_epsilon, stream);
-    saved_query_pre_norm.reshape({batch, sequence, options.num_query_heads, options.head_dim});
-    saved_key_pre_norm.reshape({batch, sequence, options.num_kv_heads, options.head_dim});
-
-    rmsnorm_forward(backward.attention_norm_output, input, weights.attention_norm, options.rms_epsilon, stream);
-    backward.grad_query.reshape({rows, options.num_query_heads * options.head_dim});
-    backward.grad_key.reshape({rows, options.num_kv_heads * options.head_dim});
-    backward.grad_value.reshape({rows, options.num_kv_heads * options.head_dim});
-    linear_backward(backward.grad_attention_norm_input, gradients.q_projection, backward.hidden_bias, backward.grad_query,
-                    backward.attention_norm_output, weights.q_projection, gemm_context, stream, linear_options);
-    linear_options.accumulate_input = true;
-    linear_backward(backward.grad_attention_norm_input, gradients.k_projection, backward.kv_bias, backward.grad_key,
-                    backward.attention_norm_output, weights.k_projection, gemm_context, stream, linear_options);
-    linear_backward(backward.grad_attention_norm_input, gradients.v_projection, backward.kv_bias, backward.grad_value,
-                    backward.attention_norm_output, weights.v_projection, gemm_context, stream, linear_options);
-    linear_options.accumulate_input = false;
-    backward.grad_query_pre_rope.reshape({batch, sequence, options.num_query_heads, options.head_dim});
-    backward.grad_key_pre_rope.reshape({batch, sequence, options.num_kv_heads, options.head_dim});
-    backward.grad_value.reshape({batch, sequence, options.num_kv_heads, options.head_dim});
-    backward.grad_query.reshape({batch, sequence, options.num_query_heads, options.head_dim});
-    backward.grad_key.reshape({batch, sequence, options.num_kv_heads, options.head_dim});
-    rmsnorm_backward(backward.grad_residual, gradients.attention_norm, backward.grad_attention_norm_input, input,
-                     weights.attention_norm, options.rms_epsilon, stream);
-    add_inplace(grad_input, backward.grad_residual, stream);
-}
-
+// ---- (2) the call table, walked through the wrappers ---------------------------------------------
 int failures = 0;
 void expect(bool ok, const std::string& what) {
     if (!ok) {
@@ -159,11 +107,113 @@ void expect(bool ok, const std::string& what) {
 void ok(int status, const char* what) {
     if (status != CGPTX_OK) throw std::runtime_error(std::string(what) + ": " + cgptx_last_error());
 }
+void check_hip(hipError_t status, const char* what) {
+    if (status != hipSuccess) throw std::runtime_error(std::string(what) + ": " + hipGetErrorString(status));
+}
 std::vector<std::uint8_t> bytes_of(const void* device, std::size_t bytes) {
     std::vector<std::uint8_t> host(bytes);
     check_hip(hipMemcpy(host.data(), device, bytes, hipMemcpyDeviceToHost), "hipMemcpy");
     return host;
 }
+
+struct Caller {
+    hipStream_t stream;
+    GemmContext gemm_context;
+    std::map<std::size_t, Tensor> bias_scratch;  // linear_backward's bias gradient, which the block throws away
+
+    static Dtype dtype_of(const cgptx_call_record& r) { return r.dtype == CGPTX_F16 ? Dtype::F16 : (r.dtype == CGPTX_BF16 ? Dtype::BF16 : Dtype::F32); }
+    static Tensor view(const cgptx_call_record& r, int index, std::vector<std::size_t> shape) {
+        return Tensor::device_view(std::move(shape), const_cast<void*>(r.tensors[index]), dtype_of(r));
+    }
+    static Tensor view_f32(const cgptx_call_record& r, int index, std::vector<std::size_t> shape) {
+        return Tensor::device_view(std::move(shape), const_cast<void*>(r.tensors[index]), Dtype::F32);
+    }
+    static Ids ids(const cgptx_call_record& r, int index) { return static_cast<Ids>(r.tensors[index]); }
+
+    void call(const cgptx_call_record& r) {
+        const std::string name(r.op);
+        const auto* d = r.dims;
+        if (name == "embedding_forward") {
+            Tensor out = view(r, 0, {d[0], d[2]});
+            embedding_forward(out, ids(r, 1), d[0], view(r, 2, {d[1], d[2]}), stream);
+        } else if (name == "rmsnorm_forward") {
+            Tensor out = view(r, 0, {d[0], d[1]});
+            rmsnorm_forward(out, view(r, 1, {d[0], d[1]}), view(r, 2, {d[1]}), r.scalar, stream);
+        } else if (name == "linear_forward") {
+            Tensor out = view(r, 0, {d[0], d[2]});
+            linear_forward(out, view(r, 1, {d[0], d[1]}), view(r, 2, {d[2], d[1]}), gemm_context, stream);
+        } else if (name == "rope_forward") {
+            Tensor q = view(r, 0, {d[0], d[1], d[2], d[4]}), k = view(r, 1, {d[0], d[1], d[3], d[4]});
+            rope_forward(q, k, view(r, 2, {d[7], d[5] / 2}), view(r, 3, {d[7], d[5] / 2}), stream, RopeOptions{d[5], d[6]});
+        } else if (name == "flash_gqa_attention_forward_with_lse") {
+            Tensor out = view(r, 0, {d[0], d[1], d[3], d[5]}), lse = view_f32(r, 1, {d[0], d[1], d[3]});
+            flash_gqa_attention_forward_with_lse(out, lse, view(r, 2, {d[0], d[1], d[3], d[5]}), view(r, 3, {d[0], d[2], d[4], d[5]}),
+                                                 view(r, 4, {d[0], d[2], d[4], d[5]}), stream, attention_options(r));
+        } else if (name == "swiglu_forward") {
+            Tensor out = view(r, 0, {d[0]});
+            swiglu_forward(out, view(r, 1, {d[0]}), view(r, 2, {d[0]}), stream);
+        } else if (name == "add") {  // the block's own residual helper, not an operator of include/ops
+            ok(cgptx_add(const_cast<void*>(r.tensors[0]), r.tensors[1], r.tensors[2], d[0], r.dtype, stream), "add");
+        } else if (name == "cross_entropy_forward_backward") {
+            Tensor loss = view_f32(r, 0, {1}), gradient = view(r, 1, {d[0], d[1]});
+            cross_entropy_forward_backward(loss, gradient, view(r, 2, {d[0], d[1]}), ids(r, 3), d[0], stream, r.scalar);
+        } else if (name == "cut_cross_entropy_forward_backward") {
+            if (r.scalar != 1.0f) throw std::runtime_error("cut_cross_entropy_forward_backward takes no gradient scale");
+            Tensor loss = view_f32(r, 0, {1}), dx = view(r, 1, {d[0], d[1]}), dc = view(r, 2, {d[2], d[1]});
+            cut_cross_entropy_forward_backward(loss, dx, dc, view(r, 3, {d[0], d[1]}), view(r, 4, {d[2], d[1]}), ids(r, 5), d[0], stream);
+        } else if (name == "linear_backward") {
+            Tensor dx = view(r, 0, {d[0], d[1]}), dw = view(r, 1, {d[2], d[1]});
+            auto found = bias_scratch.find(d[2]);
+            if (found == bias_scratch.end()) found = bias_scratch.emplace(d[2], Tensor({d[2]}, dtype_of(r))).first;
+            LinearBackwardOptions options;
+            options.accumulate_input = r.flags[0] != 0;
+            linear_backward(dx, dw, found->second, view(r, 2, {d[0], d[2]}), view(r, 3, {d[0], d[1]}), view(r, 4, {d[2], d[1]}),
+                            gemm_context, stream, options);
+        } else if (name == "rmsnorm_backward") {
+            Tensor dx = view(r, 0, {d[0], d[1]}), dw = view(r, 1, {d[1]});
+            // The saved input is const for the caller and reshaped in place before the call, as the block does
+            // with its q / k tensors before their per-head norm gradients.
+            const Tensor saved = view(r, 3, {d[0] * d[1]});
+            const_cast<Tensor&>(saved).reshape({d[0], d[1]});
+            rmsnorm_backward(dx, dw, view(r, 2, {d[0], d[1]}), saved, view(r, 4, {d[1]}), r.scalar, stream);
+        } else if (name == "swiglu_backward") {
+            Tensor dg = view(r, 0, {d[0]}), du = view(r, 1, {d[0]});
+            SwiGLUBackwardOptions options;
+            options.accumulate_gate = r.flags[0] != 0;
+            options.accumulate_up = r.flags[1] != 0;
+            swiglu_backward(dg, du, view(r, 2, {d[0]}), view(r, 3, {d[0]}), view(r, 4, {d[0]}), stream, options);
+        } else if (name == "flash_gqa_attention_backward_with_lse") {
+            Tensor dq = view(r, 0, {d[0], d[1], d[3], d[5]}), dk = view(r, 1, {d[0], d[2], d[4], d[5]}),
+                   dv = view(r, 2, {d[0], d[2], d[4], d[5]});
+            flash_gqa_attention_backward_with_lse(dq, dk, dv, view(r, 3, {d[0], d[1], d[3], d[5]}), view(r, 4, {d[0], d[1], d[3], d[5]}),
+                                                  view_f32(r, 5, {d[0], d[1], d[3]}), view(r, 6, {d[0], d[1], d[3], d[5]}),
+                                                  view(r, 7, {d[0], d[2], d[4], d[5]}), view(r, 8, {d[0], d[2], d[4], d[5]}), stream,
+                                                  attention_options(r), r.flags[1] != 0);
+        } else if (name == "rope_backward") {
+            Tensor dq = view(r, 0, {d[0], d[1], d[2], d[4]}), dk = view(r, 1, {d[0], d[1], d[3], d[4]});
+            rope_backward(dq, dk, view(r, 2, {d[0], d[1], d[2], d[4]}), view(r, 3, {d[0], d[1], d[3], d[4]}),
+                          view(r, 4, {d[7], d[5] / 2}), view(r, 5, {d[7], d[5] / 2}), stream, RopeOptions{d[5], d[6]});
+        } else if (name == "embedding_backward") {
+            Tensor dw = view(r, 0, {d[1], d[2]});
+            EmbeddingBackwardOptions options;
+            options.bounds_check = r.flags[0] != 0;
+            options.accumulate_weight = r.flags[1] != 0;
+            embedding_backward(dw, view(r, 1, {d[0], d[2]}), ids(r, 2), d[0], stream, options);
+        } else {
+            throw std::runtime_error("call table names an operator this caller does not know: " + name);
+        }
+    }
+    static FlashAttentionOptions attention_options(const cgptx_call_record& r) {
+        FlashAttentionOptions o{};
+        o.num_query_heads = r.dims[3];
+        o.num_kv_heads = r.dims[4];
+        o.head_dim = r.dims[5];
+        o.attention_scale = r.scalar;
+        o.causal = r.flags[0] != 0;
+        o.query_position_offset = r.dims[6];
+        return o;
+    }
+};
 
 }  // namespace
 
@@ -171,7 +221,6 @@ int main() {
     try {
         setenv("CGPTX_FUSE", "0", 1);  // the library step as the reference's call sequence
         constexpr std::size_t B = 2, T = 48, L = 2, H = 256, I = 512, HQ = 4, HKV = 2, D = 64, V = 512, N = B * T;
-        constexpr Dtype dtype = Dtype::BF16;
         cgptx_model_config config{};
         config.vocabulary_size = V;
         config.num_layers = L;
@@ -194,86 +243,54 @@ int main() {
         ok(cgptx_model_set_tokens(model, tokens.data(), targets.data()), "set_tokens");
         hipStream_t stream = nullptr;
         check_hip(hipStreamCreate(&stream), "hipStreamCreate");
+        ok(cgptx_model_record_calls(model, 1), "record_calls");
         ok(cgptx_model_forward_backward(model, 64.0f, CGPTX_LOSS_DENSE, 0, stream), "forward_backward");
         check_hip(hipStreamSynchronize(stream), "sync");
 
-        // The first block's weights and the gradients the library step computed for them.
-        std::map<std::string, std::pair<void*, std::vector<std::uint8_t>>> parameters;  // short name -> (weight, gradient bytes)
-        const std::string prefix = "model.layers.0.";
+        // What the library step left: every parameter gradient, the gradient of the first hidden state, the loss.
+        struct Result {
+            std::string name;
+            void* device;
+            std::vector<std::uint8_t> want;
+        };
+        std::vector<Result> results;
         for (std::size_t i = 0; i < cgptx_model_parameter_count(model); ++i) {
             const char* name = nullptr;
             void *value = nullptr, *gradient = nullptr;
             std::size_t count = 0;
             ok(cgptx_model_parameter(model, i, &name, &value, &gradient, &count), "model_parameter");
-            const std::string full(name);
-            if (full.rfind(prefix, 0) == 0) parameters[full.substr(prefix.size())] = {value, bytes_of(gradient, count * 2)};
+            results.push_back({std::string("gradient of ") + name, gradient, bytes_of(gradient, count * 2)});
         }
-        auto named = [&](const char* name, std::vector<std::size_t> shape, Dtype t = dtype) {
+        for (const char* name : {"grad.hidden.0", "loss"}) {
             void* data = nullptr;
             std::size_t count = 0;
             ok(cgptx_model_activation(model, name, &data, &count), name);
-            Tensor view = Tensor::device_view(std::move(shape), data, t);
-            if (view.numel() != count) throw std::runtime_error(std::string(name) + ": unexpected size");
-            return view;
+            const std::size_t bytes = std::string(name) == "loss" ? sizeof(float) : count * 2;
+            results.push_back({name, data, bytes_of(data, bytes)});
+        }
+
+        std::vector<cgptx_call_record> table(cgptx_model_call_count(model));
+        for (std::size_t i = 0; i < table.size(); ++i) ok(cgptx_model_call(model, i, &table[i]), "model_call");
+        std::map<std::string, int> seen;
+        for (const auto& r : table) ++seen[r.op];
+        // Per block the reference makes 7 linear_backward calls (down, gate, up, o, q, k, v) and 4 norm gradients;
+        // the model adds the classifier's and the final norm's.
+        expect(seen["linear_backward"] == 7 * L + 1 && seen["rmsnorm_backward"] == 4 * L + 1 &&
+                   seen["flash_gqa_attention_backward_with_lse"] == L && seen["rope_backward"] == L && seen["swiglu_backward"] == L &&
+                   seen["embedding_backward"] == 1 && seen["cross_entropy_forward_backward"] == 1,
+               "the call table holds the reference's backward calls");
+
+        Caller caller{stream, GemmContext{}, {}};
+        auto run = [&] {
+            for (const auto& r : table) caller.call(r);
         };
-        auto weight = [&](const char* name, std::vector<std::size_t> shape) {
-            return Tensor::device_view(std::move(shape), parameters.at(name).first, dtype);
-        };
-        const Tensor input = named("hidden.0", {N, H}), grad_output = named("grad.hidden.1", {N, H});
-        const std::vector<std::uint8_t> want_grad_input = bytes_of(named("grad.hidden.0", {N, H}).raw_data(), N * H * 2);
-        const Tensor cos_cache = named("rope.cos", {T, D / 2}), sin_cache = named("rope.sin", {T, D / 2});
-        Tensor gate_up = named("layer.0.gate_up", {2, N, I});  // CGPTX_FUSE=0: [gate; up], each [N, I]
-        TransformerBlockWorkspace forward{
-            named("layer.0.ffn_norm_output", {N, H}),
-            named("layer.0.query_pre_norm", {B, T, HQ, D}),
-            named("layer.0.key_pre_norm", {B, T, HKV, D}),
-            named("layer.0.query", {B, T, HQ, D}),
-            named("layer.0.key", {B, T, HKV, D}),
-            named("layer.0.value", {B, T, HKV, D}),
-            named("layer.0.attention_output", {B, T, HQ, D}),
-            named("layer.0.logsumexp", {B, T, HQ}, Dtype::F32),
-            Tensor::device_view({N, I}, gate_up.raw_data(), dtype),
-            Tensor::device_view({N, I}, static_cast<char*>(gate_up.raw_data()) + N * I * 2, dtype),
-            named("layer.0.activated", {N, I})};
-        const Tensor w_attention_norm = weight("input_layernorm.weight", {H}), w_q = weight("self_attn.q_proj.weight", {HQ * D, H}),
-                     w_k = weight("self_attn.k_proj.weight", {HKV * D, H}), w_q_norm = weight("self_attn.q_norm.weight", {D}),
-                     w_k_norm = weight("self_attn.k_norm.weight", {D}), w_v = weight("self_attn.v_proj.weight", {HKV * D, H}),
-                     w_o = weight("self_attn.o_proj.weight", {H, HQ * D}), w_ffn_norm = weight("post_attention_layernorm.weight", {H}),
-                     w_gate = weight("mlp.gate_proj.weight", {I, H}), w_up = weight("mlp.up_proj.weight", {I, H}),
-                     w_down = weight("mlp.down_proj.weight", {H, I});
-        const TransformerBlockWeights weights{w_attention_norm, w_q, w_k, w_q_norm, w_k_norm, w_v, w_o, w_ffn_norm, w_gate, w_up, w_down};
-        auto fresh = [&](std::vector<std::size_t> shape) { return Tensor(std::move(shape), dtype); };
-        Tensor g_attention_norm = fresh({H}), g_q = fresh({HQ * D, H}), g_k = fresh({HKV * D, H}), g_q_norm = fresh({D}),
-               g_k_norm = fresh({D}), g_v = fresh({HKV * D, H}), g_o = fresh({H, HQ * D}), g_ffn_norm = fresh({H}),
-               g_gate = fresh({I, H}), g_up = fresh({I, H}), g_down = fresh({H, I});
-        const TransformerBlockGradients gradients{g_attention_norm, g_q, g_k, g_q_norm, g_k_norm, g_v, g_o, g_ffn_norm, g_gate, g_up, g_down};
-        TransformerBlockBackwardWorkspace backward{
-            fresh({N, I}), fresh({N, I}), fresh({N, I}), fresh({N, H}), fresh({N, H}), fresh({N, H}),
-            fresh({B, T, HQ, D}), fresh({B, T, HQ, D}), fresh({B, T, HKV, D}), fresh({B, T, HKV, D}),
-            fresh({B, T, HQ, D}), fresh({B, T, HKV, D}), fresh({N, H}), fresh({N, H}), fresh({H}), fresh({I}), fresh({HKV * D})};
-        Tensor grad_input = fresh({N, H});
-        const TransformerBlockOptions options{H, I, HQ, HKV, D, D, 1e-5f};
-        const GemmContext gemm_context;
-        const std::map<std::string, Tensor*> produced = {
-            {"input_layernorm.weight", &g_attention_norm}, {"self_attn.q_proj.weight", &g_q}, {"self_attn.k_proj.weight", &g_k},
-            {"self_attn.q_norm.weight", &g_q_norm}, {"self_attn.k_norm.weight", &g_k_norm}, {"self_attn.v_proj.weight", &g_v},
-            {"self_attn.o_proj.weight", &g_o}, {"post_attention_layernorm.weight", &g_ffn_norm}, {"mlp.gate_proj.weight", &g_gate},
-            {"mlp.up_proj.weight", &g_up}, {"mlp.down_proj.weight", &g_down}};
         auto clear_outputs = [&] {
-            for (const auto& [name, tensor] : produced) check_hip(hipMemset(tensor->raw_data(), 0xFF, tensor->nbytes()), "hipMemset");
-            check_hip(hipMemset(grad_input.raw_data(), 0xFF, grad_input.nbytes()), "hipMemset");
+            for (const auto& r : results) check_hip(hipMemset(r.device, 0xFF, r.want.size()), "hipMemset");
         };
         auto compare = [&](const char* pass) {
             check_hip(hipStreamSynchronize(stream), "sync");
-            for (const auto& [name, tensor] : produced)
-                expect(bytes_of(tensor->raw_data(), tensor->nbytes()) == parameters.at(name).second,
-                       std::string(pass) + ": gradient of " + name + " differs from the library step");
-            expect(bytes_of(grad_input.raw_data(), grad_input.nbytes()) == want_grad_input,
-                   std::string(pass) + ": grad_input differs from the library step");
-        };
-        auto run = [&] {
-            transformer_block_backward(grad_input, grad_output, input, weights, gradients, forward, backward, cos_cache, sin_cache,
-                                       gemm_context, stream, options, 0);
+            for (const auto& r : results)
+                expect(bytes_of(r.device, r.want.size()) == r.want, std::string(pass) + ": " + r.name + " differs from the library step");
         };
 
         clear_outputs();

@@ -69,10 +69,23 @@ def test_interface_program_replays_reference_known_answers():
 
 
 @pytest.mark.gpu
-def test_block_backward_written_against_the_headers_matches_the_library_step():
-    """tests/cpp/block_backward_test.cpp: the reference's transformer_block_backward call sequence
-    (src/core/transformer_block.cu:644-748) against include/ only, eagerly and from a HipGraph capture, bit for bit
-    equal to the library's step run as the reference's call sequence (CGPTX_FUSE=0)."""
+def test_token_batches_upload_through_the_data_header():
+    """tests/cpp/data_upload_test.cpp: data::Batch / data::DeviceBatch / data::upload_batch
+    (include/data/dataset_loader.h) over the library's upload entry points: alternating page-locked batches arrive
+    bit for bit, device buffers keep their address, shape mismatches throw, copies are deep, moves carry the
+    pending upload."""
+    binary = ROOT / "tests" / "cpp" / "data_upload_test.bin"
+    assert binary.exists(), "build it with `python -m cgpt_amd.build` (there is no fallback)"
+    proc = subprocess.run([str(binary)], capture_output=True, text=True, timeout=120)
+    assert proc.returncode == 0, proc.stdout + proc.stderr
+    assert "0 failure(s)" in proc.stdout
+
+
+@pytest.mark.gpu
+def test_callers_of_the_headers_reproduce_the_library_step():
+    """tests/cpp/block_backward_test.cpp: the wrappers accept the reference's argument lists (compile-time), and
+    the library's own table of operator calls (the step as the reference's call sequence, CGPTX_FUSE=0), made
+    through include/ops/** eagerly and from a HipGraph capture, gives the library step's gradients bit for bit."""
     binary = ROOT / "tests" / "cpp" / "block_backward_test.bin"
     assert binary.exists(), "build it with `python -m cgpt_amd.build` (there is no fallback)"
     proc = subprocess.run([str(binary)], capture_output=True, text=True, timeout=120)

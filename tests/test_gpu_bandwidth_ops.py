@@ -54,9 +54,10 @@ def test_rmsnorm_backward_reference_test_inputs(device, dtype, tol):
 
 
 def test_rmsnorm_backward_is_deterministic_and_full_size(device):
-    """[32768, 1024] bf16 (the training shape), the QK-norm shape [65536, 128] and the 768-wide shapes ([32768, 768];
-    [131072, 64] for its 4 kv-heads of 64): run twice, bit-identical, and equal to the CPU checker."""
-    for rows, hidden in ((32768, 1024), (65536, 128), (32768, 768), (131072, 64)):
+    """[32768, 1024] bf16 (the training shape), the QK-norm shapes [262144, 128] (q: the 8 heads of every token, the pass
+    a step runs once per layer) and [65536, 128] (k), and the 768-wide shapes ([32768, 768]; [131072, 64] for its 4
+    kv-heads of 64): run twice, bit-identical, and equal to the CPU checker."""
+    for rows, hidden in ((32768, 1024), (262144, 128), (65536, 128), (32768, 768), (131072, 64)):
         dtype = torch.bfloat16
         x, dy = randn((rows, hidden), dtype, 11), randn((rows, hidden), dtype, 12)
         w = (1.0 + 0.1 * randn((hidden,), torch.float32, 13)).to(dtype)

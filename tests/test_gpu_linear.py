@@ -138,6 +138,48 @@ def test_linear_backward_layer_shapes_of_the_104m_model(device):
         check_against_float64(outs[0][1], dw64, dtype, f"dW {fout}x{fin}", rows)
 
 
+@pytest.mark.parametrize("fout,fin", [(256, 1024), (1024, 1024), (4096, 1024), (1024, 2048), (32000, 1024)],
+                         ids=["kv-256x1024", "q-o-1024x1024", "gate_up-4096x1024", "down-1024x2048", "lm_head-32000x1024"])
+def test_linear_backward_at_the_32768_training_rows_sampled_against_float64(device, fout, fin):
+    """linear_backward at the real row count of a B=32, T=1024 step (the weight gradient's split-K depth is the 32768
+    rows; the classifier shape is the one the cut cross-entropy contracts), bf16. Checked against float64 dot products
+    on samples that touch every output tile: 256 rows of dX (two per 256-row tile, all columns), 64 rows and 64 columns
+    of dW (all of the other index, i.e. sums over all 32768 rows), with the tolerance of the 16-bit parity bar relative
+    to each result's scale. Inputs are made on the device; only the sampled slices travel to the host."""
+    dtype = torch.bfloat16
+    rows = 32768
+    gen = torch.Generator(device=device).manual_seed(fout + fin)
+    x = torch.randn(rows, fin, device=device, generator=gen).to(dtype)
+    w = (torch.randn(fout, fin, device=device, generator=gen) * 0.02).to(dtype)
+    dy = torch.randn(rows, fout, device=device, generator=gen).to(dtype)
+    gi = torch.empty(rows, fin, dtype=dtype, device=device)
+    gw = torch.empty(fout, fin, dtype=dtype, device=device)
+    ops.linear_backward(gi, gw, None, dy, x, w)
+    torch.cuda.synchronize()
+    rng = np.random.default_rng(fout * 7 + fin)
+    # dX rows: two per 256-row tile.
+    picked = np.sort(np.concatenate([tile * 256 + rng.choice(256, 2, replace=False) for tile in range(rows // 256)]))
+    index = torch.as_tensor(picked, device=device)
+    want = to_np(dy[index]) @ to_np(w)
+    check_against_float64(gi[index], want, dtype, f"dX rows {fout}x{fin}", fout)
+    # dW rows (outputs o) and columns (inputs i), each a sum over all rows: accumulated over row chunks on the host.
+    some_out = np.sort(rng.choice(fout, 64, replace=False))
+    some_in = np.sort(rng.choice(fin, 64, replace=False))
+    out_index, in_index = torch.as_tensor(some_out, device=device), torch.as_tensor(some_in, device=device)
+    want_rows = np.zeros((64, fin))
+    want_cols = np.zeros((fout, 64))
+    for r0 in range(0, rows, 2048):
+        dy_chunk, x_chunk = dy[r0:r0 + 2048], x[r0:r0 + 2048]
+        want_rows += to_np(dy_chunk[:, out_index]).T @ to_np(x_chunk)
+        want_cols += to_np(dy_chunk).T @ to_np(x_chunk[:, in_index])
+    check_against_float64(gw[out_index], want_rows, dtype, f"dW rows {fout}x{fin}", rows)
+    check_against_float64(gw[:, in_index], want_cols, dtype, f"dW columns {fout}x{fin}", rows)
+    # dX columns over all rows for the layer shapes (the classifier's dY is too large to widen on the host).
+    if fout <= 4096:
+        want_dx_cols = np.concatenate([to_np(dy[r0:r0 + 4096]) @ to_np(w[:, in_index]) for r0 in range(0, rows, 4096)])
+        check_against_float64(gi[:, in_index], want_dx_cols, dtype, f"dX columns {fout}x{fin}", fout)
+
+
 def test_linear_argument_errors(device):
     x, w, dy = torch.zeros(4, 8, device=device), torch.zeros(3, 8, device=device), torch.zeros(4, 3, device=device)
     gi, gw, gb = torch.zeros_like(x), torch.zeros_like(w), torch.zeros(3, device=device)

@@ -103,18 +103,23 @@ def params_from_model(model, cfg):
 
 
 def compare_gradients(got, want, tol, loss_scale):
+    worst = [0.0, ""]
+
     def one(g, w, name):
         w = np.asarray(w).reshape(-1)
         scale = max(np.abs(w).max(), 1e-3 * loss_scale)
         got_flat = to_np(g).reshape(-1)
         err = np.abs(got_flat - w).max() / scale
         assert np.isfinite(got_flat).all(), name
+        if err > worst[0]:
+            worst[:] = [err, name]
         assert err <= tol, f"{name}: error {err:.3e} of the tensor's scale"
     one(got["embedding"], want["embedding"], "embedding")
     one(got["final_norm"], want["final_norm"], "final_norm")
     for l, (g, w) in enumerate(zip(got["layers"], want["layers"])):
         for key in model64.LAYER_KEYS:
             one(g[key], w[key], f"layer{l}.{key}")
+    print(f"[parity] composed step: worst gradient error {worst[0]:.3e} of its tensor's scale ({worst[1]}; bound {tol:.1e})")
 
 
 MODEL_CFG = dict(vocab=96, layers=2, hidden=64, inter=128, hq=2, hkv=1, d=32, eps=1e-5)
@@ -133,7 +138,8 @@ def test_gpu_step_matches_float64_composition(device, dtype, loss_mode, shape):
     """Hidden 64, 2:1 heads of 32, T=24, B=2, two layers (and the wide-head variant above): every parameter
     gradient of the GPU step against the float64 composition that rounds each operator output to the storage
     dtype where the GPU stores it.
-    Tolerance: 5e-2 of each tensor's largest gradient entry (2e-2 per operator, several operators deep)."""
+    Tolerance: 3e-2 of each tensor's largest gradient entry (the operators' own bar is 2e-2, and a gradient here has
+    passed through several of them; the observed worst is printed)."""
     cfg, batch, seq = shape
     loss_scale = 64.0
     model = build(device, dtype, batch, seq, cfg)
@@ -150,7 +156,7 @@ def test_gpu_step_matches_float64_composition(device, dtype, loss_mode, shape):
     for l in range(cfg["layers"] + 1):
         hidden = to_np(model.activation(f"hidden.{l}")).reshape(batch * seq, cfg["hidden"])
         assert np.abs(hidden - saved["hidden"][l]).max() <= 4e-2 * max(1.0, np.abs(saved["hidden"][l]).max())
-    compare_gradients(grads, want, 5e-2, loss_scale)
+    compare_gradients(grads, want, 3e-2, loss_scale)
     model.close()
 
 
@@ -190,7 +196,7 @@ def test_gpu_step_matches_float64_composition_on_random_configurations(device, s
     for l in range(cfg["layers"] + 1):
         hidden = to_np(model.activation(f"hidden.{l}")).reshape(batch * seq, cfg["hidden"])
         assert np.abs(hidden - saved["hidden"][l]).max() <= (4e-2 if sixteen else 1e-4) * max(1.0, np.abs(saved["hidden"][l]).max())
-    compare_gradients(grads, want, 5e-2 if sixteen else 1e-3, loss_scale)
+    compare_gradients(grads, want, 3e-2 if sixteen else 1e-3, loss_scale)
     model.close()
 
 

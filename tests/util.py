@@ -6,6 +6,9 @@ import torch
 
 # Tolerances of the parity bar: max |a-b| / max(1, |b|).
 TOL = {torch.float32: 1e-4, torch.float16: 2e-2, torch.bfloat16: 2e-2}
+# Bounds of the one-normalisation comparison (assert_scaled_close): half the element-wise bar for 16-bit storage
+# (the worst error any attention or cut-cross-entropy case shows is 5.5e-3 of the tensor's scale).
+STOL = {torch.float32: 1e-4, torch.float16: 1e-2, torch.bfloat16: 1e-2}
 DTYPES = [torch.float32, torch.float16, torch.bfloat16]
 DTYPE_IDS = ["f32", "f16", "bf16"]
 
