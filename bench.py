@@ -228,6 +228,24 @@ def _isolated_rest(torch, ops, want, record, rnd, timed, stream, out, N, H, I, V
         t = timed(torch, torch.cuda.current_stream(), lambda: target.copy_(source), launches=5, warm=1)
         record("copy 1 GiB (torch)", "hbm", 2.0 * (1 << 30), t, "1 GiB read, 1 GiB written")
         del source, target
+    if want("adamw"):
+        # The preset's parameter list (2 + 11 per layer tensors): all of it in three launches.
+        layers = 8
+        QW, KW = H, H // 4
+        shapes = [(V, H), (H,)] + layers * [(H,), (QW, H), (KW, H), (H // 8,), (H // 8,), (KW, H), (H, QW), (H,), (I, H), (I, H), (H, I)]
+        entries = []
+        for shape in shapes:
+            parameter = rnd(*shape, scale=0.02)
+            entries.append(ops.AdamWBatchEntry(parameter, rnd(*shape), ops.AdamWState.for_parameter(parameter)))
+        count = sum(e.parameter.numel() for e in entries)
+        workspace = ops.AdamWWorkspace()
+        options = ops.AdamWOptions(learning_rate=3e-4, beta1=0.9, beta2=0.95, epsilon=1e-8, weight_decay=0.1,
+                                   loss_scale=1024.0, max_grad_norm=1.0)
+        t = timed(torch, stream, lambda: ops.adamw_step_many_async(entries, options, workspace, stream), launches=5, warm=1)
+        record(f"adamw_step_many_async {count} parameters in {len(entries)} tensors", "hbm", 30.0 * count, t,
+               "30 B/parameter: 16-bit gradient read twice (norm, update), fp32 master and both moments read and written, "
+               "16-bit parameter written")
+        del entries, workspace
     if want("dense_cross_entropy"):
         rows = N // 2
         logits = rnd(rows, V)
@@ -240,7 +258,8 @@ def _isolated_rest(torch, ops, want, record, rnd, timed, stream, out, N, H, I, V
 def published_kernel_shapes(torch, stream, seed):
     """The launches of the reference's own kernel table (kernel_profile.md:9-25: B = 1, T = 512, 32:8 heads, D = 128,
     hidden 4096, measured by its authors on a 192 GB/s GPU) on this GPU: average us over 50 back-to-back calls beside
-    the published milliseconds. These launches are small (2 to 100 MB): they measure launch latency as much as rate."""
+    the published milliseconds. Context only (--kernels-only published): other hardware, not a configuration of the
+    benchmark, and launches so small (2 to 100 MB) that they measure launch latency as much as rate."""
     from cgpt_amd import ops
 
     gen = torch.Generator(device="cuda").manual_seed(seed)
@@ -251,8 +270,7 @@ def published_kernel_shapes(torch, stream, seed):
     out = {}
 
     def record(name, published_ms, seconds):
-        out[name] = {"us": round(seconds * 1e6, 1), "published_ms": published_ms,
-                     "speedup": round(published_ms * 1e-3 / seconds, 1)}
+        out[name] = {"us": round(seconds * 1e6, 1), "published_ms_on_other_hardware": published_ms}
 
     for dtype, label, ms in ((torch.float16, "F16", 0.1228), (torch.bfloat16, "BF16", 0.1230)):
         x, dy, w = rnd(512, 4096, dtype=dtype), rnd(512, 4096, dtype=dtype), rnd(4096, dtype=dtype)
@@ -289,16 +307,36 @@ def published_kernel_shapes(torch, stream, seed):
     return out
 
 
+def source_digest(name):
+    """sha256 of a kernel source file (the summaries under profiles/ record the one they were made with)."""
+    import hashlib
+
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "cgpt_amd", "csrc", name)
+    with open(path, "rb") as handle:
+        return hashlib.sha256(handle.read()).hexdigest()
+
+
 def measured_traffic():
-    """HBM bytes per launch of the probe kernel from the committed counter summary, or None."""
+    """(HBM bytes per launch of the probe kernel from the committed counter summary or None, note). The summary
+    names the sha256 of the kernel source it was measured with; when the source has changed since, the figure is
+    reported with a warning (stderr and `traffic_note`) instead of silently."""
+    value, recorded = None, None
     try:
         with open(TRAFFIC_FILE) as handle:
             for line in handle:
                 if line.startswith("traffic_bytes_per_launch"):
-                    return float(line.split("=")[1].split()[0])
+                    value = float(line.split("=")[1].split()[0])
+                if line.startswith("gemm_hip_sha256"):
+                    recorded = line.split("=")[1].strip()
     except OSError:
-        pass
-    return None
+        return None, "no counter summary found"
+    if value is None:
+        return None, "the counter summary holds no traffic figure"
+    if recorded is None or recorded != source_digest("gemm.hip"):
+        note = "STALE: cgpt_amd/csrc/gemm.hip has changed since profiles/gemm_dx_256x256_gate_projection_pmc.txt was measured"
+        print("bench.py: warning: roofline.traffic is " + note, file=sys.stderr)
+        return value, note
+    return value, "measured with the current cgpt_amd/csrc/gemm.hip"
 
 
 def cpu_model_name():
@@ -409,7 +447,7 @@ def main() -> int:
     parser.add_argument("--seed", type=int, default=0)
     parser.add_argument("--kernels-only", metavar="NAME", default=None,
                         help="run only the isolated operator launches whose name contains NAME (rmsnorm, rope, "
-                             "attention, swiglu, embedding, cut_cross_entropy, dense_cross_entropy, copy, secondary, published; several "
+                             "attention, swiglu, embedding, cut_cross_entropy, dense_cross_entropy, adamw, copy, secondary, published; several "
                              "separated by commas; '' = all) and print "
                              "their table: the target of per-kernel rocprofv3 runs")
     parser.add_argument("--probe-data", choices=["random", "zeros"], default="random",
@@ -427,6 +465,9 @@ def main() -> int:
 
     import torch
 
+    import ctypes
+
+    from cgpt_amd import capi
     from cgpt_amd.model import LOSS_CUT, LOSS_DENSE, Model, ModelConfig
     from cgpt_amd.ops import AdamWOptions
 
@@ -515,16 +556,56 @@ def main() -> int:
             launches[label] = {"m": m_, "n": n_, "k": k_, "calls": calls, "us_per_call": round(ms * 1e3 / calls, 1),
                                "tflops": round(tflops, 1), "frac": round(tflops / PEAK_BF16_TFLOPS, 4)}
     family = {kind: per_kind[kind]["frac"] for kind in ("gemm_fwd", "gemm_dx", "gemm_dw") if kind in per_kind}
+    # All event-timed launches of the probe kernel's instantiation in the step (plain, unsegmented dX with 256 x 256
+    # tiles: the gate/up and the output projection's input gradients, one each per layer), FLOPs over time.
+    same_kernel = [launches[label] for label in ("gemm_dx.gate_up", "gemm_dx.o") if label in launches]
+    weighted_flops = sum(2.0 * e["m"] * e["n"] * e["k"] * e["calls"] for e in same_kernel)
+    weighted_seconds = sum(e["us_per_call"] * 1e-6 * e["calls"] for e in same_kernel)
+    weighted_frac = weighted_flops / weighted_seconds / 1e12 / PEAK_BF16_TFLOPS if weighted_seconds > 0 else None
+    traffic, traffic_note = measured_traffic()
+    scratch_bytes = int(capi.lib().cgptx_scratch_bytes(ctypes.c_void_p(stream.cuda_stream)))
     kernels = {} if args.no_kernel_table else isolated_kernels(torch, cfg, args.batch, args.seq, dtype, stream, args.seed)
-    published = {} if args.no_kernel_table else published_kernel_shapes(torch, stream, args.seed)
-    # AdamW over all parameters (3 launches for all tensors): 30 B/parameter with 16-bit gradients and parameters.
-    options_probe = options
-    adamw_seconds = timed(torch, stream, lambda: model.optimizer_step(options_probe, stream), launches=5, warm=1)
+    # AdamW over the model's own parameters (3 launches for all tensors): 30 B/parameter with 16-bit gradients and
+    # parameters. (--kernels-only adamw runs the same update on a parameter list of its own.)
+    adamw_seconds = timed(torch, stream, lambda: model.optimizer_step(options, stream), launches=5, warm=1)
     adamw_bytes = 30.0 * model.num_parameters
     kernels["adamw_step_many_async"] = {
         "shape": f"{model.num_parameters} parameters in {2 + 11 * cfg.num_layers} tensors", "bound": "hbm", "us": round(adamw_seconds * 1e6, 1),
         "rate": round(adamw_bytes / adamw_seconds / 1e9, 1), "unit": "GB/s",
         "frac": round(adamw_bytes / adamw_seconds / 1e9 / PEAK_HBM_GBS, 4)}
+    num_parameters = model.num_parameters
+    model.close()
+    del model
+    capi.call("cgptx_release_scratch")
+    torch.cuda.empty_cache()
+
+    def secondary_step(batch, seq, step_dtype, step_loss):
+        """ms per step of another configuration of the same model (3 warm-up, 10 timed steps, hipGraph)."""
+        other = Model(ModelConfig(dtype=step_dtype), batch, seq, seed=args.seed, device=device)
+        other.set_tokens(rng.integers(0, cfg.vocabulary_size, size=(batch, seq)), rng.integers(0, cfg.vocabulary_size, size=(batch, seq)))
+        for _ in range(3):
+            other.train_step(options, step_loss, True, stream)
+        other.status(stream)
+        torch.cuda.synchronize()
+        begin = time.perf_counter()
+        for _ in range(10):
+            other.train_step(options, step_loss, True, stream)
+        stream.synchronize()
+        torch.cuda.synchronize()
+        seconds = (time.perf_counter() - begin) / 10
+        loss, finite, _ = other.status(stream)
+        other.close()
+        capi.call("cgptx_release_scratch")
+        torch.cuda.empty_cache()
+        return {"ms_per_step": round(seconds * 1e3, 3), "tokens_per_s": round(batch * seq / seconds, 1), "loss_last": loss,
+                "all_finite": bool(finite)}
+
+    secondary = {}
+    if args.shape == "104m" and not args.no_kernel_table:
+        secondary["bf16, B=8, T=4096, cut cross-entropy (the long-context variant of the configuration)"] = \
+            secondary_step(8, 4096, torch.bfloat16, LOSS_CUT)
+        secondary["f16, B=32, T=1024, dense cross-entropy (storage and loss of the reference's own published run)"] = \
+            secondary_step(32, 1024, torch.float16, LOSS_DENSE)
 
     result = {
         "metric": f"train tokens/sec, {args.shape} fwd+bwd+AdamW B={args.batch} T={args.seq}",
@@ -541,12 +622,18 @@ def main() -> int:
         "data": "synthetic",
         "config": {"workload": f"full {args.shape} train step (embedding, {cfg.num_layers} blocks, {args.loss} cross-entropy, backward, "
                                f"AdamW), B={args.batch}, T={args.seq}, hipGraph={'on' if use_graph else 'off'}",
-                   "parameters": model.num_parameters, "global_batch": args.batch, "seq_len": args.seq,
+                   "parameters": num_parameters, "global_batch": args.batch, "seq_len": args.seq,
                    "loss_scale": 1024.0},
+        "scratch_bytes": scratch_bytes,
+        "scratch_note": "device memory the operators of the step took beyond the caller's tensors (one arena per stream, sized "
+                        "by the largest request): with the cut cross-entropy it is the logits chunk, rows x vocabulary in "
+                        "the storage dtype",
+        "secondary_steps": secondary,
         "loss_after_warmup": loss_after_warmup, "loss_last": last_loss, "all_finite": bool(finite and finite_after),
         "optimizer_steps": steps_done,
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / PEAK_BF16_TFLOPS, "traffic": measured_traffic(),
+                     "frac": achieved / PEAK_BF16_TFLOPS, "traffic": traffic, "traffic_note": traffic_note,
+                     "frac_time_weighted": weighted_frac,
                      "kernel": PROBE_KERNEL, "launch_shape": probe["shape"],
                      "launch_us": in_step_seconds * 1e6, "launches_timed": cfg.num_layers,
                      "flops_per_launch": probe["flops"], "algorithmic_bytes_per_launch": probe["algorithmic_bytes"],
@@ -563,13 +650,12 @@ def main() -> int:
                              "breakdown), next to the best launch quoted as `frac`; gemm_launches = every contraction "
                              "by position in that pass; kernels = each backward operator alone at the configuration's "
                              "shape, 20 back-to-back launches between HIP events on the launch stream; "
-                             "published_kernel_shapes = the launches of the reference's own kernel table "
-                             "(kernel_profile.md:9-25, other hardware) on this GPU",
+                             "frac_time_weighted = FLOPs over time of all event-timed launches of the probe kernel's "
+                             "instantiation in the step (dX of the gate/up and of the output projection, every layer), "
+                             "beside the best launch quoted as `frac`",
                      "family_step_wide": family,
-                     "breakdown": per_kind, "gemm_launches": launches, "kernels": kernels,
-                     "published_kernel_shapes": published},
+                     "breakdown": per_kind, "gemm_launches": launches, "kernels": kernels},
     }
-    model.close()
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(args.seed)
     print(json.dumps(result))

@@ -114,7 +114,7 @@ PROTOTYPES = {
 }
 
 SIZE_FUNCTIONS = {"cgptx_model_parameter_count": [_vp], "cgptx_model_num_parameters": [_vp],
-                  "cgptx_model_profile_count": [_vp], "cgptx_model_call_count": [_vp]}
+                  "cgptx_model_profile_count": [_vp], "cgptx_model_call_count": [_vp], "cgptx_scratch_bytes": [_vp]}
 
 STRING_FUNCTIONS = ("cgptx_last_error", "cgptx_version")
 

@@ -4,12 +4,17 @@
 // preparation, batched update) and 269-435 (host entry points). The reference
 // launches two kernels per tensor (181 launches for the 104m model); here the
 // whole parameter list is covered by three launches:
-//   1. stats:   every block owns one 4096-element chunk of one tensor, reads the
-//               gradient with 128-bit loads and writes one partial Σ(g/scale)²;
-//               a non-finite value sets an integer flag.
+//   1. stats:   the tensors are cut into 4096-element chunks; a block takes eight
+//               consecutive chunks, requests all their 128-bit gradient loads
+//               before it adds anything and writes one partial Σ(g/scale)² per
+//               chunk; a non-finite value sets an integer flag.
 //   2. prepare: one block sums the partials in a fixed order (in double), decides
 //               skip / step++ / bias corrections / clip factor on the device.
-//   3. update:  same chunking; reads g, m, v, master, writes m, v, master, param.
+//   3. update:  one chunk per block; reads g, m, v, master, writes m, v, master, param.
+// The non-finite flag exists twice and the calls alternate between the two (the
+// call counter lives on the device, so a captured sequence alternates as well):
+// prepare clears the one the next call will use, which saves a launch that only
+// cleared a flag.
 // The block → (tensor, offset) map is a binary search in a small prefix table
 // that lives in the workspace. HBM traffic per parameter: g twice, m/v/master
 // read+write, param write = 30 B with 16-bit params.
@@ -45,12 +50,14 @@ struct Hyper {
 
 // Device-side scalars of one workspace.
 struct DeviceState {
-    unsigned int non_finite;
+    unsigned int non_finite;           // this call skips its update (set by prepare, read by update and the host)
     unsigned int observed_non_finite;
     unsigned long long step;
     float scalars[4];  // bias_correction1, bias_correction2, clip, unused
     float squared_norm;
-    float pad;
+    unsigned int calls;                // completed prepare passes; its parity picks the flag a call uses
+    unsigned int found_non_finite[2];  // set by the statistics pass of a call, cleared by the previous call's prepare
+    unsigned int pad[2];
 };
 
 __device__ __forceinline__ int find_entry(const unsigned int* __restrict__ chunk_begin, int entries,
@@ -74,86 +81,184 @@ __device__ __forceinline__ float block_sum(float v, float* stage) {
     return total;
 }
 
+constexpr int kStatsChunks = 4;  // consecutive chunks per block of the statistics pass
+
+// g / loss_scale. A power-of-two scale (the usual choice) divides exactly by multiplying with its reciprocal,
+// which takes one instruction instead of a dozen; any other scale is divided by, so that the value is the one
+// the update uses.
+struct Unscale {
+    float scale, reciprocal;
+    bool exact;  // reciprocal is a power of two
+};
+__device__ __forceinline__ float unscale(float g, const Unscale& s) { return s.exact ? g * s.reciprocal : g / s.scale; }
+
+// A non-finite gradient makes its sum non-finite (and so does an overflowing sum): the sums are checked, not
+// every element; the squared norm of a pass that found one is not used.
+// Σ (g / loss_scale)² over the calling thread's elements of one chunk (vector v = thread, thread + 256, ... of the
+// chunk, then the elements past the last whole vector), in that order; `bad` is set by a non-finite value.
+// Vector loads are requested together, before any arithmetic.
 template <typename T>
-__device__ __forceinline__ void stats_chunk(const T* __restrict__ g, unsigned long long begin, unsigned long long end,
-                                            float inv_scale_unused, float loss_scale, float& sum, bool& bad) {
+__device__ __forceinline__ float stats_chunk(const T* __restrict__ g, unsigned long long begin, unsigned long long end,
+                                             const Unscale& scale, bool& bad) {
     constexpr int VEC = kVec128<T>;
+    constexpr int kPasses = kChunk / (kThreads * VEC) > 0 ? kChunk / (kThreads * VEC) : 1;
     const bool aligned = (reinterpret_cast<std::uintptr_t>(g + begin) & 15u) == 0;
     const unsigned long long count = end - begin;
     const unsigned long long vectors = aligned ? count / VEC : 0;
-    for (unsigned long long v = threadIdx.x; v < vectors; v += kThreads) {
-        const vec_t<float, VEC> x = vec_to_f32<T, VEC>(load_vec<T, VEC>(g + begin + v * VEC));
+    float sum = 0.0f;
+    vec_t<T, VEC> held[kPasses];
+#pragma unroll
+    for (int k = 0; k < kPasses; ++k) {
+        const unsigned long long v = static_cast<unsigned long long>(k) * kThreads + threadIdx.x;
+        if (v < vectors) held[k] = load_vec<T, VEC>(g + begin + v * VEC);
+    }
+#pragma unroll
+    for (int k = 0; k < kPasses; ++k) {
+        const unsigned long long v = static_cast<unsigned long long>(k) * kThreads + threadIdx.x;
+        if (v >= vectors) continue;
+        const vec_t<float, VEC> x = vec_to_f32<T, VEC>(held[k]);
 #pragma unroll
         for (int e = 0; e < VEC; ++e) {
-            const float grad = x[e] / loss_scale;
-            if (isfinite(grad)) sum = fmaf(grad, grad, sum); else bad = true;
+            const float grad = unscale(x[e], scale);
+            sum = fmaf(grad, grad, sum);
         }
     }
     for (unsigned long long i = begin + vectors * VEC + threadIdx.x; i < end; i += kThreads) {
-        const float grad = to_f32(g[i]) / loss_scale;
-        if (isfinite(grad)) sum = fmaf(grad, grad, sum); else bad = true;
+        const float grad = unscale(to_f32(g[i]), scale);
+        sum = fmaf(grad, grad, sum);
+    }
+    if (!isfinite(sum)) bad = true;
+    return sum;
+}
+
+// kStatsChunks whole chunks of one tensor, 16-byte aligned: every load of the block is requested before the first
+// addition. The additions per chunk are those of stats_chunk, in its order.
+template <typename T>
+__device__ __forceinline__ void stats_run(const T* __restrict__ g, const Unscale& scale, float (&sums)[kStatsChunks], bool& bad) {
+    constexpr int VEC = kVec128<T>;
+    constexpr int kPasses = kChunk / (kThreads * VEC);
+    static_assert(kPasses >= 1 && kPasses * kThreads * VEC == kChunk, "a chunk is a whole number of block-wide vector passes");
+    vec_t<T, VEC> held[kStatsChunks][kPasses];
+#pragma unroll
+    for (int c = 0; c < kStatsChunks; ++c)
+#pragma unroll
+        for (int k = 0; k < kPasses; ++k) held[c][k] = load_vec<T, VEC>(g + c * kChunk + (k * kThreads + threadIdx.x) * VEC);
+#pragma unroll
+    for (int c = 0; c < kStatsChunks; ++c) {
+        float sum = 0.0f;
+#pragma unroll
+        for (int k = 0; k < kPasses; ++k) {
+            const vec_t<float, VEC> x = vec_to_f32<T, VEC>(held[c][k]);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                const float grad = unscale(x[e], scale);
+                sum = fmaf(grad, grad, sum);
+            }
+        }
+        if (!isfinite(sum)) bad = true;
+        sums[c] = sum;
     }
 }
 
 __global__ __launch_bounds__(kThreads) void adamw_stats_kernel(const DeviceEntry* __restrict__ entries,
                                                               const unsigned int* __restrict__ chunk_begin,
-                                                              int entry_count, float loss_scale,
+                                                              int entry_count, unsigned int total_chunks, float loss_scale,
                                                               float* __restrict__ partial, DeviceState* state) {
-    __shared__ float stage[kThreads / kWave];
+    __shared__ float stage[kStatsChunks][kThreads / kWave];
     __shared__ int any_bad;
     if (threadIdx.x == 0) any_bad = 0;
     __syncthreads();
-    const int e = find_entry(chunk_begin, entry_count, blockIdx.x);
-    const DeviceEntry entry = entries[e];
-    const unsigned long long begin = static_cast<unsigned long long>(blockIdx.x - chunk_begin[e]) * kChunk;
-    const unsigned long long end = begin + kChunk < entry.count ? begin + kChunk : entry.count;
-    float sum = 0.0f;
+    const unsigned int first_chunk = blockIdx.x * kStatsChunks;
+    // The tensor of the block's first chunk is found by bisection, those of the following chunks by stepping on.
+    int e = find_entry(chunk_begin, entry_count, first_chunk);
+    float sums[kStatsChunks];
     bool bad = false;
-    switch (entry.dtype) {
-        case CGPTX_F16: stats_chunk(static_cast<const f16_t*>(entry.gradient), begin, end, 0.f, loss_scale, sum, bad); break;
-        case CGPTX_BF16: stats_chunk(static_cast<const bf16_t*>(entry.gradient), begin, end, 0.f, loss_scale, sum, bad); break;
-        default: stats_chunk(static_cast<const float*>(entry.gradient), begin, end, 0.f, loss_scale, sum, bad); break;
+    int exponent = 0;
+    const Unscale scale{loss_scale, 1.0f / loss_scale, frexpf(loss_scale, &exponent) == 0.5f};
+    const DeviceEntry head = entries[e];
+    const unsigned long long head_begin = static_cast<unsigned long long>(first_chunk - chunk_begin[e]) * kChunk;
+    const std::size_t elem = head.dtype == CGPTX_F32 ? 4 : 2;
+    const bool whole_run = head_begin + static_cast<unsigned long long>(kStatsChunks) * kChunk <= head.count &&
+                           ((reinterpret_cast<std::uintptr_t>(head.gradient) + head_begin * elem) & 15u) == 0;
+    if (whole_run) {
+        switch (head.dtype) {
+            case CGPTX_F16: stats_run(static_cast<const f16_t*>(head.gradient) + head_begin, scale, sums, bad); break;
+            case CGPTX_BF16: stats_run(static_cast<const bf16_t*>(head.gradient) + head_begin, scale, sums, bad); break;
+            default: stats_run(static_cast<const float*>(head.gradient) + head_begin, scale, sums, bad); break;
+        }
+    } else {
+#pragma unroll
+        for (int c = 0; c < kStatsChunks; ++c) {
+            const unsigned int chunk = first_chunk + c;
+            sums[c] = 0.0f;
+            if (chunk >= total_chunks) continue;
+            while (chunk >= chunk_begin[e + 1]) ++e;
+            const DeviceEntry entry = entries[e];
+            const unsigned long long begin = static_cast<unsigned long long>(chunk - chunk_begin[e]) * kChunk;
+            const unsigned long long end = begin + kChunk < entry.count ? begin + kChunk : entry.count;
+            switch (entry.dtype) {
+                case CGPTX_F16: sums[c] = stats_chunk(static_cast<const f16_t*>(entry.gradient), begin, end, scale, bad); break;
+                case CGPTX_BF16: sums[c] = stats_chunk(static_cast<const bf16_t*>(entry.gradient), begin, end, scale, bad); break;
+                default: sums[c] = stats_chunk(static_cast<const float*>(entry.gradient), begin, end, scale, bad); break;
+            }
+        }
     }
     if (bad) any_bad = 1;  // benign race: every writer stores 1
-    const float total = block_sum(sum, stage);
-    if (threadIdx.x == 0) {
-        partial[blockIdx.x] = total;
-        if (any_bad) atomicExch(&state->non_finite, 1u);
+    // One partial per chunk: lanes of a wavefront by butterfly, then the wavefronts in order.
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+#pragma unroll
+    for (int c = 0; c < kStatsChunks; ++c) {
+        const float v = wave_sum(sums[c]);
+        if (lane == 0) stage[c][wave] = v;
     }
+    __syncthreads();
+    if (threadIdx.x < kStatsChunks && first_chunk + threadIdx.x < total_chunks) {
+        float total = 0.0f;
+#pragma unroll
+        for (int w = 0; w < kThreads / kWave; ++w) total += stage[threadIdx.x][w];
+        partial[first_chunk + threadIdx.x] = total;
+    }
+    if (threadIdx.x == 0 && any_bad) atomicExch(&state->found_non_finite[state->calls & 1u], 1u);
 }
 
 // One block. Fixed-order sum of the partials, then the decision logic of
 // adamw_prepare_step_kernel (src/optim/adamw.cu:166-187).
-__global__ __launch_bounds__(kThreads) void adamw_prepare_kernel(const float* __restrict__ partial,
-                                                                unsigned int partial_count, DeviceState* state,
-                                                                float beta1, float beta2, float max_grad_norm,
-                                                                int advance_step) {
-    __shared__ double stage[kThreads];
+constexpr int kPrepareThreads = 1024;
+__global__ __launch_bounds__(kPrepareThreads) void adamw_prepare_kernel(const float* __restrict__ partial,
+                                                                       unsigned int partial_count, DeviceState* state,
+                                                                       float beta1, float beta2, float max_grad_norm,
+                                                                       int advance_step) {
+    __shared__ double stage[kPrepareThreads];
     // Four independent sums per thread keep four loads in flight (one block adds some 25,000 partials for the 104m
     // model); the order of the additions is fixed by the partial count alone.
     double s0 = 0.0, s1 = 0.0, s2 = 0.0, s3 = 0.0;
     unsigned int i = threadIdx.x;
-    for (; i + 3 * kThreads < partial_count; i += 4 * kThreads) {
+    for (; i + 3 * kPrepareThreads < partial_count; i += 4 * kPrepareThreads) {
         s0 += static_cast<double>(partial[i]);
-        s1 += static_cast<double>(partial[i + kThreads]);
-        s2 += static_cast<double>(partial[i + 2 * kThreads]);
-        s3 += static_cast<double>(partial[i + 3 * kThreads]);
+        s1 += static_cast<double>(partial[i + kPrepareThreads]);
+        s2 += static_cast<double>(partial[i + 2 * kPrepareThreads]);
+        s3 += static_cast<double>(partial[i + 3 * kPrepareThreads]);
     }
-    for (; i < partial_count; i += kThreads) s0 += static_cast<double>(partial[i]);
+    for (; i < partial_count; i += kPrepareThreads) s0 += static_cast<double>(partial[i]);
     stage[threadIdx.x] = (s0 + s1) + (s2 + s3);
     __syncthreads();
-    for (int stride = kThreads / 2; stride > 0; stride >>= 1) {
+    for (int stride = kPrepareThreads / 2; stride > 0; stride >>= 1) {
         if (threadIdx.x < stride) stage[threadIdx.x] += stage[threadIdx.x + stride];
         __syncthreads();
     }
     if (threadIdx.x != 0) return;
     const float squared = static_cast<float>(stage[0]);
     state->squared_norm = squared;
-    if (state->non_finite != 0u || !isfinite(squared)) {
+    const unsigned int parity = state->calls & 1u;
+    const bool found = state->found_non_finite[parity] != 0u;
+    state->found_non_finite[parity ^ 1u] = 0u;  // the flag of the next call
+    state->calls += 1u;
+    if (found || !isfinite(squared)) {
         state->non_finite = 1u;
         state->observed_non_finite = 1u;
         return;
     }
+    state->non_finite = 0u;
     if (advance_step) {
         const unsigned long long next_step = state->step + 1ull;
         state->step = next_step;
@@ -166,11 +271,6 @@ __global__ __launch_bounds__(kThreads) void adamw_prepare_kernel(const float* __
         const float norm = sqrtf(squared);
         state->scalars[2] = norm > max_grad_norm ? max_grad_norm / norm : 1.0f;
     }
-}
-
-__global__ void adamw_reset_kernel(DeviceState* state) {
-    state->non_finite = 0u;
-    state->squared_norm = 0.0f;
 }
 
 __device__ __forceinline__ void adamw_element(float grad_raw, float& m, float& v, float& master, const Hyper& h,
@@ -412,12 +512,10 @@ extern "C" int cgptx_adamw_step_many_async(cgptx_adamw_workspace* ws, const cgpt
     }
     const Hyper h = to_hyper(*options);
     const int n = static_cast<int>(entry_count);
-    hipLaunchKernelGGL(adamw_reset_kernel, dim3(1), dim3(1), 0, stream, ws->state);
+    hipLaunchKernelGGL(adamw_stats_kernel, dim3((ws->total_chunks + kStatsChunks - 1) / kStatsChunks), dim3(kThreads), 0, stream,
+                       ws->entries, ws->chunk_begin, n, ws->total_chunks, h.loss_scale, ws->partial, ws->state);
     CGPTX_LAUNCH_CHECK();
-    hipLaunchKernelGGL(adamw_stats_kernel, dim3(ws->total_chunks), dim3(kThreads), 0, stream, ws->entries,
-                       ws->chunk_begin, n, h.loss_scale, ws->partial, ws->state);
-    CGPTX_LAUNCH_CHECK();
-    hipLaunchKernelGGL(adamw_prepare_kernel, dim3(1), dim3(kThreads), 0, stream, ws->partial, ws->total_chunks,
+    hipLaunchKernelGGL(adamw_prepare_kernel, dim3(1), dim3(kPrepareThreads), 0, stream, ws->partial, ws->total_chunks,
                        ws->state, h.beta1, h.beta2, h.max_grad_norm, 1);
     CGPTX_LAUNCH_CHECK();
     hipLaunchKernelGGL(adamw_update_kernel, dim3(ws->total_chunks), dim3(kThreads), 0, stream, ws->entries,
@@ -472,10 +570,11 @@ extern "C" int cgptx_adamw_step(void* parameter, const void* gradient, float* ma
     CGPTX_HIP(hipMemcpy(d_entry, &h_entry, sizeof(h_entry), hipMemcpyHostToDevice));
     CGPTX_HIP(hipMemcpy(d_begin, h_begin, sizeof(h_begin), hipMemcpyHostToDevice));
     const Hyper h = to_hyper(*options);
-    hipLaunchKernelGGL(adamw_stats_kernel, dim3(static_cast<unsigned int>(chunks)), dim3(kThreads), 0, stream,
-                       d_entry, d_begin, 1, h.loss_scale, partial, state);
+    hipLaunchKernelGGL(adamw_stats_kernel, dim3(static_cast<unsigned int>((chunks + kStatsChunks - 1) / kStatsChunks)),
+                       dim3(kThreads), 0, stream, d_entry, d_begin, 1, static_cast<unsigned int>(chunks), h.loss_scale, partial,
+                       state);
     CGPTX_LAUNCH_CHECK();
-    hipLaunchKernelGGL(adamw_prepare_kernel, dim3(1), dim3(kThreads), 0, stream, partial,
+    hipLaunchKernelGGL(adamw_prepare_kernel, dim3(1), dim3(kPrepareThreads), 0, stream, partial,
                        static_cast<unsigned int>(chunks), state, h.beta1, h.beta2, h.max_grad_norm, 0);
     CGPTX_LAUNCH_CHECK();
     // Bias corrections in double on the host, as adamw_step does (src/optim/adamw.cu:413-415).

@@ -5,13 +5,15 @@
 //   z = X·Cᵀ, loss = mean_r(logsumexp z_r − z_{r,y_r}),
 //   dX = (softmax(z) − onehot)·C / rows, dC = (softmax(z) − onehot)ᵀ·X / rows.
 // The reference recomputes full dot products per thread (O(rows·hidden²·vocab)), which
-// cannot run at training size. Here rows are processed in chunks: one MFMA contraction
-// produces the chunk's logits into scratch, the softmax kernel turns them into the
-// scaled logit gradient in place, and two more contractions consume that gradient
-// (dX for the chunk's rows; dC accumulated in fp32 across chunks, so the classifier
-// gradient is rounded once). Scratch is chunk·vocab logits + vocab·hidden fp32,
-// independent of the number of rows, and three vocabulary-sized contractions are done
-// instead of four because the chunk's logits stay resident between loss and gradient.
+// cannot run at training size. Here rows are processed in chunks of at most 1 GiB of logits: one
+// MFMA contraction produces the chunk's logits into scratch, the softmax kernel turns them into
+// the scaled logit gradient in place, and two more contractions consume that gradient (dX for the
+// chunk's rows; dC accumulated in fp32 across chunks — the last chunk's contraction adds the
+// accumulator in its epilogue — so the classifier gradient is rounded once; a single chunk writes
+// it straight out of its contraction, which rounds the same sum in another order of additions).
+// Scratch is chunk·vocab logits + vocab·hidden fp32, independent of the number of rows, and three
+// vocabulary-sized contractions are done instead of four because the chunk's logits stay resident
+// between loss and gradient.
 //
 // Extensions over the reference: any storage dtype, a gradient scale (loss scaling),
 // and accumulate_classifier for tied embeddings.
@@ -22,27 +24,6 @@
 #include <cmath>
 #include <cstdlib>
 #include <limits>
-
-namespace cgptx {
-namespace {
-
-constexpr int kThreads = 256;
-
-// out = (accumulate ? out : 0) + acc, element-wise, acc in fp32.
-template <typename T>
-__global__ __launch_bounds__(kThreads) void finish_classifier_kernel(T* __restrict__ out,
-                                                                    const float* __restrict__ acc,
-                                                                    std::size_t count, int accumulate) {
-    for (std::size_t i = static_cast<std::size_t>(blockIdx.x) * kThreads + threadIdx.x; i < count;
-         i += static_cast<std::size_t>(gridDim.x) * kThreads) {
-        float v = acc[i];
-        if (accumulate) v += to_f32(out[i]);
-        out[i] = from_f32<T>(v);
-    }
-}
-
-}  // namespace
-}  // namespace cgptx
 
 extern "C" int cgptx_cut_cross_entropy_forward_backward(float* loss, void* input_gradient, void* classifier_gradient,
                                                         const void* input, const void* classifier,
@@ -63,15 +44,15 @@ extern "C" int cgptx_cut_cross_entropy_forward_backward(float* loss, void* input
         return fail(CGPTX_OVERFLOW, std::string(name) + ": dimension exceeds int range");
     auto stream = static_cast<hipStream_t>(stream_);
     const std::size_t elem = dtype_size(dtype);
-    // Chunk so that the logits scratch stays within 2 GiB whatever the number of rows (a small fraction of this
-    // GPU's memory; CGPTX_CUT_CE_LOGITS_BYTES, read per call, sets another bound), while each chunk still gives
-    // the three contractions enough 256x256 tiles to fill the chip. The rows are split evenly over the chunks.
-    // 32768 rows at V=32000 are one chunk: the classifier gradient then comes straight out of its contraction,
-    // rounded once, without the fp32 accumulator and the pass that folds it into the gradient.
-    // The bound itself stays 1 MiB under 2^31: the streamed contraction kernels address an operand with 32-bit
-    // byte offsets below that, and a chunk beyond it would fall back to the plain kernels.
+    // Rows are processed in chunks so that the logits scratch stays within 1 GiB whatever the number of rows
+    // (CGPTX_CUT_CE_LOGITS_BYTES, read per call, sets another bound, up to 2 GiB - 1 MiB: the streamed contraction
+    // kernels address an operand with 32-bit byte offsets below that). The rows are split evenly over the chunks.
+    // At V = 32000 in 16-bit storage the bound gives chunks of 16384 rows, which still fill the chip: 64 x 4 tiles
+    // of a chunk's input gradient, one per compute unit. Measured at [32768, 1024] x [32000, 1024]: 1 GiB costs
+    // nothing against one 2 GiB chunk (6.04 - 6.12 against 6.03 - 6.05 ms), 512 MiB 3.5 % (the input gradient of an
+    // 8192-row chunk has to be split along K), 256 MiB 8 %.
     constexpr std::size_t kMaxLogitsBytes = (std::size_t{1} << 31) - (std::size_t{1} << 20);
-    std::size_t logits_bytes = kMaxLogitsBytes;
+    std::size_t logits_bytes = std::size_t{1} << 30;
     if (const char* text = std::getenv("CGPTX_CUT_CE_LOGITS_BYTES")) {
         const unsigned long long asked = std::strtoull(text, nullptr, 0);
         if (asked > 0) logits_bytes = std::min<std::size_t>(static_cast<std::size_t>(asked), kMaxLogitsBytes);
@@ -85,14 +66,20 @@ extern "C" int cgptx_cut_cross_entropy_forward_backward(float* loss, void* input
     const std::size_t loss_bytes = (rows * sizeof(float) + 255) & ~std::size_t{255};
     const std::size_t acc_bytes = single ? 0 : (vocab * hidden * sizeof(float) + 255) & ~std::size_t{255};
     const std::size_t logit_bytes = (chunk * vocab * elem + 255) & ~std::size_t{255};
+    // A chunk's input gradient has few output tiles ([chunk, hidden]) and a long K (the vocabulary): with several
+    // chunks it is split along K into up to `units / tiles` slices, whose fp32 partial tiles need room of their own.
+    const std::size_t dx_tiles = ((chunk + 255) / 256) * ((hidden + 255) / 256);
+    const std::size_t dx_slices = single ? 1 : std::max<std::size_t>(1, static_cast<std::size_t>(compute_units()) / std::max<std::size_t>(dx_tiles, 1));
+    const std::size_t split_bytes = dx_slices > 1 ? (dx_slices * chunk * hidden * sizeof(float) + 255) & ~std::size_t{255} : 0;
     void* mem = nullptr;
-    // Arena layout: [row_loss | acc | logits]. The contractions below run with no_split, so they
-    // never ask the arena for split-K scratch of their own.
-    if (int s = scratch(stream, loss_bytes + acc_bytes + logit_bytes, &mem)) return s;
+    // Arena layout: [row_loss | acc | split-K partials | logits]. The contractions below run with no_split: they
+    // never ask the arena for scratch of their own, and split only into the room given to them here.
+    if (int s = scratch(stream, loss_bytes + acc_bytes + split_bytes + logit_bytes, &mem)) return s;
     auto* base = static_cast<char*>(mem);
     auto* row_loss = reinterpret_cast<float*>(base);
     auto* acc = reinterpret_cast<float*>(base + loss_bytes);
-    void* logits = base + loss_bytes + acc_bytes;
+    void* split_room = split_bytes != 0 ? base + loss_bytes + acc_bytes : nullptr;
+    void* logits = base + loss_bytes + acc_bytes + split_bytes;
     const float factor = gradient_scale / static_cast<float>(rows);
     for (std::size_t r0 = 0; r0 < rows; r0 += chunk) {
         const std::size_t r = std::min(chunk, rows - r0);
@@ -125,11 +112,17 @@ extern "C" int cgptx_cut_cross_entropy_forward_backward(float* loss, void* input
         dx.b_k_contiguous = false;
         dx.dtype = dtype;
         dx.no_split = true;
+        dx.split_workspace = split_room;
+        dx.split_workspace_bytes = split_bytes;
         if (int s = gemm(dx, stream)) return s;
-        GemmArgs dc;  // acc[V, H] (+)= dZᵀ[V, r]·X[r, H], fp32; a single chunk writes the gradient itself
+        // dC = Σ_chunks dZᵀ[V, r]·X[r, H]: all chunks but the last add their product to acc (fp32; the first one
+        // starts it), the last one adds acc to its own and writes the gradient, rounded once. A single chunk
+        // writes the gradient itself.
+        const bool last = r0 + chunk >= rows;
+        GemmArgs dc;
         dc.a = logits;
         dc.b = x;
-        dc.c = single ? classifier_gradient : static_cast<void*>(acc);
+        dc.c = last ? classifier_gradient : static_cast<void*>(acc);
         dc.m = vocab;
         dc.n = hidden;
         dc.k = r;
@@ -138,21 +131,15 @@ extern "C" int cgptx_cut_cross_entropy_forward_backward(float* loss, void* input
         dc.ldc = hidden;
         dc.a_k_contiguous = false;
         dc.b_k_contiguous = false;
-        dc.accumulate = single ? accumulate_classifier != 0 : r0 != 0;
-        dc.c_is_f32 = !single;
+        dc.accumulate = last ? accumulate_classifier != 0 : r0 != 0;
+        dc.c_is_f32 = !last;
+        if (last && !single) {
+            dc.addend_f32 = acc;
+            dc.ld_addend = hidden;
+        }
         dc.dtype = dtype;
         dc.no_split = true;
         if (int s = gemm(dc, stream)) return s;
     }
-    if (int s = mean_reduce(loss, row_loss, rows, stream)) return s;
-    if (single) return CGPTX_OK;
-    const std::size_t count = vocab * hidden;
-    const std::size_t blocks = std::min<std::size_t>((count + kThreads - 1) / kThreads,
-                                                     static_cast<std::size_t>(compute_units()) * 16);
-    return dispatch_dtype(dtype, [&]<typename T>() -> int {
-        hipLaunchKernelGGL((finish_classifier_kernel<T>), dim3(static_cast<unsigned int>(blocks)), dim3(kThreads), 0,
-                           stream, static_cast<T*>(classifier_gradient), acc, count, accumulate_classifier);
-        CGPTX_LAUNCH_CHECK();
-        return CGPTX_OK;
-    });
+    return mean_reduce(loss, row_loss, rows, stream);
 }

@@ -30,12 +30,40 @@ constexpr int kWavesPerBlock = kThreads / kWave;
 // offsets[id] .. offsets[id + 1] is id's segment of `order`; ids >= vocab belong to nobody and are skipped.
 constexpr int kGroupThreads = 1024;
 constexpr unsigned int kGroupMaxIds = 32768;  // LDS histogram entries of one workgroup (128 KiB)
+constexpr int kGroupBatch = 8;                // 128-bit id loads a thread keeps in flight
+
+// The id list is walked in batches of kGroupBatch x 4 ids per thread, all of a batch's loads requested before the
+// first id is looked at (one dependent load per id would cost a memory round trip each). visit(id, t) sees every
+// token once; the order within a workgroup does not matter to any caller.
+template <typename Visit>
+__device__ __forceinline__ void for_each_id(const std::uint32_t* __restrict__ ids, unsigned int count, bool aligned, Visit&& visit) {
+    using u32x4 = vec_t<unsigned int, 4>;
+    const unsigned int quads = aligned ? count / 4 : 0;
+    const auto* wide = reinterpret_cast<const u32x4*>(ids);
+    for (unsigned int base = 0; base < quads; base += kGroupBatch * kGroupThreads) {
+        u32x4 held[kGroupBatch];
+#pragma unroll
+        for (int k = 0; k < kGroupBatch; ++k) {
+            const unsigned int q = base + k * kGroupThreads + threadIdx.x;
+            if (q < quads) held[k] = wide[q];
+        }
+#pragma unroll
+        for (int k = 0; k < kGroupBatch; ++k) {
+            const unsigned int q = base + k * kGroupThreads + threadIdx.x;
+            if (q < quads) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) visit(held[k][e], 4 * q + e);
+            }
+        }
+    }
+    for (unsigned int t = 4 * quads + threadIdx.x; t < count; t += kGroupThreads) visit(ids[t], t);
+}
 
 __global__ __launch_bounds__(kGroupThreads) void embedding_group_kernel(unsigned int* __restrict__ offsets,
                                                                        unsigned int* __restrict__ order,
                                                                        const std::uint32_t* __restrict__ ids,
                                                                        unsigned int count, unsigned int vocab,
-                                                                       unsigned int ids_per_group) {
+                                                                       unsigned int ids_per_group, bool aligned) {
     extern __shared__ unsigned int bins[];  // [ids_per_group]
     __shared__ unsigned int wave_totals[kGroupThreads / kWave];
     __shared__ unsigned int smaller_total;
@@ -46,11 +74,10 @@ __global__ __launch_bounds__(kGroupThreads) void embedding_group_kernel(unsigned
     if (tid == 0) smaller_total = 0;
     __syncthreads();
     unsigned int smaller = 0;
-    for (unsigned int t = tid; t < count; t += kGroupThreads) {
-        const unsigned int id = ids[t];
+    for_each_id(ids, count, aligned, [&](unsigned int id, unsigned int) {
         if (id < lo) ++smaller;
         else if (id - lo < width) atomicAdd(&bins[id - lo], 1u);
-    }
+    });
 #pragma unroll
     for (int offset = kWave / 2; offset > 0; offset >>= 1) smaller += __shfl_xor(smaller, offset, kWave);
     if (lane == 0 && smaller != 0) atomicAdd(&smaller_total, smaller);
@@ -80,10 +107,9 @@ __global__ __launch_bounds__(kGroupThreads) void embedding_group_kernel(unsigned
     }
     if (lo + width == vocab && tid == kGroupThreads - 1) offsets[vocab] = running;  // the piece that ends the last range
     __syncthreads();
-    for (unsigned int t = tid; t < count; t += kGroupThreads) {
-        const unsigned int id = ids[t];
+    for_each_id(ids, count, aligned, [&](unsigned int id, unsigned int t) {
         if (id >= lo && id - lo < width) order[atomicAdd(&bins[id - lo], 1u)] = t;
-    }
+    });
 }
 
 // ---- rows: one wavefront per vocabulary row -------------------------------------------------------
@@ -225,7 +251,7 @@ extern "C" int cgptx_embedding_backward(void* grad_weight, const void* grad_outp
         }
     }
     hipLaunchKernelGGL(embedding_group_kernel, dim3(groups), dim3(kGroupThreads), group_lds, stream, offsets, order, token_ids,
-                       count, v, ids_per_group);
+                       count, v, ids_per_group, is_aligned16(token_ids));
     CGPTX_LAUNCH_CHECK();
     return dispatch_dtype(dtype, [&]<typename T>() -> int {
         auto* dw = static_cast<T*>(grad_weight);

@@ -109,6 +109,8 @@ struct KernelArgs {
     void* c;            // T* (or float* when c_f32), or float partials when split
     const void* bias;
     const void* residual;  // T*, row stride ldr, or null
+    const float* addend;   // fp32 [M, N], row stride ld_addend, added before anything else, or null
+    long ld_addend;
     int m, n, k;
     long lda, ldb, ldc, ldr;
     int tiles_m, tiles_n;
@@ -833,7 +835,7 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
             return;
         }
         bool plain = false;
-        if constexpr (!SPLIT) plain = p.bias == nullptr && p.residual == nullptr && !p.accumulate && !p.c_f32;
+        if constexpr (!SPLIT) plain = p.bias == nullptr && p.residual == nullptr && p.addend == nullptr && !p.accumulate && !p.c_f32;
         if (plain) {
             // Straight-line code, no per-lane predicates or address arithmetic (with one wavefront per
             // SIMD every branch and every dependent wait is exposed): the stores go through a buffer
@@ -911,6 +913,11 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
                     vec_t<float, 4> v1 = *reinterpret_cast<const vec_t<float, 4>*>(hi);
                     if (m >= p.m || c_col >= c_cols) return;
                     {
+                        if (p.addend != nullptr) {
+                            const float* addend = p.addend + static_cast<long>(m) * p.ld_addend + n;
+                            v0 += *reinterpret_cast<const vec_t<float, 4>*>(addend);
+                            v1 += *reinterpret_cast<const vec_t<float, 4>*>(addend + 4);
+                        }
                         if (p.bias != nullptr) {
                             const T* bias = static_cast<const T*>(p.bias) + n;
                             v0 += vec_to_f32<T, 4>(load_vec<T, 4>(bias));
@@ -1125,6 +1132,7 @@ __global__ __launch_bounds__(kGenericTile* kGenericTile / 4) void gemm_generic_k
             const long m = m0 + ty + 16 * i, n = n0 + tx + 16 * j;
             if (m >= p.m || n >= p.n) continue;
             float v = acc[i][j];
+            if (p.addend != nullptr) v += p.addend[m * p.ld_addend + n];
             if (p.bias != nullptr) v += to_f32(static_cast<const T*>(p.bias)[n]);
             if (p.residual != nullptr) v += to_f32(static_cast<const T*>(p.residual)[static_cast<long>(m) * p.ldr + n]);
             if (p.c_f32) {
@@ -1188,7 +1196,7 @@ int launch_layout(const KernelArgs& p, bool a_k, bool b_k, int slices, hipStream
     }
     if (p.saved != nullptr) return fail(CGPTX_RUNTIME, "gemm: the SwiGLU gradient epilogue needs 256-wide unsplit tiles");
     if constexpr (!SPLIT) {
-        if (a_k && b_k && p.bias == nullptr && !p.c_f32) {
+        if (a_k && b_k && p.bias == nullptr && p.addend == nullptr && !p.c_f32) {
             if (p.residual != nullptr && !p.accumulate) return launch_mfma<T, BM, BN, true, true, false, false, true>(p, slices, stream);
             if (p.residual == nullptr && p.accumulate && p.c_seg.count == 0) {
                 // C += A·B in the storage dtype is the same epilogue with C as its own residual
@@ -1227,7 +1235,8 @@ int run_config(const GemmArgs& g, KernelArgs p, hipStream_t stream) {
     const long want_blocks = static_cast<long>(compute_units()) * (BM == 256 ? 1 : 2);
     int slices = 1;
     const bool k_segments = g.a_k_contiguous && g.a_segments.count > 0;
-    if (!g.no_split && g.residual == nullptr && g.swiglu_out == nullptr && g.swiglu_saved == nullptr &&
+    const bool may_split = !g.no_split || g.split_workspace != nullptr;
+    if (may_split && g.residual == nullptr && g.addend_f32 == nullptr && g.swiglu_out == nullptr && g.swiglu_saved == nullptr &&
         g.c_segments.count == 0 && !k_segments &&
         tiles < want_blocks && k_tiles >= 32) {
         // As many slices as fit the CU slots in one go: one item more than that would cost a
@@ -1235,11 +1244,14 @@ int run_config(const GemmArgs& g, KernelArgs p, hipStream_t stream) {
         slices = static_cast<int>(std::min<long>(want_blocks / tiles, k_tiles / 16));
         if (slices < 1) slices = 1;
     }
+    if (g.no_split && static_cast<std::size_t>(slices) * g.m * g.n * sizeof(float) > g.split_workspace_bytes) slices = 1;
     p.k_tiles_per_slice = (k_tiles + slices - 1) / slices;
     slices = (k_tiles + p.k_tiles_per_slice - 1) / p.k_tiles_per_slice;
     if (slices == 1) return launch_layout<T, BM, BN, false>(p, g.a_k_contiguous, g.b_k_contiguous, 1, stream);
-    void* mem = nullptr;
-    if (int s = scratch(stream, static_cast<std::size_t>(slices) * g.m * g.n * sizeof(float), &mem)) return s;
+    void* mem = g.no_split ? g.split_workspace : nullptr;
+    if (mem == nullptr) {
+        if (int s = scratch(stream, static_cast<std::size_t>(slices) * g.m * g.n * sizeof(float), &mem)) return s;
+    }
     KernelArgs split = p;
     split.c = mem;
     if (int s = launch_layout<T, BM, BN, true>(split, g.a_k_contiguous, g.b_k_contiguous, slices, stream)) return s;
@@ -1300,6 +1312,8 @@ int run_typed(const GemmArgs& g, hipStream_t stream) {
     p.bias = g.bias;
     p.residual = g.residual;
     p.ldr = static_cast<long>(g.ldr);
+    p.addend = g.addend_f32;
+    p.ld_addend = static_cast<long>(g.ld_addend);
     p.m = static_cast<int>(g.m);
     p.n = static_cast<int>(g.n);
     p.k = static_cast<int>(g.k);
@@ -1347,6 +1361,7 @@ int run_typed(const GemmArgs& g, hipStream_t stream) {
                is_aligned16(g.a) && is_aligned16(g.b) && (g.ldc * c_elem) % 16 == 0 && is_aligned16(g.c) &&
                (g.bias == nullptr || (reinterpret_cast<std::uintptr_t>(g.bias) & 7u) == 0) &&
                (g.residual == nullptr || ((reinterpret_cast<std::uintptr_t>(g.residual) & 7u) == 0 && g.ldr % 4 == 0)) &&
+               (g.addend_f32 == nullptr || (is_aligned16(g.addend_f32) && g.ld_addend % 4 == 0)) &&
                !(!g.a_k_contiguous && g.b_k_contiguous) && offsets_fit_32bit(g, sizeof(T));
     }
     if (!fast && segmented) return fail(CGPTX_INVALID_ARGUMENT, "gemm: segmented operands need the aligned MFMA path");
@@ -1367,7 +1382,8 @@ int run_typed(const GemmArgs& g, hipStream_t stream) {
         const int forced = forced_tile();
         const long units = compute_units();
         const bool fills = big_tiles * 5 >= units * 4;
-        const bool splits = !g.no_split && g.residual == nullptr && g.c_segments.count == 0 && big_tiles >= 8 &&
+        const bool splits = (!g.no_split || g.split_workspace != nullptr) && g.residual == nullptr && g.addend_f32 == nullptr &&
+                            g.c_segments.count == 0 && big_tiles >= 8 &&
                             g.k / kBK >= static_cast<std::size_t>(32 * ((units + big_tiles - 1) / big_tiles));
         const bool big = g.swiglu_out != nullptr || g.swiglu_saved != nullptr || forced == 256 || (forced == 0 && (fills || splits));
         if (big) return run_config<T, 256, 256>(g, p, stream);

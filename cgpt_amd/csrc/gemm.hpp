@@ -27,6 +27,8 @@ struct GemmArgs {
     void* c = nullptr;
     const void* bias = nullptr;
     const void* residual = nullptr;
+    const float* addend_f32 = nullptr;  // optional fp32 [M, N] (row stride ld_addend) added to the product first
+    std::size_t ld_addend = 0;
     std::size_t m = 0, n = 0, k = 0;
     std::size_t lda = 0, ldb = 0, ldc = 0, ldr = 0;
     bool a_k_contiguous = true;
@@ -34,6 +36,10 @@ struct GemmArgs {
     bool accumulate = false;
     bool c_is_f32 = false;
     bool no_split = false;  // never use split-K scratch (the caller owns the arena)
+    // Memory for split-K partial tiles from a caller that owns the arena (used instead of the arena when the
+    // launch is split along K; a launch whose partials would not fit runs unsplit).
+    void* split_workspace = nullptr;
+    std::size_t split_workspace_bytes = 0;
     int dtype = CGPTX_BF16;
     // Column segments of A as stored (its K range when k-contiguous, its M range otherwise) and of
     // C (written through; not combined with split-K, residual or fp32 output). Segment widths are

@@ -89,6 +89,15 @@ extern "C" const char* cgptx_last_error(void) { return cgptx::g_last_error.c_str
 
 extern "C" const char* cgptx_version(void) { return "cgptx 0.1 (gfx950)"; }
 
+extern "C" size_t cgptx_scratch_bytes(cgptx_stream stream) {
+    using namespace cgptx;
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess) return 0;
+    std::lock_guard<std::mutex> lock(g_arena_mutex);
+    const auto it = g_arenas.find({device, static_cast<hipStream_t>(stream)});
+    return it == g_arenas.end() ? 0 : it->second.bytes;
+}
+
 extern "C" int cgptx_release_scratch(void) {
     using namespace cgptx;
     int device = 0;

@@ -358,6 +358,13 @@ bool fused_swiglu() {
     return text == nullptr || text[0] != '0';
 }
 
+// Whether the down projection's input gradient also turns its result into the gradient of [gate | up] in its
+// epilogue (CGPTX_FUSE_SWIGLU_GRAD=0 keeps the separate operator in the backward pass only, for comparisons).
+bool fused_swiglu_gradient() {
+    const char* text = std::getenv("CGPTX_FUSE_SWIGLU_GRAD");  // read per enqueue
+    return text == nullptr || text[0] != '0';
+}
+
 // Whether the norm-backward passes of the step leave their weight-gradient reductions to one pair of launches at
 // the end of the backward pass (CGPTX_FUSE_DGAMMA=0 keeps the two small launches after each pass, for comparisons:
 // same additions in the same order, same bits).
@@ -656,7 +663,7 @@ int enqueue_forward_backward(cgptx_model* m, float loss_scale, int loss_mode, hi
         const auto& w = m->layers[reverse];
         const auto& a = m->acts[reverse];
         void* x = m->hidden[reverse];
-        if (fused_swiglu()) {
+        if (fused_swiglu() && fused_swiglu_gradient()) {
             // The SwiGLU gradient rides in the epilogue of the down projection's input gradient.
             CGPTX_OP("gemm_dx.down", cgptx_linear_swiglu_backward(m->d_gate_up, m->d_act, current, w.down.value, a.gate_up, N, I, H, dt, s));
             CGPTX_OP("gemm_dw.down", cgptx_linear_backward(nullptr, w.down.gradient, nullptr, current, a.act, w.down.value, N, I, H, 0, 0, 0, dt, s));

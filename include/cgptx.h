@@ -49,6 +49,10 @@ const char* cgptx_last_error(void);
 const char* cgptx_version(void);
 /* Releases every scratch arena of the current device (synchronises the device). */
 int cgptx_release_scratch(void);
+/* Bytes of the scratch arena bound to (current device, stream): the largest request any operator has made on
+ * that stream so far, rounded up to 1 MiB; 0 when the stream has none. For a train step it is dominated by the
+ * logits chunk of the cut cross-entropy (rows x vocabulary in the storage dtype, up to 2 GiB - 1 MiB). */
+size_t cgptx_scratch_bytes(cgptx_stream stream);
 
 /* ------------------------------------------------------------------ backward */
 

@@ -81,11 +81,37 @@ def test_equivalent_to_dense_cross_entropy_plus_linear_backward(device, monkeypa
     assert again[0] == loss and torch.equal(again[1], dx) and torch.equal(again[2], dc)
 
 
+@pytest.mark.parametrize("rows", [1024, 1025, 1281, 2049], ids=["at-the-bound", "one-row-over", "ragged-second-chunk", "three-chunks"])
+def test_row_counts_on_both_sides_of_the_chunk_bound(device, monkeypatch, rows):
+    """CGPTX_CUT_CE_LOGITS_BYTES = 64 MiB at V = 32000 in bf16 allows 1024 rows per chunk: 1024 rows are one chunk
+    (the classifier gradient straight out of its contraction), 1025 rows two chunks of 768 and 257 rows, 2049 three.
+    Loss, dX and dC against float64 on every side of the bound; both gradient paths round the same fp32 sums once."""
+    monkeypatch.setenv("CGPTX_CUT_CE_LOGITS_BYTES", str(64 << 20))
+    dtype = torch.bfloat16
+    hidden, vocab = 64, 32000
+    x, c = randn((rows, hidden), dtype, 40 + rows), randn((vocab, hidden), dtype, 41, 0.05)
+    targets = randint(vocab, (rows,), 42)
+    loss, dx, dc = run(device, x.to(device), c.to(device), targets.to(device), 64.0)
+    z = to_np(x) @ to_np(c).T
+    lse = np.log(np.exp(z - z.max(axis=1, keepdims=True)).sum(axis=1)) + z.max(axis=1)
+    want_loss = float((lse - z[np.arange(rows), targets.numpy()]).mean())
+    prob = np.exp(z - lse[:, None])
+    prob[np.arange(rows), targets.numpy()] -= 1.0
+    prob *= 64.0 / rows
+    assert abs(loss - want_loss) <= 1e-4 * want_loss
+    assert_scaled_close(dx, prob @ to_np(c), STOL[dtype], f"dX, {rows} rows")
+    assert_scaled_close(dc, prob.T @ to_np(x), STOL[dtype], f"dC, {rows} rows")
+
+
+@pytest.mark.parametrize("logits_bytes", [None, 2 << 30], ids=["two-chunks-by-default", "one-chunk"])
 @pytest.mark.parametrize("hidden", [1024, 768], ids=["preset-1024", "secondary-768"])
-def test_training_shape_against_the_dense_path_and_float64_rows(device, hidden):
-    """[32768, hidden] x [32000, hidden] bf16, loss scale 1024: loss, dX and dC against the dense path (logits
-    contraction, cross-entropy operator, linear_backward), the dX rows of 256 rows against float64 (a row's gradient
+def test_training_shape_against_the_dense_path_and_float64_rows(device, monkeypatch, hidden, logits_bytes):
+    """[32768, hidden] x [32000, hidden] bf16, loss scale 1024, with the default bound on the logits scratch (two
+    chunks of 16384 rows) and as one chunk: loss, dX and dC against the dense path (logits contraction,
+    cross-entropy operator, linear_backward), the dX rows of 256 rows against float64 (a row's gradient
     does not depend on the other rows), and two runs are bit-identical."""
+    if logits_bytes is not None:
+        monkeypatch.setenv("CGPTX_CUT_CE_LOGITS_BYTES", str(logits_bytes))
     dtype = torch.bfloat16
     rows, vocab = 32768, 32000
     x, c = randn((rows, hidden), dtype, 31), randn((vocab, hidden), dtype, 32, 0.02)
