@@ -57,7 +57,11 @@ struct DeviceState {
     float squared_norm;
     unsigned int calls;                // completed prepare passes; its parity picks the flag a call uses
     unsigned int found_non_finite[2];  // set by the statistics pass of a call, cleared by the previous call's prepare
-    unsigned int pad[2];
+    // The options of the call in progress. The three kernels read them from here, not from their arguments, so
+    // that a captured sequence of them follows a learning rate that changes from step to step: the caller
+    // writes the options (adamw_set_hyper_kernel, outside the capture) before every launch of the graph.
+    Hyper hyper;
+    unsigned int pad;
 };
 
 __device__ __forceinline__ int find_entry(const unsigned int* __restrict__ chunk_begin, int entries,
@@ -160,10 +164,13 @@ __device__ __forceinline__ void stats_run(const T* __restrict__ g, const Unscale
     }
 }
 
+__global__ void adamw_set_hyper_kernel(DeviceState* state, Hyper hyper) { state->hyper = hyper; }
+
 __global__ __launch_bounds__(kThreads) void adamw_stats_kernel(const DeviceEntry* __restrict__ entries,
                                                               const unsigned int* __restrict__ chunk_begin,
-                                                              int entry_count, unsigned int total_chunks, float loss_scale,
+                                                              int entry_count, unsigned int total_chunks,
                                                               float* __restrict__ partial, DeviceState* state) {
+    const float loss_scale = state->hyper.loss_scale;
     __shared__ float stage[kStatsChunks][kThreads / kWave];
     __shared__ int any_bad;
     if (threadIdx.x == 0) any_bad = 0;
@@ -226,7 +233,6 @@ __global__ __launch_bounds__(kThreads) void adamw_stats_kernel(const DeviceEntry
 constexpr int kPrepareThreads = 1024;
 __global__ __launch_bounds__(kPrepareThreads) void adamw_prepare_kernel(const float* __restrict__ partial,
                                                                        unsigned int partial_count, DeviceState* state,
-                                                                       float beta1, float beta2, float max_grad_norm,
                                                                        int advance_step) {
     __shared__ double stage[kPrepareThreads];
     // Four independent sums per thread keep four loads in flight (one block adds some 25,000 partials for the 104m
@@ -259,6 +265,7 @@ __global__ __launch_bounds__(kPrepareThreads) void adamw_prepare_kernel(const fl
         return;
     }
     state->non_finite = 0u;
+    const float beta1 = state->hyper.beta1, beta2 = state->hyper.beta2, max_grad_norm = state->hyper.max_grad_norm;
     if (advance_step) {
         const unsigned long long next_step = state->step + 1ull;
         state->step = next_step;
@@ -353,9 +360,10 @@ __device__ __forceinline__ void update_chunk(const DeviceEntry& entry, unsigned 
 
 __global__ __launch_bounds__(kThreads) void adamw_update_kernel(const DeviceEntry* __restrict__ entries,
                                                                const unsigned int* __restrict__ chunk_begin,
-                                                               int entry_count, Hyper h,
+                                                               int entry_count,
                                                                const DeviceState* __restrict__ state) {
     if (state->non_finite != 0u) return;
+    const Hyper h = state->hyper;
     const float bc1 = state->scalars[0], bc2 = state->scalars[1], clip = state->scalars[2];
     const int e = find_entry(chunk_begin, entry_count, blockIdx.x);
     const DeviceEntry entry = entries[e];
@@ -489,39 +497,73 @@ extern "C" int cgptx_adamw_workspace_destroy(cgptx_adamw_workspace* ws) {
     return CGPTX_OK;
 }
 
-extern "C" int cgptx_adamw_step_many_async(cgptx_adamw_workspace* ws, const cgptx_adamw_entry* entries,
-                                           size_t entry_count, const cgptx_adamw_options* options,
-                                           uint64_t initial_step, cgptx_stream stream_) {
-    using namespace cgptx;
+namespace cgptx {
+
+// The two halves of adamw_step_many_async, for callers that record the update into a graph: the options travel to
+// the device outside the recording (they change from step to step: the learning rate), the three launches inside.
+int adamw_set_options(cgptx_adamw_workspace* ws, const cgptx_adamw_options* options, hipStream_t stream) {
     const char* name = "adamw_step_many_async";
     if (int s = validate_options(options, name)) return s;
+    if (ws == nullptr) return fail(CGPTX_INVALID_ARGUMENT, std::string(name) + ": null workspace");
+    hipLaunchKernelGGL(adamw_set_hyper_kernel, dim3(1), dim3(1), 0, stream, ws->state, to_hyper(*options));
+    CGPTX_LAUNCH_CHECK();
+    return CGPTX_OK;
+}
+
+int adamw_enqueue(cgptx_adamw_workspace* ws, const cgptx_adamw_entry* entries, std::size_t entry_count,
+                  std::uint64_t initial_step, hipStream_t stream) {
+    const char* name = "adamw_step_many_async";
     if (ws == nullptr) return fail(CGPTX_INVALID_ARGUMENT, std::string(name) + ": null workspace");
     if (entries == nullptr || entry_count == 0)
         return fail(CGPTX_INVALID_ARGUMENT, std::string(name) + ": empty parameter list");
     for (std::size_t i = 0; i < entry_count; ++i)
         if (int s = validate_entry(entries[i], name)) return s;
-    auto stream = static_cast<hipStream_t>(stream_);
-    if (!ws->initialized) {
-        if (int s = bind_entries(ws, entries, entry_count, stream)) return s;
-        DeviceState init{};
-        init.step = initial_step;
-        CGPTX_HIP(hipMemcpy(ws->state, &init, sizeof(init), hipMemcpyHostToDevice));
-        ws->initialized = true;
-    } else if (!same_entries(ws->bound, entries, entry_count)) {
+    if (!ws->initialized) return fail(CGPTX_INVALID_ARGUMENT, std::string(name) + ": the workspace has no entries bound yet");
+    if (!same_entries(ws->bound, entries, entry_count))
         return fail(CGPTX_INVALID_ARGUMENT, std::string(name) + ": workspace entries changed");
-    }
-    const Hyper h = to_hyper(*options);
+    (void)initial_step;
     const int n = static_cast<int>(entry_count);
     hipLaunchKernelGGL(adamw_stats_kernel, dim3((ws->total_chunks + kStatsChunks - 1) / kStatsChunks), dim3(kThreads), 0, stream,
-                       ws->entries, ws->chunk_begin, n, ws->total_chunks, h.loss_scale, ws->partial, ws->state);
+                       ws->entries, ws->chunk_begin, n, ws->total_chunks, ws->partial, ws->state);
     CGPTX_LAUNCH_CHECK();
     hipLaunchKernelGGL(adamw_prepare_kernel, dim3(1), dim3(kPrepareThreads), 0, stream, ws->partial, ws->total_chunks,
-                       ws->state, h.beta1, h.beta2, h.max_grad_norm, 1);
+                       ws->state, 1);
     CGPTX_LAUNCH_CHECK();
     hipLaunchKernelGGL(adamw_update_kernel, dim3(ws->total_chunks), dim3(kThreads), 0, stream, ws->entries,
-                       ws->chunk_begin, n, h, ws->state);
+                       ws->chunk_begin, n, ws->state);
     CGPTX_LAUNCH_CHECK();
     return CGPTX_OK;
+}
+
+// Binds the entry list on first use (device copies of the list: allocates and synchronises, so never under capture).
+int adamw_bind(cgptx_adamw_workspace* ws, const cgptx_adamw_entry* entries, std::size_t entry_count,
+               std::uint64_t initial_step, hipStream_t stream) {
+    const char* name = "adamw_step_many_async";
+    if (ws == nullptr) return fail(CGPTX_INVALID_ARGUMENT, std::string(name) + ": null workspace");
+    if (entries == nullptr || entry_count == 0)
+        return fail(CGPTX_INVALID_ARGUMENT, std::string(name) + ": empty parameter list");
+    for (std::size_t i = 0; i < entry_count; ++i)
+        if (int s = validate_entry(entries[i], name)) return s;
+    if (ws->initialized) return CGPTX_OK;
+    if (int s = bind_entries(ws, entries, entry_count, stream)) return s;
+    DeviceState init{};
+    init.step = initial_step;
+    CGPTX_HIP(hipMemcpy(ws->state, &init, sizeof(init), hipMemcpyHostToDevice));
+    ws->initialized = true;
+    return CGPTX_OK;
+}
+
+}  // namespace cgptx
+
+extern "C" int cgptx_adamw_step_many_async(cgptx_adamw_workspace* ws, const cgptx_adamw_entry* entries,
+                                           size_t entry_count, const cgptx_adamw_options* options,
+                                           uint64_t initial_step, cgptx_stream stream_) {
+    using namespace cgptx;
+    auto stream = static_cast<hipStream_t>(stream_);
+    if (int s = validate_options(options, "adamw_step_many_async")) return s;
+    if (int s = adamw_bind(ws, entries, entry_count, initial_step, stream)) return s;
+    if (int s = adamw_set_options(ws, options, stream)) return s;
+    return adamw_enqueue(ws, entries, entry_count, initial_step, stream);
 }
 
 extern "C" int cgptx_adamw_check(cgptx_adamw_workspace* ws, int* all_finite, uint64_t* step, cgptx_stream stream_) {
@@ -564,18 +606,18 @@ extern "C" int cgptx_adamw_step(void* parameter, const void* gradient, float* ma
     const DeviceEntry h_entry{parameter, gradient, master_parameter, first_moment, second_moment,
                               static_cast<unsigned long long>(count), dtype, 0};
     const unsigned int h_begin[2] = {0u, static_cast<unsigned int>(chunks)};
+    const Hyper h = to_hyper(*options);
     DeviceState init{};
+    init.hyper = h;
     CGPTX_HIP(hipStreamSynchronize(stream));
     CGPTX_HIP(hipMemcpy(state, &init, sizeof(init), hipMemcpyHostToDevice));
     CGPTX_HIP(hipMemcpy(d_entry, &h_entry, sizeof(h_entry), hipMemcpyHostToDevice));
     CGPTX_HIP(hipMemcpy(d_begin, h_begin, sizeof(h_begin), hipMemcpyHostToDevice));
-    const Hyper h = to_hyper(*options);
     hipLaunchKernelGGL(adamw_stats_kernel, dim3(static_cast<unsigned int>((chunks + kStatsChunks - 1) / kStatsChunks)),
-                       dim3(kThreads), 0, stream, d_entry, d_begin, 1, static_cast<unsigned int>(chunks), h.loss_scale, partial,
-                       state);
+                       dim3(kThreads), 0, stream, d_entry, d_begin, 1, static_cast<unsigned int>(chunks), partial, state);
     CGPTX_LAUNCH_CHECK();
     hipLaunchKernelGGL(adamw_prepare_kernel, dim3(1), dim3(kPrepareThreads), 0, stream, partial,
-                       static_cast<unsigned int>(chunks), state, h.beta1, h.beta2, h.max_grad_norm, 0);
+                       static_cast<unsigned int>(chunks), state, 0);
     CGPTX_LAUNCH_CHECK();
     // Bias corrections in double on the host, as adamw_step does (src/optim/adamw.cu:413-415).
     const float bc1 = static_cast<float>(1.0 - std::pow(static_cast<double>(h.beta1), static_cast<double>(next_step)));
@@ -583,7 +625,7 @@ extern "C" int cgptx_adamw_step(void* parameter, const void* gradient, float* ma
     hipLaunchKernelGGL(adamw_set_scalars_kernel, dim3(1), dim3(1), 0, stream, state, bc1, bc2);
     CGPTX_LAUNCH_CHECK();
     hipLaunchKernelGGL(adamw_update_kernel, dim3(static_cast<unsigned int>(chunks)), dim3(kThreads), 0, stream,
-                       d_entry, d_begin, 1, h, state);
+                       d_entry, d_begin, 1, state);
     CGPTX_LAUNCH_CHECK();
     CGPTX_HIP(hipStreamSynchronize(stream));
     DeviceState result{};

@@ -178,6 +178,17 @@ int rmsnorm_backward_dual(void* grad_input, void* grad_weight_a, void* grad_weig
                           const void* residual, std::size_t rows, std::size_t hidden, float epsilon, int dtype,
                           hipStream_t stream, ColumnReduceSink* sink = nullptr);
 
+// ---- the batched AdamW update in parts, for a caller that records it into a graph ----------------------------
+// adamw_bind: first use of a workspace (device copies of the entry list; allocates and synchronises). adamw_set_options:
+// one small launch that writes the options where the update's kernels read them; it stays outside a recording, since
+// the learning rate changes from step to step. adamw_enqueue: the three launches of the update, recordable.
+// cgptx_adamw_step_many_async is the three of them in a row.
+int adamw_bind(cgptx_adamw_workspace* workspace, const cgptx_adamw_entry* entries, std::size_t entry_count,
+               std::uint64_t initial_step, hipStream_t stream);
+int adamw_set_options(cgptx_adamw_workspace* workspace, const cgptx_adamw_options* options, hipStream_t stream);
+int adamw_enqueue(cgptx_adamw_workspace* workspace, const cgptx_adamw_entry* entries, std::size_t entry_count,
+                  std::uint64_t initial_step, hipStream_t stream);
+
 // ---- scratch arena ----------------------------------------------------------
 // Returns `bytes` of device scratch bound to (current device, stream), 256-byte
 // aligned. Grows by reallocation on eager calls; refuses to grow during capture.

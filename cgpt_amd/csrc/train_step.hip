@@ -11,8 +11,10 @@
 //   * the attention-norm output is kept instead of being recomputed in the backward;
 //   * bias gradients, which the reference computes into scratch and never uses
 //     (the model has no biases), are not computed;
-//   * forward + loss + backward are captured into one hipGraph after one eager run;
-//     every scratch request was sized by that eager run, so replay allocates nothing.
+//   * forward + loss + backward, and in a train step the AdamW update behind them, are captured into
+//     one hipGraph after one eager run; every scratch request was sized by that eager run, so replay
+//     allocates nothing. The optimizer's options reach its kernels through device memory, written
+//     ahead of each replay.
 #include "cgptx_train.h"
 #include "common.hpp"
 #include "gemm.hpp"
@@ -112,11 +114,15 @@ struct cgptx_model {
     std::uint64_t initial_step = 0;  // step count the optimizer workspace starts from when it is first used
     std::vector<cgptx_adamw_entry> entries;
     // captured graph
-    hipGraphExec_t graph_exec = nullptr;
-    float graph_loss_scale = 0.0f;
-    int graph_loss_mode = -1;
-    hipStream_t graph_stream = nullptr;
-    std::uint64_t graph_scratch_generation = 0;  // scratch arena block the recorded kernels point into
+    // Recorded steps: [0] forward + loss + backward, [1] the same followed by the AdamW update.
+    struct RecordedStep {
+        hipGraphExec_t exec = nullptr;
+        float loss_scale = 0.0f;
+        int loss_mode = -1;
+        hipStream_t stream = nullptr;
+        std::uint64_t scratch_generation = 0;  // scratch arena block the recorded kernels point into
+    };
+    RecordedStep recorded[2];
     // weight-gradient reductions of the norm-backward passes, run as one pair of launches per step
     cgptx::ColumnReduceSink norm_reductions;
     cgptx::ColumnReduceEntry* norm_reduction_table = nullptr;       // device copy of the entries
@@ -384,9 +390,9 @@ int finish_norm_reductions(cgptx_model* m, hipStream_t stream) {
     // A recorded step holds the addresses of the table and of the sink's memory and the number of entries: it is
     // recorded again after any of them changes.
     auto drop_recorded_step = [&]() {
-        if (m->graph_exec != nullptr) {
-            (void)hipGraphExecDestroy(m->graph_exec);
-            m->graph_exec = nullptr;
+        for (auto& step : m->recorded) {
+            if (step.exec != nullptr) (void)hipGraphExecDestroy(step.exec);
+            step.exec = nullptr;
         }
     };
     if (!sink.entries.empty()) {
@@ -752,7 +758,8 @@ int validate_config(const cgptx_model_config& c, std::size_t batch, std::size_t 
 extern "C" int cgptx_model_destroy(cgptx_model* m) {
     if (m == nullptr) return CGPTX_OK;
     (void)hipDeviceSynchronize();
-    if (m->graph_exec != nullptr) (void)hipGraphExecDestroy(m->graph_exec);
+    for (auto& step : m->recorded)
+        if (step.exec != nullptr) (void)hipGraphExecDestroy(step.exec);
     if (m->optimizer != nullptr) (void)cgptx_adamw_workspace_destroy(m->optimizer);
     for (void* p : m->allocations) (void)hipFree(p);
     if (m->norm_reductions.memory != nullptr) (void)hipFree(m->norm_reductions.memory);
@@ -1062,30 +1069,38 @@ extern "C" int cgptx_token_upload_async(uint32_t* device_inputs, uint32_t* devic
     return CGPTX_OK;
 }
 
-extern "C" int cgptx_model_forward_backward(cgptx_model* m, float loss_scale, int loss_mode, int use_graph,
-                                            cgptx_stream stream_) {
-    using namespace cgptx;
-    if (m == nullptr) return fail(CGPTX_INVALID_ARGUMENT, "model_forward_backward: null model");
+namespace cgptx {
+namespace {
+
+// Forward + loss + backward and, with_optimizer, the three launches of the AdamW update behind them (its options
+// are on the device already: adamw_set_options).
+int enqueue_step(cgptx_model* m, float loss_scale, int loss_mode, bool with_optimizer, hipStream_t stream) {
+    if (int s = enqueue_forward_backward(m, loss_scale, loss_mode, stream)) return s;
+    if (!with_optimizer) return CGPTX_OK;
+    return adamw_enqueue(m->optimizer, m->entries.data(), m->entries.size(), m->initial_step, stream);
+}
+
+int run_step(cgptx_model* m, float loss_scale, int loss_mode, int use_graph, bool with_optimizer, hipStream_t stream) {
     if (!std::isfinite(loss_scale) || loss_scale <= 0.0f)
         return fail(CGPTX_INVALID_ARGUMENT, "model_forward_backward: loss scale must be finite and positive");
     if (loss_mode != CGPTX_LOSS_DENSE && loss_mode != CGPTX_LOSS_CUT)
         return fail(CGPTX_INVALID_ARGUMENT, "model_forward_backward: unknown loss mode");
-    auto stream = static_cast<hipStream_t>(stream_);
     if (loss_mode == CGPTX_LOSS_DENSE && m->logits == nullptr) {
         const std::size_t bytes = m->rows * m->config.vocabulary_size * dtype_size(m->config.dtype);
         if (int s = allocate(m, &m->logits, bytes)) return s;
         if (int s = allocate(m, &m->grad_logits, bytes)) return s;
     }
-    if (!use_graph) return enqueue_forward_backward(m, loss_scale, loss_mode, stream);
+    if (!use_graph) return enqueue_step(m, loss_scale, loss_mode, with_optimizer, stream);
     if (stream == nullptr)
         return fail(CGPTX_INVALID_ARGUMENT, "model_forward_backward: graph capture needs a non-default stream");
-    const bool have_graph = m->graph_exec != nullptr && m->graph_loss_scale == loss_scale &&
-                            m->graph_loss_mode == loss_mode && m->graph_stream == stream &&
+    cgptx_model::RecordedStep& step = m->recorded[with_optimizer ? 1 : 0];
+    const bool have_graph = step.exec != nullptr && step.loss_scale == loss_scale && step.loss_mode == loss_mode &&
+                            step.stream == stream &&
                             // The recorded kernels hold addresses inside the stream's scratch arena: a graph
                             // whose arena block has since been reallocated or released is recorded again.
-                            m->graph_scratch_generation == scratch_generation(stream);
+                            step.scratch_generation == scratch_generation(stream);
     if (have_graph) {
-        CGPTX_HIP(hipGraphLaunch(m->graph_exec, stream));
+        CGPTX_HIP(hipGraphLaunch(step.exec, stream));
         return CGPTX_OK;
     }
     // Eager run first: it sizes every scratch arena and does this call's work. Then record the
@@ -1096,13 +1111,16 @@ extern "C" int cgptx_model_forward_backward(cgptx_model* m, float loss_scale, in
         // pass records them and writes their table, which a capture cannot do.
         if (int s = enqueue_forward_backward(m, loss_scale, loss_mode, stream)) return s;
     }
+    if (with_optimizer) {
+        if (int s = adamw_enqueue(m->optimizer, m->entries.data(), m->entries.size(), m->initial_step, stream)) return s;
+    }
     CGPTX_HIP(hipStreamSynchronize(stream));
-    if (m->graph_exec != nullptr) {
-        CGPTX_HIP(hipGraphExecDestroy(m->graph_exec));
-        m->graph_exec = nullptr;
+    if (step.exec != nullptr) {
+        CGPTX_HIP(hipGraphExecDestroy(step.exec));
+        step.exec = nullptr;
     }
     CGPTX_HIP(hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal));
-    const int status = enqueue_forward_backward(m, loss_scale, loss_mode, stream);
+    const int status = enqueue_step(m, loss_scale, loss_mode, with_optimizer, stream);
     hipGraph_t graph = nullptr;
     const hipError_t end = hipStreamEndCapture(stream, &graph);
     if (status != CGPTX_OK) {
@@ -1110,14 +1128,24 @@ extern "C" int cgptx_model_forward_backward(cgptx_model* m, float loss_scale, in
         return status;
     }
     CGPTX_HIP(end);
-    const hipError_t inst = hipGraphInstantiate(&m->graph_exec, graph, nullptr, nullptr, 0);
+    const hipError_t inst = hipGraphInstantiate(&step.exec, graph, nullptr, nullptr, 0);
     (void)hipGraphDestroy(graph);
     CGPTX_HIP(inst);
-    m->graph_loss_scale = loss_scale;
-    m->graph_loss_mode = loss_mode;
-    m->graph_stream = stream;
-    m->graph_scratch_generation = scratch_generation(stream);
+    step.loss_scale = loss_scale;
+    step.loss_mode = loss_mode;
+    step.stream = stream;
+    step.scratch_generation = scratch_generation(stream);
     return CGPTX_OK;
+}
+
+}  // namespace
+}  // namespace cgptx
+
+extern "C" int cgptx_model_forward_backward(cgptx_model* m, float loss_scale, int loss_mode, int use_graph,
+                                            cgptx_stream stream_) {
+    using namespace cgptx;
+    if (m == nullptr) return fail(CGPTX_INVALID_ARGUMENT, "model_forward_backward: null model");
+    return run_step(m, loss_scale, loss_mode, use_graph, false, static_cast<hipStream_t>(stream_));
 }
 
 extern "C" int cgptx_model_optimizer_step(cgptx_model* m, const cgptx_adamw_options* options, cgptx_stream stream) {
@@ -1127,12 +1155,16 @@ extern "C" int cgptx_model_optimizer_step(cgptx_model* m, const cgptx_adamw_opti
                                        stream);
 }
 
+// With use_graph the AdamW update is part of the recorded step: its options (the learning rate changes from step to
+// step) are written to the device by one small launch ahead of the graph, and the update's kernels read them there.
 extern "C" int cgptx_model_train_step(cgptx_model* m, const cgptx_adamw_options* options, int loss_mode,
-                                      int use_graph, cgptx_stream stream) {
+                                      int use_graph, cgptx_stream stream_) {
     using namespace cgptx;
     if (m == nullptr || options == nullptr) return fail(CGPTX_INVALID_ARGUMENT, "model_train_step: null argument");
-    if (int s = cgptx_model_forward_backward(m, options->loss_scale, loss_mode, use_graph, stream)) return s;
-    return cgptx_model_optimizer_step(m, options, stream);
+    auto stream = static_cast<hipStream_t>(stream_);
+    if (int s = adamw_bind(m->optimizer, m->entries.data(), m->entries.size(), m->initial_step, stream)) return s;
+    if (int s = adamw_set_options(m->optimizer, options, stream)) return s;
+    return run_step(m, options->loss_scale, loss_mode, use_graph, true, stream);
 }
 
 extern "C" int cgptx_model_status(cgptx_model* m, float* loss, int* all_finite, uint64_t* step,

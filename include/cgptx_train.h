@@ -5,7 +5,7 @@
  *   forward   src/core/transformer_model.cu:195-241, src/core/transformer_block.cu:405-611
  *   backward  src/core/transformer_model.cu:336-381, src/core/transformer_block.cu:644-748
  *   step      train/train.cpp:536-556 (forward + loss + backward replayed from one
- *             captured graph, AdamW enqueued after it)
+ *             captured graph; here the AdamW update is recorded with them)
  * The block is the reference's parallel-residual block with per-head QK-norm:
  *   out = x + Wo·Attn(rope(norm_q(Wq·n_a)), rope(norm_k(Wk·n_a)), Wv·n_a) + Wd·swiglu(Wg·n_f, Wu·n_f),
  *   n_a = RMSNorm_a(x), n_f = RMSNorm_f(x); embeddings are tied to the classifier.
@@ -99,7 +99,10 @@ int cgptx_model_forward_backward(cgptx_model* model, float loss_scale, int loss_
 /* Enqueues the global-norm AdamW update over all parameters (adamw_step_many_async). */
 int cgptx_model_optimizer_step(cgptx_model* model, const cgptx_adamw_options* options, cgptx_stream stream);
 
-/* forward_backward followed by optimizer_step. */
+/* forward_backward followed by optimizer_step (train/train.cpp:536-556). With use_graph the three launches of
+ * the AdamW update are part of the recorded step: the options, which change from step to step (the learning rate),
+ * are written to the device by one small launch ahead of the graph, and the update's kernels read them there — same
+ * results as the eager step, bit for bit, including skipped (non-finite) steps. */
 int cgptx_model_train_step(cgptx_model* model, const cgptx_adamw_options* options, int loss_mode, int use_graph,
                            cgptx_stream stream);
 

@@ -258,6 +258,50 @@ def test_train_steps_reduce_the_loss_and_count_steps(device):
 
 
 @pytest.mark.gpu
+def test_recorded_train_step_follows_a_changing_learning_rate_and_skips_like_the_eager_one(device):
+    """With use_graph the AdamW update is part of the recorded step and reads its options on the device. Two models
+    from one seed take the same eight steps, one eagerly and one from the recording, with a learning rate, weight
+    decay and clipping norm that change every step and one step whose gradients are made non-finite (both must skip
+    it and count it): parameters, master copies and moments agree bit for bit after every step."""
+    cfg = MODEL_CFG
+    from cgpt_amd.ops import AdamWOptions
+
+    batch, seq = 2, 24
+    rng = np.random.default_rng(17)
+    tokens = rng.integers(0, cfg["vocab"], size=(batch, seq))
+    targets = rng.integers(0, cfg["vocab"], size=(batch, seq))
+    stream = torch.cuda.Stream(device=device)
+    models = [build(device, torch.bfloat16, batch, seq, cfg, seed=3) for _ in range(2)]
+    for model in models:
+        model.set_tokens(tokens, targets)
+    saved = None
+    for step in range(8):
+        options = AdamWOptions(learning_rate=1e-2 / (1 + step), beta1=0.9, beta2=0.95, weight_decay=0.1 * (step % 3),
+                               loss_scale=256.0, max_grad_norm=[1.0, float("inf"), 0.5][step % 3])
+        if step == 4:  # a weight that overflows the forward pass: every gradient becomes non-finite
+            saved = [models[i].parameters()[1][1].clone() for i in range(2)]
+            for model in models:
+                model.parameters()[1][1].fill_(float("inf"))
+            torch.cuda.synchronize()
+        for use_graph, model in zip((False, True), models):
+            model.train_step(options, loss_mode=1, use_graph=use_graph, stream=stream)
+        states = [model.status(stream) for model in models]
+        assert states[0][1:] == states[1][1:], f"step {step}: {states}"
+        assert states[0][1] == (step != 4), f"step {step}: finite flag {states[0][1]}"
+        if step == 4:
+            for i, model in enumerate(models):
+                model.parameters()[1][1].copy_(saved[i])
+            torch.cuda.synchronize()
+        for index, ((name, p0, _), (_, p1, _)) in enumerate(zip(models[0].parameters(), models[1].parameters())):
+            assert torch.equal(p0, p1), f"step {step}: {name} differs between the eager and the recorded step"
+            for a, b in zip(models[0].optimizer_state(index), models[1].optimizer_state(index)):
+                assert torch.equal(a, b), f"step {step}: optimizer state of {name} differs"
+    assert models[0].status(stream)[2] == 7  # eight calls, one skipped
+    for model in models:
+        model.close()
+
+
+@pytest.mark.gpu
 def test_model_argument_errors(device):
     from cgpt_amd.model import Model, ModelConfig
 
