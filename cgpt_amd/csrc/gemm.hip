@@ -38,9 +38,9 @@
 //     fp32 partial tiles go to scratch and a second kernel adds them in slice order
 //     (deterministic), applying accumulate and the dtype conversion.
 //
-// Shapes the MFMA path does not cover (K not a multiple of 32, leading dimensions
-// or pointers not 16-byte aligned, fp32 storage) run on a plain LDS-tiled fp32
-// kernel with the same semantics.
+// Shapes the streamed path does not cover (K not a multiple of 32, leading dimensions
+// or pointers not 16-byte aligned, fp32 storage) run on an fp32 matrix-core kernel
+// (v_mfma_f32_32x32x2_f32, register-staged operand tiles) with the same semantics.
 #include "gemm.hpp"
 
 #include <algorithm>
@@ -1088,59 +1088,116 @@ __global__ __launch_bounds__(kThreads) void splitk_reduce_kernel(void* __restric
     }
 }
 
-// ---- plain fp32 kernel for everything the MFMA path does not take -------------
-constexpr int kGenericTile = 32;
+// ---- fp32 matrix-core kernel for everything the streamed 16-bit path does not take ---------------
+// fp32 storage (the reference serves it through its tensor-core library too: src/ops/linear.cu:634-667,
+// src/ops/backward/linear_backward.cu:79-82), and 16-bit storage whose K is not a multiple of 32 or whose rows are
+// not 16-byte aligned. Any shape, any alignment, all three operand layouts: a 128 x 128 tile of C per block, K in
+// steps of 16; the four wavefronts own 64 x 64 each and multiply with v_mfma_f32_32x32x2_f32 on fp32 operands
+// (16-bit storage is widened on the way into LDS, so the products are exact and the sums fp32, as in the streamed
+// kernels). Operand tiles go through registers into a K-major LDS layout ([k][m], [k][n]) — the fragment of an
+// MFMA step is then 32 consecutive floats per half-wavefront — with the next tile's loads in flight during the
+// multiplication; rows, columns and K positions past the matrices read as zeros.
+constexpr int kF32Tile = 128;  // rows and columns of C per block
+constexpr int kF32K = 16;      // K per LDS stage
+constexpr int kF32Pad = 4;
+using acc16_t = vec_t<float, 16>;
 
 template <typename T>
-__global__ __launch_bounds__(kGenericTile* kGenericTile / 4) void gemm_generic_kernel(KernelArgs p, int a_k, int b_k) {
-    // 32x32 tile of C per block of 16x16 threads, 2x2 outputs per thread, K step 32.
-    __shared__ float as[kGenericTile][kGenericTile + 1];
-    __shared__ float bs[kGenericTile][kGenericTile + 1];
+__global__ __launch_bounds__(kThreads) void gemm_f32_mfma_kernel(KernelArgs p, int a_k, int b_k) {
+    __shared__ float as[2][kF32K][kF32Tile + kF32Pad];
+    __shared__ float bs[2][kF32K][kF32Tile + kF32Pad];
     const T* A = static_cast<const T*>(p.a);
     const T* B = static_cast<const T*>(p.b);
-    const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
-    const long m0 = static_cast<long>(blockIdx.y) * kGenericTile, n0 = static_cast<long>(blockIdx.x) * kGenericTile;
-    float acc[2][2] = {{0.0f, 0.0f}, {0.0f, 0.0f}};
-    for (long k0 = 0; k0 < p.k; k0 += kGenericTile) {
-        for (int e = threadIdx.x; e < kGenericTile * kGenericTile; e += kGenericTile * kGenericTile / 4) {
-            const int r = e / kGenericTile, c = e % kGenericTile;  // r: m (or n), c: k
-            const long m = m0 + r, n = n0 + r, k = k0 + c;
-            float av = 0.0f, bv = 0.0f;
-            if (k < p.k) {
-                if (m < p.m) av = to_f32(a_k ? A[m * p.lda + k] : A[k * p.lda + m]);
-                if (n < p.n) bv = to_f32(b_k ? B[n * p.ldb + k] : B[k * p.ldb + n]);
-            }
-            as[r][c] = av;
-            bs[r][c] = bv;
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int wm = wave >> 1, wn = wave & 1;
+    const long m0 = static_cast<long>(blockIdx.y) * kF32Tile, n0 = static_cast<long>(blockIdx.x) * kF32Tile;
+    constexpr int kPerThread = kF32Tile * kF32K / kThreads;  // elements of each operand tile a thread moves
+    float a_regs[kPerThread], b_regs[kPerThread];
+    // Element e of a thread's share: consecutive threads walk the operand's contiguous index.
+    auto coordinates = [&](int e, bool k_contiguous, int& row, int& k) {
+        const int index = threadIdx.x + e * kThreads;
+        if (k_contiguous) {
+            row = index / kF32K;
+            k = index % kF32K;
+        } else {
+            k = index / kF32Tile;
+            row = index % kF32Tile;
         }
-        __syncthreads();
-#pragma unroll 8
-        for (int k = 0; k < kGenericTile; ++k) {
-            const float a0 = as[ty][k], a1 = as[ty + 16][k];
-            const float b0 = bs[tx][k], b1 = bs[tx + 16][k];
-            acc[0][0] = fmaf(a0, b0, acc[0][0]);
-            acc[0][1] = fmaf(a0, b1, acc[0][1]);
-            acc[1][0] = fmaf(a1, b0, acc[1][0]);
-            acc[1][1] = fmaf(a1, b1, acc[1][1]);
+    };
+    auto fetch = [&](long k0) {
+#pragma unroll
+        for (int e = 0; e < kPerThread; ++e) {
+            int row, k;
+            coordinates(e, a_k != 0, row, k);
+            const long m = m0 + row, ka = k0 + k;
+            a_regs[e] = (m < p.m && ka < p.k) ? to_f32(a_k ? A[m * p.lda + ka] : A[ka * p.lda + m]) : 0.0f;
+            coordinates(e, b_k != 0, row, k);
+            const long n = n0 + row, kb = k0 + k;
+            b_regs[e] = (n < p.n && kb < p.k) ? to_f32(b_k ? B[n * p.ldb + kb] : B[kb * p.ldb + n]) : 0.0f;
         }
-        __syncthreads();
+    };
+    auto deposit = [&](int stage) {
+#pragma unroll
+        for (int e = 0; e < kPerThread; ++e) {
+            int row, k;
+            coordinates(e, a_k != 0, row, k);
+            as[stage][k][row] = a_regs[e];
+            coordinates(e, b_k != 0, row, k);
+            bs[stage][k][row] = b_regs[e];
+        }
+    };
+    acc16_t acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = acc16_t(0.0f);
+    fetch(0);
+    deposit(0);
+    __syncthreads();
+    int stage = 0;
+    for (long k0 = 0; k0 < p.k; k0 += kF32K) {
+        const bool more = k0 + kF32K < p.k;
+        if (more) fetch(k0 + kF32K);  // in flight during the multiplication below
+#pragma unroll
+        for (int kk = 0; kk < kF32K; kk += 2) {
+            // MFMA step of k = 2: lane l holds row (column) l % 32 at k = l / 32.
+            float a[2], b[2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) a[i] = as[stage][kk + (lane >> 5)][wm * 64 + i * 32 + (lane & 31)];
+#pragma unroll
+            for (int j = 0; j < 2; ++j) b[j] = bs[stage][kk + (lane >> 5)][wn * 64 + j * 32 + (lane & 31)];
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
+        }
+        if (more) {
+            deposit(stage ^ 1);  // nobody reads that stage: the barrier below closed its last use
+            __syncthreads();
+            stage ^= 1;
+        }
     }
+    // Register r of a block holds row 8 (r / 4) + 4 (lane / 32) + r % 4 of column lane % 32.
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
-            const long m = m0 + ty + 16 * i, n = n0 + tx + 16 * j;
-            if (m >= p.m || n >= p.n) continue;
-            float v = acc[i][j];
-            if (p.addend != nullptr) v += p.addend[m * p.ld_addend + n];
-            if (p.bias != nullptr) v += to_f32(static_cast<const T*>(p.bias)[n]);
-            if (p.residual != nullptr) v += to_f32(static_cast<const T*>(p.residual)[static_cast<long>(m) * p.ldr + n]);
-            if (p.c_f32) {
-                float* out = static_cast<float*>(p.c) + m * p.ldc + n;
-                *out = p.accumulate ? v + *out : v;
-            } else {
-                T* out = static_cast<T*>(p.c) + m * p.ldc + n;
-                *out = from_f32<T>(p.accumulate ? v + to_f32(*out) : v);
+            const long n = n0 + wn * 64 + j * 32 + (lane & 31);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const long m = m0 + wm * 64 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                if (m >= p.m || n >= p.n) continue;
+                float v = acc[i][j][r];
+                if (p.addend != nullptr) v += p.addend[m * p.ld_addend + n];
+                if (p.bias != nullptr) v += to_f32(static_cast<const T*>(p.bias)[n]);
+                if (p.residual != nullptr) v += to_f32(static_cast<const T*>(p.residual)[m * p.ldr + n]);
+                if (p.c_f32) {
+                    float* out = static_cast<float*>(p.c) + m * p.ldc + n;
+                    *out = p.accumulate ? v + *out : v;
+                } else {
+                    T* out = static_cast<T*>(p.c) + m * p.ldc + n;
+                    *out = from_f32<T>(p.accumulate ? v + to_f32(*out) : v);
+                }
             }
         }
     }
@@ -1366,10 +1423,11 @@ int run_typed(const GemmArgs& g, hipStream_t stream) {
     }
     if (!fast && segmented) return fail(CGPTX_INVALID_ARGUMENT, "gemm: segmented operands need the aligned MFMA path");
     if (!fast) {
-        const dim3 grid(static_cast<unsigned int>((g.n + kGenericTile - 1) / kGenericTile),
-                        static_cast<unsigned int>((g.m + kGenericTile - 1) / kGenericTile));
-        hipLaunchKernelGGL((gemm_generic_kernel<T>), grid, dim3(kGenericTile * kGenericTile / 4), 0, stream, p,
-                           g.a_k_contiguous ? 1 : 0, g.b_k_contiguous ? 1 : 0);
+        const dim3 grid(static_cast<unsigned int>((g.n + kF32Tile - 1) / kF32Tile),
+                        static_cast<unsigned int>((g.m + kF32Tile - 1) / kF32Tile));
+        if (grid.y > 65535u) return fail(CGPTX_OVERFLOW, "gemm: too many rows for the fp32 kernel's grid");
+        hipLaunchKernelGGL((gemm_f32_mfma_kernel<T>), grid, dim3(kThreads), 0, stream, p, g.a_k_contiguous ? 1 : 0,
+                           g.b_k_contiguous ? 1 : 0);
         CGPTX_LAUNCH_CHECK();
         return CGPTX_OK;
     }
