@@ -556,6 +556,21 @@ def main() -> int:
             launches[label] = {"m": m_, "n": n_, "k": k_, "calls": calls, "us_per_call": round(ms * 1e3 / calls, 1),
                                "tflops": round(tflops, 1), "frac": round(tflops / PEAK_BF16_TFLOPS, 4)}
     family = {kind: per_kind[kind]["frac"] for kind in ("gemm_fwd", "gemm_dx", "gemm_dw") if kind in per_kind}
+    # Launches that carry a SwiGLU operator in their epilogue (no separate swiglu time in the breakdown then): their
+    # time also pays for that operator's traffic, so the families are given without them as well.
+    carriers = (("gemm_fwd", "gemm_fwd.gate_up", "swiglu_fwd", "SwiGLU forward"),
+                ("gemm_dx", "gemm_dx.down", "swiglu_bwd", "SwiGLU gradient"))
+    for kind, label, operator, what in carriers:
+        if operator in breakdown or label not in launches or kind not in breakdown or operator not in work:
+            continue
+        entry = launches[label]
+        carried = work[operator][1] / cfg.num_layers
+        entry["carries"] = (f"{what}: {carried / 1e6:.0f} MB of operator traffic per launch "
+                            f"({carried / (PEAK_HBM_GBS * 1e9) * 1e6:.0f} us at {PEAK_HBM_GBS / 1e3:.0f} TB/s)")
+        rest_ms = breakdown[kind] - labelled[label]
+        rest_flops = work[kind][1] - 2.0 * entry["m"] * entry["n"] * entry["k"] * entry["calls"]
+        if rest_ms > 0:
+            family[f"{kind} without the launch that carries the {what}"] = round(rest_flops / (rest_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4)
     # All event-timed launches of the probe kernel's instantiation in the step (plain, unsegmented dX with 256 x 256
     # tiles: the gate/up and the output projection's input gradients, one each per layer), FLOPs over time.
     same_kernel = [launches[label] for label in ("gemm_dx.gate_up", "gemm_dx.o") if label in launches]

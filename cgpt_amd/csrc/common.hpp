@@ -137,6 +137,9 @@ struct ColumnReduceSink {
         return block;
     }
 };
+// Bytes one norm-backward pass of the given kind takes from a sink (0: that shape reduces at once, from the arena).
+enum class NormPass { plain, with_rope, dual };
+std::size_t rmsnorm_backward_sink_bytes(NormPass pass, std::size_t rows, std::size_t hidden, int dtype);
 // Runs the reductions recorded in `table` (device copy of `count` entries). max_hidden / max_slices: the largest
 // values among the entries (they size the grid).
 int run_column_reductions(const ColumnReduceEntry* table, int count, int max_hidden, int max_slices, hipStream_t stream);

@@ -813,6 +813,28 @@ int rmsnorm_backward_impl(void* grad_input, void* grad_weight, const void* grad_
 }
 }  // namespace
 
+// What one backward pass takes from a ColumnReduceSink (0 when the shape runs on kernels that do not defer their
+// reduction). The same arithmetic as in the passes below; a caller sizes its sink with it before the first pass.
+std::size_t rmsnorm_backward_sink_bytes(NormPass pass, std::size_t rows, std::size_t hidden, int dtype) {
+    if (!valid_dtype(dtype) || rows == 0 || hidden == 0 || rows > (1u << 30) || hidden > (1u << 20)) return 0;
+    const int r = static_cast<int>(rows), h = static_cast<int>(hidden);
+    std::size_t bytes = 0;
+    dispatch_dtype(dtype, [&]<typename T>() -> int {
+        const FastShape shape = pick_fast_shape<T>(h);
+        if (shape.lpr == 0) return CGPTX_OK;
+        const void* kernel = pass == NormPass::dual ? dual_kernel<T, true>(shape) : fast_kernel<T, true>(shape, pass == NormPass::with_rope);
+        if (kernel == nullptr) return CGPTX_OK;
+        const int blocks = fast_blocks(shape, r, kernel);
+        const int slices = wide_reduce_slices(blocks, h, compute_units());
+        const std::size_t partial_bytes = static_cast<std::size_t>(blocks) * hidden * sizeof(float);
+        const std::size_t second_bytes = static_cast<std::size_t>(slices) * hidden * sizeof(float);
+        bytes = pass == NormPass::dual ? 2 * partial_bytes + 2 * ((second_bytes + 255) & ~std::size_t{255}) : partial_bytes + second_bytes;
+        bytes = (bytes + 255) & ~std::size_t{255};  // ColumnReduceSink::take hands out multiples of 256
+        return CGPTX_OK;
+    });
+    return bytes;
+}
+
 int rmsnorm_backward_residual(void* grad_input, void* grad_weight, const void* grad_output, const void* input,
                               const void* weight, const void* residual, std::size_t rows, std::size_t hidden,
                               float epsilon, int dtype, hipStream_t stream, ColumnReduceSink* sink) {

@@ -380,8 +380,9 @@ cgptx::ColumnReduceSink* norm_reduction_sink(cgptx_model* m) {
 }
 
 // Runs what the passes recorded. The entries are the same from pass to pass (same buffers, same shapes), so the
-// device copy of the table is written once, outside any capture; the sink's memory is sized after the first pass
-// that found it too small (that pass reduced at once, from the arena).
+// device copy of the table is written once, by the first pass, outside any capture. The sink's memory and the
+// table are sized when the model is created; should a pass still find the memory too small (it then reduced at
+// once, from the arena), the memory grows here and the caller repeats the pass before recording it.
 int finish_norm_reductions(cgptx_model* m, hipStream_t stream) {
     auto& sink = m->norm_reductions;
     hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
@@ -868,6 +869,28 @@ extern "C" int cgptx_model_create(cgptx_model** out, const cgptx_model_config* c
         CGPTX_HIP(hipMemcpy(m->cos_cache, storage.data(), storage.size(), hipMemcpyHostToDevice));
         convert_to_storage(sine, c.dtype, storage);
         CGPTX_HIP(hipMemcpy(m->sin_cache, storage.data(), storage.size(), hipMemcpyHostToDevice));
+        // Memory for the weight-gradient partial sums of every norm-backward pass of a step, and the device table of
+        // their reductions, sized here from the shapes: the first pass then finds room, defers its reductions and is
+        // not repeated. Each pair of alternatives (per-head norms with or without the rotary embedding, the block's
+        // two norms in one pass or two) is sized for the larger one; a pass that still asks for more than this grows
+        // the memory when it ends, as before.
+        {
+            const std::size_t HQ = c.num_query_heads, HKV = c.num_kv_heads, D = c.head_dim;
+            auto bytes = [&](NormPass pass, std::size_t rows, std::size_t width) {
+                return rmsnorm_backward_sink_bytes(pass, rows, width, c.dtype);
+            };
+            const std::size_t heads = std::max(bytes(NormPass::with_rope, N * HQ, D) + bytes(NormPass::with_rope, N * HKV, D),
+                                               bytes(NormPass::plain, N * HQ, D) + bytes(NormPass::plain, N * HKV, D));
+            const std::size_t block = std::max(bytes(NormPass::dual, N, H), 2 * bytes(NormPass::plain, N, H));
+            const std::size_t total = c.num_layers * (heads + block) + bytes(NormPass::plain, N, H);
+            if (total != 0) {
+                CGPTX_HIP(hipMalloc(reinterpret_cast<void**>(&m->norm_reductions.memory), total));
+                m->norm_reductions.capacity = total;
+            }
+            m->norm_reduction_table_capacity = 4 * c.num_layers + 1;
+            CGPTX_HIP(hipMalloc(reinterpret_cast<void**>(&m->norm_reduction_table),
+                                m->norm_reduction_table_capacity * sizeof(ColumnReduceEntry)));
+        }
         CGPTX_TRY(cgptx_adamw_workspace_create(&m->optimizer));
         std::vector<Parameter*> all;
         collect(m, all);
