@@ -293,22 +293,24 @@ template <typename T>
 __device__ __forceinline__ void update_chunk(const DeviceEntry& entry, unsigned long long begin,
                                              unsigned long long end, const Hyper& h, float bc1, float bc2,
                                              float clip) {
-    constexpr int VEC = kVec128<T>;
+    constexpr int VEC = 4;  // elements per lane and access: 128 bits of each fp32 state tensor
     T* p = static_cast<T*>(entry.parameter);
     const T* g = static_cast<const T*>(entry.gradient);
-    const bool aligned = ((reinterpret_cast<std::uintptr_t>(p + begin) | reinterpret_cast<std::uintptr_t>(g + begin) |
-                           reinterpret_cast<std::uintptr_t>(entry.master + begin) |
+    const bool aligned = ((reinterpret_cast<std::uintptr_t>(p + begin) | reinterpret_cast<std::uintptr_t>(g + begin)) &
+                          (VEC * sizeof(T) - 1)) == 0 &&
+                         ((reinterpret_cast<std::uintptr_t>(entry.master + begin) |
                            reinterpret_cast<std::uintptr_t>(entry.first + begin) |
                            reinterpret_cast<std::uintptr_t>(entry.second + begin)) & 15u) == 0;
     const unsigned long long count = end - begin;
     const unsigned long long vectors = aligned ? count / VEC : 0;
-    // A thread requests everything it will touch in the chunk (kPasses vectors of the gradient and of the three fp32
-    // state tensors: 7 kPasses 128-bit loads with 16-bit gradients) before it computes anything.
+    // A thread requests everything it will touch in the chunk before it computes anything: kPasses groups of four
+    // elements, each group's position in the chunk chosen so that every access instruction of a wavefront covers one
+    // contiguous kilobyte of an fp32 state tensor (512 B of 16-bit gradients or parameters) - whole cache lines per
+    // instruction for the loads and, which matters more, for the stores.
     constexpr int kPasses = kChunk / (kThreads * VEC) > 0 ? kChunk / (kThreads * VEC) : 1;
-    constexpr int kQuads = VEC / 4;
     for (unsigned long long v0 = 0; v0 < vectors; v0 += static_cast<unsigned long long>(kPasses) * kThreads) {
         vec_t<T, VEC> gr[kPasses];
-        vec_t<float, 4> mm[kPasses][kQuads], vv[kPasses][kQuads], ww[kPasses][kQuads];
+        vec_t<float, 4> mm[kPasses], vv[kPasses], ww[kPasses];
         bool live[kPasses];
 #pragma unroll
         for (int k = 0; k < kPasses; ++k) {
@@ -317,35 +319,27 @@ __device__ __forceinline__ void update_chunk(const DeviceEntry& entry, unsigned 
             if (!live[k]) continue;
             const unsigned long long at = begin + vi * VEC;
             gr[k] = load_vec<T, VEC>(g + at);
-#pragma unroll
-            for (int q = 0; q < kQuads; ++q) {
-                mm[k][q] = load_vec<float, 4>(entry.first + at + 4 * q);
-                vv[k][q] = load_vec<float, 4>(entry.second + at + 4 * q);
-                ww[k][q] = load_vec<float, 4>(entry.master + at + 4 * q);
-            }
+            mm[k] = load_vec<float, 4>(entry.first + at);
+            vv[k] = load_vec<float, 4>(entry.second + at);
+            ww[k] = load_vec<float, 4>(entry.master + at);
         }
 #pragma unroll
         for (int k = 0; k < kPasses; ++k) {
             if (!live[k]) continue;
             const unsigned long long at = begin + (v0 + static_cast<unsigned long long>(k) * kThreads + threadIdx.x) * VEC;
             const vec_t<float, VEC> grad = vec_to_f32<T, VEC>(gr[k]);
-            vec_t<float, VEC> updated;
 #pragma unroll
-            for (int q = 0; q < kQuads; ++q) {
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    float m = mm[k][q][e], v = vv[k][q][e], w = ww[k][q][e];
-                    adamw_element(grad[4 * q + e], m, v, w, h, bc1, bc2, clip);
-                    mm[k][q][e] = m;
-                    vv[k][q][e] = v;
-                    ww[k][q][e] = w;
-                    updated[4 * q + e] = w;
-                }
-                store_vec<float, 4>(entry.first + at + 4 * q, mm[k][q]);
-                store_vec<float, 4>(entry.second + at + 4 * q, vv[k][q]);
-                store_vec<float, 4>(entry.master + at + 4 * q, ww[k][q]);
+            for (int e = 0; e < 4; ++e) {
+                float m = mm[k][e], v = vv[k][e], w = ww[k][e];
+                adamw_element(grad[e], m, v, w, h, bc1, bc2, clip);
+                mm[k][e] = m;
+                vv[k][e] = v;
+                ww[k][e] = w;
             }
-            store_vec<T, VEC>(p + at, vec_from_f32<T, VEC>(updated));
+            store_vec<float, 4>(entry.first + at, mm[k]);
+            store_vec<float, 4>(entry.second + at, vv[k]);
+            store_vec<float, 4>(entry.master + at, ww[k]);
+            store_vec<T, VEC>(p + at, vec_from_f32<T, VEC>(ww[k]));
         }
     }
     for (unsigned long long i = begin + vectors * VEC + threadIdx.x; i < end; i += kThreads) {
