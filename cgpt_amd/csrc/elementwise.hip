@@ -119,6 +119,11 @@ __global__ __launch_bounds__(kThreads) void rope_pair_kernel(T* __restrict__ out
     }
 }
 
+bool rope_is_empty(std::size_t batch, std::size_t sequence, std::size_t query_heads, std::size_t kv_heads,
+                   std::size_t head_dim) {
+    return batch == 0 || sequence == 0 || query_heads == 0 || kv_heads == 0 || head_dim == 0;
+}
+
 int validate_rope(const char* name, const void* q, const void* k, const void* c, const void* s, std::size_t batch,
                   std::size_t sequence, std::size_t query_heads, std::size_t kv_heads, std::size_t head_dim,
                   std::size_t& rotary_dim, std::size_t position_offset, std::size_t cache_positions, int dtype) {
@@ -386,6 +391,8 @@ extern "C" int cgptx_rope_backward(void* grad_query, void* grad_key, const void*
                                    size_t head_dim, size_t rotary_dim, size_t position_offset, size_t cache_positions,
                                    int dtype, cgptx_stream stream) {
     using namespace cgptx;
+    // Tensors without elements: nothing to do, as in the reference (src/ops/backward/rope_backward.cu:243-245, 326-328).
+    if (valid_dtype(dtype) && rope_is_empty(batch, sequence, query_heads, kv_heads, head_dim)) return CGPTX_OK;
     if (grad_rotated_query == nullptr || grad_rotated_key == nullptr)
         return fail(CGPTX_INVALID_ARGUMENT, "rope_backward: null tensor");
     if (int s = validate_rope("rope_backward", grad_query, grad_key, cos_cache, sin_cache, batch, sequence,
@@ -401,6 +408,8 @@ extern "C" int cgptx_rope_forward(void* query, void* key, const void* cos_cache,
                                   size_t rotary_dim, size_t position_offset, size_t cache_positions, int dtype,
                                   cgptx_stream stream) {
     using namespace cgptx;
+    // Tensors without elements: nothing to do, as in the reference (src/ops/rope.cu:606-608).
+    if (valid_dtype(dtype) && rope_is_empty(batch, sequence, query_heads, kv_heads, head_dim)) return CGPTX_OK;
     if (int s = validate_rope("rope_forward", query, key, cos_cache, sin_cache, batch, sequence, query_heads,
                               kv_heads, head_dim, rotary_dim, position_offset, cache_positions, dtype))
         return s;
@@ -413,9 +422,9 @@ extern "C" int cgptx_swiglu_backward(void* grad_gate, void* grad_up, const void*
                                      cgptx_stream stream) {
     using namespace cgptx;
     if (!valid_dtype(dtype)) return fail(CGPTX_INVALID_ARGUMENT, "swiglu_backward: unsupported dtype");
+    if (count == 0) return CGPTX_OK;  // nothing to do, as in the reference (src/ops/backward/swiglu_backward.cu:772-774)
     if (grad_gate == nullptr || grad_up == nullptr || grad_output == nullptr || gate == nullptr || up == nullptr)
         return fail(CGPTX_INVALID_ARGUMENT, "swiglu_backward: null tensor");
-    if (count == 0) return fail(CGPTX_INVALID_ARGUMENT, "swiglu_backward: empty tensor");
     return dispatch_dtype(dtype, [&]<typename T>() -> int {
         return launch_swiglu_backward<T>(static_cast<T*>(grad_gate), static_cast<T*>(grad_up),
                                          static_cast<const T*>(grad_output), static_cast<const T*>(gate),
@@ -429,9 +438,9 @@ extern "C" int cgptx_swiglu_backward_packed(void* grad_gate_up, const void* grad
                                             cgptx_stream stream) {
     using namespace cgptx;
     if (!valid_dtype(dtype)) return fail(CGPTX_INVALID_ARGUMENT, "swiglu_backward: unsupported dtype");
+    if (rows == 0 || hidden == 0) return CGPTX_OK;  // nothing to do (src/ops/backward/swiglu_backward.cu:839-841)
     if (grad_gate_up == nullptr || grad_output == nullptr || gate_up == nullptr)
         return fail(CGPTX_INVALID_ARGUMENT, "swiglu_backward: null tensor");
-    if (rows == 0 || hidden == 0) return fail(CGPTX_INVALID_ARGUMENT, "swiglu_backward: empty tensor");
     return dispatch_dtype(dtype, [&]<typename T>() -> int {
         auto* out = static_cast<T*>(grad_gate_up);
         auto* in = static_cast<const T*>(gate_up);
@@ -446,8 +455,9 @@ extern "C" int cgptx_swiglu_forward(void* output, const void* gate, const void* 
                                     cgptx_stream stream) {
     using namespace cgptx;
     if (!valid_dtype(dtype)) return fail(CGPTX_INVALID_ARGUMENT, "swiglu_forward: unsupported dtype");
-    if (output == nullptr || gate == nullptr || up == nullptr || count == 0)
-        return fail(CGPTX_INVALID_ARGUMENT, "swiglu_forward: null or empty tensor");
+    if (count == 0) return CGPTX_OK;  // nothing to do, as in the reference (src/ops/swiglu.cu:530-532)
+    if (output == nullptr || gate == nullptr || up == nullptr)
+        return fail(CGPTX_INVALID_ARGUMENT, "swiglu_forward: null tensor");
     return dispatch_dtype(dtype, [&]<typename T>() -> int {
         const bool vector_ok = is_aligned16(output) && is_aligned16(gate) && is_aligned16(up);
         hipLaunchKernelGGL((swiglu_forward_kernel<T>), dim3(grid_for(count / kVec128<T> + 1)), dim3(kThreads), 0,
@@ -462,8 +472,9 @@ extern "C" int cgptx_swiglu_forward_packed(void* output, const void* gate_up, si
                                            cgptx_stream stream) {
     using namespace cgptx;
     if (!valid_dtype(dtype)) return fail(CGPTX_INVALID_ARGUMENT, "swiglu_forward: unsupported dtype");
-    if (output == nullptr || gate_up == nullptr || rows == 0 || hidden == 0)
-        return fail(CGPTX_INVALID_ARGUMENT, "swiglu_forward: null or empty tensor");
+    if (rows == 0 || hidden == 0) return CGPTX_OK;  // nothing to do (src/ops/swiglu.cu:581-583)
+    if (output == nullptr || gate_up == nullptr)
+        return fail(CGPTX_INVALID_ARGUMENT, "swiglu_forward: null tensor");
     if (rows > std::numeric_limits<std::size_t>::max() / (2 * hidden))
         return fail(CGPTX_OVERFLOW, "swiglu_forward: element count overflows");
     return dispatch_dtype(dtype, [&]<typename T>() -> int {

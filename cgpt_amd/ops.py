@@ -188,6 +188,8 @@ def swiglu_backward_packed(grad_gate_up, grad_output, gate_up, stream=None,
     if gate_up.dim() < 1 or gate_up.shape[-1] != 2 * hidden or gate_up.numel() != 2 * grad_output.numel() or \
             grad_gate_up.shape != gate_up.shape:
         raise ValueError(f"{name}: invalid fused tensors")
+    if grad_output.numel() == 0:
+        return  # nothing to do (src/ops/backward/swiglu_backward.cu:839-841)
     capi.call("cgptx_swiglu_backward_packed", _ptr(grad_gate_up), _ptr(grad_output), _ptr(gate_up),
               grad_output.numel() // hidden, hidden, int(options.accumulate_gate_up), _code(gate_up), _stream(stream))
 
@@ -501,6 +503,8 @@ def swiglu_forward(output, gate, up=None, stream=None):
         if output.dim() != gate_up.dim() or tuple(output.shape[:-1]) != tuple(gate_up.shape[:-1]) or \
                 output.shape[-1] != hidden:
             raise ValueError(f"{name}: output shape must match gate_up except for its last dimension")
+        if output.numel() == 0:
+            return  # nothing to do (src/ops/swiglu.cu:581-583)
         capi.call("cgptx_swiglu_forward_packed", _ptr(output), _ptr(gate_up), output.numel() // hidden, hidden,
                   _code(gate_up), _stream(stream))
         return

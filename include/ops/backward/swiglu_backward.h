@@ -32,6 +32,7 @@ inline void swiglu_backward(Tensor& grad_gate_up, const Tensor& grad_output, con
     require_same_shape(op, gate_up, {&grad_gate_up});
     if (gate_up.dim() == 0 || gate_up.shape().back() % 2 != 0 || grad_output.numel() * 2 != gate_up.numel())
         throw std::invalid_argument("swiglu_backward: gate_up must hold [gate | up] for every grad_output row");
+    if (grad_output.numel() == 0) return;  // nothing to do (src/ops/backward/swiglu_backward.cu:839-841)
     const std::size_t hidden = gate_up.shape().back() / 2;
     check(cgptx_swiglu_backward_packed(grad_gate_up.raw_data(), grad_output.raw_data(), gate_up.raw_data(),
                                        grad_output.numel() / hidden, hidden, options.accumulate_gate_up,

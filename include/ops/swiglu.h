@@ -25,6 +25,7 @@ inline void swiglu_forward(Tensor& output, const Tensor& gate_up, hipStream_t st
     const std::size_t hidden = gate_up.shape().back() / 2;
     if (output.dim() != gate_up.dim() || output.shape().back() != hidden || output.numel() * 2 != gate_up.numel())
         throw std::invalid_argument("swiglu_forward: output shape must match gate_up except for its last dimension");
+    if (output.numel() == 0) return;  // nothing to do (src/ops/swiglu.cu:581-583)
     check(cgptx_swiglu_forward_packed(output.raw_data(), gate_up.raw_data(), output.numel() / hidden, hidden,
                                       dtype_code(gate_up.dtype()), stream));
 }

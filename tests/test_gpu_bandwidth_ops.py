@@ -246,6 +246,28 @@ def test_swiglu_forward_packed_parity(device, rows, hidden, dtype):
         ops.swiglu_forward(dout, dev(gu, device)[:, : 2 * hidden - 1].contiguous())
 
 
+@pytest.mark.parametrize("dtype", DTYPES, ids=DTYPE_IDS)
+def test_tensors_without_elements_are_accepted_and_nothing_is_written(device, dtype):
+    """The reference returns early for RoPE and SwiGLU tensors with no elements (src/ops/rope.cu:606-608,
+    src/ops/backward/rope_backward.cu:326-328, src/ops/swiglu.cu:530-532 and 581-583,
+    src/ops/backward/swiglu_backward.cu:772-774 and 839-841): zero rows, a zero batch or a zero sequence are not
+    errors. A guard tensor next to the calls keeps its contents."""
+    guard = torch.full((64,), 3.0, dtype=dtype, device=device)
+    empty = torch.zeros(0, 16, dtype=dtype, device=device)
+    ops.swiglu_backward(empty.clone(), empty.clone(), empty, empty, empty)
+    ops.swiglu_forward(empty.clone(), empty, empty)
+    packed = torch.zeros(0, 32, dtype=dtype, device=device)
+    ops.swiglu_backward_packed(packed.clone(), empty, packed)
+    ops.swiglu_forward(empty.clone(), packed)
+    cos = torch.zeros(4, 4, dtype=dtype, device=device)
+    for shape_q, shape_k in (((0, 4, 2, 8), (0, 4, 1, 8)), ((2, 0, 2, 8), (2, 0, 1, 8))):
+        q, k = torch.zeros(shape_q, dtype=dtype, device=device), torch.zeros(shape_k, dtype=dtype, device=device)
+        ops.rope_backward(q.clone(), k.clone(), q, k, cos, cos)
+        ops.rope_forward(q, k, cos, cos)
+    torch.cuda.synchronize()
+    assert torch.equal(guard, torch.full_like(guard, 3.0))
+
+
 def test_swiglu_argument_errors(device):
     a = torch.zeros(4, 4, device=device)
     with pytest.raises(ValueError):
