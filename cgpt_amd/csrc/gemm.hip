@@ -667,6 +667,17 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
             v0 = *reinterpret_cast<const vec_t<float, 4>*>(base + (((f_col / 4) ^ sw(row)) * 16));
             v1 = *reinterpret_cast<const vec_t<float, 4>*>(base + (((f_col / 4 + 1) ^ sw(row)) * 16));
         };
+        // The same staged half, dealt out so that every store instruction of fp32 values covers whole cache lines: lane l
+        // of round u takes columns 4 (l % 8) .. + 3 and, for its second store, the four columns 32 further on, of row
+        // 8u + l/8 (with eight consecutive fp32 columns per lane, each store instruction would write every other 16 bytes
+        // of a line, and lines reach memory in parts).
+        const int l_col = (lane % kGroups) * 4;  // first column of the lane's first quad within the staged half
+        auto read_staged_lines = [&](int u, vec_t<float, 4>& v0, vec_t<float, 4>& v1) __attribute__((always_inline)) {
+            const int row = u * kRowsF + f_row;
+            const unsigned char* base = region + row * kRowBytes;
+            v0 = *reinterpret_cast<const vec_t<float, 4>*>(base + (((l_col / 4) ^ sw(row)) * 16));
+            v1 = *reinterpret_cast<const vec_t<float, 4>*>(base + (((l_col / 4 + kGroups) ^ sw(row)) * 16));
+        };
         // Descriptor over a wavefront's part of a row-major matrix (see the 16-bit case above).
         auto part_rsrc = [&](const void* origin, long ld, int elem, int rows_left, int cols_left) __attribute__((always_inline)) {
             const long extent = rows_left > 0 && cols_left > 0 ? (static_cast<long>(rows_left - 1) * ld + cols_left) * elem : 0;
@@ -885,16 +896,18 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
 #pragma unroll
                 for (int half = 0; half < 2; ++half) {
                     stage.template operator()<float, TN / 2>(r, half * (TN / 2));
-                    const int col = half * (WN / 2) + f_col;
-                    const int voffset = col < cols_left ? f_row * row_bytes + col * 4 : std::numeric_limits<int>::min();
+                    const int col = half * (WN / 2) + l_col;
+                    constexpr int kSecond = kGroups * 4;  // columns between a lane's two quads
+                    const int voffset0 = col < cols_left ? f_row * row_bytes + col * 4 : std::numeric_limits<int>::min();
+                    const int voffset1 = col + kSecond < cols_left ? f_row * row_bytes + (col + kSecond) * 4 : std::numeric_limits<int>::min();
                     vec_t<float, 4> v0[kRoundsF], v1[kRoundsF];
 #pragma unroll
-                    for (int u = 0; u < kRoundsF; ++u) read_staged(u, v0[u], v1[u]);
+                    for (int u = 0; u < kRoundsF; ++u) read_staged_lines(u, v0[u], v1[u]);
 #pragma unroll
                     for (int u = 0; u < kRoundsF; ++u) {
                         const int soffset = (r * 32 + u * kRowsF) * row_bytes;
-                        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v0[u]), rsrc, voffset, soffset, 0);
-                        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v1[u]), rsrc, voffset + 16, soffset, 0);
+                        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v0[u]), rsrc, voffset0, soffset, 0);
+                        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v1[u]), rsrc, voffset1, soffset, 0);
                     }
                 }
             }
