@@ -59,7 +59,7 @@ constexpr int kBK = 32;          // K step per LDS stage
 // blocks own a CU (5 x 32 KiB), 128x128 blocks run two per CU (5 x 16 KiB each).
 constexpr int stages_for(int /*bm*/, int /*bn*/) { return 5; }
 constexpr int kXcds = 8;
-constexpr int kGroupRows = 8;    // tile-rows per L2 locality group
+
 
 using acc_t = vec_t<float, 4>;
 
@@ -119,9 +119,10 @@ struct KernelArgs {
     int accumulate;
     int c_f32;
     KernelSegments a_seg, c_seg;  // column segments of A (as stored) and of C; count 0 = one buffer
-    // ceil(2^32 / (kGroupRows * tiles_n)) when multiplying by it divides every item index of the
+    // ceil(2^32 / (group rows * tiles_n)) when multiplying by it divides every item index of the
     // launch exactly, else 0 (the kernel then divides).
     unsigned int group_reciprocal;
+    int group_rows_log2;  // tile-rows per L2 locality group: 1 << group_rows_log2
     void* act;      // SWIGLU kernels: [M, inter] = silu(gate) * up, T*
     long ld_act;
     const void* saved;  // GRAD kernels: the forward's [M, 2 * inter] = [gate | up], T*
@@ -374,7 +375,7 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
     const int wm = wave >> 1, wn = wave & 1;
 
     // Work items are numbered slice-major (all tiles of K slice 0, then of slice 1, ...), tiles in
-    // groups of kGroupRows tile-rows, down the rows first. Blocks are dealt round-robin to the 8
+    // groups of 1 << group_rows_log2 tile-rows, down the rows first. Blocks are dealt round-robin to the 8
     // XCDs, so XCD x takes the x-th eighth of the items and its blocks walk it side by side: the
     // items in flight on one XCD are neighbours and share A and B panels in that XCD's L2.
     const int tiles = p.tiles_m * p.tiles_n;
@@ -396,14 +397,15 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
         Item w;
         w.slice = p.slices == 1 ? 0 : index / tiles;
         const int logical = index - w.slice * tiles;
-        const int group_size = kGroupRows * p.tiles_n;
+        const int group_rows = 1 << p.group_rows_log2;
+        const int group_size = p.tiles_n << p.group_rows_log2;
         const int group = p.group_reciprocal != 0u
                               ? static_cast<int>(__umulhi(static_cast<unsigned int>(logical), p.group_reciprocal))
                               : logical / group_size;
-        const int first_m = group * kGroupRows;
-        const int rows_in_group = min(p.tiles_m - first_m, kGroupRows);
+        const int first_m = group << p.group_rows_log2;
+        const int rows_in_group = min(p.tiles_m - first_m, group_rows);
         const int in_group = logical - group * group_size;
-        const int column = rows_in_group == kGroupRows ? in_group / kGroupRows : in_group / rows_in_group;
+        const int column = rows_in_group == group_rows ? in_group >> p.group_rows_log2 : in_group / rows_in_group;
         w.m0 = (first_m + in_group - column * rows_in_group) * BM;
         w.n0 = column * BN;
         w.kt_begin = w.slice * p.k_tiles_per_slice;
@@ -1235,7 +1237,13 @@ int launch_mfma(const KernelArgs& p, int slices, hipStream_t stream) {
     const long items = static_cast<long>(p.tiles_m) * p.tiles_n * slices;
     {
         // x * ceil(2^32 / d) >> 32 == x / d for every x with x * d < 2^32.
-        const unsigned long divisor = static_cast<unsigned long>(kGroupRows) * static_cast<unsigned long>(p.tiles_n);
+        // Tile-rows per L2 locality group. 8 (x 4 tile-columns = the 32 tiles in flight on an XCD) shares operand
+        // panels best. The SwiGLU-gradient epilogue moves four times the bytes of a plain one, two loads and two
+        // stores of whole [gate | up] rows: there the tiles in flight on an XCD are better spread along the rows
+        // (2 tile-rows x all 8 tile-columns of the training shape: 250 -> 212 us per launch; 1, 2 and 4 tile-rows
+        // measure the same, every other kernel is at its best with 8).
+        args.group_rows_log2 = GRAD ? 1 : 3;
+        const unsigned long divisor = (1ul << args.group_rows_log2) * static_cast<unsigned long>(p.tiles_n);
         const unsigned long tiles = static_cast<unsigned long>(p.tiles_m) * static_cast<unsigned long>(p.tiles_n);
         const bool exact = divisor > 1 && tiles * divisor < (1ul << 32);
         args.group_reciprocal = exact ? static_cast<unsigned int>(((1ul << 32) + divisor - 1) / divisor) : 0u;
