@@ -16,7 +16,8 @@
 //   * The kernel is persistent: one block per CU slot walks its share of the work items
 //     (output tile x K slice). The 8 XCDs (blocks are dealt round-robin to them) each take
 //     a contiguous eighth of the items, ordered in groups of 8 tile-rows, so that the
-//     tiles in flight on one XCD share A and B panels in that XCD's L2.
+//     tiles in flight on one XCD share A and B panels in that XCD's L2 (2 tile-rows for
+//     the kernel whose epilogue reads and writes whole rows of a wider matrix).
 //   * Operand tiles go global -> LDS with buffer_load ... lds (no staging registers, no
 //     LDS stores, one loop-invariant per-lane offset) into a ring of five LDS stages:
 //     one being multiplied, up to three K tiles in flight, one being refilled. LDS rows
