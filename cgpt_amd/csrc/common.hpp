@@ -58,17 +58,42 @@ __device__ __forceinline__ void store_vec(T* p, vec_t<T, N> v) {
     *reinterpret_cast<vec_t<T, N>*>(p) = v;
 }
 
-// Butterfly reductions across `width` adjacent lanes (width a power of two <= 64).
+// The value of lane (lane ^ offset) for offset 8, 4, 2 or 1 inside a row of 16 lanes, taken through the data-parallel
+// operand path of the vector unit instead of the LDS crossbar. Offsets 8, 2 and 1 are exact lane exchanges (a row
+// rotation by 8, two quad permutations). Offset 4 is a row rotation by 4, which hands lane i the value of lane
+// (i ^ 4) or (i ^ 4 ^ 8): the same bits whenever lanes i and i ^ 8 hold equal values, which is the case right after
+// the offset-8 step of a butterfly that runs from large offsets to small ones.
+template <int offset>
+__device__ __forceinline__ float row_exchange(float v) {
+    static_assert(offset == 8 || offset == 4 || offset == 2 || offset == 1);
+    constexpr int control = offset == 8 ? 0x128 : offset == 4 ? 0x124 : offset == 2 ? 0x4E : 0xB1;
+    const int bits = __builtin_bit_cast(int, v);
+    return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(bits, control, 0xF, 0xF, true));
+}
+
+// Butterfly reductions across `width` adjacent lanes (width a power of two <= 64), from the largest offset down.
+// Steps across rows of 16 lanes go through the LDS crossbar, the last four stay in the vector unit; the result has
+// the bits of the plain butterfly (a + b and max(a, b) do not depend on which of the two equal partners is read).
 template <int width = kWave>
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
-    for (int offset = width / 2; offset > 0; offset >>= 1) v += __shfl_xor(v, offset, kWave);
+    for (int offset = width / 2; offset > 8; offset >>= 1) v += __shfl_xor(v, offset, kWave);
+    if constexpr (width >= 16) v += row_exchange<8>(v);
+    if constexpr (width >= 16) v += row_exchange<4>(v);
+    else if constexpr (width >= 8) v += __shfl_xor(v, 4, kWave);
+    if constexpr (width >= 4) v += row_exchange<2>(v);
+    if constexpr (width >= 2) v += row_exchange<1>(v);
     return v;
 }
 template <int width = kWave>
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll
-    for (int offset = width / 2; offset > 0; offset >>= 1) v = fmaxf(v, __shfl_xor(v, offset, kWave));
+    for (int offset = width / 2; offset > 8; offset >>= 1) v = fmaxf(v, __shfl_xor(v, offset, kWave));
+    if constexpr (width >= 16) v = fmaxf(v, row_exchange<8>(v));
+    if constexpr (width >= 16) v = fmaxf(v, row_exchange<4>(v));
+    else if constexpr (width >= 8) v = fmaxf(v, __shfl_xor(v, 4, kWave));
+    if constexpr (width >= 4) v = fmaxf(v, row_exchange<2>(v));
+    if constexpr (width >= 2) v = fmaxf(v, row_exchange<1>(v));
     return v;
 }
 

@@ -27,6 +27,10 @@ namespace {
 
 constexpr int kThreads = 256;
 constexpr int kWavesPerBlock = kThreads / kWave;
+// Groups of four rows a wavefront of the dense norm + rotary kernel requests at a time: the backward pass holds three
+// times the registers per group, and more of them in flight cost it more in resident wavefronts than they bring.
+template <bool Backward>
+constexpr int kRopeDenseUnroll = Backward ? 2 : 4;
 
 // Rotary embedding applied to the rows on the way (rows are heads of head_dim = hidden elements):
 // forward  y = rope(round(rmsnorm(x)));  backward  the incoming gradient is rotated back (and
@@ -193,6 +197,153 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_rows_kernel(
 #pragma unroll
             for (int s = 0; s < kWavesPerBlock; ++s) v += stage[s][col];
             partial[static_cast<std::size_t>(blockIdx.x) * hidden + col] = v;
+        }
+    }
+}
+
+// The fused per-head norm + rotary pass at the shape a training step gives it: rows of exactly 16 vectors (head_dim 128
+// in 16-bit storage), all of them rotated, a multiple of four rows, tensors and tables below 4 GiB. Same arithmetic,
+// in the same order, as rmsnorm_rows_kernel<T, 16, 1, Backward, true>; what differs is the bookkeeping, which at 2 KiB
+// of rows per wavefront and trip is what that kernel spends most of its instructions on: no per-lane predicates, 32-bit
+// byte offsets that advance by a constant, and the token position carried from trip to trip (head index and position
+// advance by constants with one carry each) instead of two integer divisions per trip. A trip requests U groups of
+// four rows before it uses the first, so that a wavefront has U times the bytes in flight.
+template <typename T, bool Backward, int U>
+__global__ __launch_bounds__(kThreads) void rmsnorm_rope_dense_kernel(
+    T* out, float* __restrict__ partial, const T* dy /* may be out itself */, const T* __restrict__ x,
+    const T* __restrict__ w, int rows, float inv_hidden, float eps, RopeArgs rope) {
+    constexpr int VEC = kVec128<T>;
+    constexpr int HALF = VEC / 2;
+    constexpr int LPR = 16;
+    constexpr int RPW = kWave / LPR;
+    constexpr int HIDDEN = LPR * VEC;
+    using F = vec_t<float, VEC>;
+    using H = vec_t<float, HALF>;
+
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    const int sub = lane % LPR;
+    const int rsel = lane / LPR;
+    const F wv = vec_to_f32<T, VEC>(load_vec<T, VEC>(w + sub * VEC));
+    F acc(0.0f);
+
+    const int groups = rows / RPW;
+    const int wave_global = blockIdx.x * kWavesPerBlock + wave;
+    const int wave_count = gridDim.x * kWavesPerBlock;
+    const int first_row = wave_global * RPW + rsel;
+    const int stride_rows = wave_count * RPW;
+    int head = first_row % rope.heads;
+    int pos = (first_row / rope.heads) % rope.sequence;
+    const int head_step = stride_rows % rope.heads;
+    const int pos_step = (stride_rows / rope.heads) % rope.sequence;
+    unsigned offset = (static_cast<unsigned>(first_row) * HIDDEN + sub * VEC) * static_cast<unsigned>(sizeof(T));
+    const unsigned offset_step = static_cast<unsigned>(stride_rows) * HIDDEN * static_cast<unsigned>(sizeof(T));
+    const unsigned table_lane = sub * HALF * static_cast<unsigned>(sizeof(T));
+    constexpr unsigned kTableRow = (HIDDEN / 2) * sizeof(T);
+    const auto at = [](const void* base, unsigned bytes) {
+        return reinterpret_cast<const T*>(static_cast<const char*>(base) + bytes);
+    };
+
+    struct Fetched {
+        vec_t<T, VEC> x, g;
+        vec_t<T, HALF> c, s;
+        unsigned offset;
+    };
+    // Requests the operands of the group at `offset` / `pos` and moves both on to the wavefront's next group.
+    const auto fetch = [&]() {
+        Fetched f;
+        const unsigned table = static_cast<unsigned>(rope.position_offset + pos) * kTableRow + table_lane;
+        f.c = load_vec<T, HALF>(at(rope.cos_cache, table));
+        f.s = load_vec<T, HALF>(at(rope.sin_cache, table));
+        f.x = load_vec<T, VEC>(at(x, offset));
+        if constexpr (Backward) f.g = load_vec<T, VEC>(at(dy, offset));
+        f.offset = offset;
+        offset += offset_step;
+        head += head_step;
+        const int carry = head >= rope.heads ? 1 : 0;
+        head -= carry ? rope.heads : 0;
+        pos += pos_step + carry;
+        pos -= pos >= rope.sequence ? rope.sequence : 0;
+        return f;
+    };
+    const auto finish = [&](const Fetched& f) {
+        const H c = vec_to_f32<T, HALF>(f.c);
+        const H s = vec_to_f32<T, HALF>(f.s);
+        const F xv = vec_to_f32<T, VEC>(f.x);
+        F gv;
+        if constexpr (Backward) {
+            // The incoming gradient rotated back and rounded: what the separate rotary operator would have stored.
+            const F raw = vec_to_f32<T, VEC>(f.g);
+            F turned;
+#pragma unroll
+            for (int p = 0; p < HALF; ++p) {
+                float a, b;
+                rotate_pair<true>(raw[2 * p], raw[2 * p + 1], c[p], s[p], a, b);
+                turned[2 * p] = a;
+                turned[2 * p + 1] = b;
+            }
+            gv = vec_to_f32<T, VEC>(vec_from_f32<T, VEC>(turned));
+        }
+        float ss = 0.0f, dd = 0.0f;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            ss = fmaf(xv[e], xv[e], ss);
+            if constexpr (Backward) dd = fmaf(gv[e] * wv[e], xv[e], dd);
+        }
+        ss = wave_sum<LPR>(ss);
+        const float inv = 1.0f / sqrtf(ss * inv_hidden + eps);
+        F r;
+        if constexpr (Backward) {
+            dd = wave_sum<LPR>(dd);
+            const float corr = dd * inv * inv * inv * inv_hidden;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                r[e] = gv[e] * wv[e] * inv - xv[e] * corr;
+                acc[e] = fmaf(gv[e], xv[e] * inv, acc[e]);
+            }
+        } else {
+            F y;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) y[e] = xv[e] * inv * wv[e];
+            y = vec_to_f32<T, VEC>(vec_from_f32<T, VEC>(y));  // the norm's own store, before the rotation
+#pragma unroll
+            for (int p = 0; p < HALF; ++p) {
+                float a, b;
+                rotate_pair<false>(y[2 * p], y[2 * p + 1], c[p], s[p], a, b);
+                r[2 * p] = a;
+                r[2 * p + 1] = b;
+            }
+        }
+        store_vec<T, VEC>(const_cast<T*>(at(out, f.offset)), vec_from_f32<T, VEC>(r));
+    };
+
+    int g = wave_global;
+    for (; g + (U - 1) * wave_count < groups; g += U * wave_count) {
+        Fetched f[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) f[u] = fetch();
+        __builtin_amdgcn_sched_barrier(0);  // every request of the trip goes out before the first use
+#pragma unroll
+        for (int u = 0; u < U; ++u) finish(f[u]);
+    }
+    for (; g < groups; g += wave_count) finish(fetch());
+
+    if constexpr (Backward) {
+        // Fold the four row slots of the wavefront, then the block's wavefronts.
+        __shared__ float stage[kWavesPerBlock][HIDDEN];
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            float v = acc[e];
+#pragma unroll
+            for (int across = LPR; across < kWave; across <<= 1) v += __shfl_xor(v, across, kWave);
+            if (rsel == 0) stage[wave][sub * VEC + e] = v;
+        }
+        __syncthreads();
+        for (int col = threadIdx.x; col < HIDDEN; col += kThreads) {
+            float v = 0.0f;
+#pragma unroll
+            for (int s = 0; s < kWavesPerBlock; ++s) v += stage[s][col];
+            partial[static_cast<std::size_t>(blockIdx.x) * HIDDEN + col] = v;
         }
     }
 }
@@ -421,12 +572,29 @@ FastShape pick_fast_shape(int hidden) {
     return {};
 }
 
+// Whether rmsnorm_rope_dense_kernel serves the pass: rows of exactly 16 vectors, all of them rotated, whole groups of
+// four rows, and every byte offset it forms (tensor and table) below 2^32.
+template <typename T>
+bool rope_dense(int rows, int hidden, const RopeArgs& rope) {
+    constexpr int VEC = kVec128<T>;
+    const unsigned long long tensor_bytes = static_cast<unsigned long long>(rows) * hidden * sizeof(T);
+    const unsigned long long table_bytes =
+        (static_cast<unsigned long long>(rope.position_offset) + rope.sequence) * (hidden / 2) * sizeof(T);
+    return hidden == 16 * VEC && rope.rotary_dim == hidden && rows % 4 == 0 && tensor_bytes < (1ull << 32) &&
+           table_bytes < (1ull << 32);
+}
+
 template <typename T, bool Backward>
 int launch_fast(const FastShape shape, T* out, float* partial, const T* dy, const T* residual, const T* x, const T* w,
                 int rows, int hidden, float eps, int blocks, hipStream_t stream, const RopeArgs* rope = nullptr) {
     const float inv_hidden = 1.0f / static_cast<float>(hidden);
     if (rope != nullptr) {
         if (shape.lpr != 16 || shape.k != 1) return fail(CGPTX_RUNTIME, "rmsnorm: no rotary kernel for shape");
+        if (rope_dense<T>(rows, hidden, *rope)) {
+            hipLaunchKernelGGL((rmsnorm_rope_dense_kernel<T, Backward, kRopeDenseUnroll<Backward>>), dim3(blocks), dim3(kThreads), 0, stream, out,
+                               partial, dy, x, w, rows, inv_hidden, eps, *rope);
+            return CGPTX_OK;
+        }
         hipLaunchKernelGGL((rmsnorm_rows_kernel<T, 16, 1, Backward, true>), dim3(blocks), dim3(kThreads), 0, stream, out,
                            partial, dy, residual, x, w, rows, hidden, inv_hidden, eps, *rope);
         return CGPTX_OK;
@@ -448,10 +616,12 @@ int launch_fast(const FastShape shape, T* out, float* partial, const T* dy, cons
 
 // The kernel launch_fast would launch (null when there is none).
 template <typename T, bool Backward>
-const void* fast_kernel(const FastShape shape, bool rope) {
-    if (rope)
-        return shape.lpr == 16 && shape.k == 1 ? reinterpret_cast<const void*>(&rmsnorm_rows_kernel<T, 16, 1, Backward, true>)
-                                               : nullptr;
+const void* fast_kernel(const FastShape shape, bool rope, bool dense = false) {
+    if (rope) {
+        if (shape.lpr != 16 || shape.k != 1) return nullptr;
+        return dense ? reinterpret_cast<const void*>(&rmsnorm_rope_dense_kernel<T, Backward, kRopeDenseUnroll<Backward>>)
+                     : reinterpret_cast<const void*>(&rmsnorm_rows_kernel<T, 16, 1, Backward, true>);
+    }
 #define CGPTX_RMS_CASE(L, KK) \
     if (shape.lpr == L && shape.k == KK) return reinterpret_cast<const void*>(&rmsnorm_rows_kernel<T, L, KK, Backward>);
     CGPTX_RMS_CASE(16, 1)
@@ -585,7 +755,7 @@ int rmsnorm_rope_forward(void* output, const void* input, const void* weight, co
         const FastShape shape = pick_fast_shape<T>(h);
         if (int s = launch_fast<T, false>(shape, static_cast<T*>(output), nullptr, nullptr, nullptr,
                                           static_cast<const T*>(input), static_cast<const T*>(weight), r, h, epsilon,
-                                          fast_blocks(shape, r, fast_kernel<T, false>(shape, true)), stream, &rope))
+                                          fast_blocks(shape, r, fast_kernel<T, false>(shape, true, rope_dense<T>(r, h, rope))), stream, &rope))
             return s;
         CGPTX_LAUNCH_CHECK();
         return CGPTX_OK;
@@ -605,7 +775,7 @@ int rmsnorm_rope_backward(void* grad_input, void* grad_weight, const void* grad_
     const RopeArgs rope = make_rope(cos_cache, sin_cache, heads, sequence, rotary_dim, position_offset);
     return dispatch_dtype(dtype, [&]<typename T>() -> int {
         const FastShape shape = pick_fast_shape<T>(h);
-        const int blocks = fast_blocks(shape, r, fast_kernel<T, true>(shape, true));
+        const int blocks = fast_blocks(shape, r, fast_kernel<T, true>(shape, true, rope_dense<T>(r, h, rope)));
         const int slices = wide_reduce_slices(blocks, h, compute_units());
         void* mem = nullptr;
         bool deferred = false;
@@ -824,8 +994,16 @@ std::size_t rmsnorm_backward_sink_bytes(NormPass pass, std::size_t rows, std::si
         if (shape.lpr == 0) return CGPTX_OK;
         const void* kernel = pass == NormPass::dual ? dual_kernel<T, true>(shape) : fast_kernel<T, true>(shape, pass == NormPass::with_rope);
         if (kernel == nullptr) return CGPTX_OK;
-        const int blocks = fast_blocks(shape, r, kernel);
-        const int slices = wide_reduce_slices(blocks, h, compute_units());
+        int blocks = fast_blocks(shape, r, kernel);
+        int slices = wide_reduce_slices(blocks, h, compute_units());
+        if (pass == NormPass::with_rope) {
+            // The pass picks between two kernels by properties of its rotary tables that are not known here: room
+            // for whichever of them takes more.
+            const int other = fast_blocks(shape, r, fast_kernel<T, true>(shape, true, true));
+            const int other_slices = wide_reduce_slices(other, h, compute_units());
+            blocks = other > blocks ? other : blocks;
+            slices = other_slices > slices ? other_slices : slices;
+        }
         const std::size_t partial_bytes = static_cast<std::size_t>(blocks) * hidden * sizeof(float);
         const std::size_t second_bytes = static_cast<std::size_t>(slices) * hidden * sizeof(float);
         bytes = pass == NormPass::dual ? 2 * partial_bytes + 2 * ((second_bytes + 255) & ~std::size_t{255}) : partial_bytes + second_bytes;
