@@ -340,20 +340,27 @@ def test_cpu_float32_step_matches_float64_composition():
 
 
 @pytest.mark.gpu
-def test_fused_qk_norm_rope_is_bit_identical_to_the_separate_operators(device, monkeypatch):
+@pytest.mark.parametrize("head_dim,rotary_dim,kv_heads,seq,dtype", [
+    (64, 32, 2, 48, torch.bfloat16),     # the general row kernel, part of the head rotated
+    (128, 128, 2, 48, torch.bfloat16),   # the kernel for head_dim 128; a group of four k rows spans two tokens
+    (128, 128, 1, 333, torch.float16),   # the same with one kv head (four tokens per group), several trips per wavefront
+    (128, 128, 4, 47, torch.bfloat16),   # 2 * 47 * 4 = 376 k rows and as many q rows per head group
+], ids=["d64-r32", "d128-kv2", "d128-kv1-f16", "d128-kv4"])
+def test_fused_qk_norm_rope_is_bit_identical_to_the_separate_operators(device, monkeypatch, head_dim, rotary_dim,
+                                                                      kv_heads, seq, dtype):
     """Per-head RMSNorm + rotary embedding run as one pass (forward and backward) when head_dim is
-    served by the row kernel; the pass keeps the separate operators' intermediate roundings, so a whole
+    served by the row kernels; the pass keeps the separate operators' intermediate roundings, so a whole
     step gives the same bits either way. CGPTX_FUSE_QK=0 selects the separate operators."""
     from cgpt_amd.model import LOSS_DENSE, Model, ModelConfig
-    config = ModelConfig(vocabulary_size=128, num_layers=2, hidden_size=256, intermediate_size=256, num_query_heads=4,
-                         num_kv_heads=2, head_dim=64, rotary_dim=32, dtype=torch.bfloat16)
+    config = ModelConfig(vocabulary_size=128, num_layers=2, hidden_size=4 * head_dim, intermediate_size=256,
+                         num_query_heads=4, num_kv_heads=kv_heads, head_dim=head_dim, rotary_dim=rotary_dim, dtype=dtype)
     rng = np.random.default_rng(3)
-    inputs = rng.integers(0, 128, size=2 * 48).astype(np.uint32)
-    targets = rng.integers(0, 128, size=2 * 48).astype(np.uint32)
+    inputs = rng.integers(0, 128, size=2 * seq).astype(np.uint32)
+    targets = rng.integers(0, 128, size=2 * seq).astype(np.uint32)
     results = []
     for fuse in ("1", "0"):
         monkeypatch.setenv("CGPTX_FUSE_QK", fuse)
-        model = Model(config, 2, 48, seed=4, device=device)
+        model = Model(config, 2, seq, seed=4, device=device)
         model.set_tokens(inputs, targets)
         model.forward_backward(loss_scale=4.0, loss_mode=LOSS_DENSE)
         loss = model.status()[0]
