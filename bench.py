@@ -663,7 +663,9 @@ def main() -> int:
                              "event-timed duration of its calls (the same eager pass); "
                              "family_step_wide = the contraction family's fractions over the whole step (from "
                              "breakdown), next to the best launch quoted as `frac`; gemm_launches = every contraction "
-                             "by position in that pass; kernels = each backward operator alone at the configuration's "
+                             "by position in that pass (the projections' weight gradients run as one launch over "
+                             "all layers when the model's shapes are tile-aligned: their us_per_call is that launch's "
+                             "duration divided by the layers); kernels = each backward operator alone at the configuration's "
                              "shape, 20 back-to-back launches between HIP events on the launch stream; "
                              "frac_time_weighted = FLOPs over time of all event-timed launches of the probe kernel's "
                              "instantiation in the step (dX of the gate/up and of the output projection, every layer), "

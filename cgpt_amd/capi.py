@@ -75,6 +75,7 @@ PROTOTYPES = {
     "cgptx_linear_forward": [_vp, _vp, _vp, _vp, _sz, _sz, _sz, _i, _vp],
     "cgptx_linear_swiglu_forward": [_vp, _vp, _vp, _vp, _sz, _sz, _sz, _i, _vp],
     "cgptx_linear_swiglu_backward": [_vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _i, _vp],
+    "cgptx_linear_backward_weights_stacked": [_vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz, _sz, _i, _vp],
     "cgptx_embedding_forward": [_vp, _vp, _sz, _vp, _sz, _sz, _i, _vp],
     "cgptx_flash_gqa_attention_forward": [_vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz, _sz, _f, _i, _sz, _i, _vp],
     "cgptx_add": [_vp, _vp, _vp, _sz, _i, _vp],

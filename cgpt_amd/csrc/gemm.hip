@@ -129,6 +129,11 @@ struct KernelArgs {
     const void* saved;  // GRAD kernels: the forward's [M, 2 * inter] = [gate | up], T*
     long ld_saved;
     int inter;      // SWIGLU kernels: columns of gate (= of up); n = 2 * inter
+    // Stacked products (weight-gradient layout only): rows of C per product (0 = one product) and what a and b (or
+    // A's segments) move by from one product to the next, in elements.
+    int batch_rows;
+    long a_batch_stride, b_batch_stride;
+    long a_seg_batch_stride[3];
 };
 
 // The column segment (of up to three) that holds column `col`, picked with selects: indexing the
@@ -138,6 +143,7 @@ struct SegmentPick {
     long ld;
     int first;  // first column of the segment
     int cols;
+    int index;  // which segment
 };
 __device__ __forceinline__ SegmentPick pick_segment(const KernelSegments& seg, int col) {
     const int end0 = seg.cols[0], end1 = end0 + seg.cols[1];
@@ -148,6 +154,7 @@ __device__ __forceinline__ SegmentPick pick_segment(const KernelSegments& seg, i
     pick.ld = in2 ? seg.ld[2] : in1 ? seg.ld[1] : seg.ld[0];
     pick.first = in2 ? end1 : in1 ? end0 : 0;
     pick.cols = in2 ? seg.cols[2] : in1 ? seg.cols[1] : seg.cols[0];
+    pick.index = in2 ? 2 : in1 ? 1 : 0;
     return pick;
 }
 
@@ -426,6 +433,7 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
         const int m0 = w.m0, n0 = w.n0;
         src_begin = w.kt_begin;
         src_end = w.kt_end;
+        long b_shift = 0;
         if constexpr (A_K && !SEGMENTED) {
             a_src.init(static_cast<const T*>(p.a) + static_cast<long>(m0) * p.lda, p.lda, p.m - m0, p.k, wave);
         } else if constexpr (A_K) {
@@ -448,21 +456,34 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(KernelArgs p) {
             a_end0 = segments > 1 ? cols0 : std::numeric_limits<int>::max();
             a_end1 = segments > 2 ? cols0 + cols1 : std::numeric_limits<int>::max();
         } else {
-            const T* base = static_cast<const T*>(p.a);
+            // Stacked products: the tile's rows of C name the product, and the operands move with it.
+            long product = 0;
+            int local_m0 = m0, rows = p.m;
+            if constexpr (!B_K) {
+                if (p.batch_rows > 0) {
+                    product = m0 / p.batch_rows;
+                    local_m0 = m0 - static_cast<int>(product) * p.batch_rows;
+                    rows = p.batch_rows;
+                    b_shift = product * p.b_batch_stride;
+                }
+            }
+            const T* base = static_cast<const T*>(p.a) + product * p.a_batch_stride;
             long ld = p.lda;
-            int first = 0, width = p.m;
+            int first = 0, width = rows;
             if (p.a_seg.count > 0) {
-                const SegmentPick pick = pick_segment(p.a_seg, m0);
-                base = static_cast<const T*>(pick.ptr);
+                const SegmentPick pick = pick_segment(p.a_seg, local_m0);
+                const long stride = pick.index == 2 ? p.a_seg_batch_stride[2]
+                                    : pick.index == 1 ? p.a_seg_batch_stride[1] : p.a_seg_batch_stride[0];
+                base = static_cast<const T*>(pick.ptr) + product * stride;
                 ld = pick.ld;
                 first = pick.first;
                 width = pick.cols;
             }
-            a_src.init(base + (m0 - first), ld, width - (m0 - first), p.k, wave);
+            a_src.init(base + (local_m0 - first), ld, width - (local_m0 - first), p.k, wave);
         }
         if constexpr (SWIGLU) b_src.init(static_cast<const T*>(p.b) + static_cast<long>(n0 / 2) * p.ldb, p.ldb, p.n - n0 / 2, p.k, wave);
         else if constexpr (B_K) b_src.init(static_cast<const T*>(p.b) + static_cast<long>(n0) * p.ldb, p.ldb, p.n - n0, p.k, wave);
-        else b_src.init(static_cast<const T*>(p.b) + n0, p.ldb, p.n - n0, p.k, wave);
+        else b_src.init(static_cast<const T*>(p.b) + b_shift + n0, p.ldb, p.n - n0, p.k, wave);
     };
     // K tiles past the end of the slice are still "loaded" (the loop stays free of data-dependent
     // branches and every wavefront always has the same number of loads in flight), but from an
@@ -1323,6 +1344,19 @@ int run_config(const GemmArgs& g, KernelArgs p, hipStream_t stream) {
         slices = static_cast<int>(std::min<long>(want_blocks / tiles, k_tiles / 16));
         if (slices < 1) slices = 1;
     }
+    if (g.batch_rows != 0 && may_split && k_tiles >= 32) {
+        // A stack of products brings any number of tiles: the slice count that needs the least time, counted in
+        // rounds of the persistent blocks times the length of a slice (fewer slices on a tie: fewer partial tiles).
+        double best = 0.0;
+        for (int s = 1; s <= 8 && k_tiles / s >= 16; ++s) {
+            const long rounds = (tiles * s + want_blocks - 1) / want_blocks;
+            const double time = static_cast<double>(rounds) / s * (s > 1 ? 1.02 : 1.0);
+            if (s == 1 || time < best * 0.999) {
+                best = time;
+                slices = s;
+            }
+        }
+    }
     if (g.no_split && static_cast<std::size_t>(slices) * g.m * g.n * sizeof(float) > g.split_workspace_bytes) slices = 1;
     p.k_tiles_per_slice = (k_tiles + slices - 1) / slices;
     slices = (k_tiles + p.k_tiles_per_slice - 1) / p.k_tiles_per_slice;
@@ -1413,9 +1447,17 @@ int run_typed(const GemmArgs& g, hipStream_t stream) {
         p.ld_saved = static_cast<long>(g.ld_swiglu);
         p.inter = static_cast<int>(g.n);
     }
+    if (g.batch_rows != 0) {
+        if (!gemm_takes_batch(g)) return fail(CGPTX_INVALID_ARGUMENT, "gemm: this call cannot be a stack of products");
+        p.batch_rows = static_cast<int>(g.batch_rows);
+        p.a_batch_stride = static_cast<long>(g.a_batch_stride);
+        p.b_batch_stride = static_cast<long>(g.b_batch_stride);
+        for (int s = 0; s < 3; ++s) p.a_seg_batch_stride[s] = static_cast<long>(g.a_segment_batch_stride[s]);
+    }
     const bool segmented = g.a_segments.count > 0 || g.c_segments.count > 0;
     if (segmented) {
-        if (int s = copy_segments(g.a_segments, g.a_k_contiguous ? g.k : g.m, g.a_k_contiguous ? kBK : 256, p.a_seg))
+        if (int s = copy_segments(g.a_segments, g.a_k_contiguous ? g.k : (g.batch_rows != 0 ? g.batch_rows : g.m),
+                                  g.a_k_contiguous ? kBK : 256, p.a_seg))
             return s;
         if (int s = copy_segments(g.c_segments, g.n, 256, p.c_seg)) return s;
         if (g.c_segments.count > 0 && (g.c_is_f32 || g.residual != nullptr))
@@ -1444,6 +1486,7 @@ int run_typed(const GemmArgs& g, hipStream_t stream) {
                !(!g.a_k_contiguous && g.b_k_contiguous) && offsets_fit_32bit(g, sizeof(T));
     }
     if (!fast && segmented) return fail(CGPTX_INVALID_ARGUMENT, "gemm: segmented operands need the aligned MFMA path");
+    if (!fast && g.batch_rows != 0) return fail(CGPTX_INVALID_ARGUMENT, "gemm: a stack of products needs the aligned MFMA path");
     if (!fast) {
         const dim3 grid(static_cast<unsigned int>((g.n + kF32Tile - 1) / kF32Tile),
                         static_cast<unsigned int>((g.m + kF32Tile - 1) / kF32Tile));
@@ -1465,7 +1508,8 @@ int run_typed(const GemmArgs& g, hipStream_t stream) {
         const bool splits = (!g.no_split || g.split_workspace != nullptr) && g.residual == nullptr && g.addend_f32 == nullptr &&
                             g.c_segments.count == 0 && big_tiles >= 8 &&
                             g.k / kBK >= static_cast<std::size_t>(32 * ((units + big_tiles - 1) / big_tiles));
-        const bool big = g.swiglu_out != nullptr || g.swiglu_saved != nullptr || forced == 256 || (forced == 0 && (fills || splits));
+        const bool big = g.swiglu_out != nullptr || g.swiglu_saved != nullptr || g.batch_rows != 0 || forced == 256 ||
+                         (forced == 0 && (fills || splits));
         if (big) return run_config<T, 256, 256>(g, p, stream);
         return run_config<T, 128, 128>(g, p, stream);
     }
@@ -1508,6 +1552,21 @@ bool gemm_fuses_swiglu_gradient(const GemmArgs& g) {
     if (forced_tile() == 128 || tiles * 5 < static_cast<long>(compute_units()) * 4) return false;
     constexpr std::size_t limit = (std::size_t{1} << 31) - (std::size_t{1} << 20);
     return offsets_fit_32bit(g, elem) && 256 * g.ld_swiglu * elem < limit;
+}
+
+bool gemm_takes_batch(const GemmArgs& g) {
+    if (g.batch_rows == 0) return true;
+    if (g.dtype == CGPTX_F32 || g.a_k_contiguous || g.b_k_contiguous || g.bias != nullptr || g.residual != nullptr ||
+        g.addend_f32 != nullptr || g.accumulate || g.c_is_f32 || g.c_segments.count > 0 || g.swiglu_out != nullptr ||
+        g.swiglu_saved != nullptr || g.no_split || g.c == nullptr || g.b == nullptr)
+        return false;
+    if (g.batch_rows % 256 != 0 || g.m % g.batch_rows != 0 || g.n % 8 != 0 || g.k % kBK != 0 || g.ldb % 8 != 0 ||
+        g.ldc % 8 != 0 || g.b_batch_stride % 8 != 0)
+        return false;
+    if (g.a_segments.count == 0) return g.a != nullptr && g.lda % 8 == 0 && g.a_batch_stride % 8 == 0;
+    for (int s = 0; s < g.a_segments.count && s < 3; ++s)
+        if (g.a_segment_batch_stride[s] % 8 != 0) return false;
+    return true;
 }
 
 int gemm(const GemmArgs& g, hipStream_t stream) {

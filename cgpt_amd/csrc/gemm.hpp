@@ -59,11 +59,22 @@ struct GemmArgs {
     // applied (the bits of the two separate operators). Only for calls that
     // gemm_fuses_swiglu_gradient() accepts.
     const void* swiglu_saved = nullptr;
+    // Several products of one shape in one launch (weight gradients of equal layers): C is the stack of their results,
+    // [m, n] with m = batch x batch_rows, and the rows batch_rows j .. batch_rows (j + 1) - 1 of it are
+    // A_j^T B_j with A_j = a + j a_batch_stride and B_j = b + j b_batch_stride (elements; for a segmented A every
+    // segment moves by its own stride). Only for the layout of a weight gradient (neither operand k-contiguous),
+    // 16-bit storage and batch_rows a multiple of 256; batch_rows = 0: one product. Only for calls that
+    // gemm_takes_batch() accepts.
+    std::size_t batch_rows = 0;
+    std::size_t a_batch_stride = 0, b_batch_stride = 0;
+    std::size_t a_segment_batch_stride[3] = {0, 0, 0};
 };
 
 int gemm(const GemmArgs& args, hipStream_t stream);
 // Whether gemm() serves args.swiglu_out for this call (shape, layout and alignment of the fused kernel).
 bool gemm_fuses_swiglu(const GemmArgs& args);
 bool gemm_fuses_swiglu_gradient(const GemmArgs& args);
+// Whether gemm() serves args.batch_rows for this call.
+bool gemm_takes_batch(const GemmArgs& args);
 
 }  // namespace cgptx

@@ -109,6 +109,49 @@ extern "C" int cgptx_linear_swiglu_backward(void* grad_gate_up, void* grad_activ
     return cgptx_swiglu_backward_packed(grad_gate_up, grad_activated, gate_up, rows, hidden, 0, dtype, stream_);
 }
 
+extern "C" int cgptx_linear_backward_weights_stacked(void* grad_weight, const void* grad_output, const void* input,
+                                                     size_t rows, size_t in_features, size_t out_features,
+                                                     size_t count, size_t grad_output_stride, size_t input_stride,
+                                                     int dtype, cgptx_stream stream_) {
+    using namespace cgptx;
+    if (int s = validate("linear_backward_weights_stacked", rows, in_features, out_features, dtype)) return s;
+    if (grad_weight == nullptr || grad_output == nullptr || input == nullptr)
+        return fail(CGPTX_INVALID_ARGUMENT, "linear_backward_weights_stacked: null tensor");
+    if (count == 0) return fail(CGPTX_INVALID_ARGUMENT, "linear_backward_weights_stacked: empty stack");
+    if (count > static_cast<std::size_t>(std::numeric_limits<int>::max()) / out_features)
+        return fail(CGPTX_OVERFLOW, "linear_backward_weights_stacked: dimension exceeds int range");
+    auto stream = static_cast<hipStream_t>(stream_);
+    GemmArgs g;  // rows j out .. (j + 1) out - 1 of dW = dY_jᵀ[out, rows] · X_j[rows, in]
+    g.a = grad_output;
+    g.b = input;
+    g.c = grad_weight;
+    g.m = count * out_features;
+    g.n = in_features;
+    g.k = rows;
+    g.lda = out_features;
+    g.ldb = in_features;
+    g.ldc = in_features;
+    g.a_k_contiguous = false;
+    g.b_k_contiguous = false;
+    g.dtype = dtype;
+    g.batch_rows = out_features;
+    g.a_batch_stride = grad_output_stride;
+    g.b_batch_stride = input_stride;
+    if (count > 1 && gemm_takes_batch(g) && is_aligned16(grad_output) && is_aligned16(input) && is_aligned16(grad_weight) &&
+        rows % 32 == 0)
+        return gemm(g, stream);
+    // Shapes the stacked launch does not take: one weight gradient after the other.
+    const std::size_t elem = dtype_size(dtype);
+    for (std::size_t j = 0; j < count; ++j) {
+        if (int s = cgptx_linear_backward(nullptr, static_cast<char*>(grad_weight) + j * out_features * in_features * elem,
+                                          nullptr, static_cast<const char*>(grad_output) + j * grad_output_stride * elem,
+                                          static_cast<const char*>(input) + j * input_stride * elem, nullptr, rows,
+                                          in_features, out_features, 0, 0, 0, dtype, stream_))
+            return s;
+    }
+    return CGPTX_OK;
+}
+
 extern "C" int cgptx_linear_backward(void* grad_input, void* grad_weight, void* grad_bias, const void* grad_output,
                                      const void* input, const void* weight, size_t rows, size_t in_features,
                                      size_t out_features, int accumulate_input, int accumulate_weight,

@@ -110,6 +110,19 @@ struct cgptx_model {
     void *d_normalized = nullptr, *grad_a = nullptr, *grad_b = nullptr, *d_act = nullptr, *d_gate_up = nullptr,
          *d_norm_in = nullptr, *d_norm_in_f = nullptr, *d_attn_out = nullptr, *d_q = nullptr,
          *d_k = nullptr, *d_v = nullptr, *d_q_pre = nullptr, *d_k_pre = nullptr;
+    // Weight gradients of the projections for all layers at once, at the end of the backward pass (stacked_dw): what
+    // those four launches read and write lies layer after layer in one block per tensor kind, and the backward pass
+    // keeps every layer's output gradients instead of reusing one set of buffers.
+    struct Stack {
+        char* base = nullptr;
+        std::size_t stride = 0;  // bytes from one layer to the next
+        void* at(std::size_t layer) const { return base + layer * stride; }
+    };
+    bool stacked_dw = false;
+    Stack qkv_gradients, o_gradients, gate_up_gradients, down_gradients;  // [layers][out, in], no gaps
+    Stack norm_a_all, attn_out_all, norm_f_all, act_all;                  // the forward's inputs of those projections
+    Stack d_hidden_all;                                                   // layers + 1 residual-stream gradients
+    Stack d_gate_up_all, d_q_all, d_k_all, d_v_all;
     cgptx_adamw_workspace* optimizer = nullptr;
     std::uint64_t initial_step = 0;  // step count the optimizer workspace starts from when it is first used
     std::vector<cgptx_adamw_entry> entries;
@@ -330,6 +343,54 @@ int qkv_backward_weight(void* qkv_gradient, const void* dq, const void* dk, cons
     g.b = x;
     g.c = qkv_gradient;
     g.m = QW + 2 * KW;
+    g.n = H;
+    g.k = rows;
+    g.ldb = H;
+    g.ldc = H;
+    g.a_k_contiguous = false;
+    g.b_k_contiguous = false;
+    g.dtype = dt;
+    return gemm(g, stream);
+}
+
+// Whether the projections' weight gradients of all layers run as four launches at the end of the backward pass
+// instead of four per layer (CGPTX_STACK_DW=0 keeps them per layer, for comparisons). One layer's weight
+// gradients have far fewer tiles than the chip has compute units, so each of them splits its sum over the rows into
+// partial tiles that a second launch adds up; the layers' tiles together fill the chip several times over and
+// (almost) nothing is split. Needs 16-bit storage, tile-aligned weight shapes and at least two layers; costs the
+// memory of every layer's output gradients.
+bool stackable_weight_gradients(const cgptx_model_config& c, std::size_t rows) {
+    const char* text = std::getenv("CGPTX_STACK_DW");  // read when the model is created
+    if (text != nullptr && text[0] == '0') return false;
+    const std::size_t H = c.hidden_size, I = c.intermediate_size;
+    const std::size_t QW = c.num_query_heads * c.head_dim, KW = c.num_kv_heads * c.head_dim;
+    return c.dtype != CGPTX_F32 && c.num_layers >= 2 && rows % 32 == 0 && H % 256 == 0 && QW % 256 == 0 && KW % 256 == 0 &&
+           (2 * I) % 256 == 0 && I % 8 == 0;
+}
+
+// Rows j out .. of grad_weights = dY_jᵀ·X_j for every layer j: see cgptx_linear_backward_weights_stacked.
+int stacked_weight_gradients(const cgptx_model::Stack& grad_weights, const void* dy, std::size_t dy_stride_bytes,
+                             const cgptx_model::Stack& x, std::size_t rows, std::size_t in_features, std::size_t out_features,
+                             std::size_t layers, int dt, hipStream_t stream) {
+    const std::size_t elem = dtype_size(dt);
+    return cgptx_linear_backward_weights_stacked(grad_weights.base, dy, x.base, rows, in_features, out_features, layers,
+                                                 dy_stride_bytes / elem, x.stride / elem, dt, static_cast<cgptx_stream>(stream));
+}
+
+// [dWq; dWk; dWv] = [dq | dk | dv]ᵀ·X for every layer in one launch.
+int stacked_qkv_weight_gradients(const cgptx_model* m, std::size_t rows, std::size_t H, std::size_t QW, std::size_t KW, int dt,
+                                 hipStream_t stream) {
+    const std::size_t elem = dtype_size(dt);
+    GemmArgs g;
+    g.a_segments = qkv_segments(m->d_q_all.base, m->d_k_all.base, m->d_v_all.base, QW, KW);
+    g.a_segment_batch_stride[0] = m->d_q_all.stride / elem;
+    g.a_segment_batch_stride[1] = m->d_k_all.stride / elem;
+    g.a_segment_batch_stride[2] = m->d_v_all.stride / elem;
+    g.b = m->norm_a_all.base;
+    g.b_batch_stride = m->norm_a_all.stride / elem;
+    g.c = m->qkv_gradients.base;
+    g.batch_rows = QW + 2 * KW;
+    g.m = m->config.num_layers * (QW + 2 * KW);
     g.n = H;
     g.k = rows;
     g.ldb = H;
@@ -660,8 +721,12 @@ int enqueue_forward_backward(cgptx_model* m, float loss_scale, int loss_mode, hi
     }
 
     // ----------------------------------------------------------------- backward
-    void* current = m->grad_a;
-    void* previous = m->grad_b;
+    // With the weight gradients left to the end, layer l keeps its output gradients: the residual stream's in slot
+    // l + 1 of d_hidden_all (slot l receives the block's input gradient), [dgate | dup], dq, dk and dv in slot l of
+    // their stacks. Otherwise one set of buffers serves every layer.
+    const bool stacked = m->stacked_dw && fused_qkv;
+    void* current = stacked ? m->d_hidden_all.at(c.num_layers) : m->grad_a;
+    void* previous = stacked ? nullptr : m->grad_b;
     ColumnReduceSink* sink = norm_reduction_sink(m);
     m->norm_reductions.begin();
     CGPTX_OP("rmsnorm_bwd", rmsnorm_backward_residual(current, m->final_norm.gradient, m->d_normalized, last, m->final_norm.value,
@@ -670,13 +735,21 @@ int enqueue_forward_backward(cgptx_model* m, float loss_scale, int loss_mode, hi
         const auto& w = m->layers[reverse];
         const auto& a = m->acts[reverse];
         void* x = m->hidden[reverse];
+        void* d_gate_up = stacked ? m->d_gate_up_all.at(reverse) : m->d_gate_up;
+        void* d_q = stacked ? m->d_q_all.at(reverse) : m->d_q;
+        void* d_k = stacked ? m->d_k_all.at(reverse) : m->d_k;
+        void* d_v = stacked ? m->d_v_all.at(reverse) : m->d_v;
+        if (stacked) previous = m->d_hidden_all.at(reverse);
         if (fused_swiglu() && fused_swiglu_gradient()) {
             // The SwiGLU gradient rides in the epilogue of the down projection's input gradient.
-            CGPTX_OP("gemm_dx.down", cgptx_linear_swiglu_backward(m->d_gate_up, m->d_act, current, w.down.value, a.gate_up, N, I, H, dt, s));
-            CGPTX_OP("gemm_dw.down", cgptx_linear_backward(nullptr, w.down.gradient, nullptr, current, a.act, w.down.value, N, I, H, 0, 0, 0, dt, s));
+            CGPTX_OP("gemm_dx.down", cgptx_linear_swiglu_backward(d_gate_up, m->d_act, current, w.down.value, a.gate_up, N, I, H, dt, s));
+            if (!stacked)
+                CGPTX_OP("gemm_dw.down", cgptx_linear_backward(nullptr, w.down.gradient, nullptr, current, a.act, w.down.value, N, I, H, 0, 0, 0, dt, s));
         } else {
-            CGPTX_TRY(linear_backward_split(m, m->d_act, w.down.gradient, current, a.act, w.down.value, N, I, H, 0, dt, stream, "gemm_dx.down", "gemm_dw.down"));
-            CGPTX_OP("swiglu_bwd", cgptx_swiglu_backward_packed(m->d_gate_up, m->d_act, a.gate_up, N, I, 0, dt, s));
+            CGPTX_OP("gemm_dx.down", cgptx_linear_backward(m->d_act, nullptr, nullptr, current, a.act, w.down.value, N, I, H, 0, 0, 0, dt, s));
+            if (!stacked)
+                CGPTX_OP("gemm_dw.down", cgptx_linear_backward(nullptr, w.down.gradient, nullptr, current, a.act, w.down.value, N, I, H, 0, 0, 0, dt, s));
+            CGPTX_OP("swiglu_bwd", cgptx_swiglu_backward_packed(d_gate_up, m->d_act, a.gate_up, N, I, 0, dt, s));
         }
         // The gradient of the residual stream collects the two norm branches: in one pass at the end of
         // the block when the shape allows (previous = current + d(ffn norm) + d(attention norm)), else as
@@ -684,38 +757,42 @@ int enqueue_forward_backward(cgptx_model* m, float loss_scale, int loss_mode, hi
         const bool dual_norms = fused_block_norms(m, previous, m->d_norm_in, m->d_norm_in_f, x, current) &&
                                 is_aligned16(w.attention_norm.value) && is_aligned16(w.ffn_norm.value);
         void* d_norm_f = dual_norms ? m->d_norm_in_f : m->d_norm_in;
-        CGPTX_TRY(linear_backward_split(m, d_norm_f, w.gate.gradient, m->d_gate_up, a.norm_f, w.gate.value, N, H, 2 * I, 0, dt, stream,
-                                        "gemm_dx.gate_up", "gemm_dw.gate_up"));
+        CGPTX_OP("gemm_dx.gate_up", cgptx_linear_backward(d_norm_f, nullptr, nullptr, d_gate_up, a.norm_f, w.gate.value, N, H, 2 * I, 0, 0, 0, dt, s));
+        if (!stacked)
+            CGPTX_OP("gemm_dw.gate_up", cgptx_linear_backward(nullptr, w.gate.gradient, nullptr, d_gate_up, a.norm_f, w.gate.value, N, H, 2 * I, 0, 0, 0, dt, s));
         if (!dual_norms) {
             CGPTX_OP("rmsnorm_bwd", rmsnorm_backward_residual(previous, w.ffn_norm.gradient, m->d_norm_in, x, w.ffn_norm.value,
                                                               current, N, H, eps, dt, stream, sink));
         }
-        CGPTX_TRY(linear_backward_split(m, m->d_attn_out, w.o.gradient, current, a.attn_out, w.o.value, N, QW, H, 0, dt, stream, "gemm_dx.o", "gemm_dw.o"));
-        CGPTX_OP("attn_bwd", cgptx_flash_gqa_attention_backward_with_lse(m->d_q, m->d_k, m->d_v, m->d_attn_out, a.attn_out,
+        CGPTX_OP("gemm_dx.o", cgptx_linear_backward(m->d_attn_out, nullptr, nullptr, current, a.attn_out, w.o.value, N, QW, H, 0, 0, 0, dt, s));
+        if (!stacked)
+            CGPTX_OP("gemm_dw.o", cgptx_linear_backward(nullptr, w.o.gradient, nullptr, current, a.attn_out, w.o.value, N, QW, H, 0, 0, 0, dt, s));
+        CGPTX_OP("attn_bwd", cgptx_flash_gqa_attention_backward_with_lse(d_q, d_k, d_v, m->d_attn_out, a.attn_out,
                                                               a.lse, a.q, a.k, a.v, m->batch, m->sequence,
                                                               m->sequence, HQ, HKV, D, 0.0f, 1, 0, 0, dt, s));
         // In place over the attention gradients (a lane reads and writes the same elements).
-        if (fused_qk_norm_rope(m, m->d_q, m->d_q, a.q_pre, w.q_norm.value) &&
-            fused_qk_norm_rope(m, m->d_k, m->d_k, a.k_pre, w.k_norm.value)) {
-            CGPTX_OP("rmsnorm_bwd", rmsnorm_rope_backward(m->d_q, w.q_norm.gradient, m->d_q, a.q_pre, w.q_norm.value, m->cos_cache,
+        if (fused_qk_norm_rope(m, d_q, d_q, a.q_pre, w.q_norm.value) &&
+            fused_qk_norm_rope(m, d_k, d_k, a.k_pre, w.k_norm.value)) {
+            CGPTX_OP("rmsnorm_bwd", rmsnorm_rope_backward(d_q, w.q_norm.gradient, d_q, a.q_pre, w.q_norm.value, m->cos_cache,
                                                           m->sin_cache, N * HQ, D, HQ, m->sequence, c.rotary_dim, 0, eps, dt, stream, sink));
-            CGPTX_OP("rmsnorm_bwd", rmsnorm_rope_backward(m->d_k, w.k_norm.gradient, m->d_k, a.k_pre, w.k_norm.value, m->cos_cache,
+            CGPTX_OP("rmsnorm_bwd", rmsnorm_rope_backward(d_k, w.k_norm.gradient, d_k, a.k_pre, w.k_norm.value, m->cos_cache,
                                                           m->sin_cache, N * HKV, D, HKV, m->sequence, c.rotary_dim, 0, eps, dt, stream, sink));
         } else {
-            CGPTX_OP("rope_bwd", cgptx_rope_backward(m->d_q_pre, m->d_k_pre, m->d_q, m->d_k, m->cos_cache, m->sin_cache, m->batch,
+            CGPTX_OP("rope_bwd", cgptx_rope_backward(m->d_q_pre, m->d_k_pre, d_q, d_k, m->cos_cache, m->sin_cache, m->batch,
                                           m->sequence, HQ, HKV, D, c.rotary_dim, 0, m->sequence, dt, s));
-            CGPTX_OP("rmsnorm_bwd", rmsnorm_backward_residual(m->d_q, w.q_norm.gradient, m->d_q_pre, a.q_pre, w.q_norm.value, nullptr,
+            CGPTX_OP("rmsnorm_bwd", rmsnorm_backward_residual(d_q, w.q_norm.gradient, m->d_q_pre, a.q_pre, w.q_norm.value, nullptr,
                                                               N * HQ, D, eps, dt, stream, sink));
-            CGPTX_OP("rmsnorm_bwd", rmsnorm_backward_residual(m->d_k, w.k_norm.gradient, m->d_k_pre, a.k_pre, w.k_norm.value, nullptr,
+            CGPTX_OP("rmsnorm_bwd", rmsnorm_backward_residual(d_k, w.k_norm.gradient, m->d_k_pre, a.k_pre, w.k_norm.value, nullptr,
                                                               N * HKV, D, eps, dt, stream, sink));
         }
         if (fused_qkv) {
-            CGPTX_OP("gemm_dx.qkv", qkv_backward_input(m->d_norm_in, m->d_q, m->d_k, m->d_v, w.q.value, N, H, QW, KW, dt, stream));
-            CGPTX_OP("gemm_dw.qkv", qkv_backward_weight(w.q.gradient, m->d_q, m->d_k, m->d_v, a.norm_a, N, H, QW, KW, dt, stream));
+            CGPTX_OP("gemm_dx.qkv", qkv_backward_input(m->d_norm_in, d_q, d_k, d_v, w.q.value, N, H, QW, KW, dt, stream));
+            if (!stacked)
+                CGPTX_OP("gemm_dw.qkv", qkv_backward_weight(w.q.gradient, d_q, d_k, d_v, a.norm_a, N, H, QW, KW, dt, stream));
         } else {
-            CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.q.gradient, m->d_q, a.norm_a, w.q.value, N, H, QW, 0, dt, stream, "gemm_dx.qkv", "gemm_dw.qkv"));
-            CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.k.gradient, m->d_k, a.norm_a, w.k.value, N, H, KW, 1, dt, stream, "gemm_dx.qkv", "gemm_dw.qkv"));
-            CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.v.gradient, m->d_v, a.norm_a, w.v.value, N, H, KW, 1, dt, stream, "gemm_dx.qkv", "gemm_dw.qkv"));
+            CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.q.gradient, d_q, a.norm_a, w.q.value, N, H, QW, 0, dt, stream, "gemm_dx.qkv", "gemm_dw.qkv"));
+            CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.k.gradient, d_k, a.norm_a, w.k.value, N, H, KW, 1, dt, stream, "gemm_dx.qkv", "gemm_dw.qkv"));
+            CGPTX_TRY(linear_backward_split(m, m->d_norm_in, w.v.gradient, d_v, a.norm_a, w.v.value, N, H, KW, 1, dt, stream, "gemm_dx.qkv", "gemm_dw.qkv"));
         }
         if (dual_norms) {
             CGPTX_OP("rmsnorm_bwd", rmsnorm_backward_dual(previous, w.attention_norm.gradient, w.ffn_norm.gradient, m->d_norm_in,
@@ -725,7 +802,18 @@ int enqueue_forward_backward(cgptx_model* m, float loss_scale, int loss_mode, hi
             CGPTX_OP("rmsnorm_bwd", rmsnorm_backward_residual(previous, w.attention_norm.gradient, m->d_norm_in, x,
                                                               w.attention_norm.value, previous, N, H, eps, dt, stream, sink));
         }
-        std::swap(current, previous);
+        if (stacked) current = previous;
+        else std::swap(current, previous);
+    }
+    if (stacked) {
+        // Layer l's output projections read the residual stream's gradient at the block's output: slot l + 1.
+        const std::size_t L = c.num_layers;
+        const void* d_out = m->d_hidden_all.at(1);
+        CGPTX_OP("gemm_dw.down", stacked_weight_gradients(m->down_gradients, d_out, m->d_hidden_all.stride, m->act_all, N, I, H, L, dt, stream));
+        CGPTX_OP("gemm_dw.gate_up", stacked_weight_gradients(m->gate_up_gradients, m->d_gate_up_all.base, m->d_gate_up_all.stride,
+                                                             m->norm_f_all, N, H, 2 * I, L, dt, stream));
+        CGPTX_OP("gemm_dw.o", stacked_weight_gradients(m->o_gradients, d_out, m->d_hidden_all.stride, m->attn_out_all, N, QW, H, L, dt, stream));
+        CGPTX_OP("gemm_dw.qkv", stacked_qkv_weight_gradients(m, N, H, QW, KW, dt, stream));
     }
     // Tied embedding: the classifier gradient is already in place; add the lookup's gradient
     // (src/core/transformer_model.cu:375-380).
@@ -791,6 +879,35 @@ extern "C" int cgptx_model_create(cgptx_model** out, const cgptx_model_config* c
         CGPTX_TRY(make_parameter(m, m->final_norm, "model.norm.weight", H, 1, 0.0f, seed, 1));
         m->layers.resize(c.num_layers);
         m->acts.resize(c.num_layers);
+        m->stacked_dw = stackable_weight_gradients(c, N);
+        if (m->stacked_dw) {
+            const std::size_t L = c.num_layers;
+            auto stack = [&](cgptx_model::Stack& st, std::size_t bytes, std::size_t count) -> int {
+                st.stride = bytes;
+                return allocate_typed(m, &st.base, bytes * count);
+            };
+            CGPTX_TRY(stack(m->qkv_gradients, (QW + 2 * KW) * H * elem, L));
+            CGPTX_TRY(stack(m->o_gradients, H * QW * elem, L));
+            CGPTX_TRY(stack(m->gate_up_gradients, 2 * I * H * elem, L));
+            CGPTX_TRY(stack(m->down_gradients, H * I * elem, L));
+            CGPTX_TRY(stack(m->norm_a_all, N * H * elem, L));
+            CGPTX_TRY(stack(m->attn_out_all, N * QW * elem, L));
+            CGPTX_TRY(stack(m->norm_f_all, N * H * elem, L));
+            CGPTX_TRY(stack(m->act_all, N * I * elem, L));
+            CGPTX_TRY(stack(m->d_hidden_all, N * H * elem, L + 1));
+            CGPTX_TRY(stack(m->d_gate_up_all, N * 2 * I * elem, L));
+            CGPTX_TRY(stack(m->d_q_all, N * QW * elem, L));
+            CGPTX_TRY(stack(m->d_k_all, N * KW * elem, L));
+            CGPTX_TRY(stack(m->d_v_all, N * KW * elem, L));
+        }
+        // A tensor of layer l: its slot in the stack of its kind, or an allocation of its own.
+        auto place = [&](void** out, const cgptx_model::Stack& st, std::size_t l, std::size_t bytes) -> int {
+            if (m->stacked_dw) {
+                *out = st.at(l);
+                return CGPTX_OK;
+            }
+            return allocate(m, out, bytes);
+        };
         for (std::size_t l = 0; l < c.num_layers; ++l) {
             auto& w = m->layers[l];
             const std::string prefix = "model.layers." + std::to_string(l) + ".";
@@ -798,9 +915,11 @@ extern "C" int cgptx_model_create(cgptx_model** out, const cgptx_model_config* c
             CGPTX_TRY(make_parameter(m, w.attention_norm, prefix + "input_layernorm.weight", H, 1, 0, seed, id));
             // q, k and v share one [QW + 2 KW, H] block (values and gradients): the three projections of
             // the normalized input run as one contraction whose output columns go to three buffers.
-            char *qkv_value = nullptr, *qkv_gradient = nullptr;
+            char* qkv_value = nullptr;
+            void* qkv_gradient_slot = nullptr;
             CGPTX_TRY(allocate_typed(m, &qkv_value, (QW + 2 * KW) * H * elem));
-            CGPTX_TRY(allocate_typed(m, &qkv_gradient, (QW + 2 * KW) * H * elem));
+            CGPTX_TRY(place(&qkv_gradient_slot, m->qkv_gradients, l, (QW + 2 * KW) * H * elem));
+            char* qkv_gradient = static_cast<char*>(qkv_gradient_slot);
             CGPTX_TRY(make_parameter(m, w.q, prefix + "self_attn.q_proj.weight", QW * H, 0, stddev, seed, id + 1, qkv_value,
                                      qkv_gradient));
             CGPTX_TRY(make_parameter(m, w.k, prefix + "self_attn.k_proj.weight", KW * H, 0, stddev, seed, id + 2,
@@ -809,31 +928,37 @@ extern "C" int cgptx_model_create(cgptx_model** out, const cgptx_model_config* c
             CGPTX_TRY(make_parameter(m, w.k_norm, prefix + "self_attn.k_norm.weight", c.head_dim, 1, 0, seed, id + 4));
             CGPTX_TRY(make_parameter(m, w.v, prefix + "self_attn.v_proj.weight", KW * H, 0, stddev, seed, id + 5,
                                      qkv_value + (QW + KW) * H * elem, qkv_gradient + (QW + KW) * H * elem));
-            CGPTX_TRY(make_parameter(m, w.o, prefix + "self_attn.o_proj.weight", H * QW, 0, residual_stddev, seed, id + 6));
+            void* o_gradient = nullptr;
+            if (m->stacked_dw) o_gradient = m->o_gradients.at(l);
+            CGPTX_TRY(make_parameter(m, w.o, prefix + "self_attn.o_proj.weight", H * QW, 0, residual_stddev, seed, id + 6, nullptr,
+                                     o_gradient));
             CGPTX_TRY(make_parameter(m, w.ffn_norm, prefix + "post_attention_layernorm.weight", H, 1, 0, seed, id + 7));
             // gate and up share one [2I, H] block (values and gradients), so that the block's three
             // contractions with them each run as one [.., 2I] product on the packed activations.
             void *gate_up_value = nullptr, *gate_up_gradient = nullptr;
             CGPTX_TRY(allocate(m, &gate_up_value, 2 * I * H * elem));
-            CGPTX_TRY(allocate(m, &gate_up_gradient, 2 * I * H * elem));
+            CGPTX_TRY(place(&gate_up_gradient, m->gate_up_gradients, l, 2 * I * H * elem));
             CGPTX_TRY(make_parameter(m, w.gate, prefix + "mlp.gate_proj.weight", I * H, 0, stddev, seed, id + 8,
                                      gate_up_value, gate_up_gradient));
             CGPTX_TRY(make_parameter(m, w.up, prefix + "mlp.up_proj.weight", I * H, 0, stddev, seed, id + 9,
                                      static_cast<char*>(gate_up_value) + I * H * elem,
                                      static_cast<char*>(gate_up_gradient) + I * H * elem));
-            CGPTX_TRY(make_parameter(m, w.down, prefix + "mlp.down_proj.weight", H * I, 0, residual_stddev, seed, id + 10));
+            void* down_gradient = nullptr;
+            if (m->stacked_dw) down_gradient = m->down_gradients.at(l);
+            CGPTX_TRY(make_parameter(m, w.down, prefix + "mlp.down_proj.weight", H * I, 0, residual_stddev, seed, id + 10, nullptr,
+                                     down_gradient));
             auto& a = m->acts[l];
-            CGPTX_TRY(allocate(m, &a.norm_a, N * H * elem));
+            CGPTX_TRY(place(&a.norm_a, m->norm_a_all, l, N * H * elem));
             CGPTX_TRY(allocate(m, &a.q_pre, N * QW * elem));
             CGPTX_TRY(allocate(m, &a.k_pre, N * KW * elem));
             CGPTX_TRY(allocate(m, &a.q, N * QW * elem));
             CGPTX_TRY(allocate(m, &a.k, N * KW * elem));
             CGPTX_TRY(allocate(m, &a.v, N * KW * elem));
-            CGPTX_TRY(allocate(m, &a.attn_out, N * QW * elem));
+            CGPTX_TRY(place(&a.attn_out, m->attn_out_all, l, N * QW * elem));
             CGPTX_TRY(allocate_typed(m, &a.lse, N * c.num_query_heads * sizeof(float)));
-            CGPTX_TRY(allocate(m, &a.norm_f, N * H * elem));
+            CGPTX_TRY(place(&a.norm_f, m->norm_f_all, l, N * H * elem));
             CGPTX_TRY(allocate(m, &a.gate_up, N * 2 * I * elem));
-            CGPTX_TRY(allocate(m, &a.act, N * I * elem));
+            CGPTX_TRY(place(&a.act, m->act_all, l, N * I * elem));
         }
         m->hidden.resize(c.num_layers + 1);
         for (auto& h : m->hidden) CGPTX_TRY(allocate(m, &h, N * H * elem));

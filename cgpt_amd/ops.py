@@ -563,6 +563,27 @@ def linear_swiglu_backward(grad_gate_up, grad_activated, grad_output, weight, ga
               _ptr(gate_up), grad_output.numel() // out_features, hidden, out_features, _code(grad_output), _stream(stream))
 
 
+def linear_backward_weights_stacked(grad_weight, grad_output, input, stream=None):
+    """The weight gradients of several layers of one shape in one launch: grad_output [count, rows, out], input
+    [count, rows, in], grad_weight [count, out, in] — `count` calls of linear_backward
+    (include/ops/backward/linear_backward.h:36-46) for the weight gradient only."""
+    name = "linear_backward_weights_stacked"
+    _require_device(name, grad_weight)
+    if grad_output.device.type != "cuda" or input.device.type != "cuda":  # layers may be slices of larger blocks
+        raise ValueError(f"{name}: all tensors must be device tensors")
+    _same_dtype(name, grad_weight, grad_output, input)
+    if grad_weight.dim() != 3 or grad_output.dim() != 3 or input.dim() != 3 or \
+            grad_output.shape[0] != grad_weight.shape[0] or input.shape[0] != grad_weight.shape[0] or \
+            grad_output.shape[1] != input.shape[1] or grad_output.shape[2] != grad_weight.shape[1] or \
+            input.shape[2] != grad_weight.shape[2] or not grad_weight.is_contiguous() or \
+            grad_output.stride()[1:] != (grad_output.shape[2], 1) or input.stride()[1:] != (input.shape[2], 1):
+        raise ValueError(f"{name}: incompatible tensors")
+    count, out_features, in_features = grad_weight.shape
+    capi.call("cgptx_linear_backward_weights_stacked", _ptr(grad_weight), _ptr(grad_output), _ptr(input),
+              input.shape[1], in_features, out_features, count, grad_output.stride(0), input.stride(0),
+              _code(grad_output), _stream(stream))
+
+
 def embedding_forward(output, device_token_ids, token_count, weight, stream=None):
     """include/ops/embedding.h."""
     name = "embedding_forward"

@@ -287,6 +287,19 @@ int cgptx_linear_swiglu_backward(void* grad_gate_up, void* grad_activated, const
                                  const void* weight, const void* gate_up, size_t rows,
                                  size_t hidden, size_t out_features, int dtype, cgptx_stream stream);
 
+/* The weight gradients of `count` layers of one shape in one launch — `count` calls of linear_backward
+ * (include/ops/backward/linear_backward.h:36-46) that ask for the weight gradient only, as
+ * src/core/transformer_block.cu:660-745 makes them for every block of a model: layer j reads grad_output +
+ * j * grad_output_stride ([rows, out_features]) and input + j * input_stride ([rows, in_features]), strides in
+ * elements, and writes rows j * out_features .. of grad_weight ([count * out_features, in_features]). One launch
+ * over all layers' tiles fills the chip without splitting the row sum of each product into partial tiles; shapes it
+ * does not take (fp32 storage, out_features not a multiple of 256, unaligned tensors) run as `count` separate
+ * weight gradients. */
+int cgptx_linear_backward_weights_stacked(void* grad_weight, const void* grad_output, const void* input,
+                                          size_t rows, size_t in_features, size_t out_features, size_t count,
+                                          size_t grad_output_stride, size_t input_stride, int dtype,
+                                          cgptx_stream stream);
+
 /* embedding_forward — include/ops/embedding.h. out[t,:] = W[id_t,:]; ids >= vocab give a zero row. */
 int cgptx_embedding_forward(void* output, const uint32_t* token_ids,
                             size_t token_count, const void* weight,

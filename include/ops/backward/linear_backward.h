@@ -31,3 +31,23 @@ inline void linear_backward(Tensor& grad_input, Tensor& grad_weight, Tensor& gra
                                 weight.size(0), options.accumulate_input, options.accumulate_weight,
                                 options.accumulate_bias, dtype_code(input.dtype()), stream));
 }
+
+// The weight gradients of several layers of one shape in one launch: grad_output [count, rows, out], input
+// [count, rows, in], grad_weight [count, out, in], all contiguous — `count` calls of linear_backward that ask for the
+// weight gradient only, as the reference's block backward makes them for every block of a model
+// (src/core/transformer_block.cu:660-745). No single reference function corresponds.
+inline void linear_backward_weights_stacked(Tensor& grad_weight, const Tensor& grad_output, const Tensor& input,
+                                            const GemmContext&, hipStream_t stream = nullptr) {
+    using namespace cgptx_detail;
+    const char* op = "linear_backward_weights_stacked";
+    require_device(op, {&grad_weight, &grad_output, &input});
+    require_same_dtype(op, input, {&grad_weight, &grad_output});
+    if (grad_weight.dim() != 3 || grad_output.dim() != 3 || input.dim() != 3 || grad_output.size(0) != grad_weight.size(0) ||
+        input.size(0) != grad_weight.size(0) || grad_output.size(1) != input.size(1) ||
+        grad_output.size(2) != grad_weight.size(1) || input.size(2) != grad_weight.size(2))
+        throw std::invalid_argument("linear_backward_weights_stacked: incompatible tensors");
+    check(cgptx_linear_backward_weights_stacked(grad_weight.raw_data(), grad_output.raw_data(), input.raw_data(), input.size(1),
+                                                input.size(2), grad_output.size(2), grad_weight.size(0),
+                                                grad_output.size(1) * grad_output.size(2), input.size(1) * input.size(2),
+                                                dtype_code(input.dtype()), stream));
+}

@@ -180,6 +180,59 @@ def test_linear_backward_at_the_32768_training_rows_sampled_against_float64(devi
         check_against_float64(gi[:, in_index], want_dx_cols, dtype, f"dX columns {fout}x{fin}", fout)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32], ids=["bf16", "f16", "f32"])
+@pytest.mark.parametrize("count,rows,fout,fin", [
+    (8, 2048, 256, 512),    # 16 tiles: the launch splits the row sum
+    (3, 1056, 512, 264),    # ragged columns, three slices' worth of K tiles
+    (5, 4096, 768, 1024),   # 60 tiles
+    (40, 1024, 2048, 256),  # 320 tiles: more than one round of the persistent blocks
+    (2, 520, 96, 200),      # out_features not a multiple of 256: separate weight gradients
+    (1, 2048, 256, 512),    # a stack of one
+], ids=["8x256x512", "3x512x264", "5x768x1024", "40x2048x256", "fallback", "single"])
+def test_linear_backward_weights_stacked_matches_float64_and_integers(device, count, rows, fout, fin, dtype):
+    """The weight gradients of several layers in one launch against float64 products (the bound of the single
+    weight gradient), and exact on small integers whatever the number of slices the launch picks."""
+    g = torch.Generator().manual_seed(11)
+    dy = (torch.randn((count, rows, fout), generator=g) * 1.0).to(dtype)
+    x = (torch.randn((count, rows, fin), generator=g) * 1.0).to(dtype)
+    gw = torch.full((count, fout, fin), 7.0, dtype=dtype, device=device)
+    ops.linear_backward_weights_stacked(gw, dev(dy, device), dev(x, device))
+    for j in range(count):
+        want = to_np(dy[j]).T @ to_np(x[j])
+        check_against_float64(gw[j].cpu(), want, dtype, f"dW of layer {j}", rows)
+    # twice, bit-identical
+    again = torch.empty_like(gw)
+    ops.linear_backward_weights_stacked(again, dev(dy, device), dev(x, device))
+    assert torch.equal(gw, again)
+    if dtype != torch.float32:
+        dy = torch.randint(-1, 2, (count, rows, fout), generator=g).to(dtype)
+        x = torch.randint(-2, 3, (count, rows, fin), generator=g).to(dtype)
+        ops.linear_backward_weights_stacked(gw, dev(dy, device), dev(x, device))
+        for j in range(count):
+            want = torch.tensor(to_np(dy[j]).T @ to_np(x[j])).to(dtype)
+            assert np.array_equal(to_np(gw[j]), to_np(want)), f"layer {j}"
+
+
+def test_linear_backward_weights_stacked_with_strided_layers_and_errors(device):
+    """Layers taken out of larger blocks (strides beyond rows x features), and the argument checks."""
+    dtype = torch.bfloat16
+    count, rows, fout, fin = 4, 1024, 256, 256
+    g = torch.Generator().manual_seed(12)
+    dy_block = torch.randn((count, rows + 64, fout), generator=g).to(dtype).to(device)
+    x_block = torch.randn((count, rows + 32, fin), generator=g).to(dtype).to(device)
+    dy, x = dy_block[:, :rows], x_block[:, :rows]
+    gw = torch.empty((count, fout, fin), dtype=dtype, device=device)
+    ops.linear_backward_weights_stacked(gw, dy, x)
+    for j in range(count):
+        check_against_float64(gw[j].cpu(), to_np(dy[j]).T @ to_np(x[j]), dtype, f"dW of layer {j}", rows)
+    with pytest.raises(ValueError):
+        ops.linear_backward_weights_stacked(gw, dy[:3], x)
+    with pytest.raises(ValueError):
+        ops.linear_backward_weights_stacked(gw, dy, x[:, :, :128])
+    with pytest.raises(ValueError):
+        ops.linear_backward_weights_stacked(gw.cpu(), dy, x)
+
+
 def test_linear_argument_errors(device):
     x, w, dy = torch.zeros(4, 8, device=device), torch.zeros(3, 8, device=device), torch.zeros(4, 3, device=device)
     gi, gw, gb = torch.zeros_like(x), torch.zeros_like(w), torch.zeros(3, device=device)

@@ -130,10 +130,16 @@ MODEL_CFG = dict(vocab=96, layers=2, hidden=64, inter=128, hq=2, hkv=1, d=32, ep
 WIDE_CFG = dict(vocab=96, layers=1, hidden=256, inter=128, hq=2, hkv=2, d=128, eps=1e-5)
 
 
+# Three layers with tile-aligned projections (256-wide q, k, v, hidden and [gate | up]) and 64 rows: the shape class in
+# which the projections' weight gradients of all layers run as four launches at the end of the backward pass.
+STACKED_CFG = dict(vocab=96, layers=3, hidden=256, inter=128, hq=2, hkv=2, d=128, eps=1e-5)
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
 @pytest.mark.parametrize("loss_mode", [0, 1], ids=["dense", "cut"])
-@pytest.mark.parametrize("shape", [(MODEL_CFG, 2, 24), (WIDE_CFG, 2, 32)], ids=["heads32", "heads128-fused-qkv"])
+@pytest.mark.parametrize("shape", [(MODEL_CFG, 2, 24), (WIDE_CFG, 2, 32), (STACKED_CFG, 2, 32)],
+                         ids=["heads32", "heads128-fused-qkv", "stacked-weight-gradients"])
 def test_gpu_step_matches_float64_composition(device, dtype, loss_mode, shape):
     """Hidden 64, 2:1 heads of 32, T=24, B=2, two layers (and the wide-head variant above): every parameter
     gradient of the GPU step against the float64 composition that rounds each operator output to the storage
@@ -463,6 +469,55 @@ def test_block_norms_in_one_pass_match_the_separate_operators(device, monkeypatc
         separate = results[1][1][name]
         scale = separate.abs().max().item() + 1e-12
         assert (fused - separate).abs().max().item() <= 2e-2 * scale, name
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+def test_weight_gradients_of_all_layers_in_one_launch_agree_with_the_launches_per_layer(device, monkeypatch, dtype):
+    """Tile-aligned models leave the projections' weight gradients to the end of the backward pass and compute
+    them for all layers at once (CGPTX_STACK_DW=0 keeps one launch per layer and projection). Nothing else
+    changes: loss, activations and every other gradient are bit-identical; the projections' weight gradients are
+    the same sums over the rows taken in a different number of slices, equal to storage precision; eager and
+    recorded passes of the stacked step give the same bits."""
+    from cgpt_amd.model import LOSS_CUT, Model, ModelConfig
+    config = ModelConfig(vocabulary_size=256, num_layers=4, hidden_size=512, intermediate_size=256, num_query_heads=4,
+                         num_kv_heads=2, head_dim=128, rotary_dim=128, dtype=dtype)
+    batch, seq = 2, 96
+    rng = np.random.default_rng(9)
+    inputs = rng.integers(0, 256, size=batch * seq).astype(np.uint32)
+    targets = rng.integers(0, 256, size=batch * seq).astype(np.uint32)
+    results = {}
+    stream = torch.cuda.Stream(device=device)
+    for stack in ("1", "0"):
+        monkeypatch.setenv("CGPTX_STACK_DW", stack)
+        model = Model(config, batch, seq, seed=8, device=device)
+        model.set_tokens(inputs, targets)
+        model.forward_backward(16.0, LOSS_CUT, use_graph=False, stream=stream)
+        stream.synchronize()
+        eager = {n: g.clone() for n, _, g in model.parameters()}
+        for use_graph in (True, True):
+            for _, _, g in model.parameters():
+                g.zero_()
+            torch.cuda.synchronize()
+            model.forward_backward(16.0, LOSS_CUT, use_graph=use_graph, stream=stream)
+            stream.synchronize()
+            for n, _, g in model.parameters():
+                assert torch.equal(g, eager[n]), f"{n}: recorded pass differs from the eager one (stack={stack})"
+        results[stack] = (model.status(stream)[0], eager, model.activation(f"hidden.{config.num_layers}").clone())
+        model.close()
+    assert results["1"][0] == results["0"][0]
+    assert torch.equal(results["1"][2], results["0"][2])
+    projections = ("q_proj", "k_proj", "v_proj", "o_proj", "gate_proj", "up_proj", "down_proj")
+    seen = 0
+    for name, stacked in results["1"][1].items():
+        separate = results["0"][1][name]
+        if any(part in name for part in projections):
+            seen += 1
+            scale = separate.float().abs().max().item() + 1e-12
+            assert (stacked.float() - separate.float()).abs().max().item() <= 1e-2 * scale, name
+        else:
+            assert torch.equal(stacked, separate), name
+    assert seen == 7 * config.num_layers
 
 
 HEADLINE = dict(vocabulary_size=32000, num_layers=8, hidden_size=1024, intermediate_size=2048, num_query_heads=8,
