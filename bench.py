@@ -119,6 +119,9 @@ def gemm_shapes(cfg, batch, seq):
         shapes[f"gemm_fwd.{name}"] = (N, o, i)   # Y[N, out] = X[N, in] W^T
         shapes[f"gemm_dx.{name}"] = (N, i, o)    # dX[N, in] = dY[N, out] W
         shapes[f"gemm_dw.{name}"] = (o, i, N)    # dW[out, in] = dY^T X
+    # The stacked weight gradients pair the q projection with the output projection (one shape) and leave [k; v].
+    shapes["gemm_dw.q_o"] = (QW + H, H, N)
+    shapes["gemm_dw.kv"] = (QKV - QW, H, N)
     return shapes
 
 

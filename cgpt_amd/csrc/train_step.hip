@@ -119,10 +119,20 @@ struct cgptx_model {
         void* at(std::size_t layer) const { return base + layer * stride; }
     };
     bool stacked_dw = false;
-    Stack qkv_gradients, o_gradients, gate_up_gradients, down_gradients;  // [layers][out, in], no gaps
-    Stack norm_a_all, attn_out_all, norm_f_all, act_all;                  // the forward's inputs of those projections
-    Stack d_hidden_all;                                                   // layers + 1 residual-stream gradients
-    Stack d_gate_up_all, d_q_all, d_k_all, d_v_all;
+    // The q and the output projection have one shape ([hidden, hidden], since hidden = query heads x head_dim), and so
+    // have their inputs and output gradients: both projections of all layers form one stack of 2 x layers products —
+    // slot l belongs to layer l's q projection, slot layers + l to its output projection.
+    Stack q_o_gradients, kv_gradients, gate_up_gradients, down_gradients;  // [slots][out, in], no gaps
+    Stack q_o_inputs;    // slot l: attention norm output, slot layers + l: attention output
+    Stack norm_f_all, act_all;
+    // slot l: dq of layer l; slot layers + l: the residual stream's gradient at layer l's output (slot 2 x layers: at
+    // the first layer's input, read by the embedding's gradient)
+    Stack q_o_output_gradients;
+    Stack d_gate_up_all, d_k_all, d_v_all;
+    std::size_t stacked_layers = 0;
+    void* d_hidden_slot(std::size_t index) const {  // gradient of hidden[index]
+        return index == 0 ? q_o_output_gradients.at(2 * stacked_layers) : q_o_output_gradients.at(stacked_layers + index - 1);
+    }
     cgptx_adamw_workspace* optimizer = nullptr;
     std::uint64_t initial_step = 0;  // step count the optimizer workspace starts from when it is first used
     std::vector<cgptx_adamw_entry> entries;
@@ -377,20 +387,23 @@ int stacked_weight_gradients(const cgptx_model::Stack& grad_weights, const void*
                                                  dy_stride_bytes / elem, x.stride / elem, dt, static_cast<cgptx_stream>(stream));
 }
 
-// [dWq; dWk; dWv] = [dq | dk | dv]ᵀ·X for every layer in one launch.
-int stacked_qkv_weight_gradients(const cgptx_model* m, std::size_t rows, std::size_t H, std::size_t QW, std::size_t KW, int dt,
-                                 hipStream_t stream) {
+// [dWk; dWv] = [dk | dv]ᵀ·X for every layer in one launch (dk and dv lie in separate buffers).
+int stacked_kv_weight_gradients(const cgptx_model* m, std::size_t rows, std::size_t H, std::size_t KW, int dt,
+                                hipStream_t stream) {
     const std::size_t elem = dtype_size(dt);
     GemmArgs g;
-    g.a_segments = qkv_segments(m->d_q_all.base, m->d_k_all.base, m->d_v_all.base, QW, KW);
-    g.a_segment_batch_stride[0] = m->d_q_all.stride / elem;
-    g.a_segment_batch_stride[1] = m->d_k_all.stride / elem;
-    g.a_segment_batch_stride[2] = m->d_v_all.stride / elem;
-    g.b = m->norm_a_all.base;
-    g.b_batch_stride = m->norm_a_all.stride / elem;
-    g.c = m->qkv_gradients.base;
-    g.batch_rows = QW + 2 * KW;
-    g.m = m->config.num_layers * (QW + 2 * KW);
+    g.a_segments.count = 2;
+    g.a_segments.ptr[0] = m->d_k_all.base;
+    g.a_segments.ptr[1] = m->d_v_all.base;
+    g.a_segments.ld[0] = g.a_segments.cols[0] = KW;
+    g.a_segments.ld[1] = g.a_segments.cols[1] = KW;
+    g.a_segment_batch_stride[0] = m->d_k_all.stride / elem;
+    g.a_segment_batch_stride[1] = m->d_v_all.stride / elem;
+    g.b = m->q_o_inputs.base;  // slots 0 .. layers - 1: the attention norm's output
+    g.b_batch_stride = m->q_o_inputs.stride / elem;
+    g.c = m->kv_gradients.base;
+    g.batch_rows = 2 * KW;
+    g.m = m->config.num_layers * 2 * KW;
     g.n = H;
     g.k = rows;
     g.ldb = H;
@@ -722,10 +735,10 @@ int enqueue_forward_backward(cgptx_model* m, float loss_scale, int loss_mode, hi
 
     // ----------------------------------------------------------------- backward
     // With the weight gradients left to the end, layer l keeps its output gradients: the residual stream's in slot
-    // l + 1 of d_hidden_all (slot l receives the block's input gradient), [dgate | dup], dq, dk and dv in slot l of
-    // their stacks. Otherwise one set of buffers serves every layer.
+    // own slot (the slot of the block's input receives the block's input gradient), [dgate | dup], dq, dk and dv in slot l
+    // of their stacks. Otherwise one set of buffers serves every layer.
     const bool stacked = m->stacked_dw && fused_qkv;
-    void* current = stacked ? m->d_hidden_all.at(c.num_layers) : m->grad_a;
+    void* current = stacked ? m->d_hidden_slot(c.num_layers) : m->grad_a;
     void* previous = stacked ? nullptr : m->grad_b;
     ColumnReduceSink* sink = norm_reduction_sink(m);
     m->norm_reductions.begin();
@@ -736,10 +749,10 @@ int enqueue_forward_backward(cgptx_model* m, float loss_scale, int loss_mode, hi
         const auto& a = m->acts[reverse];
         void* x = m->hidden[reverse];
         void* d_gate_up = stacked ? m->d_gate_up_all.at(reverse) : m->d_gate_up;
-        void* d_q = stacked ? m->d_q_all.at(reverse) : m->d_q;
+        void* d_q = stacked ? m->q_o_output_gradients.at(reverse) : m->d_q;
         void* d_k = stacked ? m->d_k_all.at(reverse) : m->d_k;
         void* d_v = stacked ? m->d_v_all.at(reverse) : m->d_v;
-        if (stacked) previous = m->d_hidden_all.at(reverse);
+        if (stacked) previous = m->d_hidden_slot(reverse);
         if (fused_swiglu() && fused_swiglu_gradient()) {
             // The SwiGLU gradient rides in the epilogue of the down projection's input gradient.
             CGPTX_OP("gemm_dx.down", cgptx_linear_swiglu_backward(d_gate_up, m->d_act, current, w.down.value, a.gate_up, N, I, H, dt, s));
@@ -806,14 +819,16 @@ int enqueue_forward_backward(cgptx_model* m, float loss_scale, int loss_mode, hi
         else std::swap(current, previous);
     }
     if (stacked) {
-        // Layer l's output projections read the residual stream's gradient at the block's output: slot l + 1.
+        // The down projection reads the residual stream's gradient at each block's output (slots layers .. of the q / output
+        // stack); the q and output projections of all layers are one stack of 2 x layers products.
         const std::size_t L = c.num_layers;
-        const void* d_out = m->d_hidden_all.at(1);
-        CGPTX_OP("gemm_dw.down", stacked_weight_gradients(m->down_gradients, d_out, m->d_hidden_all.stride, m->act_all, N, I, H, L, dt, stream));
+        CGPTX_OP("gemm_dw.down", stacked_weight_gradients(m->down_gradients, m->d_hidden_slot(1), m->q_o_output_gradients.stride,
+                                                          m->act_all, N, I, H, L, dt, stream));
         CGPTX_OP("gemm_dw.gate_up", stacked_weight_gradients(m->gate_up_gradients, m->d_gate_up_all.base, m->d_gate_up_all.stride,
                                                              m->norm_f_all, N, H, 2 * I, L, dt, stream));
-        CGPTX_OP("gemm_dw.o", stacked_weight_gradients(m->o_gradients, d_out, m->d_hidden_all.stride, m->attn_out_all, N, QW, H, L, dt, stream));
-        CGPTX_OP("gemm_dw.qkv", stacked_qkv_weight_gradients(m, N, H, QW, KW, dt, stream));
+        CGPTX_OP("gemm_dw.q_o", stacked_weight_gradients(m->q_o_gradients, m->q_o_output_gradients.base, m->q_o_output_gradients.stride,
+                                                         m->q_o_inputs, N, H, H, 2 * L, dt, stream));
+        CGPTX_OP("gemm_dw.kv", stacked_kv_weight_gradients(m, N, H, KW, dt, stream));
     }
     // Tied embedding: the classifier gradient is already in place; add the lookup's gradient
     // (src/core/transformer_model.cu:375-380).
@@ -886,17 +901,16 @@ extern "C" int cgptx_model_create(cgptx_model** out, const cgptx_model_config* c
                 st.stride = bytes;
                 return allocate_typed(m, &st.base, bytes * count);
             };
-            CGPTX_TRY(stack(m->qkv_gradients, (QW + 2 * KW) * H * elem, L));
-            CGPTX_TRY(stack(m->o_gradients, H * QW * elem, L));
+            m->stacked_layers = L;
+            CGPTX_TRY(stack(m->q_o_gradients, H * H * elem, 2 * L));
+            CGPTX_TRY(stack(m->kv_gradients, 2 * KW * H * elem, L));
             CGPTX_TRY(stack(m->gate_up_gradients, 2 * I * H * elem, L));
             CGPTX_TRY(stack(m->down_gradients, H * I * elem, L));
-            CGPTX_TRY(stack(m->norm_a_all, N * H * elem, L));
-            CGPTX_TRY(stack(m->attn_out_all, N * QW * elem, L));
+            CGPTX_TRY(stack(m->q_o_inputs, N * H * elem, 2 * L));
             CGPTX_TRY(stack(m->norm_f_all, N * H * elem, L));
             CGPTX_TRY(stack(m->act_all, N * I * elem, L));
-            CGPTX_TRY(stack(m->d_hidden_all, N * H * elem, L + 1));
+            CGPTX_TRY(stack(m->q_o_output_gradients, N * H * elem, 2 * L + 1));
             CGPTX_TRY(stack(m->d_gate_up_all, N * 2 * I * elem, L));
-            CGPTX_TRY(stack(m->d_q_all, N * QW * elem, L));
             CGPTX_TRY(stack(m->d_k_all, N * KW * elem, L));
             CGPTX_TRY(stack(m->d_v_all, N * KW * elem, L));
         }
@@ -913,23 +927,31 @@ extern "C" int cgptx_model_create(cgptx_model** out, const cgptx_model_config* c
             const std::string prefix = "model.layers." + std::to_string(l) + ".";
             const std::uint64_t id = 2 + l * 11;
             CGPTX_TRY(make_parameter(m, w.attention_norm, prefix + "input_layernorm.weight", H, 1, 0, seed, id));
-            // q, k and v share one [QW + 2 KW, H] block (values and gradients): the three projections of
-            // the normalized input run as one contraction whose output columns go to three buffers.
-            char* qkv_value = nullptr;
-            void* qkv_gradient_slot = nullptr;
+            // q, k and v share one [QW + 2 KW, H] block of values: the three projections of the normalized input run as
+            // one contraction whose output columns go to three buffers. Their gradients share such a block too when
+            // every layer computes its own weight gradients; with the stacked launches q's lies in the q / output
+            // stack and [k; v]'s in a stack of its own.
+            char *qkv_value = nullptr, *q_gradient = nullptr, *k_gradient = nullptr, *v_gradient = nullptr;
             CGPTX_TRY(allocate_typed(m, &qkv_value, (QW + 2 * KW) * H * elem));
-            CGPTX_TRY(place(&qkv_gradient_slot, m->qkv_gradients, l, (QW + 2 * KW) * H * elem));
-            char* qkv_gradient = static_cast<char*>(qkv_gradient_slot);
+            if (m->stacked_dw) {
+                q_gradient = static_cast<char*>(m->q_o_gradients.at(l));
+                k_gradient = static_cast<char*>(m->kv_gradients.at(l));
+                v_gradient = k_gradient + KW * H * elem;
+            } else {
+                CGPTX_TRY(allocate_typed(m, &q_gradient, (QW + 2 * KW) * H * elem));
+                k_gradient = q_gradient + QW * H * elem;
+                v_gradient = k_gradient + KW * H * elem;
+            }
             CGPTX_TRY(make_parameter(m, w.q, prefix + "self_attn.q_proj.weight", QW * H, 0, stddev, seed, id + 1, qkv_value,
-                                     qkv_gradient));
+                                     q_gradient));
             CGPTX_TRY(make_parameter(m, w.k, prefix + "self_attn.k_proj.weight", KW * H, 0, stddev, seed, id + 2,
-                                     qkv_value + QW * H * elem, qkv_gradient + QW * H * elem));
+                                     qkv_value + QW * H * elem, k_gradient));
             CGPTX_TRY(make_parameter(m, w.q_norm, prefix + "self_attn.q_norm.weight", c.head_dim, 1, 0, seed, id + 3));
             CGPTX_TRY(make_parameter(m, w.k_norm, prefix + "self_attn.k_norm.weight", c.head_dim, 1, 0, seed, id + 4));
             CGPTX_TRY(make_parameter(m, w.v, prefix + "self_attn.v_proj.weight", KW * H, 0, stddev, seed, id + 5,
-                                     qkv_value + (QW + KW) * H * elem, qkv_gradient + (QW + KW) * H * elem));
+                                     qkv_value + (QW + KW) * H * elem, v_gradient));
             void* o_gradient = nullptr;
-            if (m->stacked_dw) o_gradient = m->o_gradients.at(l);
+            if (m->stacked_dw) o_gradient = m->q_o_gradients.at(c.num_layers + l);
             CGPTX_TRY(make_parameter(m, w.o, prefix + "self_attn.o_proj.weight", H * QW, 0, residual_stddev, seed, id + 6, nullptr,
                                      o_gradient));
             CGPTX_TRY(make_parameter(m, w.ffn_norm, prefix + "post_attention_layernorm.weight", H, 1, 0, seed, id + 7));
@@ -948,13 +970,13 @@ extern "C" int cgptx_model_create(cgptx_model** out, const cgptx_model_config* c
             CGPTX_TRY(make_parameter(m, w.down, prefix + "mlp.down_proj.weight", H * I, 0, residual_stddev, seed, id + 10, nullptr,
                                      down_gradient));
             auto& a = m->acts[l];
-            CGPTX_TRY(place(&a.norm_a, m->norm_a_all, l, N * H * elem));
+            CGPTX_TRY(place(&a.norm_a, m->q_o_inputs, l, N * H * elem));
             CGPTX_TRY(allocate(m, &a.q_pre, N * QW * elem));
             CGPTX_TRY(allocate(m, &a.k_pre, N * KW * elem));
             CGPTX_TRY(allocate(m, &a.q, N * QW * elem));
             CGPTX_TRY(allocate(m, &a.k, N * KW * elem));
             CGPTX_TRY(allocate(m, &a.v, N * KW * elem));
-            CGPTX_TRY(place(&a.attn_out, m->attn_out_all, l, N * QW * elem));
+            CGPTX_TRY(place(&a.attn_out, m->q_o_inputs, c.num_layers + l, N * QW * elem));
             CGPTX_TRY(allocate_typed(m, &a.lse, N * c.num_query_heads * sizeof(float)));
             CGPTX_TRY(place(&a.norm_f, m->norm_f_all, l, N * H * elem));
             CGPTX_TRY(allocate(m, &a.gate_up, N * 2 * I * elem));
