@@ -109,6 +109,29 @@ def test_linear_backward_random_shapes(device, seed):
     assert_scaled_close(y, oracle64.linear_forward(to_np(x), to_np(w)), STOL[dtype], "Y")
 
 
+@pytest.mark.parametrize("seed", SEEDS[:24])
+def test_stacked_weight_gradients_random_shapes(device, seed):
+    """Weight gradients of several layers in one call: tile-aligned shapes take the stacked launch (any number of
+    K slices and rounds), the others one weight gradient per layer; layers may be slices of larger blocks."""
+    rng = np.random.default_rng(8000 + seed)
+    dtype = case_dtype(rng)
+    aligned = bool(rng.integers(0, 4))
+    count = int(rng.integers(1, 7))
+    if aligned:
+        rows, fin, fout = int(rng.integers(1, 60)) * 32, int(rng.integers(1, 40)) * 8, int(rng.integers(1, 5)) * 256
+    else:
+        rows, fin, fout = (int(rng.integers(1, 500)) for _ in range(3))
+    extra_rows = int(rng.integers(0, 3)) * 8  # rows of the block a layer is a slice of, beyond the layer's own
+    print(f"stacked dW count={count} rows={rows} in={fin} out={fout} extra_rows={extra_rows} {dtype}", flush=True)
+    dy_block = randn((count, rows + extra_rows, fout), dtype, seed).to(device)
+    x_block = randn((count, rows + extra_rows, fin), dtype, seed + 1).to(device)
+    dy, x = dy_block[:, :rows], x_block[:, :rows]
+    gw = torch.full((count, fout, fin), 5.0, dtype=dtype, device=device)
+    ops.linear_backward_weights_stacked(gw, dy, x)
+    for j in range(count):
+        assert_scaled_close(gw[j], to_np(dy[j]).T @ to_np(x[j]), STOL[dtype], f"dW of layer {j}")
+
+
 @pytest.mark.parametrize("seed", SEEDS)
 def test_attention_random_shapes(device, seed):
     rng = np.random.default_rng(4000 + seed)
