@@ -99,6 +99,15 @@ void linear_backward_known_answers() {
     Tensor wrong = Tensor::zeros({2, 4});
     expect(throws<std::invalid_argument>([&] { linear_backward(wrong, gw, gb, dy, x, w, context); }),
            "linear_backward shape mismatch -> invalid_argument");
+    // The same case as layer 0 of a stack of two, with its negated output gradient as layer 1.
+    Tensor xs = device_f32({2, 2, 3}, {1, 2, 3, 4, 5, 6, 1, 2, 3, 4, 5, 6});
+    Tensor dys = device_f32({2, 2, 2}, {2, -1, 3, 4, -2, 1, -3, -4});
+    Tensor gws = Tensor::zeros({2, 2, 3});
+    linear_backward_weights_stacked(gws, dys, xs, context);
+    expect(close(host_f32(gws), {14, 19, 24, 15, 18, 21, -14, -19, -24, -15, -18, -21}, 0), "linear_backward_weights_stacked");
+    Tensor short_stack = Tensor::zeros({1, 2, 3});
+    expect(throws<std::invalid_argument>([&] { linear_backward_weights_stacked(short_stack, dys, xs, context); }),
+           "linear_backward_weights_stacked mismatched stack -> invalid_argument");
 }
 
 // tests/cross_entropy_test.cu:33-63 — values, gradient scale 1024, target-count mismatch.
